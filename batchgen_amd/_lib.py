@@ -1,0 +1,104 @@
+"""ctypes binding of libbgmoe.so (the C ABI declared in include/bgmoe.h).
+
+There is no fallback: if the library is missing or a symbol is absent the
+import of an op module fails with ImportError / RuntimeError, and every call
+that returns a non-zero status raises RuntimeError with the library's message.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libbgmoe.so")
+
+vp = C.c_void_p
+i32 = C.c_int
+i64 = C.c_int64
+f32 = C.c_float
+sz = C.c_size_t
+
+
+class Fp8Weight(C.Structure):
+    """bgmoe_fp8_weight"""
+    _fields_ = [("w", vp), ("w_group_stride", i64), ("w_ptrs", vp), ("scale", vp),
+                ("scale_group_stride", i64), ("scale_nb_stride", i64), ("scale_ptrs", vp)]
+
+
+class Fp8Act(C.Structure):
+    """bgmoe_fp8_act"""
+    _fields_ = [("x", vp), ("scale", vp), ("scale_row_stride", i64), ("scale_kb_stride", i64)]
+
+
+_SIGS = {
+    "bgmoe_last_error": (C.c_char_p, []),
+    "bgmoe_version": (i32, []),
+    "bgmoe_fused_gate": (i32, [vp, vp, i32, i32, i32, i32, i32, f32, i32, vp, vp, vp]),
+    "bgmoe_gate_sigmoid_topk": (i32, [vp, i64, vp, i32, i32, i32, f32, vp, i32, vp, vp, vp, i32, vp, i32, i32, vp]),
+    "bgmoe_act_quant_rows": (i32, [vp, i64, i32, vp, vp, i64, i64, vp]),
+    "bgmoe_act_quant_3d": (i32, [vp, vp, i32, i32, i32, vp, vp, vp]),
+    "bgmoe_act_quant_ragged": (i32, [vp, vp, vp, i32, i64, i32, vp, vp, i32, vp]),
+    "bgmoe_silu_mul_3d": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
+    "bgmoe_fused_silu_quant_3d": (i32, [vp, vp, vp, i32, i32, i32, vp, vp, vp]),
+    "bgmoe_dispatch_workspace_bytes": (sz, [i64, i32]),
+    "bgmoe_dispatch_scatter_3d": (i32, [vp, vp, i32, i32, i32, vp, i32, i32, i32, vp, vp, vp, vp, sz, vp]),
+    "bgmoe_dispatch_scatter_ragged": (i32, [vp, vp, i32, i32, i32, vp, i64, i32, i32, vp, vp, vp, vp, i32, vp, sz, vp]),
+    "bgmoe_scatter_quant": (i32, [vp, vp, i32, i32, i32, vp, vp, i64, i64, vp]),
+    "bgmoe_reduce_weighted_scatter": (i32, [vp, vp, vp, i32, i32, i32, vp, i32, vp, i32, vp]),
+    "bgmoe_reduce_weighted_scatter_fp32": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
+    "bgmoe_reduce_weighted_scatter_bf16_ordered": (i32, [vp, vp, vp, vp, i32, i32, i32, vp, vp]),
+    "bgmoe_compact_expert_data": (i32, [vp, i32, vp, vp, vp, vp, vp]),
+    "bgmoe_fp8_grouped_gemm": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), vp, vp, i32, i64, i32, i32, vp, vp]),
+    "bgmoe_fp8_fused_s1": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), C.POINTER(Fp8Weight), vp, vp, i32,
+                                 i64, i32, i32, vp, vp, vp, i64, i64, vp]),
+}
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is not built; run `python -m batchgen_amd.build` "
+                "(hipcc, gfx950). There is no CPU fallback.")
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGS.items():
+            try:
+                fn = getattr(handle, name)
+            except AttributeError as exc:
+                raise RuntimeError(f"libbgmoe.so has no symbol {name}; rebuild batchgen_amd") from exc
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def register(name: str, restype, argtypes):
+    """Declare one more exported symbol (used by modules that add entry points)."""
+    _SIGS[name] = (restype, argtypes)
+    if _lib is not None:
+        fn = getattr(_lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+
+
+def check(status: int) -> None:
+    if status != 0:
+        msg = lib().bgmoe_last_error()
+        raise RuntimeError((msg or b"unknown error").decode("utf-8", "replace"))
+
+
+def ptr(t):
+    """Device pointer of a torch tensor (None -> NULL)."""
+    return None if t is None else t.data_ptr()
+
+
+def stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def exported_symbols():
+    return sorted(_SIGS)

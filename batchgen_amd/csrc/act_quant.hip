@@ -1,0 +1,257 @@
+// Per-row, per-128 e4m3fn activation quantisation for gfx950: one wave64 per
+// row, 16-byte loads, wave-shuffle amax, IEEE division, hardware RNE convert.
+//
+// One kernel serves every entry point; they differ in which rows are live
+// (plain / masked by count / ragged spans / gathered through topk_pos) and in
+// where a row's scales go (strides).  HBM-bound: 2 B read + 1 B written per
+// element (+4 B per 128).
+#include "bgmoe_common.h"
+
+namespace {
+
+enum RowMode { kPlain = 0, kMasked = 1, kRagged = 2, kGather = 3 };
+
+struct QuantArgs {
+  const uint16_t* x;     // gate when up != nullptr
+  const uint16_t* up;    // optional: value = bf16(silu(x) * up)
+  uint8_t* y;            // may be nullptr (silu_mul only)
+  float* scale;
+  uint16_t* h_out;       // optional bf16 copy of the value that is quantised
+  int64_t jobs;          // rows (or pairs in gather mode)
+  int k;
+  int64_t srow, skb;
+  const int32_t* counts; // masked: tokens_per_expert
+  int mtp;
+  const int32_t* seqlens;
+  const int32_t* cu;
+  int e;
+  int row_align;
+  int64_t max_rows;
+  const int32_t* topk_pos;
+  int topk;
+};
+
+// state of a destination row: 0 = leave untouched, 1 = valid, 2 = alignment pad
+__device__ __forceinline__ int ragged_row_state(const QuantArgs& a, int64_t row) {
+  const int64_t first = a.cu[0];
+  const int64_t last = a.cu[a.e];
+  if (row < first || row >= last || row >= a.max_rows) return 0;
+  int lo = 0, hi = a.e - 1;
+  while (lo < hi) {                 // rightmost group whose start is <= row
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int64_t)a.cu[mid] <= row) lo = mid; else hi = mid - 1;
+  }
+  const int64_t rel = row - a.cu[lo];
+  const int64_t valid = a.seqlens[lo];
+  const int64_t span = (valid + a.row_align - 1) / a.row_align * a.row_align;
+  if (rel >= span) return 0;
+  return rel < valid ? 1 : 2;
+}
+
+template <bool VEC8>
+__device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64_t dst, bool pad) {
+  const int lane = lane_id();
+  const int k = a.k;
+  const uint16_t* xr = a.x + src * (int64_t)k;
+  const uint16_t* ur = a.up ? a.up + src * (int64_t)k : nullptr;
+  uint8_t* yr = a.y ? a.y + dst * (int64_t)k : nullptr;
+  uint16_t* hr = a.h_out ? a.h_out + dst * (int64_t)k : nullptr;
+  float* sr = a.scale ? a.scale + dst * a.srow : nullptr;
+
+  if constexpr (VEC8) {
+    // 64 lanes x 8 elements = 4 blocks of 128 per step; 16 lanes share a block
+    const int steps = (k + 511) / 512;
+    for (int s = 0; s < steps; ++s) {
+      const int c0 = s * 512 + lane * 8;
+      const bool in = c0 < k;
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+      if (in && !pad) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(xr + c0);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          v[2 * i] = bf16_bits_to_f32(w[i] & 0xffffu);
+          v[2 * i + 1] = bf16_bits_to_f32(w[i] >> 16);
+        }
+        if (ur) {
+          const uint4 rawu = *reinterpret_cast<const uint4*>(ur + c0);
+          const uint32_t wu[4] = {rawu.x, rawu.y, rawu.z, rawu.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            v[2 * i] = bf16_round_f32(silu_f32(v[2 * i]) * bf16_bits_to_f32(wu[i] & 0xffffu));
+            v[2 * i + 1] = bf16_round_f32(silu_f32(v[2 * i + 1]) * bf16_bits_to_f32(wu[i] >> 16));
+          }
+          if (hr) {
+            uint4 o;
+            o.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+            o.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+            o.z = f32_to_bf16_bits(v[4]) | (f32_to_bf16_bits(v[5]) << 16);
+            o.w = f32_to_bf16_bits(v[6]) | (f32_to_bf16_bits(v[7]) << 16);
+            *reinterpret_cast<uint4*>(hr + c0) = o;
+          }
+        }
+      }
+      if (yr == nullptr) continue;
+      float amax = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+      amax = wave_max_xor<16>(amax);
+      const float sc = quant_scale_from_amax(amax);
+      if (in) {
+        float q[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = clamp448(v[i] / sc);
+        uint2 o;
+        o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
+        o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
+        *reinterpret_cast<uint2*>(yr + c0) = o;
+        if ((lane & 15) == 0) sr[(int64_t)(c0 >> 7) * a.skb] = sc;
+      }
+    }
+  } else {
+    // any k: one 128-block per step, two columns per lane
+    const int kb = (k + 127) / 128;
+    for (int b = 0; b < kb; ++b) {
+      const int c0 = b * 128 + lane * 2;
+      float v[2] = {0.0f, 0.0f};
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if (c0 + i < k && !pad) {
+          float g = bf16_bits_to_f32(xr[c0 + i]);
+          if (ur) {
+            g = bf16_round_f32(silu_f32(g) * bf16_bits_to_f32(ur[c0 + i]));
+            if (hr) hr[c0 + i] = (uint16_t)f32_to_bf16_bits(g);
+          }
+          v[i] = g;
+        }
+      }
+      if (yr == nullptr) continue;
+      float amax = fmaxf(fabsf(v[0]), fabsf(v[1]));
+      amax = wave_max_xor<64>(amax);
+      const float sc = quant_scale_from_amax(amax);
+      const uint32_t p = pack4_e4m3(clamp448(v[0] / sc), clamp448(v[1] / sc), 0.0f, 0.0f);
+      if (c0 < k) yr[c0] = (uint8_t)(p & 0xff);
+      if (c0 + 1 < k) yr[c0 + 1] = (uint8_t)((p >> 8) & 0xff);
+      if (lane == 0) sr[(int64_t)b * a.skb] = sc;
+    }
+  }
+}
+
+template <int MODE, bool VEC8>
+__global__ __launch_bounds__(256) void act_quant_kernel(QuantArgs a) {
+  const int wave = threadIdx.x >> 6;
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  for (int64_t job = (int64_t)blockIdx.x * 4 + wave; job < a.jobs; job += stride) {
+    int64_t src = job, dst = job;
+    bool pad = false;
+    if constexpr (MODE == kMasked) {
+      const int e = (int)(job / a.mtp);
+      const int t = (int)(job - (int64_t)e * a.mtp);
+      if (t >= a.counts[e]) continue;
+    } else if constexpr (MODE == kRagged) {
+      const int st = ragged_row_state(a, job);
+      if (st == 0) continue;
+      pad = st == 2;
+    } else if constexpr (MODE == kGather) {
+      const int p = a.topk_pos[job];
+      if (p < 0) continue;
+      src = job / a.topk;
+      dst = p;
+    }
+    quant_row<VEC8>(a, src, dst, pad);
+  }
+}
+
+template <int MODE>
+int launch(const QuantArgs& a, hipStream_t st) {
+  if (a.jobs <= 0 || a.k <= 0) return BGMOE_OK;
+  int64_t blocks = (a.jobs + 3) / 4;
+  if (blocks > 16384) blocks = 16384;
+  auto aligned = [](const void* p, size_t n) { return p == nullptr || ((uintptr_t)p % n) == 0; };
+  const bool vec = (a.k % 8 == 0) && aligned(a.x, 16) && aligned(a.up, 16) && aligned(a.y, 8) &&
+                   aligned(a.h_out, 16);
+  if (vec)
+    hipLaunchKernelGGL((act_quant_kernel<MODE, true>), dim3((unsigned)blocks), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((act_quant_kernel<MODE, false>), dim3((unsigned)blocks), dim3(256), 0, st, a);
+  return bgmoe_check_launch("act_quant");
+}
+
+}  // namespace
+
+extern "C" int bgmoe_act_quant_rows(const uint16_t* x, int64_t rows, int k, uint8_t* y, float* scale,
+                                    int64_t scale_row_stride, int64_t scale_kb_stride,
+                                    bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(rows >= 0 && k >= 0, "act_quant_rows: negative size");
+  BGMOE_REQUIRE(rows == 0 || k == 0 || (x && y && scale), "act_quant_rows: null pointer");
+  QuantArgs a{};
+  a.x = x; a.y = y; a.scale = scale; a.jobs = rows; a.k = k;
+  a.srow = scale_row_stride; a.skb = scale_kb_stride;
+  return launch<kPlain>(a, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_act_quant_3d(const uint16_t* x, const int32_t* tokens_per_expert, int e, int mtp,
+                                  int k, uint8_t* y, float* scale, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(e >= 0 && mtp >= 0 && k >= 0, "act_quant_3d: negative size");
+  if ((int64_t)e * mtp == 0 || k == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(x && y && scale && tokens_per_expert, "act_quant_3d: null pointer");
+  QuantArgs a{};
+  a.x = x; a.y = y; a.scale = scale; a.jobs = (int64_t)e * mtp; a.k = k;
+  a.skb = 1; a.srow = (k + 127) / 128; a.counts = tokens_per_expert; a.mtp = mtp;
+  return launch<kMasked>(a, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_act_quant_ragged(const uint16_t* x, const int32_t* seqlens,
+                                      const int32_t* cu_seqlens, int e, int64_t max_rows, int k,
+                                      uint8_t* y, float* scale_t, int row_align,
+                                      bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(e > 0, "act_quant_ragged: need at least one group");
+  BGMOE_REQUIRE(row_align > 0 && (row_align & (row_align - 1)) == 0,
+                "act_quant_ragged: row_align must be a positive power of two, got %d", row_align);
+  BGMOE_REQUIRE(max_rows >= 0 && k >= 0, "act_quant_ragged: negative size");
+  if (max_rows == 0 || k == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(x && y && scale_t && seqlens && cu_seqlens, "act_quant_ragged: null pointer");
+  QuantArgs a{};
+  a.x = x; a.y = y; a.scale = scale_t; a.jobs = max_rows; a.k = k;
+  a.srow = 1; a.skb = max_rows;
+  a.seqlens = seqlens; a.cu = cu_seqlens; a.e = e; a.row_align = row_align; a.max_rows = max_rows;
+  return launch<kRagged>(a, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_silu_mul_3d(const uint16_t* gate, const uint16_t* up,
+                                 const int32_t* tokens_per_expert, int e, int mtp, int k,
+                                 uint16_t* out, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(e >= 0 && mtp >= 0 && k >= 0, "silu_mul_3d: negative size");
+  if ((int64_t)e * mtp == 0 || k == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(gate && up && out && tokens_per_expert, "silu_mul_3d: null pointer");
+  QuantArgs a{};
+  a.x = gate; a.up = up; a.h_out = out; a.jobs = (int64_t)e * mtp; a.k = k;
+  a.counts = tokens_per_expert; a.mtp = mtp;
+  return launch<kMasked>(a, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_fused_silu_quant_3d(const uint16_t* gate, const uint16_t* up,
+                                         const int32_t* tokens_per_expert, int e, int mtp, int k,
+                                         uint8_t* y, float* scale, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(e >= 0 && mtp >= 0 && k >= 0, "fused_silu_quant_3d: negative size");
+  if ((int64_t)e * mtp == 0 || k == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(gate && up && y && scale && tokens_per_expert, "fused_silu_quant_3d: null pointer");
+  QuantArgs a{};
+  a.x = gate; a.up = up; a.y = y; a.scale = scale; a.jobs = (int64_t)e * mtp; a.k = k;
+  a.skb = 1; a.srow = (k + 127) / 128; a.counts = tokens_per_expert; a.mtp = mtp;
+  return launch<kMasked>(a, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h,
+                                   uint8_t* y, float* scale, int64_t scale_row_stride,
+                                   int64_t scale_kb_stride, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n >= 0 && k > 0 && h >= 0, "scatter_quant: bad size");
+  if (n == 0 || h == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(x && y && scale && topk_pos, "scatter_quant: null pointer");
+  QuantArgs a{};
+  a.x = x; a.y = y; a.scale = scale; a.jobs = (int64_t)n * k; a.k = h;
+  a.srow = scale_row_stride; a.skb = scale_kb_stride; a.topk_pos = topk_pos; a.topk = k;
+  return launch<kGather>(a, bgmoe_stream(stream));
+}

@@ -1,0 +1,70 @@
+// Shared device helpers for the gfx950 MoE kernels (wave64, OCP fp8).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/bgmoe.h"
+
+#define BGMOE_WAVE 64
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef short shortx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+// ---- error plumbing (host) ---------------------------------------------------
+void bgmoe_set_error(const char* fmt, ...);
+int bgmoe_check_launch(const char* what);
+
+#define BGMOE_REQUIRE(cond, ...)            \
+  do {                                      \
+    if (!(cond)) {                          \
+      bgmoe_set_error(__VA_ARGS__);         \
+      return BGMOE_ERR_ARG;                 \
+    }                                       \
+  } while (0)
+
+static inline hipStream_t bgmoe_stream(bgmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- bf16 <-> fp32 -----------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// round-to-nearest-even; NaN stays NaN (quiet)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+__device__ __forceinline__ float bf16_round_f32(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
+
+// ---- fp8 e4m3fn (OCP on gfx950), RNE; inputs already clamped to +-448 ---------
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d) {
+  int v = 0;
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, v, false);
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (uint32_t)v;
+}
+
+// clamp as fmaxf(fminf(q, 448), -448): a NaN q becomes +448, as in the reference quantiser
+__device__ __forceinline__ float clamp448(float q) { return fmaxf(fminf(q, 448.0f), -448.0f); }
+
+// scale of one 128-block from its amax: fmaxf(amax, 1e-12f) * (1.0f / 448.0f)
+__device__ __forceinline__ float quant_scale_from_amax(float amax) {
+  constexpr float kInv448 = 1.0f / 448.0f;
+  return fmaxf(amax, 1e-12f) * kInv448;
+}
+
+// ---- wave helpers ---------------------------------------------------------------
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (BGMOE_WAVE - 1); }
+
+template <int WIDTH>
+__device__ __forceinline__ float wave_max_xor(float v) {
+#pragma unroll
+  for (int off = WIDTH / 2; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, BGMOE_WAVE));
+  return v;
+}
+
+__device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }

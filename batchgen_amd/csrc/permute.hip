@@ -1,0 +1,316 @@
+// Expert permute for gfx950: a STABLE counting sort of the (token, k) pairs by
+// local expert id.  Slot of pair i inside its expert = number of pairs j < i of
+// the same expert, so the permutation is a pure function of topk_ids (the
+// reference claims slots with a global atomic counter, i.e. arrival order).
+//
+// Pairs are cut into chunks of 2048; a block owns a chunk, each of its four
+// waves owns 512 consecutive pairs and walks them 64 at a time.  Ranks come
+// from ballots (which lanes hold my expert?) plus wave-private LDS counters --
+// LDS atomics are used only for histograms, never to claim a slot.
+//
+//   nk <= 2048 : one launch does histogram, prefix and ranks (decode).
+//   otherwise  : hist per chunk -> one-block scan -> ranks per chunk.
+// The row copy (or the quantising copy) is a separate one-wave-per-pair launch.
+#include "bgmoe_common.h"
+
+namespace {
+
+constexpr int kChunk = 2048;       // pairs per block
+constexpr int kWavePairs = 512;    // pairs per wave
+constexpr int kMaxLocal = 1024;    // local experts
+
+struct PermArgs {
+  const int32_t* ids;      // [nk]
+  int64_t nk;
+  int expert_start, e_local;
+  int mtp;                 // masked layout stride, or 0 for ragged
+  int row_align;           // ragged
+  int32_t* counts;         // [e_local]
+  int32_t* counters;       // [e_local] (may be null)
+  int32_t* cu;             // [e_local+1] (ragged; may be null for masked)
+  int32_t* pos;            // [nk]
+  int32_t* chunk_hist;     // workspace [nchunks][e_local]
+  int nchunks;
+};
+
+__device__ __forceinline__ int local_id(const PermArgs& a, int64_t i) {
+  if (i >= a.nk) return -1;
+  const int64_t le = (int64_t)a.ids[i] - a.expert_start;
+  return (le >= 0 && le < a.e_local) ? (int)le : -1;
+}
+
+__global__ __launch_bounds__(256) void perm_hist_kernel(PermArgs a) {
+  __shared__ int32_t hist[kMaxLocal];
+  for (int e = threadIdx.x; e < a.e_local; e += 256) hist[e] = 0;
+  __syncthreads();
+  const int64_t base = (int64_t)blockIdx.x * kChunk;
+  for (int j = threadIdx.x; j < kChunk; j += 256) {
+    const int le = local_id(a, base + j);
+    if (le >= 0) atomicAdd(&hist[le], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < a.e_local; e += 256)
+    a.chunk_hist[(int64_t)blockIdx.x * a.e_local + e] = hist[e];
+}
+
+// exclusive scan over chunks per expert (in place), then counts / cu_seqlens
+__global__ __launch_bounds__(1024) void perm_scan_kernel(PermArgs a) {
+  __shared__ int32_t tot[kMaxLocal];
+  const int e = threadIdx.x;
+  if (e < a.e_local) {
+    int run = 0;
+    for (int c = 0; c < a.nchunks; ++c) {
+      const int64_t o = (int64_t)c * a.e_local + e;
+      const int t = a.chunk_hist[o];
+      a.chunk_hist[o] = run;
+      run += t;
+    }
+    const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
+    tot[e] = cnt;
+    a.counts[e] = cnt;
+    if (a.counters) a.counters[e] = cnt;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0 && a.cu) {
+    int64_t off = 0;
+    for (int g = 0; g < a.e_local; ++g) {
+      a.cu[g] = (int32_t)off;
+      off += a.mtp > 0 ? (int64_t)a.mtp
+                       : (((int64_t)tot[g] + a.row_align - 1) & ~(int64_t)(a.row_align - 1));
+    }
+    a.cu[a.e_local] = (int32_t)off;
+  }
+}
+
+template <bool SINGLE>
+__global__ __launch_bounds__(256) void perm_rank_kernel(PermArgs a) {
+  __shared__ int32_t whist[4][kMaxLocal];   // per-wave histogram, then per-wave next-slot counter
+  __shared__ int32_t s_cu[SINGLE ? kMaxLocal + 1 : 1];
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int el = a.e_local;
+  for (int e = threadIdx.x; e < 4 * el; e += 256) whist[e / el][e % el] = 0;
+  __syncthreads();
+  const int64_t wbase = (int64_t)blockIdx.x * kChunk + (int64_t)wave * kWavePairs;
+  for (int s = 0; s < kWavePairs / 64; ++s) {
+    const int le = local_id(a, wbase + s * 64 + lane);
+    if (le >= 0) atomicAdd(&whist[wave][le], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < el; e += 256) {
+    int run = SINGLE ? 0 : a.chunk_hist[(int64_t)blockIdx.x * el + e];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const int t = whist[w][e];
+      whist[w][e] = run;
+      run += t;
+    }
+    if constexpr (SINGLE) {
+      const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
+      a.counts[e] = cnt;
+      if (a.counters) a.counters[e] = cnt;
+      s_cu[e + 1] = cnt;
+    }
+  }
+  __syncthreads();
+  if constexpr (SINGLE) {
+    if (threadIdx.x == 0) {
+      int64_t off = 0;
+      for (int g = 0; g < el; ++g) {
+        const int cnt = s_cu[g + 1];
+        s_cu[g] = (int32_t)off;
+        if (a.cu) a.cu[g] = (int32_t)off;
+        off += a.mtp > 0 ? (int64_t)a.mtp
+                         : (((int64_t)cnt + a.row_align - 1) & ~(int64_t)(a.row_align - 1));
+      }
+      if (a.cu) a.cu[el] = (int32_t)off;
+    }
+    __syncthreads();
+  }
+
+  int nbits = 0;
+  while ((1 << nbits) < el) ++nbits;
+  const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  for (int s = 0; s < kWavePairs / 64; ++s) {
+    const int64_t i = wbase + s * 64 + lane;
+    const int le = local_id(a, i);
+    unsigned long long peers = __ballot(le >= 0);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (le >> b) & 1;
+      const unsigned long long m = __ballot(bit);
+      peers &= bit ? m : ~m;
+    }
+    int slot = -1;
+    if (le >= 0) slot = whist[wave][le] + __popcll(peers & lt);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (le >= 0 && (peers & lt) == 0ull) whist[wave][le] += __popcll(peers);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (i < a.nk) {
+      int p = -1;
+      if (le >= 0) {
+        if (a.mtp > 0) p = slot < a.mtp ? le * a.mtp + slot : -1;
+        else p = (SINGLE ? s_cu[le] : a.cu[le]) + slot;
+      }
+      a.pos[i] = p;
+    }
+  }
+}
+
+// one wave per pair: act[pos] = x[token]
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x,
+                                                          const int32_t* __restrict__ pos,
+                                                          uint16_t* __restrict__ act, int64_t nk,
+                                                          int k, int h, int vec) {
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  for (int64_t i = (int64_t)blockIdx.x * 4 + wave; i < nk; i += stride) {
+    const int p = pos[i];
+    if (p < 0) continue;
+    const uint16_t* src = x + (i / k) * (int64_t)h;
+    uint16_t* dst = act + (int64_t)p * h;
+    if (vec) {
+      const uint4* s4 = reinterpret_cast<const uint4*>(src);
+      uint4* d4 = reinterpret_cast<uint4*>(dst);
+      for (int v = lane; v < h / 8; v += BGMOE_WAVE) d4[v] = s4[v];
+    } else {
+      for (int c = lane; c < h; c += BGMOE_WAVE) dst[c] = src[c];
+    }
+  }
+}
+
+__global__ __launch_bounds__(64) void compact_kernel(const int32_t* __restrict__ counts, int e,
+                                                     int32_t* group_size, int32_t* active_idx,
+                                                     int32_t* starts, int32_t* num_active) {
+  const int lane = lane_id();
+  const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  int written = 0, cumulative = 0;
+  for (int base = 0; base < e; base += 64) {
+    const int g = base + lane;
+    const int c = g < e ? counts[g] : 0;
+    const unsigned long long m = __ballot(c > 0);
+    // inclusive scan of c over the wave
+    int inc = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(inc, off, BGMOE_WAVE);
+      if (lane >= off) inc += up;
+    }
+    if (c > 0) {
+      const int w = written + __popcll(m & lt);
+      active_idx[w] = g;
+      group_size[w] = c;
+      starts[w] = cumulative + inc - c;
+    }
+    written += __popcll(m);
+    cumulative += __shfl(inc, 63, BGMOE_WAVE);
+  }
+  if (lane == 0) *num_active = written;
+}
+
+int run_index(PermArgs& a, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  if (a.nk <= kChunk) {
+    a.nchunks = 1;
+    hipLaunchKernelGGL((perm_rank_kernel<true>), dim3(1), dim3(256), 0, st, a);
+    return bgmoe_check_launch("dispatch(single)");
+  }
+  a.nchunks = (int)((a.nk + kChunk - 1) / kChunk);
+  const size_t need = (size_t)a.nchunks * a.e_local * sizeof(int32_t);
+  if (workspace == nullptr || workspace_bytes < need) {
+    bgmoe_set_error("dispatch: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    return BGMOE_ERR_WORKSPACE;
+  }
+  a.chunk_hist = (int32_t*)workspace;
+  hipLaunchKernelGGL(perm_hist_kernel, dim3(a.nchunks), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(perm_scan_kernel, dim3(1), dim3(1024), 0, st, a);
+  hipLaunchKernelGGL((perm_rank_kernel<false>), dim3(a.nchunks), dim3(256), 0, st, a);
+  return bgmoe_check_launch("dispatch");
+}
+
+int run_gather(const uint16_t* x, const int32_t* pos, uint16_t* act, int64_t nk, int k, int h,
+               hipStream_t st) {
+  if (nk == 0 || h == 0) return BGMOE_OK;
+  int64_t blocks = (nk + 3) / 4;
+  if (blocks > 65536) blocks = 65536;
+  const int vec = (h % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)act % 16 == 0);
+  hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, st, x, pos, act, nk,
+                     k, h, vec);
+  return bgmoe_check_launch("dispatch(gather)");
+}
+
+}  // namespace
+
+extern "C" size_t bgmoe_dispatch_workspace_bytes(int64_t nk, int num_local_experts) {
+  if (nk <= kChunk || num_local_experts <= 0) return 0;
+  return (size_t)((nk + kChunk - 1) / kChunk) * (size_t)num_local_experts * sizeof(int32_t);
+}
+
+extern "C" int bgmoe_dispatch_scatter_3d(const uint16_t* x, const int32_t* topk_ids, int n, int k,
+                                         int h, uint16_t* act_buffer, int expert_start,
+                                         int num_local_experts, int max_tokens_padded,
+                                         int32_t* expert_counts, int32_t* expert_counters,
+                                         int32_t* topk_pos, void* workspace, size_t workspace_bytes,
+                                         bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n >= 0 && k > 0 && h >= 0, "dispatch_scatter_3d: bad sizes n=%d k=%d h=%d", n, k, h);
+  BGMOE_REQUIRE(num_local_experts > 0 && num_local_experts <= kMaxLocal,
+                "dispatch_scatter_3d: num_local_experts=%d outside [1,%d]", num_local_experts, kMaxLocal);
+  BGMOE_REQUIRE(max_tokens_padded > 0, "dispatch_scatter_3d: max_tokens_padded must be positive");
+  BGMOE_REQUIRE((int64_t)num_local_experts * max_tokens_padded <= 2147483647LL,
+                "dispatch_scatter_3d: E_local*max_tokens_padded exceeds int32");
+  BGMOE_REQUIRE(expert_counts && topk_pos, "dispatch_scatter_3d: null output");
+  BGMOE_REQUIRE(n == 0 || topk_ids, "dispatch_scatter_3d: null topk_ids");
+  PermArgs a{};
+  a.ids = topk_ids; a.nk = (int64_t)n * k; a.expert_start = expert_start;
+  a.e_local = num_local_experts; a.mtp = max_tokens_padded; a.row_align = 1;
+  a.counts = expert_counts; a.counters = expert_counters; a.cu = nullptr; a.pos = topk_pos;
+  int rc = run_index(a, workspace, workspace_bytes, bgmoe_stream(stream));
+  if (rc != BGMOE_OK || act_buffer == nullptr) return rc;
+  BGMOE_REQUIRE(n == 0 || x, "dispatch_scatter_3d: null x");
+  return run_gather(x, topk_pos, act_buffer, a.nk, k, h, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_dispatch_scatter_ragged(const uint16_t* x, const int32_t* topk_ids, int n, int k,
+                                             int h, uint16_t* act_buffer, int64_t act_rows,
+                                             int expert_start, int num_local_experts,
+                                             int32_t* expert_counts, int32_t* expert_counters,
+                                             int32_t* topk_pos, int32_t* cu_seqlens, int row_align,
+                                             void* workspace, size_t workspace_bytes,
+                                             bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(row_align > 0 && (row_align & (row_align - 1)) == 0,
+                "dispatch_scatter_ragged: row_align must be a positive power of two, got %d", row_align);
+  BGMOE_REQUIRE(n >= 0 && k > 0 && h >= 0, "dispatch_scatter_ragged: bad sizes n=%d k=%d h=%d", n, k, h);
+  BGMOE_REQUIRE(num_local_experts > 0 && num_local_experts <= kMaxLocal,
+                "dispatch_scatter_ragged: num_local_experts=%d outside [1,%d]", num_local_experts, kMaxLocal);
+  BGMOE_REQUIRE(expert_start >= 0, "dispatch_scatter_ragged: expert_start out of range: %d", expert_start);
+  const int64_t nk = (int64_t)n * k;
+  const int64_t cap_rows = (nk + (int64_t)(row_align - 1) * (nk < num_local_experts ? nk : num_local_experts)) /
+                           row_align * row_align;
+  BGMOE_REQUIRE(cap_rows <= 2147483647LL, "dispatch_scatter_ragged: N*K too large: %lld", (long long)nk);
+  if (act_buffer)
+    BGMOE_REQUIRE(act_rows >= cap_rows, "dispatch_scatter_ragged: act_buffer rows (%lld) must be in [%lld, INT32_MAX]",
+                  (long long)act_rows, (long long)cap_rows);
+  BGMOE_REQUIRE(expert_counts && topk_pos && cu_seqlens, "dispatch_scatter_ragged: null output");
+  BGMOE_REQUIRE(n == 0 || topk_ids, "dispatch_scatter_ragged: null topk_ids");
+  PermArgs a{};
+  a.ids = topk_ids; a.nk = nk; a.expert_start = expert_start; a.e_local = num_local_experts;
+  a.mtp = 0; a.row_align = row_align; a.counts = expert_counts; a.counters = expert_counters;
+  a.cu = cu_seqlens; a.pos = topk_pos;
+  int rc = run_index(a, workspace, workspace_bytes, bgmoe_stream(stream));
+  if (rc != BGMOE_OK || act_buffer == nullptr) return rc;
+  BGMOE_REQUIRE(n == 0 || x, "dispatch_scatter_ragged: null x");
+  return run_gather(x, topk_pos, act_buffer, nk, k, h, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_compact_expert_data(const int32_t* expert_counts, int e, int32_t* group_size,
+                                         int32_t* activated_group_idx, int32_t* group_start_indices,
+                                         int32_t* num_active, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(e >= 0, "compact_expert_data: e < 0");
+  BGMOE_REQUIRE(num_active, "compact_expert_data: null num_active");
+  BGMOE_REQUIRE(e == 0 || (expert_counts && group_size && activated_group_idx && group_start_indices),
+                "compact_expert_data: null pointer");
+  hipLaunchKernelGGL(compact_kernel, dim3(1), dim3(64), 0, bgmoe_stream(stream), expert_counts, e,
+                     group_size, activated_group_idx, group_start_indices, num_active);
+  return bgmoe_check_launch("compact_expert_data");
+}

@@ -1,0 +1,275 @@
+// Sigmoid + bias-corrected top-k routers for gfx950: ONE wave64 per token.
+// A token's experts live in registers (expert id = i*64 + lane, VPL values per
+// lane); every arg-max round is a lane-local scan plus a 6-step butterfly with
+// the rule "larger value wins, equal values go to the lower expert id", which
+// gives a unique winner whatever the reduction tree.
+#include <math.h>
+
+#include "bgmoe_common.h"
+
+namespace {
+
+constexpr float kNegInf = -__builtin_huge_valf();
+
+// correctly rounded fp32 sigmoid: evaluate in fp64, round once
+__device__ __forceinline__ float sigmoid_cr(float x) {
+  return (float)(1.0 / (1.0 + exp(-(double)x)));
+}
+
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float ov = __shfl_xor(v, off, BGMOE_WAVE);
+    const int oi = __shfl_xor(idx, off, BGMOE_WAVE);
+    if (ov > v || (ov == v && oi < idx)) {
+      v = ov;
+      idx = oi;
+    }
+  }
+}
+
+struct RouterArgs {
+  const float* in;        // scores or logits, row stride `stride`
+  int64_t stride;
+  const float* bias;
+  int n, e, top_k;
+  float rsf;
+  int apply_sigmoid;
+  // grouped
+  int n_group, topk_group;
+  // outputs
+  int32_t* ids32;
+  int64_t* ids64;
+  float* w;
+  // padding
+  const int32_t* num_valid;
+  const int64_t* rank_counts;
+  int rows_per_rank;
+  // latent epilogue
+  uint16_t* latent_out;
+  int latent_offset, latent_size;
+};
+
+// GROUPED: moe_fused_gate semantics (floor -1e9, w = raw * (rsf / (sum + 1e-20)))
+// else    : gate_sigmoid_topk semantics (floor -FLT_MAX, w = raw * (1/(sum+1e-20)) * rsf)
+template <int VPL, bool GROUPED>
+__global__ __launch_bounds__(256) void router_kernel(RouterArgs a) {
+  extern __shared__ float s_lds[];   // GROUPED: [4][e] biased scores
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int token = blockIdx.x * 4 + wave;
+  if (token >= a.n) return;          // whole wave; no block-level barrier is used below
+
+  if constexpr (!GROUPED) {
+    bool pad = false;
+    if (a.num_valid) {
+      pad = token >= *a.num_valid;
+    } else if (a.rank_counts) {
+      const int r = token / a.rows_per_rank;
+      pad = (int64_t)(token - r * a.rows_per_rank) >= a.rank_counts[r];
+    }
+    if (pad) {
+      if (lane < a.top_k) {
+        if (a.ids64) a.ids64[(int64_t)token * a.top_k + lane] = -1;
+        else a.ids32[(int64_t)token * a.top_k + lane] = -1;
+        a.w[(int64_t)token * a.top_k + lane] = 0.0f;
+      }
+      if (a.latent_out)
+        for (int i = lane; i < a.latent_size; i += BGMOE_WAVE)
+          a.latent_out[(int64_t)token * a.latent_size + i] = 0;
+      return;
+    }
+  }
+
+  const float* row = a.in + (int64_t)token * a.stride;
+  float raw[VPL], key[VPL];
+  const float floor_v = GROUPED ? -1e9f : -3.402823466e+38f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int ex = i * BGMOE_WAVE + lane;
+    if (ex < a.e) {
+      const float x = row[ex];
+      raw[i] = a.apply_sigmoid ? sigmoid_cr(x) : x;
+      const float s = raw[i] + a.bias[ex];
+      key[i] = s > floor_v ? s : kNegInf;     // NaN and <= floor are never candidates
+    } else {
+      raw[i] = 0.0f;
+      key[i] = kNegInf;
+    }
+  }
+
+  if constexpr (!GROUPED) {
+    if (a.latent_out) {
+      const float* lat = row + a.latent_offset;
+      for (int i = lane; i < a.latent_size; i += BGMOE_WAVE)
+        a.latent_out[(int64_t)token * a.latent_size + i] = (uint16_t)f32_to_bf16_bits(lat[i]);
+    }
+  }
+
+  if constexpr (GROUPED) {
+    // group score = sum of the group's two largest biased scores (strict '>' scan from -1e9)
+    float* s = s_lds + wave * a.e;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int ex = i * BGMOE_WAVE + lane;
+      if (ex < a.e) s[ex] = key[i] == kNegInf ? -1e9f : key[i];
+    }
+    // the slice is private to this wave: order its LDS writes before the reads below
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int epg = a.e / a.n_group;
+    float gscore = kNegInf;
+    if (lane < a.n_group) {
+      float m1 = -1e9f, m2 = -1e9f;
+      for (int i = 0; i < epg; ++i) {
+        const float v = s[lane * epg + i];
+        if (v > m1) { m2 = m1; m1 = v; }
+        else if (v > m2) { m2 = v; }
+      }
+      const float g = m1 + m2;
+      gscore = g > -1e9f ? g : kNegInf;
+    }
+    unsigned long long gmask = 0ull;
+    for (int r = 0; r < a.topk_group; ++r) {
+      float v = gscore;
+      int idx = v == kNegInf ? 0x7fffffff : lane;
+      wave_argmax(v, idx);
+      if (v != kNegInf) {
+        gmask |= 1ull << idx;
+        if (lane == idx) gscore = kNegInf;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int ex = i * BGMOE_WAVE + lane;
+      const int g = ex < a.e ? ex / epg : 0;
+      if (!((gmask >> g) & 1ull)) key[i] = kNegInf;
+    }
+  }
+
+  float total = 0.0f;
+  int my_id = -1;
+  float my_raw = 0.0f;
+  for (int r = 0; r < a.top_k; ++r) {
+    float v = kNegInf;
+    int idx = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      if (key[i] > v) {                       // ascending ids per lane: strict '>' keeps the lowest
+        v = key[i];
+        idx = i * BGMOE_WAVE + lane;
+      }
+    }
+    wave_argmax(v, idx);
+    float rv = 0.0f;
+    int id = -1;
+    if (v != kNegInf) {
+      id = idx;
+      const int owner = idx & (BGMOE_WAVE - 1);
+      const int slot = idx >> 6;
+      float mine = 0.0f;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        if (i == slot) {
+          mine = raw[i];
+          if (lane == owner) key[i] = kNegInf;
+        }
+      }
+      rv = __shfl(mine, owner, BGMOE_WAVE);
+    }
+    total = total + rv;                        // route order, from 0.0f
+    if (lane == r) {
+      my_id = id;
+      my_raw = rv;
+    }
+  }
+
+  if (lane < a.top_k) {
+    float wv;
+    if constexpr (GROUPED) {
+      const float scale = a.rsf / (total + 1e-20f);
+      wv = my_raw * scale;
+    } else {
+      const float inv = 1.0f / (total + 1e-20f);
+      wv = my_raw * inv;
+      wv = wv * a.rsf;
+    }
+    const int64_t o = (int64_t)token * a.top_k + lane;
+    if (a.ids64) a.ids64[o] = my_id;
+    else a.ids32[o] = my_id;
+    a.w[o] = wv;
+  }
+}
+
+template <bool GROUPED>
+int launch_router(const RouterArgs& a, hipStream_t st) {
+  if (a.n == 0) return BGMOE_OK;
+  const dim3 grid((a.n + 3) / 4), block(256);
+  const size_t lds = GROUPED ? (size_t)4 * a.e * sizeof(float) : 0;
+  const int vpl = (a.e + 63) / 64;
+#define BGMOE_ROUTER_CASE(V)                                                              \
+  hipLaunchKernelGGL((router_kernel<V, GROUPED>), grid, block, lds, st, a)
+  if (vpl <= 1) BGMOE_ROUTER_CASE(1);
+  else if (vpl <= 2) BGMOE_ROUTER_CASE(2);
+  else if (vpl <= 4) BGMOE_ROUTER_CASE(4);
+  else if (vpl <= 8) BGMOE_ROUTER_CASE(8);
+  else BGMOE_ROUTER_CASE(16);
+#undef BGMOE_ROUTER_CASE
+  return bgmoe_check_launch("router");
+}
+
+}  // namespace
+
+extern "C" int bgmoe_fused_gate(const float* scores, const float* bias, int n, int e, int n_group,
+                                int topk_group, int top_k, float routed_scaling_factor,
+                                int apply_sigmoid, int32_t* topk_ids, float* topk_weights,
+                                bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n >= 0, "fused_gate: n < 0");
+  BGMOE_REQUIRE(e >= 1 && e <= 1024, "fused_gate: n_routed_experts=%d outside [1,1024]", e);
+  BGMOE_REQUIRE(n_group >= 1 && n_group <= 64, "fused_gate: n_group=%d outside [1,64]", n_group);
+  BGMOE_REQUIRE(e % n_group == 0, "fused_gate: n_routed_experts (%d) must be divisible by n_group (%d)",
+                e, n_group);
+  BGMOE_REQUIRE(topk_group >= 1 && topk_group <= n_group, "fused_gate: topk_group=%d outside [1,%d]",
+                topk_group, n_group);
+  BGMOE_REQUIRE(top_k >= 1 && top_k <= 32 && top_k <= e, "fused_gate: unsupported top_k=%d", top_k);
+  if (n == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(scores && bias && topk_ids && topk_weights, "fused_gate: null pointer");
+  RouterArgs a{};
+  a.in = scores; a.stride = e; a.bias = bias; a.n = n; a.e = e; a.top_k = top_k;
+  a.rsf = routed_scaling_factor; a.apply_sigmoid = apply_sigmoid;
+  a.n_group = n_group; a.topk_group = topk_group; a.ids32 = topk_ids; a.w = topk_weights;
+  return launch_router<true>(a, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_gate_sigmoid_topk(const float* logits, int64_t logits_stride, const float* bias,
+                                       int n, int e, int k, float routed_scaling_factor,
+                                       void* topk_ids, int ids_are_int64, float* topk_weights,
+                                       const int32_t* num_valid_tokens,
+                                       const int64_t* rank_token_counts, int rows_per_rank,
+                                       uint16_t* latent_out, int latent_offset, int latent_size,
+                                       bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n >= 0, "gate_sigmoid_topk: n < 0");
+  BGMOE_REQUIRE(e >= 1 && e <= 1024, "gate_sigmoid_topk: E=%d exceeds MAX_EXPERTS=1024", e);
+  BGMOE_REQUIRE(k == 2 || k == 4 || k == 8 || k == 16, "gate_sigmoid_topk: Unsupported k=%d. Supported: 2, 4, 8, 16", k);
+  BGMOE_REQUIRE(e >= k, "gate_sigmoid_topk: E=%d must be at least k=%d", e, k);
+  BGMOE_REQUIRE(logits_stride >= e, "gate_sigmoid_topk: row stride %lld < E=%d", (long long)logits_stride, e);
+  BGMOE_REQUIRE(!(num_valid_tokens && rank_token_counts),
+                "gate_sigmoid_topk: num_valid_tokens and rank_token_counts are mutually exclusive");
+  BGMOE_REQUIRE(!rank_token_counts || rows_per_rank > 0, "gate_sigmoid_topk: rows_per_rank must be positive");
+  if (latent_out) {
+    BGMOE_REQUIRE(latent_offset >= e, "gate_sigmoid_topk: latent_offset=%d must start at or after the %d router columns", latent_offset, e);
+    BGMOE_REQUIRE((int64_t)latent_offset + latent_size <= logits_stride,
+                  "gate_sigmoid_topk: latent columns exceed the row stride");
+  }
+  if (n == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(logits && bias && topk_ids && topk_weights, "gate_sigmoid_topk: null pointer");
+  RouterArgs a{};
+  a.in = logits; a.stride = logits_stride; a.bias = bias; a.n = n; a.e = e; a.top_k = k;
+  a.rsf = routed_scaling_factor; a.apply_sigmoid = 1;
+  if (ids_are_int64) a.ids64 = (int64_t*)topk_ids; else a.ids32 = (int32_t*)topk_ids;
+  a.w = topk_weights; a.num_valid = num_valid_tokens; a.rank_counts = rank_token_counts;
+  a.rows_per_rank = rows_per_rank; a.latent_out = latent_out; a.latent_offset = latent_offset;
+  a.latent_size = latent_size;
+  return launch_router<false>(a, bgmoe_stream(stream));
+}

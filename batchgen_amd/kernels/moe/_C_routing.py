@@ -1,0 +1,141 @@
+"""gfx950 implementation of the reference extension ``batchgen_kernels.moe._C_routing``
+(bindings: batchgen_kernels/src/moe/routing/routing_extension.cc:12-105).
+
+Exports gate_sigmoid_topk, gate_sigmoid_topk_warp, dispatch_count_gather,
+reduce_weighted_scatter.  The softmax router, the router GEMM and the bias
+epilogue of that extension are not part of this build.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..._lib import check, lib, ptr, stream
+from .. import _checks as ck
+from .._workspace import dispatch_workspace
+
+
+def _padding(n, logits, num_valid_tokens, rank_token_counts, rows_per_rank):
+    """resolve_gst_padding_shape (gate_sigmoid_topk.cu:500-540)."""
+    nv = rc = None
+    rpr = 0
+    if num_valid_tokens is not None and num_valid_tokens.numel() > 0:
+        if rank_token_counts is not None and rank_token_counts.numel() > 0:
+            ck.fail("num_valid_tokens and rank_token_counts are mutually exclusive")
+        ck.cuda_tensor(logits, num_valid_tokens, torch.int32, "num_valid_tokens")
+        if num_valid_tokens.numel() != 1:
+            ck.fail("num_valid_tokens must hold one int32")
+        nv = num_valid_tokens
+    elif rank_token_counts is not None and rank_token_counts.numel() > 0:
+        ck.cuda_tensor(logits, rank_token_counts, torch.int64, "rank_token_counts")
+        rpr = int(rows_per_rank or 0)
+        if rpr <= 0:
+            ck.fail("rows_per_rank must be positive when rank_token_counts is given")
+        if rank_token_counts.numel() * rpr != n:
+            ck.fail(f"rank_token_counts ({rank_token_counts.numel()}) x rows_per_rank ({rpr}) must equal N={n}")
+        rc = rank_token_counts
+    return nv, rc, rpr
+
+
+def _gate(router_logits, e_score_correction, k, routed_scaling_factor, topk_indices, topk_weights,
+          num_valid_tokens, latent_out, latent_offset, rank_token_counts, rows_per_rank, max_e, allow_i64):
+    ck.gpu(router_logits, "router_logits")
+    ck.dtype(router_logits, torch.float32, "router_logits")
+    if router_logits.dim() != 2:
+        ck.fail("router_logits must be 2-D")
+    if router_logits.stride(1) != 1:
+        ck.fail("router_logits rows must be contiguous")
+    ck.cuda_tensor(router_logits, e_score_correction, torch.float32, "e_score_correction")
+    n, e = router_logits.shape
+    if e > max_e:
+        ck.fail(f"E={e} exceeds MAX_EXPERTS={max_e}")
+    if e < k:
+        ck.fail(f"E={e} must be at least k={k}")
+    if e_score_correction.numel() != e:
+        ck.fail("e_score_correction must have E elements")
+    dev = router_logits.device
+    if topk_indices is None or topk_indices.numel() == 0:
+        topk_indices = torch.empty((n, k), dtype=torch.int32, device=dev)
+    if topk_weights is None or topk_weights.numel() == 0:
+        topk_weights = torch.empty((n, k), dtype=torch.float32, device=dev)
+    ck.cuda_tensor(router_logits, topk_indices, (torch.int32, torch.int64) if allow_i64 else torch.int32,
+                   "topk_indices")
+    ck.cuda_tensor(router_logits, topk_weights, torch.float32, "topk_weights")
+    if tuple(topk_indices.shape) != (n, k) or tuple(topk_weights.shape) != (n, k):
+        ck.fail(f"topk_indices / topk_weights must be contiguous [{n}, {k}] tensors")
+    nv, rc, rpr = _padding(n, router_logits, num_valid_tokens, rank_token_counts, rows_per_rank)
+    lat_ptr, lat_off, lat_size = None, 0, 0
+    if latent_out is not None and latent_out.numel() > 0:
+        ck.cuda_tensor(router_logits, latent_out, torch.bfloat16, "latent_out")
+        if latent_out.dim() != 2 or latent_out.size(0) != n:
+            ck.fail(f"latent_out must have {n} rows")
+        lat_off = int(latent_offset or 0)
+        lat_size = latent_out.size(1)
+        lat_ptr = ptr(latent_out)
+    if n == 0:
+        return [topk_indices, topk_weights]
+    with torch.cuda.device(dev):
+        check(lib().bgmoe_gate_sigmoid_topk(
+            ptr(router_logits), router_logits.stride(0), ptr(e_score_correction), n, e, int(k),
+            float(routed_scaling_factor), ptr(topk_indices), int(topk_indices.dtype == torch.int64),
+            ptr(topk_weights), ptr(nv), ptr(rc), rpr, lat_ptr, lat_off, lat_size, stream()))
+    return [topk_indices, topk_weights]
+
+
+def gate_sigmoid_topk(router_logits, e_score_correction, k, routed_scaling_factor, topk_indices,
+                      topk_weights, num_valid_tokens=None, latent_out=None, latent_offset=None,
+                      rank_token_counts=None, rows_per_rank=None):
+    """Ungrouped sigmoid + bias top-k, E <= 1024 (gate_sigmoid_topk.cu:546-640)."""
+    return _gate(router_logits, e_score_correction, k, routed_scaling_factor, topk_indices, topk_weights,
+                 num_valid_tokens, latent_out, latent_offset, rank_token_counts, rows_per_rank, 1024, False)
+
+
+def gate_sigmoid_topk_warp(router_logits, e_score_correction, k, routed_scaling_factor, topk_indices,
+                           topk_weights, num_valid_tokens=None, rank_token_counts=None, rows_per_rank=None):
+    """Same routing, E <= 256, int32 or int64 ids (gate_sigmoid_topk.cu:643-714).  On gfx950 both
+    entry points run the same one-wave-per-token kernel."""
+    if topk_indices is None or topk_weights is None:
+        ck.fail("gate_sigmoid_topk_warp needs caller-owned topk_indices and topk_weights")
+    return _gate(router_logits, e_score_correction, k, routed_scaling_factor, topk_indices, topk_weights,
+                 num_valid_tokens, None, None, rank_token_counts, rows_per_rank, 256, True)
+
+
+def dispatch_count_gather(x, topk_indices, expert_start, num_local_experts, expert_counts, expert_offsets,
+                          expert_counters, dispatched_x, topk_pos, num_valid_tokens=-1):
+    """Tight (align 1) counting-sort dispatch (dispatch_count_gather.cu:145-251).
+    Returns [expert_counts, expert_offsets, topk_pos]."""
+    ck.cuda_tensor(None, x, torch.bfloat16, "x")
+    ck.cuda_tensor(x, topk_indices, torch.int32, "topk_indices")
+    n, h = x.shape
+    k = topk_indices.size(1)
+    if 0 < int(num_valid_tokens) < n:
+        n = int(num_valid_tokens)
+    for t, name in ((expert_counts, "expert_counts"), (expert_offsets, "expert_offsets"),
+                    (expert_counters, "expert_counters"), (topk_pos, "topk_pos")):
+        ck.cuda_tensor(x, t, torch.int32, name)
+    ck.cuda_tensor(x, dispatched_x, torch.bfloat16, "dispatched_x")
+    if expert_offsets.numel() < num_local_experts + 1:
+        ck.fail("expert_offsets must have num_local_experts + 1 elements")
+    ws, ws_bytes = dispatch_workspace(x.device, n * k, num_local_experts)
+    with torch.cuda.device(x.device):
+        check(lib().bgmoe_dispatch_scatter_ragged(
+            ptr(x), ptr(topk_indices), n, k, h, ptr(dispatched_x), dispatched_x.size(0), int(expert_start),
+            int(num_local_experts), ptr(expert_counts), ptr(expert_counters), ptr(topk_pos),
+            ptr(expert_offsets), 1, ptr(ws), ws_bytes, stream()))
+    return [expert_counts, expert_offsets, topk_pos]
+
+
+def reduce_weighted_scatter(expert_output, topk_pos, topk_weights, N, H, K, output, num_valid_tokens=-1):
+    """out[t] = bf16(sum_k y[pos]*w), K in {2,4,8} (reduce_weighted_scatter.cu:26-131)."""
+    if K not in (2, 4, 8):
+        ck.fail(f"Unsupported K={K}")
+    ck.cuda_tensor(None, expert_output, torch.bfloat16, "expert_output")
+    ck.cuda_tensor(expert_output, topk_pos, torch.int32, "topk_pos")
+    ck.cuda_tensor(expert_output, topk_weights, torch.float32, "topk_weights")
+    if output is None or output.numel() == 0:
+        output = torch.zeros((N, H), dtype=torch.bfloat16, device=expert_output.device)
+    ck.cuda_tensor(expert_output, output, torch.bfloat16, "output")
+    with torch.cuda.device(expert_output.device):
+        check(lib().bgmoe_reduce_weighted_scatter(ptr(expert_output), ptr(topk_pos), ptr(topk_weights), int(N),
+                                                  int(H), int(K), ptr(output), int(num_valid_tokens), None, 0,
+                                                  stream()))
+    return output

@@ -1,0 +1,235 @@
+/*
+ * bgmoe.h -- C ABI of libbgmoe.so: the MoE expert-layer hot path for AMD
+ * MI355X (gfx950).  Plain pointers and sizes only; every pointer that is not
+ * marked "host" is DEVICE memory on the current HIP device; every call
+ * enqueues on `stream` (a hipStream_t passed as void*) and returns without
+ * synchronising, reading nothing back from the device, with a launch geometry
+ * that depends on host arguments only (so a call sequence can be captured in
+ * a HIP graph and replayed with different device-side counts).
+ *
+ * Return value: BGMOE_OK, or an error code with a message available from
+ * bgmoe_last_error() (thread-local).  Argument errors are detected before
+ * anything is launched.
+ *
+ * "reference" below = batchgen-project/batchgen; each entry point names the
+ * reference op it replaces.  Paths are relative to the reference tree.
+ */
+#ifndef BGMOE_H
+#define BGMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* bgmoe_stream_t; /* hipStream_t */
+
+enum {
+  BGMOE_OK = 0,
+  BGMOE_ERR_ARG = 1,         /* bad shape / alignment / unsupported value */
+  BGMOE_ERR_HIP = 2,         /* a HIP runtime call failed                 */
+  BGMOE_ERR_WORKSPACE = 3    /* workspace too small                       */
+};
+
+const char* bgmoe_last_error(void);
+int bgmoe_version(void);
+
+/* ------------------------------------------------------------------ router */
+
+/* Group-limited top-k on (optionally already sigmoided) scores.
+ * Replaces `moe_fused_gate` (batchgen_kernels/common/mgn.py:32-65,
+ * batchgen_kernels/src/moe/mgn/moe_fused_gate.cu:83-329).
+ * scores [n,e] fp32 contiguous; bias [e]; ids [n,top_k] int32 in descending
+ * biased-score order; weights [n,top_k] fp32 = raw*rsf/(sum(raw)+1e-20).
+ * apply_sigmoid != 0: `scores` holds logits; the correctly rounded fp32
+ * sigmoid is applied first (the reference caller does torch.sigmoid before the
+ * op, batchgen/models/deepseek/deepseekv3/modeling_deepseek_v3.py:893-914).
+ * e <= 1024, n_group <= 64, e % n_group == 0, top_k <= 32. */
+int bgmoe_fused_gate(const float* scores, const float* bias, int n, int e, int n_group,
+                     int topk_group, int top_k, float routed_scaling_factor, int apply_sigmoid,
+                     int32_t* topk_ids, float* topk_weights, bgmoe_stream_t stream);
+
+/* Ungrouped sigmoid + bias top-k.
+ * Replaces `gate_sigmoid_topk` / `gate_sigmoid_topk_warp`
+ * (batchgen/moe/routing/cuda_routing.py:124-304,
+ * batchgen_kernels/src/moe/routing/gate_sigmoid_topk.cu:71-213, 546-714).
+ * logits rows may be strided (logits_stride elements, >= e).
+ * ids: int32 or int64 [n,k] (ids_are_int64).  num_valid_tokens (device int32
+ * scalar) or rank_token_counts (device int64 [ceil(n/rows_per_rank)]) mark
+ * padding rows, which get id -1 / weight 0; both may be NULL.
+ * latent_out (bf16 [n, latent_size]) optionally receives
+ * bf16(row[latent_offset : latent_offset+latent_size]); NULL to skip. */
+int bgmoe_gate_sigmoid_topk(const float* logits, int64_t logits_stride, const float* bias, int n,
+                            int e, int k, float routed_scaling_factor, void* topk_ids,
+                            int ids_are_int64, float* topk_weights,
+                            const int32_t* num_valid_tokens, const int64_t* rank_token_counts,
+                            int rows_per_rank, uint16_t* latent_out, int latent_offset,
+                            int latent_size, bgmoe_stream_t stream);
+
+/* --------------------------------------------------------- FP8 act quant */
+
+/* Per-row, per-128 e4m3fn quantisation of plain rows:
+ *   s = fmaxf(amax,1e-12f)*(1/448.f); q = clamp(x/s, +-448) -> RNE e4m3fn.
+ * Replaces `act_quant` (batchgen/quantization/act_quant.py:78-128; identical
+ * bytes and, for amax >= 2^-16, identical scales).  x [rows,k] bf16;
+ * y [rows,k] bytes; scale element (r,kb) at scale[r*srow + kb*skb]. */
+int bgmoe_act_quant_rows(const uint16_t* x, int64_t rows, int k, uint8_t* y, float* scale,
+                         int64_t scale_row_stride, int64_t scale_kb_stride, bgmoe_stream_t stream);
+
+/* Masked layout.  Replaces `act_quant_3d`
+ * (batchgen_kernels/src/moe/fp8_blockwise/fp8_blockwise_ops.cu:39-111, 519-556).
+ * x [e,mtp,k]; rows >= tokens_per_expert[e] are neither read nor written;
+ * scale [e,mtp,ceil(k/128)]. */
+int bgmoe_act_quant_3d(const uint16_t* x, const int32_t* tokens_per_expert, int e, int mtp, int k,
+                       uint8_t* y, float* scale, bgmoe_stream_t stream);
+
+/* Ragged layout.  Replaces `act_quant_ragged` (fp8_blockwise_ops.cu:151-361,
+ * 558-628).  Row r in [cu[0],cu[e]) owned by o = max{e: cu[e] <= r} is written
+ * iff r-cu[o] < align(seqlens[o],row_align); rows past seqlens[o] inside the
+ * span get bytes 0 and the all-zero-row scale; other rows are untouched and
+ * their x is not read.  scale_t is TRANSPOSED [ceil(k/128), max_rows]. */
+int bgmoe_act_quant_ragged(const uint16_t* x, const int32_t* seqlens, const int32_t* cu_seqlens,
+                           int e, int64_t max_rows, int k, uint8_t* y, float* scale_t,
+                           int row_align, bgmoe_stream_t stream);
+
+/* silu(gate)*up -> bf16 on the masked layout.  Replaces `silu_mul_3d`
+ * (fp8_blockwise_ops.cu:391-438).  gate, up, out [e,mtp,k] bf16. */
+int bgmoe_silu_mul_3d(const uint16_t* gate, const uint16_t* up, const int32_t* tokens_per_expert,
+                      int e, int mtp, int k, uint16_t* out, bgmoe_stream_t stream);
+
+/* silu(gate)*up then quantise.  Replaces `fused_silu_quant_3d`
+ * (fp8_blockwise_ops.cu:445-513) with this build's canonical rounding:
+ * h = bf16(silu_f32(gate)*up) then the act-quant above (so that the result is
+ * bit-identical to bgmoe_silu_mul_3d followed by bgmoe_act_quant_3d). */
+int bgmoe_fused_silu_quant_3d(const uint16_t* gate, const uint16_t* up,
+                              const int32_t* tokens_per_expert, int e, int mtp, int k, uint8_t* y,
+                              float* scale, bgmoe_stream_t stream);
+
+/* ------------------------------------------------------ permute / unpermute */
+
+/* Bytes of device workspace the dispatch calls need for n*k pairs. */
+size_t bgmoe_dispatch_workspace_bytes(int64_t nk, int num_local_experts);
+
+/* Masked [E_l, mtp, H] layout.  Replaces `dispatch_scatter_3d`
+ * (batchgen/moe/dispatch_scatter_3d.py:76-109,
+ * batchgen_kernels/src/moe/dispatch_scatter_3d.cu:15-137).
+ * Pair i = t*k + j with local id le = ids[i]-expert_start in [0,E_l) goes to
+ * row le*mtp + slot, slot = number of earlier pairs (smaller i) of the same
+ * expert (deterministic; the reference uses arrival order).  topk_pos[i] = row
+ * or -1.  Pairs with slot >= mtp are dropped (-1) and counts are clipped.
+ * expert_counters is written with the counts too.  act_buffer may be NULL to
+ * compute indices only. */
+int bgmoe_dispatch_scatter_3d(const uint16_t* x, const int32_t* topk_ids, int n, int k, int h,
+                              uint16_t* act_buffer, int expert_start, int num_local_experts,
+                              int max_tokens_padded, int32_t* expert_counts,
+                              int32_t* expert_counters, int32_t* topk_pos, void* workspace,
+                              size_t workspace_bytes, bgmoe_stream_t stream);
+
+/* Contiguous ragged layout.  Replaces `dispatch_scatter_ragged`
+ * (dispatch_scatter_3d.py:112-156, dispatch_scatter_3d.cu:152-358) and, with
+ * row_align = 1, `dispatch_count_gather`
+ * (batchgen_kernels/src/moe/routing/dispatch_count_gather.cu:32-251) and
+ * `fused_moe_token_dispatch` (batchgen_kernels/src/moe/mgn/fused_moe_token_dispatch.cu:172-292).
+ * cu_seqlens[e+1]-cu_seqlens[e] = align(count[e], row_align); act_rows is the
+ * capacity of act_buffer, checked against the worst case. */
+int bgmoe_dispatch_scatter_ragged(const uint16_t* x, const int32_t* topk_ids, int n, int k, int h,
+                                  uint16_t* act_buffer, int64_t act_rows, int expert_start,
+                                  int num_local_experts, int32_t* expert_counts,
+                                  int32_t* expert_counters, int32_t* topk_pos,
+                                  int32_t* cu_seqlens, int row_align, void* workspace,
+                                  size_t workspace_bytes, bgmoe_stream_t stream);
+
+/* Quantise-while-scattering: for every pair with topk_pos[i] >= 0 write the
+ * act-quant of x[i/k] to row topk_pos[i] of y / scale.  Bit-identical to a
+ * scatter followed by bgmoe_act_quant_*.  No reference counterpart as one op:
+ * it fuses `dispatch_scatter_*` with `act_quant_*` (the reference's DeepEP
+ * receive path delivers the same quantised masked layout,
+ * batchgen/moe/deepep_ll.py:331-364). */
+int bgmoe_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h,
+                        uint8_t* y, float* scale, int64_t scale_row_stride,
+                        int64_t scale_kb_stride, bgmoe_stream_t stream);
+
+/* out[t] = bf16(sum_k float(y[pos[t,k]])*w[t,k]), k ascending, pos<0 skipped.
+ * Replaces `reduce_weighted_scatter` (dispatch_scatter_3d.cu:365-395, 527-556;
+ * batchgen_kernels/src/moe/routing/reduce_weighted_scatter.cu:26-131).
+ * num_valid_tokens > 0 limits the rows written.  shared (bf16 [n,h], may be
+ * NULL) is the shared expert's output: shared_mode 0 -> bf16(bf16(sum)+shared)
+ * (the reference's bf16 tensor add), 1 -> bf16(sum+shared). */
+int bgmoe_reduce_weighted_scatter(const uint16_t* expert_out, const int32_t* topk_pos,
+                                  const float* topk_weights, int n, int h, int k, uint16_t* out,
+                                  int num_valid_tokens, const uint16_t* shared, int shared_mode,
+                                  bgmoe_stream_t stream);
+
+/* fp32 output.  Replaces `reduce_weighted_scatter_fp32` (dispatch_scatter_3d.cu:402-434). */
+int bgmoe_reduce_weighted_scatter_fp32(const uint16_t* expert_out, const int32_t* topk_pos,
+                                       const float* topk_weights, int n, int h, int k, float* out,
+                                       bgmoe_stream_t stream);
+
+/* Expert-id-ordered bf16 accumulation.  Replaces
+ * `reduce_weighted_scatter_bf16_ordered` (dispatch_scatter_3d.cu:436-525). */
+int bgmoe_reduce_weighted_scatter_bf16_ordered(const uint16_t* expert_out, const int32_t* topk_pos,
+                                               const int32_t* topk_ids, const float* topk_weights,
+                                               int n, int h, int k, uint16_t* out,
+                                               bgmoe_stream_t stream);
+
+/* Active-expert compaction.  Replaces `compact_expert_data`
+ * (batchgen_kernels/src/moe/mgn/expert_bin_count.cu:332-385): ascending expert
+ * id; outputs int32 [e]: group_size, activated_group_idx, group_start_indices;
+ * num_active int32 [1]. */
+int bgmoe_compact_expert_data(const int32_t* expert_counts, int e, int32_t* group_size,
+                              int32_t* activated_group_idx, int32_t* group_start_indices,
+                              int32_t* num_active, bgmoe_stream_t stream);
+
+/* ------------------------------------------------------------ grouped GEMM */
+
+/* Operands of one block-scaled FP8 grouped GEMM
+ *   Y[r,n] = sum_kb (sum_{k in kb} Xq[r,k]*Wq[g,n,k]) * xs[r,kb] * ws[g,n/128,kb]
+ * for rows r in [cu_seqlens[g], cu_seqlens[g]+seqlens[g]).
+ * Weights: either a stack (w + g*w_group_stride bytes) or, when w_ptrs != NULL,
+ * a device table of per-group pointers (the reference's *_ptrs forms). */
+typedef struct bgmoe_fp8_weight {
+  const uint8_t* w;              /* [groups, n, k] e4m3fn                      */
+  int64_t w_group_stride;        /* bytes between groups                      */
+  const uint8_t* const* w_ptrs;  /* device int64[groups] or NULL              */
+  const float* scale;            /* [groups, n/128, kb_stride] fp32           */
+  int64_t scale_group_stride;    /* elements between groups                   */
+  int64_t scale_nb_stride;       /* elements between 128-row blocks (>= k/128)*/
+  const float* const* scale_ptrs;/* device table or NULL                      */
+} bgmoe_fp8_weight;
+
+typedef struct bgmoe_fp8_act {
+  const uint8_t* x;              /* [m, k] e4m3fn                              */
+  const float* scale;            /* element (r,kb) at r*row_stride+kb*kb_stride */
+  int64_t scale_row_stride;
+  int64_t scale_kb_stride;
+} bgmoe_fp8_act;
+
+/* Single grouped GEMM, bf16 output [m,n].  Replaces
+ * `fp8_blockwise_grouped_gemm` / `_ptrs` (batchgen/moe/grouped_fp8_blockwise_moe.py:292-420,
+ * batchgen_kernels/src/moe/fp8_blockwise/fp8_blockwise_gemm.cu:564-900).
+ * k % 128 == 0, n % 128 == 0, groups <= 1024.  Rows outside every group's
+ * live range are not written. */
+int bgmoe_fp8_grouped_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* b,
+                           const int32_t* seqlens, const int32_t* cu_seqlens, int groups,
+                           int64_t m, int n, int k, uint16_t* out, bgmoe_stream_t stream);
+
+/* Fused stage 1: out = bf16( silu(X*Wg^T) * (X*Wu^T) ), fp32 gate and up.
+ * Replaces `fp8_blockwise_fused_s1` / `_ptrs`
+ * (grouped_fp8_blockwise_moe.py:423-560, fp8_blockwise_s1_kernel.cuh:425-607).
+ * If out_q != NULL the bf16 result is quantised in the epilogue (act-quant of
+ * each row's 128-blocks) into out_q [m,n] bytes + out_scale (strided), and
+ * `out` may be NULL: this replaces the S1 -> `act_quant_ragged` pair
+ * (batchgen/models/glm/glm5/model.py:2560-2573) bit for bit. */
+int bgmoe_fp8_fused_s1(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* gate,
+                       const bgmoe_fp8_weight* up, const int32_t* seqlens,
+                       const int32_t* cu_seqlens, int groups, int64_t m, int n, int k,
+                       uint16_t* out, uint8_t* out_q, float* out_scale,
+                       int64_t out_scale_row_stride, int64_t out_scale_nb_stride,
+                       bgmoe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BGMOE_H */

@@ -1,0 +1,218 @@
+"""HIP block-scaled FP8 grouped GEMMs vs the fp32 dequantise-then-matmul oracle.
+
+Tolerances are the reference's own gates (tests/test_moe_compact_ragged_fp8.py:370-377):
+rtol 2e-2 / atol 5e-3 for a single GEMM, rtol 5e-2 / atol 2e-2 for the fused stage 1, plus a relative
+Frobenius bound far below the 1e-2 layer budget.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as og
+from oracle import quant as oq
+from tests.util import rand_bf16, say
+
+pytestmark = pytest.mark.gpu
+
+
+def gm():
+    from batchgen_amd.kernels import load_extension
+    return load_extension("batchgen_kernels.moe._C_fp8_blockwise_gemm")
+
+
+def qops():
+    from batchgen_amd.kernels import load_extension
+    return load_extension("batchgen_kernels.moe._C_fp8_blockwise_ops")
+
+
+def _layout(counts, align):
+    counts = np.asarray(counts, dtype=np.int32)
+    al = (counts + align - 1) // align * align
+    cu = np.concatenate([[0], np.cumsum(al)]).astype(np.int32)
+    return counts, cu
+
+
+def _make(seed, counts, n, k, align=16, nmat=1):
+    g = torch.Generator().manual_seed(seed)
+    counts, cu = _layout(counts, align)
+    m = max(int(cu[-1]), 1)
+    x = rand_bf16(g, m, k)
+    xq, xs = oq.act_quant(x)
+    ws = []
+    for _ in range(nmat):
+        w = (0.02 * torch.randn(len(counts), n, k, generator=g)).numpy()
+        ws.append(oq.weight_block_quant(w))
+    return counts, cu, m, xq, xs, ws
+
+
+def _dev(dev, xq, xs, wq, wsc, pad4=True):
+    kb = xs.shape[1]
+    xq_d = torch.from_numpy(xq).to(dev).view(torch.float8_e4m3fn)
+    xs_t = torch.from_numpy(np.ascontiguousarray(xs.T)).to(dev)
+    wq_d = torch.from_numpy(wq).to(dev).view(torch.float8_e4m3fn)
+    kbp = (kb + 3) // 4 * 4 if pad4 else kb
+    wsp = np.zeros(wsc.shape[:2] + (kbp,), dtype=np.float32)
+    wsp[..., :kb] = wsc
+    return xq_d, xs_t, wq_d, torch.from_numpy(wsp).to(dev)
+
+
+EDGE = (0, 1, 15, 16, 17, 31, 32, 63, 64, 65, 127, 128)
+
+
+@pytest.mark.parametrize("counts,n,k", [
+    (EDGE, 256, 512), ((5, 0, 9, 16), 128, 1024), ((3, 200, 0, 77, 130, 1), 384, 256), ((300,), 256, 384),
+    ((8,) * 8, 7168, 2048),
+])
+def test_grouped_gemm_vs_fp32_oracle(dev, counts, n, k):
+    say("grouped_gemm", counts, n, k)
+    counts, cu, m, xq, xs, ws = _make(100 + n + k, counts, n, k)
+    wq, wsc = ws[0]
+    xq_d, xs_t, wq_d, ws_d = _dev(dev, xq, xs, wq, wsc)
+    out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+    gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev),
+                                    xs_t, ws_d, 16, out)
+    ref = og.grouped_gemm_fp8(xq, xs, wq, wsc, counts, cu, to_bf16=False)
+    o = out.float().cpu().numpy()
+    live = np.zeros(m, dtype=bool)
+    for e, c in enumerate(counts):
+        live[cu[e]:cu[e] + c] = True
+    np.testing.assert_allclose(o[live], ref[live], rtol=2e-2, atol=5e-3)
+    assert og.rel_frobenius(o[live], ref[live]) < 3e-3
+    assert np.all(o[~live] == 7.0)                       # rows outside every live range untouched
+
+
+def test_grouped_gemm_closed_form_constant_case(dev):
+    """All weights 0.25 (exact in e4m3), scales 0.01, x = 1: y = K * 0.25 * 0.01 * xs."""
+    k, n, e = 512, 256, 3
+    counts, cu = _layout((7, 0, 40), 16)
+    m = int(cu[-1])
+    xq = np.full((m, k), 0x38, dtype=np.uint8)            # 1.0
+    xs = np.full((m, k // 128), 0.5, dtype=np.float32)
+    wq = np.full((e, n, k), 0x28, dtype=np.uint8)         # 0.25
+    wsc = np.full((e, n // 128, k // 128), 0.01, dtype=np.float32)
+    xq_d, xs_t, wq_d, ws_d = _dev(dev, xq, xs, wq, wsc)
+    out = gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, torch.from_numpy(counts).to(dev),
+                                          torch.from_numpy(cu).to(dev), xs_t, ws_d, 16)
+    expect = torch.tensor(k * 0.25 * 0.01 * 0.5).to(torch.bfloat16)
+    assert torch.all(out[:7] == expect.to(dev)) and torch.all(out[32:72] == expect.to(dev))
+
+
+@pytest.mark.parametrize("counts,n,k", [
+    (EDGE, 256, 512), ((5, 0, 9, 16), 128, 1024), ((3, 200, 0, 77, 130, 1), 384, 256), ((8,) * 4, 2048, 7168),
+])
+def test_fused_s1_vs_oracle_and_requant_identity(dev, counts, n, k):
+    say("fused_s1", counts, n, k)
+    counts, cu, m, xq, xs, ws = _make(200 + n + k, counts, n, k, nmat=2)
+    (gq, gs), (uq, us) = ws
+    xq_d, xs_t, gq_d, gs_d = _dev(dev, xq, xs, gq, gs)
+    _, _, uq_d, us_d = _dev(dev, xq, xs, uq, us)
+    cnt_d, cu_d = torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev)
+    h = torch.zeros((m, n), dtype=torch.bfloat16, device=dev)
+    gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16, h)
+    gate = og.grouped_gemm_fp8(xq, xs, gq, gs, counts, cu, to_bf16=False)
+    up = og.grouped_gemm_fp8(xq, xs, uq, us, counts, cu, to_bf16=False)
+    ref = oq.silu_f32(gate) * up
+    o = h.float().cpu().numpy()
+    live = np.zeros(m, dtype=bool)
+    for e, c in enumerate(counts):
+        live[cu[e]:cu[e] + c] = True
+    np.testing.assert_allclose(o[live], ref[live], rtol=5e-2, atol=2e-2)
+    assert og.rel_frobenius(o[live], ref[live]) < 4e-3
+    # epilogue requant == separate act_quant_ragged on the bf16 output, bit for bit
+    hq = torch.zeros((m, n), dtype=torch.uint8, device=dev)
+    hs = torch.zeros((n // 128, m), dtype=torch.float32, device=dev)
+    gm().fp8_blockwise_fused_s1_quant(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, hq, hs)
+    hq2 = torch.zeros((m, n), dtype=torch.uint8, device=dev)
+    hs2 = torch.zeros((n // 128, m), dtype=torch.float32, device=dev)
+    qops().act_quant_ragged(h, cnt_d, cu_d, hq2, hs2, 1)
+    lv = torch.from_numpy(live).to(dev)
+    assert torch.equal(hq[lv], hq2[lv]) and torch.equal(hs[:, lv], hs2[:, lv])
+
+
+def test_ragged_equals_uniform_layout(dev):
+    """The same rows placed at different offsets give bit-identical results."""
+    counts = (9, 0, 33, 70)
+    n, k = 256, 512
+    c1, cu1, m1, xq1, xs1, ws = _make(5, counts, n, k, align=16)
+    wq, wsc = ws[0]
+    s_ = 128
+    cu2 = (np.arange(len(counts) + 1) * s_).astype(np.int32)
+    m2 = int(cu2[-1])
+    xq2 = np.zeros((m2, k), dtype=np.uint8)
+    xs2 = np.ones((m2, k // 128), dtype=np.float32)
+    for e, c in enumerate(counts):
+        xq2[cu2[e]:cu2[e] + c] = xq1[cu1[e]:cu1[e] + c]
+        xs2[cu2[e]:cu2[e] + c] = xs1[cu1[e]:cu1[e] + c]
+    outs = []
+    for xq, xs, cu, m in ((xq1, xs1, cu1, m1), (xq2, xs2, cu2, m2)):
+        xq_d, xs_t, wq_d, ws_d = _dev(dev, xq, xs, wq, wsc)
+        o = gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, torch.from_numpy(c1).to(dev), torch.from_numpy(cu).to(dev),
+                                            xs_t, ws_d, 16)
+        outs.append((o, cu))
+    for e, c in enumerate(counts):
+        a = outs[0][0][outs[0][1][e]:outs[0][1][e] + c]
+        b = outs[1][0][outs[1][1][e]:outs[1][1][e] + c]
+        assert torch.equal(a, b)
+
+
+def test_poisoned_padding_does_not_leak(dev):
+    """Rows past a group's count hold NaN bytes / huge scales; live rows must not change."""
+    counts = (5, 20, 100)
+    n, k = 256, 256
+    c, cu, m, xq, xs, ws = _make(6, counts, n, k, align=128)
+    wq, wsc = ws[0]
+    xq_p, xs_p = xq.copy(), xs.copy()
+    for e, cc in enumerate(counts):
+        xq_p[cu[e] + cc:cu[e + 1]] = 0x7F
+        xs_p[cu[e] + cc:cu[e + 1]] = 1e30
+    res = []
+    for a, b in ((xq, xs), (xq_p, xs_p)):
+        xq_d, xs_t, wq_d, ws_d = _dev(dev, a, b, wq, wsc)
+        res.append(gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, torch.from_numpy(c).to(dev),
+                                                   torch.from_numpy(cu).to(dev), xs_t, ws_d, 64))
+    for e, cc in enumerate(counts):
+        assert torch.equal(res[0][cu[e]:cu[e] + cc], res[1][cu[e]:cu[e] + cc])
+
+
+def test_pointer_table_equals_stacked(dev):
+    counts = (4, 0, 18, 90)
+    n, k = 256, 384
+    c, cu, m, xq, xs, ws = _make(8, counts, n, k, nmat=2)
+    (gq, gs), (uq, us) = ws
+    xq_d, xs_t, gq_d, gs_d = _dev(dev, xq, xs, gq, gs)
+    _, _, uq_d, us_d = _dev(dev, xq, xs, uq, us)
+    cnt_d, cu_d = torch.from_numpy(c).to(dev), torch.from_numpy(cu).to(dev)
+    ref = gm().fp8_blockwise_grouped_gemm(xq_d, gq_d, cnt_d, cu_d, xs_t, gs_d, 16)
+    perm = [2, 0, 3, 1]                                    # tables need not be in memory order
+    gparts = [gq_d[i].clone() for i in range(4)]
+    sparts = [gs_d[i].clone() for i in range(4)]
+    wp = torch.tensor([gparts[i].data_ptr() for i in range(4)], dtype=torch.int64, device=dev)
+    sp = torch.tensor([sparts[i].data_ptr() for i in range(4)], dtype=torch.int64, device=dev)
+    out = gm().fp8_blockwise_grouped_gemm_ptrs(xq_d, gq_d[0], wp, cnt_d, cu_d, xs_t, gs_d[0], sp, 16)
+    assert torch.equal(out, ref)
+    ref1 = gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16)
+    uparts = [uq_d[i].clone() for i in range(4)]
+    usparts = [us_d[i].clone() for i in range(4)]
+    up = torch.tensor([t.data_ptr() for t in uparts], dtype=torch.int64, device=dev)
+    usp = torch.tensor([t.data_ptr() for t in usparts], dtype=torch.int64, device=dev)
+    out1 = gm().fp8_blockwise_fused_s1_ptrs(xq_d, gq_d[0], wp, uq_d[0], up, cnt_d, cu_d, xs_t, gs_d[0], sp,
+                                            us_d[0], usp, 16)
+    live = torch.zeros(m, dtype=torch.bool)
+    for e, cc in enumerate(counts):
+        live[cu[e]:cu[e] + cc] = True
+    assert torch.equal(out1[live.to(dev)], ref1[live.to(dev)])
+    del perm
+
+
+def test_gemm_argument_errors(dev):
+    x = torch.zeros((16, 200), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    w = torch.zeros((2, 128, 200), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    sl = torch.zeros(2, dtype=torch.int32, device=dev)
+    cu = torch.zeros(3, dtype=torch.int32, device=dev)
+    xs = torch.zeros((2, 16), device=dev)
+    ws = torch.zeros((2, 1, 4), device=dev)
+    with pytest.raises(RuntimeError):
+        gm().fp8_blockwise_grouped_gemm(x, w, sl, cu, xs, ws, 16)       # K not a multiple of 128
+    w2 = torch.zeros((1025, 128, 128), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+    with pytest.raises(RuntimeError):
+        gm().fp8_blockwise_grouped_gemm(x, w2, sl, cu, xs, ws, 16)      # too many groups

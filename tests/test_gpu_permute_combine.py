@@ -1,0 +1,185 @@
+"""HIP permute / combine vs the CPU oracle: indices and outputs bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import combine as oc
+from oracle import permute as op_
+from oracle.quant import act_quant
+from tests.util import rand_bf16, say
+
+pytestmark = pytest.mark.gpu
+
+
+def ds3d():
+    from batchgen_amd.kernels import load_extension
+    return load_extension("batchgen_kernels.moe._C_dispatch_scatter_3d")
+
+
+def _ids(g, n, k, e_total, extra=None):
+    ids = torch.stack([torch.randperm(e_total, generator=g)[:k] for _ in range(n)]).to(torch.int32)
+    if extra is not None and n * k >= len(extra):
+        ids.view(-1)[: len(extra)] = torch.tensor(extra, dtype=torch.int32)
+    return ids
+
+
+CASES = [  # n, k, h, e_total, expert_start, e_local
+    (1, 4, 256, 16, 0, 16), (64, 4, 1024, 16, 0, 16), (256, 8, 7168, 256, 0, 32), (256, 8, 512, 256, 64, 32),
+    (100, 2, 131, 64, 32, 8), (700, 8, 256, 256, 0, 256), (4096, 8, 128, 256, 32, 32), (513, 16, 64, 896, 28, 28),
+]
+
+
+@pytest.mark.parametrize("n,k,h,et,es,el", CASES)
+def test_dispatch_masked(dev, n, k, h, et, es, el):
+    say("dispatch_3d", n, k, h, et, es, el)
+    g = torch.Generator().manual_seed(n * 13 + k)
+    ids = _ids(g, n, k, et, extra=[-1, 0, es - 1, es + el, 10 ** 6])
+    x = rand_bf16(g, n, h)
+    counts_o, pos_o = op_.dispatch_masked(ids.numpy(), es, el, 10 ** 9)
+    mtp = max(int(counts_o.max()), 1)
+    counts_o, pos_o = op_.dispatch_masked(ids.numpy(), es, el, mtp)
+    act = torch.zeros((el * mtp, h), dtype=torch.bfloat16, device=dev)
+    counts = torch.full((el,), -3, dtype=torch.int32, device=dev)
+    counters = torch.full((el,), -3, dtype=torch.int32, device=dev)
+    pos = torch.full((n * k,), -9, dtype=torch.int32, device=dev)
+    ds3d().dispatch_scatter_3d(x.to(dev), ids.to(dev), act, es, el, mtp, counts, counters, pos)
+    assert np.array_equal(counts.cpu().numpy(), counts_o)
+    assert np.array_equal(counters.cpu().numpy(), counts_o)
+    assert np.array_equal(pos.cpu().numpy(), pos_o)
+    ref = op_.gather_rows(x.view(torch.int16).numpy(), pos_o, k, el * mtp)
+    assert np.array_equal(act.view(torch.int16).cpu().numpy(), ref)
+
+
+def test_dispatch_masked_overflow_rows_are_dropped(dev):
+    ids = torch.zeros((10, 2), dtype=torch.int32)
+    ids[:, 1] = 1
+    x = torch.ones((10, 64), dtype=torch.bfloat16)
+    act = torch.zeros((2 * 4, 64), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty(2, dtype=torch.int32, device=dev)
+    counters = torch.empty(2, dtype=torch.int32, device=dev)
+    pos = torch.empty(20, dtype=torch.int32, device=dev)
+    ds3d().dispatch_scatter_3d(x.to(dev), ids.to(dev), act, 0, 2, 4, counts, counters, pos)
+    co, po = op_.dispatch_masked(ids.numpy(), 0, 2, 4)
+    assert counts.tolist() == [4, 4] and np.array_equal(pos.cpu().numpy(), po)
+
+
+@pytest.mark.parametrize("row_align", [1, 64, 128])
+@pytest.mark.parametrize("n,k,h,et,es,el", CASES)
+def test_dispatch_ragged(dev, n, k, h, et, es, el, row_align):
+    say("dispatch_ragged", n, k, h, et, es, el, row_align)
+    g = torch.Generator().manual_seed(n * 17 + k + row_align)
+    ids = _ids(g, n, k, et, extra=[-1, 0, es - 1, es + el, 10 ** 6])
+    x = rand_bf16(g, n, h)
+    cap = op_.ragged_capacity_rows(n, k, el, row_align)
+    counts_o, cu_o, pos_o = op_.dispatch_ragged(ids.numpy(), es, el, row_align)
+    assert cu_o[-1] <= cap
+    act = torch.zeros((max(cap, 1), h), dtype=torch.bfloat16, device=dev)
+    counts = torch.empty(el, dtype=torch.int32, device=dev)
+    counters = torch.empty(el, dtype=torch.int32, device=dev)
+    cu = torch.empty(el + 1, dtype=torch.int32, device=dev)
+    pos = torch.empty(n * k, dtype=torch.int32, device=dev)
+    if cap == 0:
+        pytest.skip("empty capacity")
+    r = ds3d().dispatch_scatter_ragged(x.to(dev), ids.to(dev), act, es, el, counts, counters, pos, cu, row_align)
+    assert r[0] is counts and r[1] is cu and r[2] is pos          # caller-owned tensors come back
+    assert np.array_equal(counts.cpu().numpy(), counts_o)
+    assert np.array_equal(cu.cpu().numpy(), cu_o)
+    assert np.array_equal(pos.cpu().numpy(), pos_o)
+    ref = op_.gather_rows(x.view(torch.int16).numpy(), pos_o, k, max(cap, 1))
+    assert np.array_equal(act.view(torch.int16).cpu().numpy(), ref)
+    # invariants the reference tests check: rows of expert e are exactly [cu[e], cu[e]+count)
+    pn = pos.cpu().numpy()
+    flat = ids.view(-1).numpy().astype(np.int64) - es
+    for e in range(el):
+        rows = np.sort(pn[(flat == e)])
+        assert np.array_equal(rows, np.arange(cu_o[e], cu_o[e] + counts_o[e]))
+
+
+def test_dispatch_ragged_rejects_small_buffer_and_bad_align(dev):
+    x = torch.zeros((8, 64), dtype=torch.bfloat16, device=dev)
+    ids = torch.zeros((8, 2), dtype=torch.int32, device=dev)
+    mk = lambda n: torch.empty(n, dtype=torch.int32, device=dev)
+    act = torch.zeros((64, 64), dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError):
+        ds3d().dispatch_scatter_ragged(x, ids, act, 0, 4, mk(4), mk(4), mk(16), mk(5), 64)   # needs 256 rows
+    with pytest.raises(RuntimeError):
+        ds3d().dispatch_scatter_ragged(x, ids, act, 0, 4, mk(4), mk(4), mk(16), mk(5), 48)
+
+
+def test_scatter_quant_equals_scatter_then_quant(dev):
+    from batchgen_amd._lib import check, lib, ptr, stream
+    g = torch.Generator().manual_seed(21)
+    n, k, h, el = 50, 4, 1024, 8
+    ids = _ids(g, n, k, 16)
+    x = rand_bf16(g, n, h)
+    counts_o, cu_o, pos_o = op_.dispatch_ragged(ids.numpy(), 0, el, 16)
+    rows = int(cu_o[-1])
+    pos = torch.from_numpy(pos_o).to(dev)
+    y = torch.zeros((rows, h), dtype=torch.uint8, device=dev)
+    s = torch.zeros((rows, h // 128), dtype=torch.float32, device=dev)
+    check(lib().bgmoe_scatter_quant(ptr(x.to(dev)), ptr(pos), n, k, h, ptr(y), ptr(s), h // 128, 1, stream()))
+    yq, sq = act_quant(x)
+    assert np.array_equal(y.cpu().numpy(), op_.gather_rows(yq, pos_o, k, rows))
+    assert np.array_equal(s.cpu().numpy(), op_.gather_rows(sq, pos_o, k, rows))
+
+
+@pytest.mark.parametrize("n,k,h", [(1, 2, 256), (64, 4, 1024), (256, 8, 7168), (33, 8, 131), (17, 4, 2880)])
+def test_reduce_weighted_scatter(dev, n, k, h):
+    say("reduce", n, k, h)
+    g = torch.Generator().manual_seed(n + k + h)
+    rows = n * k + 5
+    y = rand_bf16(g, rows, h)
+    pos = torch.randperm(rows, generator=g)[: n * k].to(torch.int32)
+    pos[torch.rand(n * k, generator=g) < 0.3] = -1
+    if n > 1:
+        pos.view(n, k)[1] = -1                                        # a token with no local expert
+    w = torch.rand(n, k, generator=g)
+    out = torch.full((n, h), 3.0, dtype=torch.bfloat16, device=dev)
+    ds3d().reduce_weighted_scatter(y.to(dev), pos.to(dev), w.to(dev), n, h, k, out)
+    ref = oc.reduce_weighted_scatter(y, pos.numpy(), w.numpy(), n, k)
+    assert np.array_equal(out.float().cpu().numpy(), ref)
+    if n > 1:
+        assert torch.all(out[1] == 0)
+    if n <= 64:
+        assert np.array_equal(ref, oc.reduce_loop(y, pos.numpy(), w.numpy(), n, k))
+    if h % 8 == 0:
+        ids = torch.stack([torch.randperm(64, generator=g)[:k] for _ in range(n)]).to(torch.int32)
+        out2 = torch.empty((n, h), dtype=torch.bfloat16, device=dev)
+        ds3d().reduce_weighted_scatter_bf16_ordered(y.to(dev), pos.to(dev), ids.to(dev), w.to(dev), n, h, k, out2)
+        ref2 = oc.reduce_weighted_scatter_bf16_ordered(y, pos.numpy(), ids.numpy(), w.numpy(), n, k)
+        assert np.array_equal(out2.float().cpu().numpy(), ref2)
+
+
+def test_reduce_fp32_k16_and_shared(dev):
+    from batchgen_amd._lib import check, lib, ptr, stream
+    g = torch.Generator().manual_seed(4)
+    n, k, h = 40, 16, 3584
+    rows = n * k
+    y = rand_bf16(g, rows, h)
+    pos = torch.randperm(rows, generator=g).to(torch.int32)
+    pos[torch.rand(rows, generator=g) < 0.5] = -1
+    w = torch.rand(n, k, generator=g)
+    out = torch.empty((n, h), dtype=torch.float32, device=dev)
+    ds3d().reduce_weighted_scatter_fp32(y.to(dev), pos.to(dev), w.to(dev), n, h, k, out)
+    ref = oc.reduce_weighted_scatter_fp32(y, pos.numpy(), w.numpy(), n, k)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    sh = rand_bf16(g, n, h)
+    for mode, name in ((0, "bf16_add"), (1, "fp32_add")):
+        ob = torch.empty((n, h), dtype=torch.bfloat16, device=dev)
+        check(lib().bgmoe_reduce_weighted_scatter(ptr(y.to(dev)), ptr(pos.to(dev)), ptr(w.to(dev)), n, h, k,
+                                                  ptr(ob), -1, ptr(sh.to(dev)), mode, stream()))
+        refb = oc.reduce_weighted_scatter(y, pos.numpy(), w.numpy(), n, k, shared=sh, shared_mode=name)
+        assert np.array_equal(ob.float().cpu().numpy(), refb)
+
+
+def test_compact_expert_data(dev):
+    from batchgen_amd.kernels import load_extension
+    m = load_extension("batchgen_kernels.common._C_mgn_ops")
+    counts = torch.tensor([0, 3, 0, 0, 5, 1] + [0] * 70 + [2], dtype=torch.int32)
+    size, idx, start, num = m.compact_expert_data(counts.to(dev))
+    nz = torch.nonzero(counts).view(-1)
+    na = int(num.item())
+    assert na == len(nz)
+    assert idx[:na].cpu().tolist() == nz.tolist()
+    assert size[:na].cpu().tolist() == counts[nz].tolist()
+    assert start[:na].cpu().tolist() == (torch.cumsum(counts[nz], 0) - counts[nz]).tolist()
