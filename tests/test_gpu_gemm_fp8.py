@@ -94,7 +94,7 @@ def test_grouped_gemm_closed_form_constant_case(dev):
     out = gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, torch.from_numpy(counts).to(dev),
                                           torch.from_numpy(cu).to(dev), xs_t, ws_d, 16)
     expect = torch.tensor(k * 0.25 * 0.01 * 0.5).to(torch.bfloat16)
-    assert torch.all(out[:7] == expect.to(dev)) and torch.all(out[32:72] == expect.to(dev))
+    assert torch.all(out[:7] == expect.to(dev)) and torch.all(out[cu[2]:cu[2] + 40] == expect.to(dev))
 
 
 @pytest.mark.parametrize("counts,n,k", [
@@ -189,7 +189,10 @@ def test_pointer_table_equals_stacked(dev):
     wp = torch.tensor([gparts[i].data_ptr() for i in range(4)], dtype=torch.int64, device=dev)
     sp = torch.tensor([sparts[i].data_ptr() for i in range(4)], dtype=torch.int64, device=dev)
     out = gm().fp8_blockwise_grouped_gemm_ptrs(xq_d, gq_d[0], wp, cnt_d, cu_d, xs_t, gs_d[0], sp, 16)
-    assert torch.equal(out, ref)
+    live = torch.zeros(m, dtype=torch.bool)
+    for e, cc in enumerate(counts):
+        live[cu[e]:cu[e] + cc] = True
+    assert torch.equal(out[live.to(dev)], ref[live.to(dev)])
     ref1 = gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16)
     uparts = [uq_d[i].clone() for i in range(4)]
     usparts = [us_d[i].clone() for i in range(4)]
@@ -197,9 +200,6 @@ def test_pointer_table_equals_stacked(dev):
     usp = torch.tensor([t.data_ptr() for t in usparts], dtype=torch.int64, device=dev)
     out1 = gm().fp8_blockwise_fused_s1_ptrs(xq_d, gq_d[0], wp, uq_d[0], up, cnt_d, cu_d, xs_t, gs_d[0], sp,
                                             us_d[0], usp, 16)
-    live = torch.zeros(m, dtype=torch.bool)
-    for e, cc in enumerate(counts):
-        live[cu[e]:cu[e] + cc] = True
     assert torch.equal(out1[live.to(dev)], ref1[live.to(dev)])
     del perm
 

@@ -117,7 +117,9 @@ def test_scatter_quant_equals_scatter_then_quant(dev):
     pos = torch.from_numpy(pos_o).to(dev)
     y = torch.zeros((rows, h), dtype=torch.uint8, device=dev)
     s = torch.zeros((rows, h // 128), dtype=torch.float32, device=dev)
-    check(lib().bgmoe_scatter_quant(ptr(x.to(dev)), ptr(pos), n, k, h, ptr(y), ptr(s), h // 128, 1, stream()))
+    x_d = x.to(dev)                                   # keep every device tensor alive across the raw call
+    check(lib().bgmoe_scatter_quant(ptr(x_d), ptr(pos), n, k, h, ptr(y), ptr(s), h // 128, 1, stream()))
+    torch.cuda.synchronize()
     yq, sq = act_quant(x)
     assert np.array_equal(y.cpu().numpy(), op_.gather_rows(yq, pos_o, k, rows))
     assert np.array_equal(s.cpu().numpy(), op_.gather_rows(sq, pos_o, k, rows))
@@ -164,10 +166,11 @@ def test_reduce_fp32_k16_and_shared(dev):
     ref = oc.reduce_weighted_scatter_fp32(y, pos.numpy(), w.numpy(), n, k)
     assert np.array_equal(out.cpu().numpy().view(np.uint32), ref.view(np.uint32))
     sh = rand_bf16(g, n, h)
+    y_d, pos_d, w_d, sh_d = y.to(dev), pos.to(dev), w.to(dev), sh.to(dev)   # alive across the raw calls
     for mode, name in ((0, "bf16_add"), (1, "fp32_add")):
         ob = torch.empty((n, h), dtype=torch.bfloat16, device=dev)
-        check(lib().bgmoe_reduce_weighted_scatter(ptr(y.to(dev)), ptr(pos.to(dev)), ptr(w.to(dev)), n, h, k,
-                                                  ptr(ob), -1, ptr(sh.to(dev)), mode, stream()))
+        check(lib().bgmoe_reduce_weighted_scatter(ptr(y_d), ptr(pos_d), ptr(w_d), n, h, k,
+                                                  ptr(ob), -1, ptr(sh_d), mode, stream()))
         refb = oc.reduce_weighted_scatter(y, pos.numpy(), w.numpy(), n, k, shared=sh, shared_mode=name)
         assert np.array_equal(ob.float().cpu().numpy(), refb)
 
