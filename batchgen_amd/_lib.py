@@ -33,6 +33,10 @@ class Fp8Act(C.Structure):
 _SIGS = {
     "bgmoe_last_error": (C.c_char_p, []),
     "bgmoe_version": (i32, []),
+    "bgmoe_prof_enable": (i32, [i32]),
+    "bgmoe_prof_kernel_count": (i32, []),
+    "bgmoe_prof_kernel_name": (C.c_char_p, [i32]),
+    "bgmoe_prof_collect": (i32, [C.POINTER(C.c_double), C.POINTER(i64), i32]),
     "bgmoe_fused_gate": (i32, [vp, vp, i32, i32, i32, i32, i32, f32, i32, vp, vp, vp]),
     "bgmoe_gate_sigmoid_topk": (i32, [vp, i64, vp, i32, i32, i32, f32, vp, i32, vp, vp, vp, i32, vp, i32, i32, vp]),
     "bgmoe_act_quant_rows": (i32, [vp, i64, i32, vp, vp, i64, i64, vp]),
@@ -102,3 +106,16 @@ def stream():
 
 def exported_symbols():
     return sorted(_SIGS)
+
+
+def prof_enable(on: bool) -> None:
+    check(lib().bgmoe_prof_enable(int(on)))
+
+
+def prof_collect():
+    """-> {kernel name: (total_ms, launches)} since the last collect (synchronises the device)."""
+    n = lib().bgmoe_prof_kernel_count()
+    ms = (C.c_double * n)()
+    cnt = (i64 * n)()
+    check(lib().bgmoe_prof_collect(ms, cnt, n))
+    return {lib().bgmoe_prof_kernel_name(i).decode(): (ms[i], int(cnt[i])) for i in range(n) if cnt[i]}

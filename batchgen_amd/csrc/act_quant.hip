@@ -29,6 +29,8 @@ struct QuantArgs {
   int64_t max_rows;
   const int32_t* topk_pos;
   int topk;
+  int64_t pairs;         // gather: jobs [0,pairs) are (token,k) pairs, jobs [pairs, jobs) copy
+  int64_t extra_start;   //         token (job - pairs) to row extra_start + (job - pairs)
 };
 
 // state of a destination row: 0 = leave untouched, 1 = valid, 2 = alignment pad
@@ -155,10 +157,15 @@ __global__ __launch_bounds__(256) void act_quant_kernel(QuantArgs a) {
       if (st == 0) continue;
       pad = st == 2;
     } else if constexpr (MODE == kGather) {
-      const int p = a.topk_pos[job];
-      if (p < 0) continue;
-      src = job / a.topk;
-      dst = p;
+      if (job < a.pairs) {
+        const int p = a.topk_pos[job];
+        if (p < 0) continue;
+        src = job / a.topk;
+        dst = p;
+      } else {
+        src = job - a.pairs;
+        dst = a.extra_start + src;
+      }
     }
     quant_row<VEC8>(a, src, dst, pad);
   }
@@ -172,6 +179,7 @@ int launch(const QuantArgs& a, hipStream_t st) {
   auto aligned = [](const void* p, size_t n) { return p == nullptr || ((uintptr_t)p % n) == 0; };
   const bool vec = (a.k % 8 == 0) && aligned(a.x, 16) && aligned(a.up, 16) && aligned(a.y, 8) &&
                    aligned(a.h_out, 16);
+  BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
   if (vec)
     hipLaunchKernelGGL((act_quant_kernel<MODE, true>), dim3((unsigned)blocks), dim3(256), 0, st, a);
   else
@@ -244,14 +252,21 @@ extern "C" int bgmoe_fused_silu_quant_3d(const uint16_t* gate, const uint16_t* u
   return launch<kMasked>(a, bgmoe_stream(stream));
 }
 
+int bgmoe_internal_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h, uint8_t* y,
+                                 float* scale, int64_t srow, int64_t skb, int extra_rows, int64_t extra_start,
+                                 hipStream_t st) {
+  QuantArgs a{};
+  a.x = x; a.y = y; a.scale = scale; a.pairs = (int64_t)n * k; a.jobs = a.pairs + extra_rows; a.k = h;
+  a.srow = srow; a.skb = skb; a.topk_pos = topk_pos; a.topk = k; a.extra_start = extra_start;
+  return launch<kGather>(a, st);
+}
+
 extern "C" int bgmoe_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h,
                                    uint8_t* y, float* scale, int64_t scale_row_stride,
                                    int64_t scale_kb_stride, bgmoe_stream_t stream) {
   BGMOE_REQUIRE(n >= 0 && k > 0 && h >= 0, "scatter_quant: bad size");
   if (n == 0 || h == 0) return BGMOE_OK;
   BGMOE_REQUIRE(x && y && scale && topk_pos, "scatter_quant: null pointer");
-  QuantArgs a{};
-  a.x = x; a.y = y; a.scale = scale; a.jobs = (int64_t)n * k; a.k = h;
-  a.srow = scale_row_stride; a.skb = scale_kb_stride; a.topk_pos = topk_pos; a.topk = k;
-  return launch<kGather>(a, bgmoe_stream(stream));
+  return bgmoe_internal_scatter_quant(x, topk_pos, n, k, h, y, scale, scale_row_stride, scale_kb_stride, 0, 0,
+                                      bgmoe_stream(stream));
 }

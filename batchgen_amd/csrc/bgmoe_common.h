@@ -25,6 +25,32 @@ int bgmoe_check_launch(const char* what);
     }                                       \
   } while (0)
 
+// ---- internal entry points shared between translation units ----------------------
+int bgmoe_internal_dispatch_index(const int32_t* ids, int64_t nk, int expert_start, int e_local, int mtp,
+                                  int row_align, int32_t* counts, int32_t* counters, int32_t* cu,
+                                  int32_t* pos, int extra_count, int64_t extra_start, void* ws,
+                                  size_t ws_bytes, hipStream_t st);
+int bgmoe_internal_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h, uint8_t* y,
+                                 float* scale, int64_t srow, int64_t skb, int extra_rows, int64_t extra_start,
+                                 hipStream_t st);
+
+// ---- optional per-launch timing (off by default; see bgmoe_prof_enable) -----------
+enum BgmoeKernelId {
+  BGMOE_K_ROUTER = 0, BGMOE_K_PERM_HIST, BGMOE_K_PERM_SCAN, BGMOE_K_PERM_RANK, BGMOE_K_GATHER_ROWS,
+  BGMOE_K_ACT_QUANT, BGMOE_K_COMBINE, BGMOE_K_COMPACT,
+  BGMOE_K_S1_SKINNY16, BGMOE_K_S1_SKINNY64, BGMOE_K_S1_TILED,
+  BGMOE_K_GEMM_SKINNY16, BGMOE_K_GEMM_SKINNY64, BGMOE_K_GEMM_TILED,
+  BGMOE_K_MXFP4_S1, BGMOE_K_MXFP4_GEMM, BGMOE_K_BF16_GEMM,
+  BGMOE_K_COUNT
+};
+extern bool g_bgmoe_prof_on;
+void bgmoe_prof_mark(int id, hipStream_t st, bool begin);
+struct BgmoeProf {
+  int id; hipStream_t st;
+  BgmoeProf(int id_, hipStream_t st_) : id(id_), st(st_) { if (g_bgmoe_prof_on) bgmoe_prof_mark(id, st, true); }
+  ~BgmoeProf() { if (g_bgmoe_prof_on) bgmoe_prof_mark(id, st, false); }
+};
+
 static inline hipStream_t bgmoe_stream(bgmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 // ---- bf16 <-> fp32 -----------------------------------------------------------

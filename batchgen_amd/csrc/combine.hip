@@ -116,6 +116,7 @@ int launch(const uint16_t* y, const int32_t* pos, const int32_t* ids, const floa
                    ((uintptr_t)shared % 16 == 0);
   const int cols = kThreads * (vec ? 8 : 1);
   const dim3 grid((h + cols - 1) / cols, n), block(kThreads);
+  BgmoeProf prof(BGMOE_K_COMBINE, st);
   if (vec)
     hipLaunchKernelGGL((combine_kernel<MODE, true>), grid, block, 0, st, y, pos, ids, w, h, k, out,
                        shared, shared_mode);

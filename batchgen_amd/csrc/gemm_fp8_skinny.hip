@@ -274,10 +274,14 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   const dim3 grid((g.n + ntile - 1) / ntile, g.groups), block(256);
   // rows per group in (0,16], (16,64]; more rows go to the LDS-tiled kernel
   g.lo = 0; g.hi = 16;
-  if (fused) hipLaunchKernelGGL((fp8_skinny_kernel<1, 3, true>), grid, block, 0, st, g);
-  else hipLaunchKernelGGL((fp8_skinny_kernel<1, 3, false>), grid, block, 0, st, g);
+  {
+    BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
+    if (fused) hipLaunchKernelGGL((fp8_skinny_kernel<1, 3, true>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((fp8_skinny_kernel<1, 3, false>), grid, block, 0, st, g);
+  }
   if (m > 16) {
     g.lo = 16; g.hi = 64;
+    BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY64 : BGMOE_K_GEMM_SKINNY64, st);
     if (fused) hipLaunchKernelGGL((fp8_skinny_kernel<2, 3, true>), grid, block, 0, st, g);
     else hipLaunchKernelGGL((fp8_skinny_kernel<2, 3, false>), grid, block, 0, st, g);
   }

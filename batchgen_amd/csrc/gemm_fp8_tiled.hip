@@ -318,6 +318,7 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   int64_t blocks = (int64_t)(g_num_cu > 0 ? g_num_cu : 256);
   if (blocks > max_items) blocks = max_items;
   if (blocks < 8) blocks = 8;
+  BgmoeProf prof(w1 ? BGMOE_K_S1_TILED : BGMOE_K_GEMM_TILED, st);
   if (w1) hipLaunchKernelGGL((fp8_tiled_kernel<true>), dim3((unsigned)blocks), dim3(256), 2 * kBufBytes, st, g);
   else hipLaunchKernelGGL((fp8_tiled_kernel<false>), dim3((unsigned)blocks), dim3(256), 2 * kBufBytes, st, g);
   return bgmoe_check_launch("fp8 grouped gemm (tiled)");

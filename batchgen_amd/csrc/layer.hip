@@ -1,0 +1,91 @@
+// Whole-layer driver: chains the kernels of one FP8 MoE layer on one stream
+// with caller-owned buffers, no allocation and no device->host reads, so the
+// sequence can be captured in a HIP graph.
+#include "bgmoe_common.h"
+
+extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(L != nullptr, "moe_fp8_layer_forward: null layer");
+  const int n = L->n, h = L->h, inter = L->inter, el = L->e_local, k = L->top_k;
+  BGMOE_REQUIRE(n >= 0 && h > 0 && inter > 0 && el > 0 && k > 0, "moe_fp8_layer_forward: bad sizes");
+  BGMOE_REQUIRE(h % 128 == 0 && inter % 128 == 0, "moe_fp8_layer_forward: H=%d and I=%d must be multiples of 128", h, inter);
+  BGMOE_REQUIRE(L->layout == 0 || L->layout == 1, "moe_fp8_layer_forward: layout must be 0 (masked) or 1 (ragged)");
+  BGMOE_REQUIRE(L->layout == 1 || L->max_tokens > 0, "moe_fp8_layer_forward: masked layout needs max_tokens");
+  BGMOE_REQUIRE(L->layout == 0 || (L->row_align > 0 && (L->row_align & (L->row_align - 1)) == 0),
+                "moe_fp8_layer_forward: row_align must be a positive power of two");
+  const int64_t nk = (int64_t)n * k;
+  int64_t need_rows;
+  if (L->layout == 0) {
+    need_rows = (int64_t)el * L->max_tokens;
+  } else {
+    const int64_t a = L->row_align;
+    need_rows = (nk + (a - 1) * (nk < el ? nk : el)) / a * a;
+  }
+  BGMOE_REQUIRE(L->cap_rows >= need_rows, "moe_fp8_layer_forward: cap_rows=%lld < %lld rows needed",
+                (long long)L->cap_rows, (long long)need_rows);
+  BGMOE_REQUIRE(L->cap_rows + n <= 2147483647LL, "moe_fp8_layer_forward: row space exceeds int32");
+  if (n == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(L->x && L->logits && L->bias && L->out, "moe_fp8_layer_forward: null input/output");
+  BGMOE_REQUIRE(L->topk_ids && L->topk_weights && L->expert_counts && L->cu_seqlens && L->topk_pos &&
+                L->xq && L->xs && L->hq && L->hs && L->y, "moe_fp8_layer_forward: null buffer");
+  const bool shared = L->has_shared != 0;
+  const bool folded = shared && L->shared_folded != 0;
+  BGMOE_REQUIRE(!folded || L->shared_inter == inter, "moe_fp8_layer_forward: a folded shared expert needs shared_inter == inter");
+  BGMOE_REQUIRE(!folded || (L->gate.w_ptrs && L->up.w_ptrs && L->down.w_ptrs),
+                "moe_fp8_layer_forward: a folded shared expert needs pointer-table weights");
+  BGMOE_REQUIRE(!shared || folded || (L->shq && L->shs), "moe_fp8_layer_forward: null shared-expert buffer");
+  hipStream_t st = bgmoe_stream(stream);
+  int rc;
+
+  // 1. router
+  if (L->n_group > 1)
+    rc = bgmoe_fused_gate(L->logits, L->bias, n, L->e_total, L->n_group, L->topk_group, k,
+                          L->routed_scaling_factor, 1, L->topk_ids, L->topk_weights, stream);
+  else
+    rc = bgmoe_gate_sigmoid_topk(L->logits, L->e_total, L->bias, n, L->e_total, k, L->routed_scaling_factor,
+                                 L->topk_ids, 0, L->topk_weights, nullptr, nullptr, 0, nullptr, 0, 0, stream);
+  if (rc != BGMOE_OK) return rc;
+
+  // 2. stable counting sort -> counts, cu_seqlens (+ the shared expert as one more group), topk_pos
+  rc = bgmoe_internal_dispatch_index(L->topk_ids, nk, L->expert_start, el, L->layout == 0 ? L->max_tokens : 0,
+                                     L->layout == 0 ? 1 : L->row_align, L->expert_counts, nullptr,
+                                     L->cu_seqlens, L->topk_pos, shared ? n : 0, L->cap_rows, L->workspace,
+                                     L->workspace_bytes, st);
+  if (rc != BGMOE_OK) return rc;
+
+  // 3. quantise while scattering; the shared expert's rows are the tokens themselves
+  const int hb = h / 128, ib = inter / 128;
+  rc = bgmoe_internal_scatter_quant(L->x, L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0,
+                                    L->cap_rows, st);
+  if (rc != BGMOE_OK) return rc;
+
+  // 4/5. gate_up + SwiGLU + requant, then down
+  const int64_t rows = L->cap_rows + (shared ? n : 0);
+  const int groups = el + (folded ? 1 : 0);
+  bgmoe_fp8_act ax{L->xq, L->xs, hb, 1};
+  rc = bgmoe_fp8_fused_s1(&ax, &L->gate, &L->up, L->expert_counts, L->cu_seqlens, groups,
+                          folded ? rows : L->cap_rows, inter, h, nullptr, L->hq, L->hs, ib, 1, stream);
+  if (rc != BGMOE_OK) return rc;
+  bgmoe_fp8_act ah{L->hq, L->hs, ib, 1};
+  rc = bgmoe_fp8_grouped_gemm(&ah, &L->down, L->expert_counts, L->cu_seqlens, groups,
+                              folded ? rows : L->cap_rows, h, inter, L->y, stream);
+  if (rc != BGMOE_OK) return rc;
+  if (shared && !folded) {
+    const int si = L->shared_inter;
+    BGMOE_REQUIRE(si > 0 && si % 128 == 0, "moe_fp8_layer_forward: shared_inter=%d must be a multiple of 128", si);
+    // Group `el` of expert_counts / cu_seqlens describes the shared rows (n rows starting at
+    // cap_rows).  shq/shs hold only those n rows, so their base pointers are shifted back by
+    // cap_rows rows: the kernels address row cu_seqlens[el] + t.
+    const int32_t* cnt1 = L->expert_counts + el;
+    bgmoe_fp8_act sx0{L->xq, L->xs, hb, 1};
+    rc = bgmoe_fp8_fused_s1(&sx0, &L->sh_gate, &L->sh_up, cnt1, L->cu_seqlens + el, 1, rows, si, h, nullptr,
+                            L->shq - L->cap_rows * si, L->shs - L->cap_rows * (si / 128), si / 128, 1, stream);
+    if (rc != BGMOE_OK) return rc;
+    bgmoe_fp8_act sh{L->shq - L->cap_rows * si, L->shs - L->cap_rows * (si / 128), si / 128, 1};
+    rc = bgmoe_fp8_grouped_gemm(&sh, &L->sh_down, cnt1, L->cu_seqlens + el, 1, rows, h, si, L->y, stream);
+    if (rc != BGMOE_OK) return rc;
+  }
+
+  // 6. weighted combine + shared expert
+  return bgmoe_reduce_weighted_scatter(L->y, L->topk_pos, L->topk_weights, n, h, k, L->out, -1,
+                                       shared ? L->y + L->cap_rows * h : nullptr, L->shared_mode, stream);
+}

@@ -31,7 +31,21 @@ struct PermArgs {
   int32_t* pos;            // [nk]
   int32_t* chunk_hist;     // workspace [nchunks][e_local]
   int nchunks;
+  int extra_count;         // >= 0: one more group (counts[e_local] = extra_count,
+  int64_t extra_start;     //       cu[e_local] = extra_start, cu[e_local+1] = extra_start + extra_count)
 };
+
+__device__ __forceinline__ void write_tail(const PermArgs& a, int64_t off) {
+  if (a.extra_count >= 0) {
+    a.counts[a.e_local] = a.extra_count;
+    if (a.cu) {
+      a.cu[a.e_local] = (int32_t)a.extra_start;
+      a.cu[a.e_local + 1] = (int32_t)(a.extra_start + a.extra_count);
+    }
+  } else if (a.cu) {
+    a.cu[a.e_local] = (int32_t)off;
+  }
+}
 
 __device__ __forceinline__ int local_id(const PermArgs& a, int64_t i) {
   if (i >= a.nk) return -1;
@@ -78,7 +92,9 @@ __global__ __launch_bounds__(1024) void perm_scan_kernel(PermArgs a) {
       off += a.mtp > 0 ? (int64_t)a.mtp
                        : (((int64_t)tot[g] + a.row_align - 1) & ~(int64_t)(a.row_align - 1));
     }
-    a.cu[a.e_local] = (int32_t)off;
+    write_tail(a, off);
+  } else if (threadIdx.x == 0) {
+    write_tail(a, 0);
   }
 }
 
@@ -123,7 +139,7 @@ __global__ __launch_bounds__(256) void perm_rank_kernel(PermArgs a) {
         off += a.mtp > 0 ? (int64_t)a.mtp
                          : (((int64_t)cnt + a.row_align - 1) & ~(int64_t)(a.row_align - 1));
       }
-      if (a.cu) a.cu[el] = (int32_t)off;
+      write_tail(a, off);
     }
     __syncthreads();
   }
@@ -213,6 +229,7 @@ __global__ __launch_bounds__(64) void compact_kernel(const int32_t* __restrict__
 int run_index(PermArgs& a, void* workspace, size_t workspace_bytes, hipStream_t st) {
   if (a.nk <= kChunk) {
     a.nchunks = 1;
+    BgmoeProf prof(BGMOE_K_PERM_RANK, st);
     hipLaunchKernelGGL((perm_rank_kernel<true>), dim3(1), dim3(256), 0, st, a);
     return bgmoe_check_launch("dispatch(single)");
   }
@@ -223,9 +240,9 @@ int run_index(PermArgs& a, void* workspace, size_t workspace_bytes, hipStream_t 
     return BGMOE_ERR_WORKSPACE;
   }
   a.chunk_hist = (int32_t*)workspace;
-  hipLaunchKernelGGL(perm_hist_kernel, dim3(a.nchunks), dim3(256), 0, st, a);
-  hipLaunchKernelGGL(perm_scan_kernel, dim3(1), dim3(1024), 0, st, a);
-  hipLaunchKernelGGL((perm_rank_kernel<false>), dim3(a.nchunks), dim3(256), 0, st, a);
+  { BgmoeProf prof(BGMOE_K_PERM_HIST, st); hipLaunchKernelGGL(perm_hist_kernel, dim3(a.nchunks), dim3(256), 0, st, a); }
+  { BgmoeProf prof(BGMOE_K_PERM_SCAN, st); hipLaunchKernelGGL(perm_scan_kernel, dim3(1), dim3(1024), 0, st, a); }
+  { BgmoeProf prof(BGMOE_K_PERM_RANK, st); hipLaunchKernelGGL((perm_rank_kernel<false>), dim3(a.nchunks), dim3(256), 0, st, a); }
   return bgmoe_check_launch("dispatch");
 }
 
@@ -235,12 +252,24 @@ int run_gather(const uint16_t* x, const int32_t* pos, uint16_t* act, int64_t nk,
   int64_t blocks = (nk + 3) / 4;
   if (blocks > 65536) blocks = 65536;
   const int vec = (h % 8 == 0) && ((uintptr_t)x % 16 == 0) && ((uintptr_t)act % 16 == 0);
+  BgmoeProf prof(BGMOE_K_GATHER_ROWS, st);
   hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, st, x, pos, act, nk,
                      k, h, vec);
   return bgmoe_check_launch("dispatch(gather)");
 }
 
 }  // namespace
+
+int bgmoe_internal_dispatch_index(const int32_t* ids, int64_t nk, int expert_start, int e_local, int mtp,
+                                  int row_align, int32_t* counts, int32_t* counters, int32_t* cu,
+                                  int32_t* pos, int extra_count, int64_t extra_start, void* ws,
+                                  size_t ws_bytes, hipStream_t st) {
+  PermArgs a{};
+  a.ids = ids; a.nk = nk; a.expert_start = expert_start; a.e_local = e_local; a.mtp = mtp;
+  a.row_align = row_align; a.counts = counts; a.counters = counters; a.cu = cu; a.pos = pos;
+  a.extra_count = extra_count; a.extra_start = extra_start;
+  return run_index(a, ws, ws_bytes, st);
+}
 
 extern "C" size_t bgmoe_dispatch_workspace_bytes(int64_t nk, int num_local_experts) {
   if (nk <= kChunk || num_local_experts <= 0) return 0;
@@ -265,6 +294,7 @@ extern "C" int bgmoe_dispatch_scatter_3d(const uint16_t* x, const int32_t* topk_
   a.ids = topk_ids; a.nk = (int64_t)n * k; a.expert_start = expert_start;
   a.e_local = num_local_experts; a.mtp = max_tokens_padded; a.row_align = 1;
   a.counts = expert_counts; a.counters = expert_counters; a.cu = nullptr; a.pos = topk_pos;
+  a.extra_count = -1;
   int rc = run_index(a, workspace, workspace_bytes, bgmoe_stream(stream));
   if (rc != BGMOE_OK || act_buffer == nullptr) return rc;
   BGMOE_REQUIRE(n == 0 || x, "dispatch_scatter_3d: null x");
@@ -296,7 +326,7 @@ extern "C" int bgmoe_dispatch_scatter_ragged(const uint16_t* x, const int32_t* t
   PermArgs a{};
   a.ids = topk_ids; a.nk = nk; a.expert_start = expert_start; a.e_local = num_local_experts;
   a.mtp = 0; a.row_align = row_align; a.counts = expert_counts; a.counters = expert_counters;
-  a.cu = cu_seqlens; a.pos = topk_pos;
+  a.cu = cu_seqlens; a.pos = topk_pos; a.extra_count = -1;
   int rc = run_index(a, workspace, workspace_bytes, bgmoe_stream(stream));
   if (rc != BGMOE_OK || act_buffer == nullptr) return rc;
   BGMOE_REQUIRE(n == 0 || x, "dispatch_scatter_ragged: null x");
@@ -310,6 +340,7 @@ extern "C" int bgmoe_compact_expert_data(const int32_t* expert_counts, int e, in
   BGMOE_REQUIRE(num_active, "compact_expert_data: null num_active");
   BGMOE_REQUIRE(e == 0 || (expert_counts && group_size && activated_group_idx && group_start_indices),
                 "compact_expert_data: null pointer");
+  BgmoeProf prof(BGMOE_K_COMPACT, bgmoe_stream(stream));
   hipLaunchKernelGGL(compact_kernel, dim3(1), dim3(64), 0, bgmoe_stream(stream), expert_counts, e,
                      group_size, activated_group_idx, group_start_indices, num_active);
   return bgmoe_check_launch("compact_expert_data");

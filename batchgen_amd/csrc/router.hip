@@ -208,6 +208,7 @@ int launch_router(const RouterArgs& a, hipStream_t st) {
   const dim3 grid((a.n + 3) / 4), block(256);
   const size_t lds = GROUPED ? (size_t)4 * a.e * sizeof(float) : 0;
   const int vpl = (a.e + 63) / 64;
+  BgmoeProf prof(BGMOE_K_ROUTER, st);
 #define BGMOE_ROUTER_CASE(V)                                                              \
   hipLaunchKernelGGL((router_kernel<V, GROUPED>), grid, block, lds, st, a)
   if (vpl <= 1) BGMOE_ROUTER_CASE(1);

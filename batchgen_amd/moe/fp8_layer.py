@@ -1,0 +1,143 @@
+"""FP8 MoE layer forward on one GPU's share of the experts.
+
+Host-side counterpart of the reference's layer glue: the abstract template
+``MoEBase`` (batchgen/moe/moe_base.py:188-264: gate -> expert compute -> shared
+expert) with the buffer discipline of ``Glm5MoE3DBuffers``
+(batchgen/models/glm/glm5/model.py:1241-1428): every buffer is allocated once
+at construction, the forward allocates nothing and never synchronises.
+The collectives of the reference template are out of scope (one GPU).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from .._lib import Fp8Weight, check, lib, ptr, stream
+from ..workloads import MoEConfig
+from .dispatch_scatter_3d import ragged_row_capacity
+
+vp, i32, i64, f32, sz = _lib.vp, _lib.i32, _lib.i64, _lib.f32, _lib.sz
+
+
+class LayerStruct(C.Structure):
+    """bgmoe_moe_fp8_layer (include/bgmoe.h)"""
+    _fields_ = [
+        ("n", i32), ("h", i32), ("inter", i32), ("e_total", i32), ("e_local", i32), ("expert_start", i32),
+        ("top_k", i32), ("n_group", i32), ("topk_group", i32), ("rsf", f32),
+        ("layout", i32), ("max_tokens", i32), ("row_align", i32),
+        ("has_shared", i32), ("shared_folded", i32), ("shared_inter", i32), ("shared_mode", i32),
+        ("cap_rows", i64),
+        ("x", vp), ("logits", vp), ("bias", vp),
+        ("gate", Fp8Weight), ("up", Fp8Weight), ("down", Fp8Weight),
+        ("sh_gate", Fp8Weight), ("sh_up", Fp8Weight), ("sh_down", Fp8Weight),
+        ("topk_ids", vp), ("topk_weights", vp), ("expert_counts", vp), ("cu_seqlens", vp), ("topk_pos", vp),
+        ("xq", vp), ("xs", vp), ("hq", vp), ("hs", vp), ("shq", vp), ("shs", vp), ("y", vp),
+        ("workspace", vp), ("workspace_bytes", sz), ("out", vp),
+    ]
+
+
+_lib.register("bgmoe_moe_fp8_layer_forward", i32, [C.POINTER(LayerStruct), vp])
+
+
+def _stack_desc(q: torch.Tensor, s: torch.Tensor) -> Fp8Weight:
+    e, n, k = q.shape
+    return Fp8Weight(ptr(q), n * k, None, ptr(s), s.size(1) * s.size(2), s.size(2), None)
+
+
+class Fp8MoELayer:
+    """forward(hidden_states [N,H] bf16, router_logits [N,E] fp32) -> [N,H] bf16.
+
+    ``weights``: dict(gate_q [E_l,I,H] e4m3fn, gate_s [E_l,I/128,H/128] fp32, up_q, up_s,
+    down_q [E_l,H,I], down_s); ``shared``: same keys with one leading group, or None.
+    ``bias``: the router's score-correction bias [E] fp32.
+    """
+
+    def __init__(self, cfg: MoEConfig, weights, shared, bias: torch.Tensor, max_tokens_in: Optional[int] = None,
+                 shared_mode: str = "bf16_add", fold_shared: bool = True):
+        self.cfg = cfg
+        dev = weights["gate_q"].device
+        self.device = dev
+        self.n_max = int(max_tokens_in or cfg.n_tokens)
+        n, h, inter, el, k = self.n_max, cfg.hidden, cfg.inter, cfg.e_local, cfg.top_k
+        self.weights, self.shared = weights, shared
+        self.bias = bias.to(dev, torch.float32).contiguous()
+        self.masked = cfg.layout == "masked"
+        self.cap_rows = el * cfg.max_tokens if self.masked else ragged_row_capacity(n, k, el, cfg.row_align)
+        has_shared = shared is not None
+        self.folded = bool(has_shared and fold_shared and cfg.shared_inter == inter)
+        rows = self.cap_rows + (n if has_shared else 0)
+        e8, f4, i4, b2 = torch.uint8, torch.float32, torch.int32, torch.bfloat16
+        self.topk_ids = torch.empty((n, k), dtype=i4, device=dev)
+        self.topk_weights = torch.empty((n, k), dtype=f4, device=dev)
+        self.expert_counts = torch.zeros(el + 1, dtype=i4, device=dev)
+        self.cu_seqlens = torch.zeros(el + 2, dtype=i4, device=dev)
+        self.topk_pos = torch.empty(n * k, dtype=i4, device=dev)
+        self.xq = torch.zeros((rows, h), dtype=e8, device=dev)
+        self.xs = torch.zeros((rows, h // 128), dtype=f4, device=dev)
+        self.hq = torch.zeros((rows, inter), dtype=e8, device=dev)
+        self.hs = torch.zeros((rows, inter // 128), dtype=f4, device=dev)
+        self.y = torch.zeros((rows, h), dtype=b2, device=dev)
+        self.out = torch.empty((n, h), dtype=b2, device=dev)
+        self.shq = self.shs = None
+        if has_shared and not self.folded:
+            self.shq = torch.zeros((n, cfg.shared_inter), dtype=e8, device=dev)
+            self.shs = torch.zeros((n, cfg.shared_inter // 128), dtype=f4, device=dev)
+        ws_bytes = int(lib().bgmoe_dispatch_workspace_bytes(n * k, el))
+        self.workspace = torch.empty(max(ws_bytes, 16), dtype=e8, device=dev)
+
+        L = LayerStruct()
+        L.h, L.inter, L.e_total, L.e_local, L.expert_start = h, inter, cfg.n_experts, el, cfg.expert_start
+        L.top_k, L.n_group, L.topk_group, L.rsf = k, cfg.n_group, cfg.topk_group, cfg.rsf
+        L.layout, L.max_tokens, L.row_align = (0 if self.masked else 1), cfg.max_tokens, max(cfg.row_align, 1)
+        L.has_shared, L.shared_folded, L.shared_inter = int(has_shared), int(self.folded), cfg.shared_inter
+        L.shared_mode = {"bf16_add": 0, "fp32_add": 1}[shared_mode]
+        L.cap_rows = self.cap_rows
+        L.bias = ptr(self.bias)
+        if self.folded:
+            # one pointer table per matrix: local experts then the shared expert
+            self._tables = {}
+            for name in ("gate", "up", "down"):
+                q, s = weights[name + "_q"], weights[name + "_s"]
+                sq, ss = shared[name + "_q"], shared[name + "_s"]
+                wp = [q[i].data_ptr() for i in range(el)] + [sq[0].data_ptr()]
+                sp = [s[i].data_ptr() for i in range(el)] + [ss[0].data_ptr()]
+                tw = torch.tensor(wp, dtype=torch.int64, device=dev)
+                ts = torch.tensor(sp, dtype=torch.int64, device=dev)
+                self._tables[name] = (tw, ts)
+                setattr(L, name, Fp8Weight(None, 0, ptr(tw), None, 0, s.size(2), ptr(ts)))
+        else:
+            for name in ("gate", "up", "down"):
+                setattr(L, name, _stack_desc(weights[name + "_q"], weights[name + "_s"]))
+            if has_shared:
+                for name in ("gate", "up", "down"):
+                    setattr(L, "sh_" + name, _stack_desc(shared[name + "_q"], shared[name + "_s"]))
+                L.shq, L.shs = ptr(self.shq), ptr(self.shs)
+        L.topk_ids, L.topk_weights = ptr(self.topk_ids), ptr(self.topk_weights)
+        L.expert_counts, L.cu_seqlens, L.topk_pos = ptr(self.expert_counts), ptr(self.cu_seqlens), ptr(self.topk_pos)
+        L.xq, L.xs, L.hq, L.hs, L.y = ptr(self.xq), ptr(self.xs), ptr(self.hq), ptr(self.hs), ptr(self.y)
+        L.workspace, L.workspace_bytes = ptr(self.workspace), self.workspace.numel()
+        L.out = ptr(self.out)
+        self._L = L
+        self._fn = lib().bgmoe_moe_fp8_layer_forward
+
+    def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+        cfg = self.cfg
+        if hidden_states.dtype != torch.bfloat16 or hidden_states.dim() != 2 or hidden_states.size(1) != cfg.hidden:
+            raise RuntimeError(f"hidden_states must be BF16 [N, {cfg.hidden}]")
+        n = hidden_states.size(0)
+        if n > self.n_max:
+            raise RuntimeError(f"{n} tokens exceed the {self.n_max} this layer's buffers were sized for")
+        if router_logits.dtype != torch.float32 or tuple(router_logits.shape) != (n, cfg.n_experts):
+            raise RuntimeError(f"router_logits must be FP32 [{n}, {cfg.n_experts}]")
+        if not (hidden_states.is_contiguous() and router_logits.is_contiguous()):
+            raise RuntimeError("hidden_states and router_logits must be contiguous")
+        L = self._L
+        L.n = n
+        L.x, L.logits = ptr(hidden_states), ptr(router_logits)
+        check(self._fn(C.byref(L), stream()))
+        return self.out[:n]
+
+    __call__ = forward

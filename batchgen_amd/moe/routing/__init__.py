@@ -1,0 +1,6 @@
+from .cuda_routing import (  # noqa: F401
+    dispatch_count_gather_cuda,
+    gate_sigmoid_topk_cuda,
+    gate_sigmoid_topk_warp_cuda,
+    reduce_weighted_scatter_cuda,
+)

@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE expert-layer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1]
+
+A step is one forward pass of the layer (router -> permute+quant -> gate_up/SwiGLU/
+requant GEMM -> down GEMM -> combine + shared expert) over one batch of synthetic
+tokens, with weights and inputs already resident in HBM.  Default workload is
+config 1 of BASELINE.json (DeepSeek-V3-shaped FP8 decode, 256 tokens, 32 of 256
+experts local, masked layout).  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
+FP8_PEAK_TFLOPS = 5000.0        # MI355X published dense FP8 MFMA peak
+
+METRIC = "MoE layer TFLOP/s (FP8 prefill) & HBM GB/s (decode), % roofline, 1xMI355X"
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 4])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def cpu_baseline(cfg, inp, w, sh, ids, wt, alg_bytes, flops):
+    """The reference's CPU-runnable PyTorch path (oracle.layer.moe_layer_l1_torch) on the host cores."""
+    import numpy as np
+    import torch
+    from oracle import layer as ol
+
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+
+    def deq(q, s):     # deepseek_v3_dequantization -> bf16, per expert to bound memory
+        n, k = q.shape[-2:]
+        v = q.to(torch.float32).view(n // 128, 128, k // 128, 128) * s[:, None, :, None]
+        return v.view(n, k).to(torch.bfloat16)
+
+    # bounded sample: at most 8192 tokens and the experts those tokens use
+    n = min(cfg.n_tokens, 8192)
+    x = inp["x"][:n].cpu()
+    ids_n, wt_n = ids[:n], wt[:n]
+    used = np.unique(ids_n)
+    experts = []
+    for e in range(cfg.e_local):
+        if (e + cfg.expert_start) in used:
+            experts.append(tuple(deq(w[k + "_q"][e].cpu(), w[k + "_s"][e].cpu()) for k in ("gate", "up", "down")))
+        else:
+            experts.append(None)
+    shared = None
+    if sh is not None:
+        shared = tuple(deq(sh[k + "_q"][0].cpu(), sh[k + "_s"][0].cpu()) for k in ("gate", "up", "down"))
+    dummy = torch.zeros(1, 1, dtype=torch.bfloat16)
+    experts = [e if e is not None else (dummy, dummy, dummy) for e in experts]
+    reps = 3
+    ol.moe_layer_l1_torch(x, ids_n, wt_n, experts, cfg.expert_start, shared)
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        ol.moe_layer_l1_torch(x, ids_n, wt_n, experts, cfg.expert_start, shared)
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[len(ts) // 2]
+    frac = n / cfg.n_tokens
+    return t, threads, cores, f"{n} of {cfg.n_tokens} tokens of the workload, all experts they route to, " \
+                              f"bf16 dequantised weights, 1 warm-up + median of {reps}", frac
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU's expert-parallel share; this build has no multi-GPU path "
+              "(run with --gpus 1).", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    from batchgen_amd import _lib, workloads as wl
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = wl.CONFIGS[a.config]
+    inp = wl.make_inputs(cfg, dev)
+    w, sh = wl.make_fp8_weights(cfg, dev)
+    layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
+    x, logits = inp["x"], inp["logits"]
+
+    for _ in range(a.warmup):
+        layer(x, logits)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(a.steps):
+        layer(x, logits)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / a.steps
+
+    counts = layer.expert_counts[:cfg.e_local].cpu().numpy()
+    active = int((counts > 0).sum())
+    rows = int(counts.sum())
+    alg_bytes = wl.algorithmic_bytes_fp8(cfg, active, rows)
+    flops = wl.flops_routed(cfg, rows) + (wl.flops_routed(cfg, cfg.n_tokens) * cfg.shared_inter // cfg.inter
+                                          if cfg.shared_inter else 0)
+    decode = cfg.layout == "masked"
+    gbps = alg_bytes / (ms * 1e-3) / 1e9
+    tflops = flops / (ms * 1e-3) / 1e12
+
+    # second timed pass with per-launch HIP events -> duration of the dominant kernel
+    _lib.prof_enable(True)
+    for _ in range(a.steps):
+        layer(x, logits)
+    prof = _lib.prof_collect()
+    _lib.prof_enable(False)
+    per_kernel = {k: v[0] / a.steps for k, v in prof.items()}          # ms per step
+    h, i = cfg.hidden, cfg.inter
+    if decode:
+        dom = "s1_skinny16"
+        served = int(((counts > 0) & (counts <= 16)).sum())
+        dom_bytes = served * (2 * h * i + 2 * (h // 128) * (i // 128) * 4) + \
+            int(counts[(counts > 0) & (counts <= 16)].sum()) * (h + h // 128 * 4 + i + i // 128 * 4)
+        dom_ms = prof[dom][0] / max(prof[dom][1], 1)
+        roof = dict(bound="hbm", kernel="fp8_skinny_kernel<1,3,fused>", achieved=dom_bytes / (dom_ms * 1e-3) / 1e9,
+                    peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=dom_bytes,
+                    avg_launch_us=dom_ms * 1e3)
+    else:
+        dom = "s1_tiled"
+        big = counts[counts > 64].sum()
+        dom_flops = int(big) * 4 * h * i + (cfg.n_tokens * 4 * h * cfg.shared_inter if cfg.shared_inter else 0)
+        dom_ms = prof[dom][0] / max(prof[dom][1], 1)
+        roof = dict(bound="mfma", kernel="fp8_tiled_kernel<fused>", achieved=dom_flops / (dom_ms * 1e-3) / 1e12,
+                    peak=FP8_PEAK_TFLOPS, unit="TFLOP/s", traffic=None, flops_per_launch=dom_flops,
+                    avg_launch_us=dom_ms * 1e3)
+    roof["frac"] = roof["achieved"] / roof["peak"]
+
+    out = {
+        "metric": METRIC,
+        "value": gbps if decode else tflops,
+        "unit": "GB/s" if decode else "TFLOP/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": cfg.name, "tokens": cfg.n_tokens, "hidden": h, "moe_intermediate": i,
+                   "experts": cfg.n_experts, "local_experts": cfg.e_local, "top_k": cfg.top_k,
+                   "layout": cfg.layout, "shared_expert": bool(cfg.shared_inter)},
+        "tokens_per_s": cfg.n_tokens / (ms * 1e-3),
+        "layer_hbm_GBps": gbps, "layer_TFLOPs": tflops,
+        "layer_frac_of_hbm_peak": gbps / HBM_PEAK_GBPS, "layer_frac_of_fp8_peak": tflops / FP8_PEAK_TFLOPS,
+        "algorithmic_bytes": alg_bytes, "flops": flops, "active_local_experts": active, "routed_rows": rows,
+        "kernel_ms_per_step": per_kernel,
+        "roofline": roof,
+    }
+    if not a.no_cpu_baseline:
+        ids = layer.topk_ids.cpu().numpy()
+        wt = layer.topk_weights.cpu().numpy()
+        t, threads, cores, sample, frac = cpu_baseline(cfg, inp, w, sh, ids, wt, alg_bytes, flops)
+        v = (alg_bytes * frac / t / 1e9) if decode else (flops * frac / t / 1e12)
+        out["cpu_baseline"] = {"value": v, "unit": out["unit"], "cores": threads, "host_cores": cores,
+                               "kind": "port", "sample": sample, "seconds": t,
+                               "tokens_per_s": cfg.n_tokens * frac / t}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

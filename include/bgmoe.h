@@ -36,6 +36,17 @@ enum {
 const char* bgmoe_last_error(void);
 int bgmoe_version(void);
 
+/* Per-launch timing for benchmarks.  bgmoe_prof_enable(1) brackets every kernel
+ * launch with HIP events on its stream; bgmoe_prof_collect synchronises the
+ * device and returns, per kernel id in [0, bgmoe_prof_kernel_count()), the total
+ * elapsed milliseconds and number of launches since the last collect.  No
+ * reference counterpart (the reference times spans with CUDA-event pairs in
+ * Python, batchgen/timing.py:1-60). */
+int bgmoe_prof_enable(int on);
+int bgmoe_prof_kernel_count(void);
+const char* bgmoe_prof_kernel_name(int id);
+int bgmoe_prof_collect(double* total_ms, int64_t* launches, int n);
+
 /* ------------------------------------------------------------------ router */
 
 /* Group-limited top-k on (optionally already sigmoided) scores.
@@ -228,6 +239,59 @@ int bgmoe_fp8_fused_s1(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* gate,
                        uint16_t* out, uint8_t* out_q, float* out_scale,
                        int64_t out_scale_row_stride, int64_t out_scale_nb_stride,
                        bgmoe_stream_t stream);
+
+/* ------------------------------------------------------------ whole layer */
+
+/* One FP8 MoE layer forward on one GPU's share of the experts:
+ *   router (sigmoid + bias, group-limited when n_group > 1, else ungrouped)
+ *   -> stable permute into the masked [E_l, max_tokens, H] layout (layout 0) or
+ *      the contiguous ragged layout (layout 1, starts aligned to row_align)
+ *   -> act-quant fused into the scatter -> fused gate_up/SwiGLU/requant GEMM
+ *   -> down GEMM -> top-k weighted combine + shared expert -> out [n,h] bf16.
+ * Replaces the op sequence of `WGMMAMoEBuffers.forward`
+ * (batchgen/moe/fp8_wgmma_pipeline.py:294-372) plus the gate and shared expert
+ * of `DeepseekV3MoE_Decoding_FP8.forward`
+ * (batchgen/models/deepseek/deepseekv3/modeling_deepseek_v3.py:1924-1940).
+ * Every buffer is caller-owned; nothing is allocated and nothing is read back.
+ *
+ * Row space of xq/xs/hq/hs/y: [0, cap_rows) routed rows, then n rows of the
+ * shared expert (identity permutation) when has_shared.
+ *   masked: cap_rows = e_local*max_tokens; ragged: cap_rows >= worst case of
+ *   bgmoe_dispatch_scatter_ragged.
+ * Weights: routed = groups [0,e_local).  shared_folded != 0: gate/up/down are
+ * pointer tables with e_local+1 entries, entry e_local being the shared expert
+ * (same inter), and all experts run in one grouped launch.  Otherwise the
+ * shared expert comes in sh_* (1 group) and runs as launches of its own. */
+typedef struct bgmoe_moe_fp8_layer {
+  int32_t n, h, inter, e_total, e_local, expert_start;
+  int32_t top_k, n_group, topk_group;
+  float routed_scaling_factor;
+  int32_t layout, max_tokens, row_align;
+  int32_t has_shared, shared_folded, shared_inter, shared_mode;
+  int64_t cap_rows;
+  const uint16_t* x;          /* [n,h] bf16            */
+  const float* logits;        /* [n,e_total] fp32      */
+  const float* bias;          /* [e_total] fp32        */
+  bgmoe_fp8_weight gate, up, down;
+  bgmoe_fp8_weight sh_gate, sh_up, sh_down;
+  int32_t* topk_ids;          /* [n,top_k]             */
+  float* topk_weights;        /* [n,top_k]             */
+  int32_t* expert_counts;     /* [e_local+1]           */
+  int32_t* cu_seqlens;        /* [e_local+2]           */
+  int32_t* topk_pos;          /* [n*top_k]             */
+  uint8_t* xq;                /* [rows,h]              */
+  float* xs;                  /* [rows,h/128]          */
+  uint8_t* hq;                /* [rows,inter]          */
+  float* hs;                  /* [rows,inter/128]      */
+  uint8_t* shq;               /* [n,shared_inter]  (unfolded shared only) */
+  float* shs;                 /* [n,shared_inter/128]                     */
+  uint16_t* y;                /* [rows,h] bf16         */
+  void* workspace;            /* bgmoe_dispatch_workspace_bytes(n*top_k, e_local) */
+  size_t workspace_bytes;
+  uint16_t* out;              /* [n,h] bf16            */
+} bgmoe_moe_fp8_layer;
+
+int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* layer, bgmoe_stream_t stream);
 
 #ifdef __cplusplus
 }

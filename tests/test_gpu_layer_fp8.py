@@ -1,0 +1,101 @@
+"""Whole FP8 MoE layer on the GPU vs the CPU oracle.
+
+Integer / byte results (router ids, counts, cu_seqlens, topk_pos, quantised activation bytes and scales) are
+bit-exact; the layer output is within 1e-2 relative Frobenius error of the fp32 dequantise-then-matmul oracle
+(the bound BASELINE.json states), in practice ~1e-3.
+"""
+import numpy as np
+import pytest
+import torch
+
+from batchgen_amd import workloads as wl
+from oracle import gemm as og
+from oracle import layer as ol
+from tests.util import say
+
+pytestmark = pytest.mark.gpu
+
+SMALL = {
+    "c0": wl.CONFIGS[0],
+    "c1_small": wl.scaled(wl.CONFIGS[1], hidden=1024, inter=512, shared_inter=512),
+    "c1_unfolded_shared": wl.scaled(wl.CONFIGS[1], hidden=512, inter=512, shared_inter=256, n_tokens=100),
+    "c2_small": wl.scaled(wl.CONFIGS[2], hidden=512, inter=256, shared_inter=256, n_tokens=3000),
+    "c4_small": wl.scaled(wl.CONFIGS[4], hidden=256, inter=256, shared_inter=256, n_tokens=2048),
+    "ungrouped_fp8": wl.scaled(wl.CONFIGS[1], hidden=512, inter=256, shared_inter=0, n_group=1, topk_group=1,
+                               n_experts=384, e_local=48, expert_start=96, n_tokens=77, max_tokens=128),
+}
+
+
+def _rcfg(cfg):
+    return dict(top_k=cfg.top_k, n_group=cfg.n_group, topk_group=cfg.topk_group, rsf=cfg.rsf)
+
+
+@pytest.mark.parametrize("name", list(SMALL))
+def test_layer_matches_oracle(dev, name):
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = SMALL[name]
+    say("layer", name)
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    wd = {k: v.to(dev) for k, v in w.items()}
+    shd = {k: v.to(dev) for k, v in sh.items()} if sh else None
+    layer = Fp8MoELayer(cfg, wd, shd, inp["bias"].to(dev))
+    out = layer(inp["x"].to(dev), inp["logits"].to(dev))
+    torch.cuda.synchronize()
+    ref = ol.moe_layer_fp8(inp["x"], inp["logits"].numpy(), inp["bias"].numpy(), _rcfg(cfg),
+                           wl.weights_to_numpy(w), cfg.expert_start, cfg.e_local, layout=cfg.layout,
+                           max_tokens=cfg.max_tokens, row_align=cfg.row_align, shared=wl.weights_to_numpy(sh))
+    el = cfg.e_local
+    assert np.array_equal(layer.topk_ids.cpu().numpy(), ref["ids"])
+    np.testing.assert_allclose(layer.topk_weights.cpu().numpy(), ref["weights"], rtol=2e-7, atol=0)
+    assert np.array_equal(layer.expert_counts[:el].cpu().numpy(), ref["counts"])
+    assert np.array_equal(layer.cu_seqlens[:el].cpu().numpy(), ref["cu"][:el])
+    assert np.array_equal(layer.topk_pos.cpu().numpy(), ref["pos"])
+    live = np.zeros(layer.cap_rows, dtype=bool)
+    for e in range(el):
+        live[ref["cu"][e]:ref["cu"][e] + ref["counts"][e]] = True
+    xq = layer.xq[:layer.cap_rows].cpu().numpy()
+    xs = layer.xs[:layer.cap_rows].cpu().numpy()
+    nrows = ref["xq"].shape[0]
+    assert np.array_equal(xq[:nrows][live[:nrows]], ref["xq"][live[:nrows]])
+    assert np.array_equal(xs[:nrows][live[:nrows]].view(np.uint32), ref["xs"][live[:nrows]].view(np.uint32))
+    if sh is not None:   # shared expert rows = quantised tokens
+        assert np.array_equal(layer.xq[layer.cap_rows:].cpu().numpy(), ref["xq_tok"])
+    err = og.rel_frobenius(out.float().cpu().numpy(), ref["out"])
+    say("   rel frobenius vs fp32 oracle:", err)
+    assert err < 1e-2
+    # intermediate requant: bytes may differ where fp32 accumulation order moves a value across a rounding
+    # boundary; they must agree almost everywhere
+    hq = layer.hq[:nrows].cpu().numpy()[live[:nrows]]
+    agree = (hq == ref["hq"][live[:nrows]]).mean() if hq.size else 1.0
+    say("   requant byte agreement:", agree)
+    assert agree > 0.97
+
+
+def test_layer_is_deterministic_and_reusable(dev):
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = SMALL["c1_small"]
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    layer = Fp8MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
+                        inp["bias"].to(dev))
+    x, lg = inp["x"].to(dev), inp["logits"].to(dev)
+    a = layer(x, lg).clone()
+    other = layer(x[:50].contiguous(), lg[:50].contiguous()).clone()      # fewer tokens, same buffers
+    b = layer(x, lg).clone()
+    assert torch.equal(a, b)
+    assert torch.equal(other, a[:50])                                     # tokens are independent
+
+
+def test_layer_rejects_bad_arguments(dev):
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = SMALL["c0"]
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    layer = Fp8MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
+                        inp["bias"].to(dev))
+    with pytest.raises(RuntimeError):
+        layer(inp["x"].to(dev).float(), inp["logits"].to(dev))
+    with pytest.raises(RuntimeError):
+        layer(torch.zeros((65, cfg.hidden), dtype=torch.bfloat16, device=dev),
+              torch.zeros((65, cfg.n_experts), device=dev))
