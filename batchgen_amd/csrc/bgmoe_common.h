@@ -51,6 +51,12 @@ struct BgmoeProf {
   ~BgmoeProf() { if (g_bgmoe_prof_on) bgmoe_prof_mark(id, st, false); }
 };
 
+// fused stage 1 when w1 != nullptr; row_bound = host-side upper bound on live rows (0 = m)
+int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
+                            const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
+                            uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
+                            int64_t row_bound, hipStream_t st);
+
 static inline hipStream_t bgmoe_stream(bgmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 
 // ---- bf16 <-> fp32 -----------------------------------------------------------
@@ -81,6 +87,22 @@ __device__ __forceinline__ float clamp448(float q) { return fmaxf(fminf(q, 448.0
 __device__ __forceinline__ float quant_scale_from_amax(float amax) {
   constexpr float kInv448 = 1.0f / 448.0f;
   return fmaxf(amax, 1e-12f) * kInv448;
+}
+
+// ---- explicit global-address-space loads --------------------------------------------
+// A pointer that was itself loaded from memory (a per-group pointer table) is a generic ("flat")
+// pointer to the compiler; flat loads count against both memory counters and force full waits.
+// These helpers assert the global address space so that the loads are global_load_* and
+// s_waitcnt vmcnt(N) can leave younger loads in flight.
+#define BGMOE_GLOBAL __attribute__((address_space(1)))
+__device__ __forceinline__ intx4 gload_x4(const void* p) {
+  return *reinterpret_cast<const BGMOE_GLOBAL intx4*>((uintptr_t)p);
+}
+__device__ __forceinline__ intx4 gload_x4_stream(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const BGMOE_GLOBAL intx4*>((uintptr_t)p));
+}
+__device__ __forceinline__ float gload_f32(const float* p) {
+  return *reinterpret_cast<const BGMOE_GLOBAL float*>((uintptr_t)p);
 }
 
 // ---- wave helpers ---------------------------------------------------------------

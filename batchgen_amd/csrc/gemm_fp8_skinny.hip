@@ -18,8 +18,19 @@
 // contiguous bytes per row.  D: lane l holds token (l % 16), features
 // 4*(l / 16) + 0..3.
 //
+// Weight layouts: TILE_MAJOR (see bgmoe.h) makes each of those loads one contiguous 1 KiB and a
+// wave's whole stream one contiguous region, which is what lets the kernel approach the HBM
+// roofline (DRAM pages are opened once); ROW_MAJOR is supported for the op-level API and reads
+// 64-byte pieces of 16 rows per load.
+//
+// Scheduling: the grid is sized for every (group, n-tile) but block b serves the b-th ACTIVE item,
+// found with a ballot scan of seqlens, so the blocks that have work are consecutive block ids and
+// the hardware dispatcher spreads them evenly over the CUs whatever the pattern of empty groups.
+//
 // Algorithmic bytes per group: n*k weight bytes (+ n*k/16384*4 scale bytes)
 // per matrix; activations (rows*k) are re-read per block from L2.
+#include <stdlib.h>
+
 #include "bgmoe_common.h"
 
 namespace {
@@ -35,6 +46,7 @@ struct SkinnyArgs {
   float* out_s;
   int64_t os_row, os_nb;
   int lo, hi;                 // this launch serves groups with lo < count <= hi
+  int64_t row_bound;          // host-side upper bound on the total live rows
 };
 
 template <int TT, int NSC>
@@ -46,32 +58,65 @@ struct Stage {
 };
 
 __device__ __forceinline__ intx8 load32(const uint8_t* p) {
-  const intx4 lo = *reinterpret_cast<const intx4*>(p);
-  const intx4 hi = *reinterpret_cast<const intx4*>(p + 64);
+  const intx4 lo = gload_x4(p);
+  const intx4 hi = gload_x4(p + 64);
   intx8 r;
   r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
   r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
   return r;
 }
 
+template <int HI>
 __device__ __forceinline__ intx8 load32_stream(const uint8_t* p) {
-  const intx4 lo = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(p));
-  const intx4 hi = __builtin_nontemporal_load(reinterpret_cast<const intx4*>(p + 64));
+  const intx4 lo = gload_x4_stream(p);
+  const intx4 hi = gload_x4_stream(p + HI);
   intx8 r;
   r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
   r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
   return r;
 }
 
-template <int TT, int NSTAGE, bool FUSED>
+// Work items of one launch: every group with lo < count <= hi contributes ceil(count / chunk_rows)
+// items (ascending group, ascending chunk).  Returns the group of item `item` and its chunk index,
+// or -1 when there are fewer items.  Wave-uniform; every wave of the block runs it redundantly.
+__device__ __forceinline__ int nth_active_item(const int32_t* seqlens, int groups, int lo, int hi,
+                                               int chunk_rows, int item, int* chunk) {
+  const int lane = threadIdx.x & 63;
+  int base = 0;
+  for (int g0 = 0; g0 < groups; g0 += 64) {
+    const int gi = g0 + lane;
+    const int c = gi < groups ? seqlens[gi] : 0;
+    const int mine = (c > lo && c <= hi) ? (c + chunk_rows - 1) / chunk_rows : 0;
+    int inc = mine;                                  // inclusive prefix sum over the wave
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(inc, off, BGMOE_WAVE);
+      if (lane >= off) inc += up;
+    }
+    const int total = __shfl(inc, 63, BGMOE_WAVE);
+    if (item < base + total) {
+      const int rel = item - base;
+      const unsigned long long hit = __ballot(mine > 0 && rel >= inc - mine && rel < inc);
+      const int src = __ffsll((long long)hit) - 1;
+      *chunk = rel - __shfl(inc - mine, src, BGMOE_WAVE);
+      return g0 + src;
+    }
+    base += total;
+  }
+  return -1;
+}
+
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
   constexpr int NT = 4;                  // weight tiles per wave
   constexpr int NSC = FUSED ? 2 : 1;     // weight-scale streams per wave
   __shared__ float s_amax[4][TT][16];
 
-  const int grp = blockIdx.y;
+  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
+  int chunk = 0;
+  const int grp = nth_active_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, blockIdx.x / ntiles, &chunk);
+  if (grp < 0) return;                            // whole block: fewer items than the grid allows
   const int cnt = g.seqlens[grp];
-  if (cnt <= g.lo || cnt > g.hi) return;          // whole block
   const int64_t row0 = g.cu[grp];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -79,7 +124,7 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
   const int kq = lane >> 4;
   const int K = g.k;
   const int KB = K >> 7;
-  const int n0 = blockIdx.x * (FUSED ? 128 : 256);
+  const int n0 = (blockIdx.x % ntiles) * (FUSED ? 128 : 256);
 
   const uint8_t* wb[2];
   const float* wsb[2];
@@ -96,7 +141,11 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
   for (int t = 0; t < NT; ++t) {
     const int nrow = FUSED ? n0 + 32 * wave + 16 * (t & 1) : n0 + 64 * wave + 16 * t;
     tv[t] = nrow < g.n;
-    wp[t] = wb[FUSED ? (t >> 1) : 0] + (int64_t)(nrow + r16) * K + 16 * kq;
+    // a tile past N streams the last valid tile instead (its results are never stored): every load
+    // below is unconditional, which lets the compiler keep precise vmcnt() waits
+    const int nr = min(nrow, g.n - 16);
+    if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) wp[t] = wb[FUSED ? (t >> 1) : 0] + (int64_t)(nr + r16) * K + 16 * kq;
+    else wp[t] = wb[FUSED ? (t >> 1) : 0] + (int64_t)(nr >> 4) * K * 16 + lane * 16;
   }
   const float* wsp[NSC];
   if constexpr (FUSED) {
@@ -107,7 +156,8 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
     wsp[0] = wsb[0] + (int64_t)nb * g.w0.scale_nb_stride;
   }
 
-  for (int t0 = 0; t0 < cnt; t0 += 16 * TT) {
+  {
+    const int t0 = chunk * 16 * TT;
     const uint8_t* xp[TT];
     const float* xsp[TT];
     bool xv[TT];
@@ -115,7 +165,7 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
     for (int tt = 0; tt < TT; ++tt) {
       const int tok = t0 + 16 * tt + r16;
       xv[tt] = tok < cnt;
-      const int64_t r = row0 + (xv[tt] ? tok : 0);
+      const int64_t r = row0 + (xv[tt] ? tok : 0);     // cnt >= 1 here
       xp[tt] = g.a.x + r * K + 16 * kq;
       xsp[tt] = g.a.scale + r * g.a.scale_row_stride;
     }
@@ -127,52 +177,50 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
       for (int t = 0; t < NT; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     Stage<TT, NSC> st[NSTAGE];
+    // tokens past the count re-read the group's first row; their columns are never stored
     auto load_stage = [&](Stage<TT, NSC>& s, int kb) {
       const int ko = kb << 7;
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        if (tv[t]) s.A[t] = load32_stream(wp[t] + ko);
-        else s.A[t] = intx8{0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) s.A[t] = load32_stream<64>(wp[t] + ko);
+        else s.A[t] = load32_stream<1024>(wp[t] + ((int64_t)kb << 11));
       }
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) {
-        if (xv[tt]) {
-          s.B[tt] = load32(xp[tt] + ko);
-          s.xs[tt] = xsp[tt][(int64_t)kb * g.a.scale_kb_stride];
-        } else {
-          s.B[tt] = intx8{0, 0, 0, 0, 0, 0, 0, 0};
-          s.xs[tt] = 0.0f;
-        }
+        s.B[tt] = load32(xp[tt] + ko);
+        s.xs[tt] = gload_f32(xsp[tt] + (int64_t)kb * g.a.scale_kb_stride);
       }
 #pragma unroll
-      for (int i = 0; i < NSC; ++i) s.ws[i] = wsp[i][kb];
+      for (int i = 0; i < NSC; ++i) s.ws[i] = gload_f32(wsp[i] + kb);
+    };
+    auto compute = [&](const Stage<TT, NSC>& c) {
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+              c.A[t], c.B[tt], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+          const float sc = c.xs[tt] * c.ws[FUSED ? (t >> 1) : 0];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[tt][t][i] = fmaf(p[i], sc, acc[tt][t][i]);
+        }
+      }
     };
 
+    // software pipeline, NSTAGE-1 K-blocks ahead; prefetches past the end re-read the last block
 #pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s)
-      if (s < KB) load_stage(st[s], s);
-
-    for (int kb0 = 0; kb0 < KB; kb0 += NSTAGE) {
+    for (int s = 0; s < NSTAGE - 1; ++s) load_stage(st[s], min(s, KB - 1));
+    const int kb_main = KB - KB % NSTAGE;
+    for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
 #pragma unroll
       for (int s = 0; s < NSTAGE; ++s) {
-        const int kb = kb0 + s;
-        if (kb < KB) {
-          if (kb + NSTAGE - 1 < KB) load_stage(st[(s + NSTAGE - 1) % NSTAGE], kb + NSTAGE - 1);
-          const Stage<TT, NSC>& c = st[s];
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) {
-#pragma unroll
-            for (int t = 0; t < NT; ++t) {
-              const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                  c.A[t], c.B[tt], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-              const float sc = c.xs[tt] * c.ws[FUSED ? (t >> 1) : 0];
-#pragma unroll
-              for (int i = 0; i < 4; ++i) acc[tt][t][i] = fmaf(p[i], sc, acc[tt][t][i]);
-            }
-          }
-        }
+        load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
+        compute(st[s]);
       }
     }
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; ++s)
+      if (kb_main + s < KB) compute(st[s]);
 
     // ---- epilogue -------------------------------------------------------------
     if constexpr (FUSED) {
@@ -222,7 +270,6 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
               g.out_s[(row0 + tok) * g.os_row + (int64_t)(n0 >> 7) * g.os_nb] = sc;
           }
         }
-        __syncthreads();   // s_amax is reused by the next pass
       }
     } else {
 #pragma unroll
@@ -269,26 +316,68 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
                            uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
                            int lo, hipStream_t st);
 
+template <int TT, int NS>
+static void launch_variant(bool fused, int layout, dim3 grid, const SkinnyArgs& g, hipStream_t st) {
+  const dim3 block(256);
+  if (fused) {
+    if (layout == BGMOE_W_TILE_MAJOR) hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, true, BGMOE_W_TILE_MAJOR>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, true, BGMOE_W_ROW_MAJOR>), grid, block, 0, st, g);
+  } else {
+    if (layout == BGMOE_W_TILE_MAJOR) hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, false, BGMOE_W_TILE_MAJOR>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, false, BGMOE_W_ROW_MAJOR>), grid, block, 0, st, g);
+  }
+}
+
+// Rows per group up to which the weight-streaming kernel is used (each 32-row chunk of a group
+// streams the group's weights once more, mostly from the last-level cache); groups with more
+// rows go to the LDS-tiled kernel.
+static int skinny_limit() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("BGMOE_SKINNY_MAX_ROWS");
+    v = e ? atoi(e) : 256;
+    if (v < 0) v = 0;
+  }
+  return v;
+}
+
 static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   const int ntile = fused ? 128 : 256;
-  const dim3 grid((g.n + ntile - 1) / ntile, g.groups), block(256);
-  // rows per group in (0,16], (16,64]; more rows go to the LDS-tiled kernel
-  g.lo = 0; g.hi = 16;
-  {
+  const int layout = g.w0.layout;
+  if (fused && g.w1.layout != layout) {
+    bgmoe_set_error("fp8_fused_s1: gate and up weights must use the same layout");
+    return BGMOE_ERR_ARG;
+  }
+  if (layout != BGMOE_W_ROW_MAJOR && layout != BGMOE_W_TILE_MAJOR) {
+    bgmoe_set_error("fp8 grouped gemm: unknown weight layout %d", layout);
+    return BGMOE_ERR_ARG;
+  }
+  const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
+  const int hi = skinny_limit();
+  if (hi > 0) {
+    constexpr int TT = 2;
+    const int64_t items = g.groups + bound / (16 * TT);           // >= sum of ceil(count / 32)
+    const dim3 grid((unsigned)(((g.n + ntile - 1) / ntile) * items));
+    g.lo = 0; g.hi = hi;
     BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
-    if (fused) hipLaunchKernelGGL((fp8_skinny_kernel<1, 3, true>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((fp8_skinny_kernel<1, 3, false>), grid, block, 0, st, g);
+    launch_variant<TT, 3>(fused, layout, grid, g, st);
+    int rc = bgmoe_check_launch("fp8 grouped gemm (skinny)");
+    if (rc != BGMOE_OK) return rc;
   }
-  if (m > 16) {
-    g.lo = 16; g.hi = 64;
-    BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY64 : BGMOE_K_GEMM_SKINNY64, st);
-    if (fused) hipLaunchKernelGGL((fp8_skinny_kernel<2, 3, true>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((fp8_skinny_kernel<2, 3, false>), grid, block, 0, st, g);
-  }
-  int rc = bgmoe_check_launch("fp8 grouped gemm (skinny)");
-  if (rc != BGMOE_OK || m <= 64) return rc;
+  if (bound <= hi) return BGMOE_OK;
   return bgmoe_launch_fp8_tiled(&g.a, &g.w0, fused ? &g.w1 : nullptr, g.seqlens, g.cu, g.groups, m, g.n,
-                                g.k, g.out, g.out_q, g.out_s, g.os_row, g.os_nb, 64, st);
+                                g.k, g.out, g.out_q, g.out_s, g.os_row, g.os_nb, hi, st);
+}
+
+int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
+                            const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
+                            uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
+                            int64_t row_bound, hipStream_t st) {
+  SkinnyArgs g{};
+  g.a = *a; g.w0 = *w0; if (w1) g.w1 = *w1;
+  g.seqlens = seqlens; g.cu = cu; g.groups = groups; g.n = n; g.k = k;
+  g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.row_bound = row_bound;
+  return launch_skinny(w1 != nullptr, g, m, st);
 }
 
 extern "C" int bgmoe_fp8_grouped_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* b,

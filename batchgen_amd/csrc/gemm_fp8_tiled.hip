@@ -42,7 +42,7 @@ struct TiledArgs {
 
 __device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
 
-template <bool FUSED>
+template <bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
   extern __shared__ __align__(16) uint8_t smem[];
   __shared__ int s_tiles[kMaxGroups + 1];       // exclusive prefix of m-tiles per group
@@ -125,13 +125,22 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
     const uint8_t* w_src[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int r = i * 32 + lrow;                 // LDS weight row 0..255
-      if constexpr (FUSED) {
-        const int nrow = min(n0 + (r & 127), g.n - 1);
-        w_src[i] = (r < 128 ? wb0 : wb1) + (int64_t)nrow * K + chunk * 16;
+      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
+        const int r = i * 32 + lrow;               // LDS weight row 0..255
+        if constexpr (FUSED) {
+          const int nrow = min(n0 + (r & 127), g.n - 1);
+          w_src[i] = (r < 128 ? wb0 : wb1) + (int64_t)nrow * K + chunk * 16;
+        } else {
+          const int nrow = min(n0 + r, g.n - 1);
+          w_src[i] = wb0 + (int64_t)nrow * K + chunk * 16;
+        }
       } else {
-        const int nrow = min(n0 + r, g.n - 1);
-        w_src[i] = wb0 + (int64_t)nrow * K + chunk * 16;
+        // tile-major source: LDS keeps the 2 KiB tile image; this thread moves 16 bytes of LDS tile
+        // 2*i + (tid >> 7) (16 weight rows each), a contiguous 2 KiB per 128 threads
+        const int lt = 2 * i + (tid >> 7);         // LDS tile 0..15
+        const int r = lt * 16;
+        const int nrow = FUSED ? min(n0 + (r & 127), g.n - 16) : min(n0 + r, g.n - 16);
+        w_src[i] = ((FUSED && r >= 128) ? wb1 : wb0) + (int64_t)(nrow >> 4) * K * 16 + (tid & 127) * 16;
       }
     }
     const float* xs_src = nullptr;
@@ -142,9 +151,10 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
     auto gload = [&](int kb) {
       const int ko = kb << 7;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) rt[i] = *reinterpret_cast<const intx4*>(tok_src[i] + ko);
+      for (int i = 0; i < 4; ++i) rt[i] = gload_x4(tok_src[i] + ko);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) rw[i] = *reinterpret_cast<const intx4*>(w_src[i] + ko);
+      for (int i = 0; i < 8; ++i)
+        rw[i] = gload_x4(w_src[i] + (LAYOUT == BGMOE_W_ROW_MAJOR ? (int64_t)ko : ((int64_t)kb << 11)));
       if (tid < TM) rxs = xs_src[(int64_t)kb * g.a.scale_kb_stride];
     };
     auto lstore = [&](int buf) {
@@ -152,8 +162,12 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) *reinterpret_cast<intx4*>(b + swz(i * 32 + lrow, chunk)) = rt[i];
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        *reinterpret_cast<intx4*>(b + kTokBytes + swz(i * 32 + lrow, chunk)) = rw[i];
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR)
+          *reinterpret_cast<intx4*>(b + kTokBytes + swz(i * 32 + lrow, chunk)) = rw[i];
+        else
+          *reinterpret_cast<intx4*>(b + kTokBytes + i * 4096 + tid * 16) = rw[i];
+      }
       if (tid < TM) reinterpret_cast<float*>(b + kTokBytes + kWBytes)[tid] = rxs;
     };
 
@@ -182,8 +196,14 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int wr = FUSED ? ((t >> 1) * 128 + 32 * wave + 16 * (t & 1) + r16) : (64 * wave + 16 * t + r16);
-        const intx4 lo = *reinterpret_cast<const intx4*>(bw + swz(wr, kq));
-        const intx4 hi = *reinterpret_cast<const intx4*>(bw + swz(wr, 4 + kq));
+        intx4 lo, hi;
+        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
+          lo = *reinterpret_cast<const intx4*>(bw + swz(wr, kq));
+          hi = *reinterpret_cast<const intx4*>(bw + swz(wr, 4 + kq));
+        } else {
+          lo = *reinterpret_cast<const intx4*>(bw + (wr >> 4) * 2048 + lane * 16);
+          hi = *reinterpret_cast<const intx4*>(bw + (wr >> 4) * 2048 + 1024 + lane * 16);
+        }
         A[t] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
 #pragma unroll
@@ -301,11 +321,16 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
       return BGMOE_ERR_HIP;
     }
     g_num_cu = prop.multiProcessorCount;
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tiled_kernel<true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kBufBytes);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&fp8_tiled_kernel<false>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kBufBytes);
-    if (e1 != hipSuccess || e2 != hipSuccess) {
+    hipError_t e1 = hipSuccess;
+    const void* fns[4] = {reinterpret_cast<const void*>(&fp8_tiled_kernel<true, 0>),
+                          reinterpret_cast<const void*>(&fp8_tiled_kernel<false, 0>),
+                          reinterpret_cast<const void*>(&fp8_tiled_kernel<true, 1>),
+                          reinterpret_cast<const void*>(&fp8_tiled_kernel<false, 1>)};
+    for (const void* f : fns) {
+      hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kBufBytes);
+      if (e != hipSuccess) e1 = e;
+    }
+    if (e1 != hipSuccess) {
       bgmoe_set_error("fp8 tiled gemm: cannot reserve %d bytes of LDS", 2 * kBufBytes);
       return BGMOE_ERR_HIP;
     }
@@ -319,7 +344,14 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   if (blocks > max_items) blocks = max_items;
   if (blocks < 8) blocks = 8;
   BgmoeProf prof(w1 ? BGMOE_K_S1_TILED : BGMOE_K_GEMM_TILED, st);
-  if (w1) hipLaunchKernelGGL((fp8_tiled_kernel<true>), dim3((unsigned)blocks), dim3(256), 2 * kBufBytes, st, g);
-  else hipLaunchKernelGGL((fp8_tiled_kernel<false>), dim3((unsigned)blocks), dim3(256), 2 * kBufBytes, st, g);
+  const dim3 grid((unsigned)blocks), block(256);
+  const bool tm = w0->layout == BGMOE_W_TILE_MAJOR;
+  if (w1) {
+    if (tm) hipLaunchKernelGGL((fp8_tiled_kernel<true, 1>), grid, block, 2 * kBufBytes, st, g);
+    else hipLaunchKernelGGL((fp8_tiled_kernel<true, 0>), grid, block, 2 * kBufBytes, st, g);
+  } else {
+    if (tm) hipLaunchKernelGGL((fp8_tiled_kernel<false, 1>), grid, block, 2 * kBufBytes, st, g);
+    else hipLaunchKernelGGL((fp8_tiled_kernel<false, 0>), grid, block, 2 * kBufBytes, st, g);
+  }
   return bgmoe_check_launch("fp8 grouped gemm (tiled)");
 }

@@ -67,23 +67,39 @@ def _act(x, x_scale, m_pad):
     return Fp8Act(ptr(x), ptr(x_scale), 1, m_pad)
 
 
-def _stacked(weight, w_scale):
+_LAYOUT = {"row_major": 0, "tile_major": 1}
+
+
+def _stacked(weight, w_scale, layout="row_major"):
     g, n, k = weight.shape
     return Fp8Weight(ptr(weight), n * k, None, ptr(w_scale), w_scale.size(1) * w_scale.size(2),
-                     w_scale.size(2), None)
+                     w_scale.size(2), None, _LAYOUT[layout], 0)
 
 
-def _table(proto_w, w_ptrs, proto_s, s_ptrs):
-    return Fp8Weight(None, 0, ptr(w_ptrs), None, 0, proto_s.size(-1), ptr(s_ptrs))
+def _table(proto_w, w_ptrs, proto_s, s_ptrs, layout="row_major"):
+    return Fp8Weight(None, 0, ptr(w_ptrs), None, 0, proto_s.size(-1), ptr(s_ptrs), _LAYOUT[layout], 0)
+
+
+def fp8_weight_repack(weight):
+    """[G, N, K] row-major e4m3fn -> tile-major resident layout (one-time, at weight load).  No
+    reference counterpart as an op; plays the role of its Marlin repack / TMA plan steps."""
+    ck.cuda_tensor(None, weight, ck.FP8_BYTES, "weight")
+    w = weight if weight.dim() == 3 else weight.unsqueeze(0)
+    g, n, k = w.shape
+    out = torch.empty_like(w)
+    with torch.cuda.device(w.device):
+        check(lib().bgmoe_fp8_weight_repack(ptr(w), ptr(out), g, n, k, stream()))
+    return out.view_as(weight)
 
 
 def fp8_blockwise_grouped_gemm(x, weight, seqlens, cu_seqlens, x_scale, w_scale, num_seq_per_group_avg,
-                               output=None, tma_desc=None, tiles=None, cu_tiles=None, update_tma=True):
+                               output=None, tma_desc=None, tiles=None, cu_tiles=None, update_tma=True,
+                               weight_layout="row_major"):
     """Y[r,n] = sum_kb (Xq[r,kb] . Wq[g,n,kb]) * xs[kb,r] * ws[g,n/128,kb] -> bf16 [m, N]."""
     m, n, k, m_pad, g = _check_inputs(x, weight, seqlens, cu_seqlens, x_scale, w_scale, output)
     if output is None:
         output = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
-    a, b = _act(x, x_scale, m_pad), _stacked(weight, w_scale)
+    a, b = _act(x, x_scale, m_pad), _stacked(weight, w_scale, weight_layout)
     with torch.cuda.device(x.device):
         check(lib().bgmoe_fp8_grouped_gemm(C.byref(a), C.byref(b), ptr(seqlens), ptr(cu_seqlens), g, m, n, k,
                                            ptr(output), stream()))
@@ -92,7 +108,7 @@ def fp8_blockwise_grouped_gemm(x, weight, seqlens, cu_seqlens, x_scale, w_scale,
 
 def fp8_blockwise_fused_s1(x, gate_weight, up_weight, seqlens, cu_seqlens, x_scale, gate_w_scale, up_w_scale,
                            num_seq_per_group_avg, output=None, tma_desc=None, tiles=None, cu_tiles=None,
-                           update_tma=True):
+                           update_tma=True, weight_layout="row_major"):
     """bf16( silu(X Wg^T) * (X Wu^T) ) -> [m, N]."""
     m, n, k, m_pad, g = _check_inputs(x, gate_weight, seqlens, cu_seqlens, x_scale, gate_w_scale, output,
                                       "gate_weight")
@@ -102,7 +118,7 @@ def fp8_blockwise_fused_s1(x, gate_weight, up_weight, seqlens, cu_seqlens, x_sca
     if output is None:
         output = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     a = _act(x, x_scale, m_pad)
-    wg, wu = _stacked(gate_weight, gate_w_scale), _stacked(up_weight, up_w_scale)
+    wg, wu = _stacked(gate_weight, gate_w_scale, weight_layout), _stacked(up_weight, up_w_scale, weight_layout)
     with torch.cuda.device(x.device):
         check(lib().bgmoe_fp8_fused_s1(C.byref(a), C.byref(wg), C.byref(wu), ptr(seqlens), ptr(cu_seqlens), g, m,
                                        n, k, ptr(output), None, None, 0, 0, stream()))
@@ -110,7 +126,7 @@ def fp8_blockwise_fused_s1(x, gate_weight, up_weight, seqlens, cu_seqlens, x_sca
 
 
 def fp8_blockwise_fused_s1_quant(x, gate_weight, up_weight, seqlens, cu_seqlens, x_scale, gate_w_scale,
-                                 up_w_scale, out_q, out_scale_t):
+                                 up_w_scale, out_q, out_scale_t, weight_layout="row_major"):
     """Fused S1 with the requant in the epilogue: out_q [m,N] bytes + TRANSPOSED scale [N/128, m].
     Same bytes as fp8_blockwise_fused_s1 followed by act_quant_ragged on the live rows."""
     m, n, k, m_pad, g = _check_inputs(x, gate_weight, seqlens, cu_seqlens, x_scale, gate_w_scale, None,
@@ -121,7 +137,7 @@ def fp8_blockwise_fused_s1_quant(x, gate_weight, up_weight, seqlens, cu_seqlens,
     if tuple(out_q.shape) != (m, n) or tuple(out_scale_t.shape) != (n // 128, m):
         ck.fail(f"out_q must be [{m}, {n}] and out_scale_t [{n // 128}, {m}]")
     a = _act(x, x_scale, m_pad)
-    wg, wu = _stacked(gate_weight, gate_w_scale), _stacked(up_weight, up_w_scale)
+    wg, wu = _stacked(gate_weight, gate_w_scale, weight_layout), _stacked(up_weight, up_w_scale, weight_layout)
     with torch.cuda.device(x.device):
         check(lib().bgmoe_fp8_fused_s1(C.byref(a), C.byref(wg), C.byref(wu), ptr(seqlens), ptr(cu_seqlens), g, m,
                                        n, k, None, ptr(out_q), ptr(out_scale_t), 1, m, stream()))

@@ -42,9 +42,26 @@ class LayerStruct(C.Structure):
 _lib.register("bgmoe_moe_fp8_layer_forward", i32, [C.POINTER(LayerStruct), vp])
 
 
-def _stack_desc(q: torch.Tensor, s: torch.Tensor) -> Fp8Weight:
+W_ROW_MAJOR, W_TILE_MAJOR = 0, 1
+
+
+def _stack_desc(q: torch.Tensor, s: torch.Tensor, layout: int = W_ROW_MAJOR) -> Fp8Weight:
     e, n, k = q.shape
-    return Fp8Weight(ptr(q), n * k, None, ptr(s), s.size(1) * s.size(2), s.size(2), None)
+    return Fp8Weight(ptr(q), n * k, None, ptr(s), s.size(1) * s.size(2), s.size(2), None, layout, 0)
+
+
+def repack_tile_major(q: torch.Tensor) -> torch.Tensor:
+    """[..., N, K] e4m3fn row-major -> the same bytes in the tile-major resident layout (see
+    include/bgmoe.h).  One-time, at weight load."""
+    if q.dim() == 2:
+        q = q.unsqueeze(0)
+    if not q.is_contiguous():
+        raise RuntimeError("weights must be contiguous")
+    e, n, k = q.shape
+    out = torch.empty_like(q)
+    with torch.cuda.device(q.device):
+        check(lib().bgmoe_fp8_weight_repack(ptr(q), ptr(out), e, n, k, stream()))
+    return out
 
 
 class Fp8MoELayer:
@@ -56,9 +73,20 @@ class Fp8MoELayer:
     """
 
     def __init__(self, cfg: MoEConfig, weights, shared, bias: torch.Tensor, max_tokens_in: Optional[int] = None,
-                 shared_mode: str = "bf16_add", fold_shared: bool = True):
+                 shared_mode: str = "bf16_add", fold_shared: bool = True, weight_layout: str = "tile_major"):
         self.cfg = cfg
         dev = weights["gate_q"].device
+        if weight_layout not in ("tile_major", "row_major"):
+            raise ValueError(f"unknown weight_layout {weight_layout!r}")
+        self.layout = W_TILE_MAJOR if weight_layout == "tile_major" else W_ROW_MAJOR
+        if self.layout == W_TILE_MAJOR:
+            # resident copy in the streaming layout; the caller may drop the row-major tensors
+            weights = dict(weights)
+            shared = dict(shared) if shared is not None else None
+            for d in (weights, shared):
+                if d is not None:
+                    for name in ("gate_q", "up_q", "down_q"):
+                        d[name] = repack_tile_major(d[name])
         self.device = dev
         self.n_max = int(max_tokens_in or cfg.n_tokens)
         n, h, inter, el, k = self.n_max, cfg.hidden, cfg.inter, cfg.e_local, cfg.top_k
@@ -107,13 +135,13 @@ class Fp8MoELayer:
                 tw = torch.tensor(wp, dtype=torch.int64, device=dev)
                 ts = torch.tensor(sp, dtype=torch.int64, device=dev)
                 self._tables[name] = (tw, ts)
-                setattr(L, name, Fp8Weight(None, 0, ptr(tw), None, 0, s.size(2), ptr(ts)))
+                setattr(L, name, Fp8Weight(None, 0, ptr(tw), None, 0, s.size(2), ptr(ts), self.layout, 0))
         else:
             for name in ("gate", "up", "down"):
-                setattr(L, name, _stack_desc(weights[name + "_q"], weights[name + "_s"]))
+                setattr(L, name, _stack_desc(weights[name + "_q"], weights[name + "_s"], self.layout))
             if has_shared:
                 for name in ("gate", "up", "down"):
-                    setattr(L, "sh_" + name, _stack_desc(shared[name + "_q"], shared[name + "_s"]))
+                    setattr(L, "sh_" + name, _stack_desc(shared[name + "_q"], shared[name + "_s"], self.layout))
                 L.shq, L.shs = ptr(self.shq), ptr(self.shs)
         L.topk_ids, L.topk_weights = ptr(self.topk_ids), ptr(self.topk_weights)
         L.expert_counts, L.cu_seqlens, L.topk_pos = ptr(self.expert_counts), ptr(self.cu_seqlens), ptr(self.topk_pos)

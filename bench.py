@@ -133,11 +133,14 @@ def main():
     h, i = cfg.hidden, cfg.inter
     if decode:
         dom = "s1_skinny16"
-        served = int(((counts > 0) & (counts <= 16)).sum())
+        # one launch streams gate+up of every active routed expert and of the shared expert once
+        # (algorithmic bytes: each weight byte once, each quantised row in, each requantised row out)
+        served = active + (1 if cfg.shared_inter else 0)
+        srows = rows + (cfg.n_tokens if cfg.shared_inter else 0)
         dom_bytes = served * (2 * h * i + 2 * (h // 128) * (i // 128) * 4) + \
-            int(counts[(counts > 0) & (counts <= 16)].sum()) * (h + h // 128 * 4 + i + i // 128 * 4)
+            srows * (h + h // 128 * 4 + i + i // 128 * 4)
         dom_ms = prof[dom][0] / max(prof[dom][1], 1)
-        roof = dict(bound="hbm", kernel="fp8_skinny_kernel<1,3,fused>", achieved=dom_bytes / (dom_ms * 1e-3) / 1e9,
+        roof = dict(bound="hbm", kernel="fp8_skinny_kernel<TT=2,NS=3,fused,tile_major>", achieved=dom_bytes / (dom_ms * 1e-3) / 1e9,
                     peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=dom_bytes,
                     avg_launch_us=dom_ms * 1e3)
     else:
@@ -163,7 +166,7 @@ def main():
         "tokens_per_s": cfg.n_tokens / (ms * 1e-3),
         "layer_hbm_GBps": gbps, "layer_TFLOPs": tflops,
         "layer_frac_of_hbm_peak": gbps / HBM_PEAK_GBPS, "layer_frac_of_fp8_peak": tflops / FP8_PEAK_TFLOPS,
-        "algorithmic_bytes": alg_bytes, "flops": flops, "active_local_experts": active, "routed_rows": rows,
+        "algorithmic_bytes": alg_bytes, "flops": flops, "active_local_experts": active, "routed_rows": rows, "expert_counts": counts.tolist(),
         "kernel_ms_per_step": per_kernel,
         "roofline": roof,
     }

@@ -208,7 +208,24 @@ typedef struct bgmoe_fp8_weight {
   int64_t scale_group_stride;    /* elements between groups                   */
   int64_t scale_nb_stride;       /* elements between 128-row blocks (>= k/128)*/
   const float* const* scale_ptrs;/* device table or NULL                      */
+  int32_t layout;                /* BGMOE_W_ROW_MAJOR or BGMOE_W_TILE_MAJOR   */
+  int32_t reserved;
 } bgmoe_fp8_weight;
+
+/* Weight byte layouts.  ROW_MAJOR is the checkpoint layout [n, k] the reference
+ * ops take.  TILE_MAJOR is this build's resident layout for weight streaming:
+ * the matrix is cut into 16-row x 128-column tiles of 2048 bytes, tile (nt, kb)
+ * at byte ((nt * k/128) + kb) * 2048; inside a tile, byte
+ * half*1024 + (q*16 + r)*16 + j holds row nt*16 + r, column kb*128 + half*64 +
+ * q*16 + j (r < 16, q < 4, j < 16, half < 2) -- the order in which one wave64
+ * reads an MFMA 16x16x128 operand with two fully contiguous 1 KiB loads.
+ * bgmoe_fp8_weight_repack converts (one-time, at weight load; the reference has
+ * the same kind of step for its own kernels: Marlin repack,
+ * batchgen/moe/fused_moe_mxfp4_resident.py:13-15, and TMA plans,
+ * batchgen/moe/grouped_fp8_blockwise_moe.py:195-247). */
+enum { BGMOE_W_ROW_MAJOR = 0, BGMOE_W_TILE_MAJOR = 1 };
+int bgmoe_fp8_weight_repack(const uint8_t* src_row_major, uint8_t* dst_tile_major, int groups, int n,
+                            int k, bgmoe_stream_t stream);
 
 typedef struct bgmoe_fp8_act {
   const uint8_t* x;              /* [m, k] e4m3fn                              */

@@ -216,3 +216,32 @@ def test_gemm_argument_errors(dev):
     w2 = torch.zeros((1025, 128, 128), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
     with pytest.raises(RuntimeError):
         gm().fp8_blockwise_grouped_gemm(x, w2, sl, cu, xs, ws, 16)      # too many groups
+
+
+def _tile_major_numpy(w):
+    """[G, N, K] bytes -> tile-major image, written from the layout's definition."""
+    g, n, k = w.shape
+    t = w.reshape(g, n // 16, 16, k // 128, 2, 4, 16)          # g, nt, r, kb, half, q, j
+    return np.ascontiguousarray(t.transpose(0, 1, 3, 4, 5, 2, 6)).reshape(g, n, k)   # g, nt, kb, half, q, r, j
+
+
+@pytest.mark.parametrize("counts,n,k", [(EDGE, 256, 512), ((3, 200, 0, 77, 130, 1), 384, 256), ((8,) * 6, 2048, 1024)])
+def test_tile_major_weights_equal_row_major(dev, counts, n, k):
+    say("tile_major", counts, n, k)
+    counts, cu, m, xq, xs, ws = _make(300 + n + k, counts, n, k, nmat=2)
+    (gq, gs), (uq, us) = ws
+    xq_d, xs_t, gq_d, gs_d = _dev(dev, xq, xs, gq, gs)
+    _, _, uq_d, us_d = _dev(dev, xq, xs, uq, us)
+    gq_t, uq_t = gm().fp8_weight_repack(gq_d), gm().fp8_weight_repack(uq_d)
+    assert np.array_equal(gq_t.view(torch.uint8).cpu().numpy(), _tile_major_numpy(gq))
+    cnt_d, cu_d = torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev)
+    live = torch.zeros(m, dtype=torch.bool)
+    for e, c in enumerate(counts):
+        live[cu[e]:cu[e] + c] = True
+    live = live.to(dev)
+    a = gm().fp8_blockwise_grouped_gemm(xq_d, gq_d, cnt_d, cu_d, xs_t, gs_d, 16)
+    b = gm().fp8_blockwise_grouped_gemm(xq_d, gq_t, cnt_d, cu_d, xs_t, gs_d, 16, weight_layout="tile_major")
+    assert torch.equal(a[live], b[live])
+    a = gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16)
+    b = gm().fp8_blockwise_fused_s1(xq_d, gq_t, uq_t, cnt_d, cu_d, xs_t, gs_d, us_d, 16, weight_layout="tile_major")
+    assert torch.equal(a[live], b[live])
