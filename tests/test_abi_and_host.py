@@ -1,0 +1,179 @@
+"""The C-ABI library and the host-side mirror of the reference interface, without a GPU: the library loads,
+exports every symbol include/bgmoe.h declares, its structs have the layout the Python binding assumes, the op
+modules export the reference extension's names, and the wrappers keep the reference's frozen parameter lists
+(tests/contracts/test_pin_moe.py of the reference) and argument policy."""
+import ctypes
+import inspect
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "bgmoe.h")
+
+
+def _declared_functions():
+    src = open(HEADER).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return sorted(set(re.findall(r"\b(bgmoe_[a-z0-9_]+)\s*\(", src)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    from batchgen_amd import _lib
+    import batchgen_amd.moe.fp8_layer  # noqa: F401
+    handle = _lib.lib()
+    names = _declared_functions()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(handle, n), f"libbgmoe.so does not export {n}"
+    assert set(_lib.exported_symbols()) <= set(names) | {"bgmoe_last_error"}
+    assert handle.bgmoe_version() >= 1
+
+
+def test_struct_layout_matches_the_header(tmp_path):
+    from batchgen_amd import _lib
+    from batchgen_amd.moe.fp8_layer import LayerStruct
+    prog = tmp_path / "sz.c"
+    prog.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "bgmoe.h"\n'
+                    'int main(){printf("%zu %zu %zu %zu %zu %zu\\n", sizeof(bgmoe_fp8_weight), sizeof(bgmoe_fp8_act),'
+                    'sizeof(bgmoe_moe_fp8_layer), offsetof(bgmoe_moe_fp8_layer, cap_rows),'
+                    'offsetof(bgmoe_moe_fp8_layer, gate), offsetof(bgmoe_moe_fp8_layer, out));return 0;}\n')
+    exe = tmp_path / "sz"
+    subprocess.run(["gcc", f"-I{os.path.join(ROOT, 'include')}", str(prog), "-o", str(exe)], check=True)
+    got = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
+    want = [ctypes.sizeof(_lib.Fp8Weight), ctypes.sizeof(_lib.Fp8Act), ctypes.sizeof(LayerStruct),
+            LayerStruct.cap_rows.offset, LayerStruct.gate.offset, LayerStruct.out.offset]
+    assert got == want
+
+
+def test_errors_are_reported_without_a_gpu():
+    """Argument errors are detected before anything is launched, so they can be exercised on the CPU."""
+    from batchgen_amd import _lib
+    h = _lib.lib()
+    assert h.bgmoe_fused_gate(None, None, 4, 16, 3, 2, 4, 1.0, 0, None, None, None) != 0
+    assert b"divisible" in h.bgmoe_last_error()
+    assert h.bgmoe_gate_sigmoid_topk(None, 16, None, 4, 16, 3, 1.0, None, 0, None, None, None, 0, None, 0, 0, None) != 0
+    assert b"Unsupported k=3" in h.bgmoe_last_error()
+    assert h.bgmoe_act_quant_ragged(None, None, None, 4, 10, 128, None, None, 48, None) != 0
+    assert b"power of two" in h.bgmoe_last_error()
+    assert h.bgmoe_dispatch_scatter_ragged(None, None, 8, 2, 64, ctypes.c_void_p(16), 64, 0, 4, ctypes.c_void_p(16),
+                                           None, ctypes.c_void_p(16), ctypes.c_void_p(16), 64, None, 0, None) != 0
+    assert b"act_buffer rows" in h.bgmoe_last_error()
+    assert h.bgmoe_dispatch_workspace_bytes(2048, 32) == 0 and h.bgmoe_dispatch_workspace_bytes(131072, 32) == 64 * 32 * 4
+    assert h.bgmoe_fp8_weight_repack(None, None, 1, 100, 128, None) != 0
+
+
+def test_loader_and_op_names():
+    from batchgen_amd.kernels import load_extension
+    want = {
+        "batchgen_kernels.common._C_mgn_ops": ["moe_fused_gate", "fused_moe_token_dispatch", "compact_expert_data",
+                                               "expert_bincount"],
+        "batchgen_kernels.moe._C_routing": ["gate_sigmoid_topk", "gate_sigmoid_topk_warp", "dispatch_count_gather",
+                                            "reduce_weighted_scatter"],
+        "batchgen_kernels.moe._C_dispatch_scatter_3d": ["dispatch_scatter_3d", "dispatch_scatter_ragged",
+                                                        "reduce_weighted_scatter", "reduce_weighted_scatter_fp32",
+                                                        "reduce_weighted_scatter_bf16_ordered"],
+        "batchgen_kernels.moe._C_fp8_blockwise_ops": ["act_quant_3d", "act_quant_ragged", "silu_mul_3d",
+                                                      "fused_silu_quant_3d"],
+        "batchgen_kernels.moe._C_fp8_blockwise_gemm": ["fp8_blockwise_grouped_gemm", "fp8_blockwise_fused_s1",
+                                                       "fp8_blockwise_grouped_gemm_ptrs",
+                                                       "fp8_blockwise_fused_s1_ptrs",
+                                                       "fp8_blockwise_prepare_s1_s3_tma"],
+    }
+    for mod, names in want.items():
+        m = load_extension(mod)
+        for n in names:
+            assert callable(getattr(m, n)), f"{mod}.{n}"
+    with pytest.raises(ImportError):
+        load_extension("batchgen_kernels.moe._C_not_built")
+
+
+# frozen parameter lists of the reference's Python wrappers (tests/contracts/test_pin_moe.py:63-140, 321-368)
+PINS = {
+    ("batchgen_amd.moe.dispatch_scatter_3d", "dispatch_scatter_3d"):
+        ["x", "topk_indices", "act_buffer", "expert_start", "num_local_experts", "max_tokens_padded",
+         "expert_counts", "expert_counters", "topk_pos"],
+    ("batchgen_amd.moe.dispatch_scatter_3d", "dispatch_scatter_ragged"):
+        ["x", "topk_indices", "act_buffer", "expert_start", "num_local_experts", "expert_counts",
+         "expert_counters", "topk_pos", "cu_seqlens", "row_align"],
+    ("batchgen_amd.moe.dispatch_scatter_3d", "reduce_weighted_scatter"):
+        ["expert_output", "topk_pos", "topk_weights", "N", "H", "K", "output"],
+    ("batchgen_amd.moe.dispatch_scatter_3d", "reduce_weighted_scatter_fp32"):
+        ["expert_output", "topk_pos", "topk_weights", "N", "H", "K", "output"],
+    ("batchgen_amd.moe.routing.cuda_routing", "dispatch_count_gather_cuda"):
+        ["x", "topk_indices", "expert_start", "num_local_experts", "expert_counts", "expert_offsets",
+         "expert_counters", "dispatched_x", "topk_pos", "num_valid_tokens"],
+    ("batchgen_amd.moe.routing.cuda_routing", "gate_sigmoid_topk_cuda"):
+        ["router_logits", "e_score_correction", "k", "routed_scaling_factor", "topk_indices", "topk_weights",
+         "num_valid_tokens", "latent_out", "latent_offset", "rank_token_counts", "rows_per_rank"],
+    ("batchgen_amd.moe.routing.cuda_routing", "gate_sigmoid_topk_warp_cuda"):
+        ["router_logits", "e_score_correction", "k", "routed_scaling_factor", "topk_indices", "topk_weights",
+         "num_valid_tokens", "rank_token_counts", "rows_per_rank"],
+    ("batchgen_amd.moe.grouped_fp8_blockwise_moe", "grouped_fp8_blockwise_gemm"):
+        ["x_fp8", "weight_3d", "seqlens", "cu_seqlens", "x_scale", "w_scale_3d", "num_seq_per_group_avg", "output",
+         "tma_desc", "tma_plan"],
+    ("batchgen_amd.moe.grouped_fp8_blockwise_moe", "grouped_fp8_blockwise_fused_s1"):
+        ["x_fp8", "gate_weight_3d", "up_weight_3d", "seqlens", "cu_seqlens", "x_scale", "gate_w_scale_3d",
+         "up_w_scale_3d", "num_seq_per_group_avg", "output", "tma_desc", "tma_plan"],
+}
+
+
+@pytest.mark.parametrize("key", list(PINS))
+def test_wrapper_signatures_are_the_reference_ones(key):
+    import importlib
+    mod, name = key
+    fn = getattr(importlib.import_module(mod), name)
+    assert list(inspect.signature(fn).parameters) == PINS[key]
+
+
+def test_gate_padding_argument_policy():
+    """cuda_routing.py:102-121 of the reference: ValueError before any launch."""
+    import torch
+    from batchgen_amd.moe.routing import gate_sigmoid_topk_cuda, gate_sigmoid_topk_warp_cuda
+    lg, b = torch.zeros(4, 16), torch.zeros(16)
+    one = torch.zeros(1, dtype=torch.int32)
+    rc = torch.zeros(2, dtype=torch.int64)
+    with pytest.raises(ValueError):
+        gate_sigmoid_topk_cuda(lg, b, 4, 1.0, num_valid_tokens=one, rank_token_counts=rc, rows_per_rank=2)
+    with pytest.raises(ValueError):
+        gate_sigmoid_topk_cuda(lg, b, 4, 1.0, rank_token_counts=rc)
+    with pytest.raises(ValueError):
+        gate_sigmoid_topk_cuda(lg, b, 4, 1.0, rank_token_counts=rc, rows_per_rank=0)
+    with pytest.raises(ValueError):
+        gate_sigmoid_topk_cuda(lg, b, 4, 1.0, rows_per_rank=2)
+    with pytest.raises(TypeError):
+        gate_sigmoid_topk_warp_cuda(lg.double(), b, 4, 1.0)
+    with pytest.raises(ValueError):
+        gate_sigmoid_topk_warp_cuda(torch.zeros(4, 300), torch.zeros(300), 4, 1.0)
+    with pytest.raises(TypeError):
+        gate_sigmoid_topk_warp_cuda(lg, b, 4, 1.0, topk_indices=torch.zeros(4, 4, dtype=torch.int16))
+
+
+def test_tile_m_buckets_and_plan_checks():
+    import torch
+    from batchgen_amd.moe import grouped_fp8_blockwise_moe as g
+    assert [g.grouped_fp8_tile_m(v) for v in (1, 16, 17, 32, 33, 48, 64, 500)] == [16, 16, 32, 32, 64, 64, 64, 64]
+    a, b = torch.zeros(4, 128), torch.zeros(4, 256)
+    plan = g.GroupedFp8TmaPlan(None, None, None, None, 16, 1, 2, a.data_ptr(), b.data_ptr(), 0, 0, 4, 128, 256, 0, 0)
+    sl, cu = torch.zeros(1, dtype=torch.int32), torch.zeros(2, dtype=torch.int32)
+    with pytest.raises(ValueError):
+        g._check_plan(plan, "s1", a, None, sl, cu, 16)                 # no output buffer
+    with pytest.raises(ValueError):
+        g._check_plan(plan, "s1", a, b, sl, cu, 16)                    # other seqlens tensors
+    with pytest.raises(ValueError):
+        g._check_plan(plan, "s1", a, b, sl, cu, 64)                    # other TileM
+
+
+def test_ragged_capacity_formula():
+    from batchgen_amd.moe.dispatch_scatter_3d import ragged_row_capacity
+    assert ragged_row_capacity(256, 8, 32, 64) == (2048 + 63 * 32) // 64 * 64
+    assert ragged_row_capacity(1, 2, 32, 64) == (2 + 63 * 2) // 64 * 64
+    assert ragged_row_capacity(16384, 8, 32, 128) == (131072 + 127 * 32) // 128 * 128
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr

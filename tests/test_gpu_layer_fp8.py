@@ -99,3 +99,34 @@ def test_layer_rejects_bad_arguments(dev):
     with pytest.raises(RuntimeError):
         layer(torch.zeros((65, cfg.hidden), dtype=torch.bfloat16, device=dev),
               torch.zeros((65, cfg.n_experts), device=dev))
+
+
+def test_config0_against_the_committed_golden_fixture(dev):
+    """Same check from files only: tests/golden/c0_layer.npz (written by tests/golden/make_c0_golden.py)."""
+    import os
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "c0_layer.npz"))
+    cfg = wl.CONFIGS[0]
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    layer = Fp8MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
+                        inp["bias"].to(dev))
+    out = layer(inp["x"].to(dev), inp["logits"].to(dev))
+    assert np.array_equal(layer.topk_ids.cpu().numpy(), gold["ids"])
+    assert np.array_equal(layer.topk_pos.cpu().numpy(), gold["pos"])
+    assert np.array_equal(layer.expert_counts[:cfg.e_local].cpu().numpy(), gold["counts"])
+    assert np.array_equal(layer.xs[layer.cap_rows:].cpu().numpy().view(np.uint32), gold["xs_tok"].view(np.uint32))
+    assert og.rel_frobenius(out.float().cpu().numpy(), gold["out"]) < 1e-2
+
+
+@pytest.mark.parametrize("layout", ["row_major", "tile_major"])
+def test_weight_layouts_give_identical_layers(dev, layout):
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = SMALL["c1_small"]
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    mk = lambda lay: Fp8MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
+                                 inp["bias"].to(dev), weight_layout=lay)
+    a = mk("row_major")(inp["x"].to(dev), inp["logits"].to(dev)).clone()
+    b = mk(layout)(inp["x"].to(dev), inp["logits"].to(dev)).clone()
+    assert torch.equal(a, b)
