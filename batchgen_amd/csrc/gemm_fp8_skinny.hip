@@ -112,11 +112,22 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
   constexpr int NSC = FUSED ? 2 : 1;     // weight-scale streams per wave
   __shared__ float s_amax[4][TT][16];
 
+  // XCD-aware block -> (group, token chunk, n-tile) map.  Blocks are dispatched round-robin over the
+  // 8 XCDs (block b runs on XCD b % 8), each with its own L2.  A group with several 32-token chunks
+  // streams the same weight tile once per chunk; the map puts all chunks of one n-tile on the SAME
+  // XCD in neighbouring blocks, so they run at the same time and share the stream through that L2:
+  // inside a group, block q -> n-tile 8*(q / (8*chunks)) + q % 8, chunk (q / 8) % chunks.
   const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
-  int chunk = 0;
-  const int grp = nth_active_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, blockIdx.x / ntiles, &chunk);
+  const int ntiles_pad = (ntiles + 7) & ~7;       // every group starts on XCD 0
+  int crow = 0;
+  const int grp = nth_active_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, blockIdx.x / ntiles_pad, &crow);
   if (grp < 0) return;                            // whole block: fewer items than the grid allows
   const int cnt = g.seqlens[grp];
+  const int chunks = (cnt + 16 * TT - 1) / (16 * TT);
+  const int q = crow * ntiles_pad + blockIdx.x % ntiles_pad;
+  const int ntile = 8 * (q / (8 * chunks)) + (q & 7);
+  const int chunk = (q >> 3) % chunks;
+  if (ntile >= ntiles) return;                    // padding of the n-tile count to a multiple of 8
   const int64_t row0 = g.cu[grp];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -124,7 +135,7 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
   const int kq = lane >> 4;
   const int K = g.k;
   const int KB = K >> 7;
-  const int n0 = (blockIdx.x % ntiles) * (FUSED ? 128 : 256);
+  const int n0 = ntile * (FUSED ? 128 : 256);
 
   const uint8_t* wb[2];
   const float* wsb[2];
@@ -355,12 +366,13 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
   const int hi = skinny_limit();
   if (hi > 0) {
-    constexpr int TT = 2;
-    const int64_t items = g.groups + bound / (16 * TT);           // >= sum of ceil(count / 32)
-    const dim3 grid((unsigned)(((g.n + ntile - 1) / ntile) * items));
+    static const int tt = getenv("BGMOE_SKINNY_TT") ? atoi(getenv("BGMOE_SKINNY_TT")) : 2;
+    const int64_t items = g.groups + bound / (16 * tt);            // >= sum of ceil(count / chunk rows)
+    const dim3 grid((unsigned)(((((g.n + ntile - 1) / ntile) + 7) & ~7) * items));
     g.lo = 0; g.hi = hi;
     BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
-    launch_variant<TT, 3>(fused, layout, grid, g, st);
+    if (tt == 4) launch_variant<4, 2>(fused, layout, grid, g, st);
+    else launch_variant<2, 3>(fused, layout, grid, g, st);
     int rc = bgmoe_check_launch("fp8 grouped gemm (skinny)");
     if (rc != BGMOE_OK) return rc;
   }

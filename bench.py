@@ -33,6 +33,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 4])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one plain copy kernel of known size (the weight re-layout kernel on a "
+                         "256 MiB buffer: 256 MiB read, 256 MiB written) so that rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE readings can be scaled")
     return ap.parse_args()
 
 
@@ -105,6 +109,11 @@ def main():
     for _ in range(a.warmup):
         layer(x, logits)
     torch.cuda.synchronize()
+    if a.copy_calibration:
+        from batchgen_amd.moe.fp8_layer import repack_tile_major
+        cal = torch.zeros((1, 32768, 8192), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
+        repack_tile_major(cal)
+        torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(a.steps):
