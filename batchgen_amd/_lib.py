@@ -26,6 +26,12 @@ class Fp8Weight(C.Structure):
                 ("layout", i32), ("reserved", i32)]
 
 
+class Mxfp4Weight(C.Structure):
+    """bgmoe_mxfp4_weight"""
+    _fields_ = [("w", vp), ("w_group_stride", i64), ("w_ptrs", vp), ("scale", vp), ("scale_group_stride", i64),
+                ("scale_ptrs", vp), ("layout", i32), ("reserved", i32)]
+
+
 class Fp8Act(C.Structure):
     """bgmoe_fp8_act"""
     _fields_ = [("x", vp), ("scale", vp), ("scale_row_stride", i64), ("scale_kb_stride", i64)]
@@ -53,6 +59,10 @@ _SIGS = {
     "bgmoe_reduce_weighted_scatter_fp32": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
     "bgmoe_reduce_weighted_scatter_bf16_ordered": (i32, [vp, vp, vp, vp, i32, i32, i32, vp, vp]),
     "bgmoe_fp8_weight_repack": (i32, [vp, vp, i32, i32, i32, vp]),
+    "bgmoe_mxfp4_weight_repack": (i32, [vp, vp, vp, vp, i32, i32, i32, vp]),
+    "bgmoe_mxfp4_grouped_gemm": (i32, [vp, C.POINTER(Mxfp4Weight), vp, vp, i32, i64, i32, i32, vp, vp, i64, vp]),
+    "bgmoe_mxfp4_fused_s1": (i32, [vp, C.POINTER(Mxfp4Weight), C.POINTER(Mxfp4Weight), vp, vp, i32, i64, i32, i32, vp,
+                                   vp, i32, i64, vp]),
     "bgmoe_compact_expert_data": (i32, [vp, i32, vp, vp, vp, vp, vp]),
     "bgmoe_fp8_grouped_gemm": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), vp, vp, i32, i64, i32, i32, vp, vp]),
     "bgmoe_fp8_fused_s1": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), C.POINTER(Fp8Weight), vp, vp, i32,

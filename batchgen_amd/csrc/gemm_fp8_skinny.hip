@@ -32,6 +32,7 @@
 #include <stdlib.h>
 
 #include "bgmoe_common.h"
+#include "bgmoe_sched.h"
 
 namespace {
 
@@ -76,58 +77,16 @@ __device__ __forceinline__ intx8 load32_stream(const uint8_t* p) {
   return r;
 }
 
-// Work items of one launch: every group with lo < count <= hi contributes ceil(count / chunk_rows)
-// items (ascending group, ascending chunk).  Returns the group of item `item` and its chunk index,
-// or -1 when there are fewer items.  Wave-uniform; every wave of the block runs it redundantly.
-__device__ __forceinline__ int nth_active_item(const int32_t* seqlens, int groups, int lo, int hi,
-                                               int chunk_rows, int item, int* chunk) {
-  const int lane = threadIdx.x & 63;
-  int base = 0;
-  for (int g0 = 0; g0 < groups; g0 += 64) {
-    const int gi = g0 + lane;
-    const int c = gi < groups ? seqlens[gi] : 0;
-    const int mine = (c > lo && c <= hi) ? (c + chunk_rows - 1) / chunk_rows : 0;
-    int inc = mine;                                  // inclusive prefix sum over the wave
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const int up = __shfl_up(inc, off, BGMOE_WAVE);
-      if (lane >= off) inc += up;
-    }
-    const int total = __shfl(inc, 63, BGMOE_WAVE);
-    if (item < base + total) {
-      const int rel = item - base;
-      const unsigned long long hit = __ballot(mine > 0 && rel >= inc - mine && rel < inc);
-      const int src = __ffsll((long long)hit) - 1;
-      *chunk = rel - __shfl(inc - mine, src, BGMOE_WAVE);
-      return g0 + src;
-    }
-    base += total;
-  }
-  return -1;
-}
-
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
   constexpr int NT = 4;                  // weight tiles per wave
   constexpr int NSC = FUSED ? 2 : 1;     // weight-scale streams per wave
   __shared__ float s_amax[4][TT][16];
 
-  // XCD-aware block -> (group, token chunk, n-tile) map.  Blocks are dispatched round-robin over the
-  // 8 XCDs (block b runs on XCD b % 8), each with its own L2.  A group with several 32-token chunks
-  // streams the same weight tile once per chunk; the map puts all chunks of one n-tile on the SAME
-  // XCD in neighbouring blocks, so they run at the same time and share the stream through that L2:
-  // inside a group, block q -> n-tile 8*(q / (8*chunks)) + q % 8, chunk (q / 8) % chunks.
   const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
-  const int ntiles_pad = (ntiles + 7) & ~7;       // every group starts on XCD 0
-  int crow = 0;
-  const int grp = nth_active_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, blockIdx.x / ntiles_pad, &crow);
-  if (grp < 0) return;                            // whole block: fewer items than the grid allows
-  const int cnt = g.seqlens[grp];
-  const int chunks = (cnt + 16 * TT - 1) / (16 * TT);
-  const int q = crow * ntiles_pad + blockIdx.x % ntiles_pad;
-  const int ntile = 8 * (q / (8 * chunks)) + (q & 7);
-  const int chunk = (q >> 3) % chunks;
-  if (ntile >= ntiles) return;                    // padding of the n-tile count to a multiple of 8
+  const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles);
+  if (it.grp < 0) return;                         // whole block: fewer items than the grid allows
+  const int grp = it.grp, cnt = it.cnt, ntile = it.ntile, chunk = it.chunk;
   const int64_t row0 = g.cu[grp];
   const int wave = threadIdx.x >> 6;
   const int lane = threadIdx.x & 63;
@@ -367,8 +326,7 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   const int hi = skinny_limit();
   if (hi > 0) {
     static const int tt = getenv("BGMOE_SKINNY_TT") ? atoi(getenv("BGMOE_SKINNY_TT")) : 2;
-    const int64_t items = g.groups + bound / (16 * tt);            // >= sum of ceil(count / chunk rows)
-    const dim3 grid((unsigned)(((((g.n + ntile - 1) / ntile) + 7) & ~7) * items));
+    const dim3 grid(bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 16 * tt));
     g.lo = 0; g.hi = hi;
     BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
     if (tt == 4) launch_variant<4, 2>(fused, layout, grid, g, st);

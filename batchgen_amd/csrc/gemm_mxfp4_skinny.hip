@@ -1,0 +1,297 @@
+// W4A16 grouped GEMM for MXFP4 weights (e2m1 values, one e8m0 scale per 32 along K) and bf16
+// activations: a weight-streaming kernel bound by HBM bandwidth (decode).
+//
+// Same work split and scheduling as the FP8 weight-streaming kernel: block = (group, 32-token chunk,
+// 128 gate + 128 up columns | 256 columns), 4 waves x four 16-row weight tiles, register prefetch.
+// Weights are dequantised IN REGISTERS: one lane's 16-byte load is one row's 32-value scale group;
+// v_cvt_scalef32_pk_bf16_fp4 turns a byte (low nibble = even K) into two bf16 already multiplied by
+// 2^(scale-127), exactly (a power-of-two times a 2-bit-mantissa value), so the MFMA consumes the
+// same bf16 weights as "dequantise, then bf16 x bf16 -> fp32 GEMM".  MFMA: v_mfma_f32_16x16x32_bf16,
+// weight tile as A, token tile as B; 4 MFMAs per 128-K block.  K permutation (same on both
+// operands): in step s of a block, lane group q = lane/16 covers k = 32q + 8s .. 32q + 8s + 7.
+//
+// Layouts (bgmoe_mxfp4_weight.layout): ROW_MAJOR = checkpoint layout, packed [n, k/2] bytes and
+// scales [n, k/32] bytes; TILE_MAJOR = per (16 rows, 128 K) tile 1024 packed bytes in lane order
+// (lane l = q*16 + r holds row r, bytes 16q..16q+15 of the row's 64-byte segment) and 64 scale bytes
+// [r][4] -- one contiguous 1 KiB load per wave and tile.
+//
+// Algorithmic bytes per group and matrix: n*k/2 + n*k/32.
+#include <stdlib.h>
+
+#include "bgmoe_common.h"
+#include "bgmoe_sched.h"
+
+namespace {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+struct Mx4Args {
+  const uint16_t* x;            // [m, k] bf16
+  bgmoe_mxfp4_weight w0, w1;
+  const int32_t* seqlens;
+  const int32_t* cu;
+  int groups, n, k;
+  uint16_t* out;                // [m, n] bf16, row r of the activation buffer -> row r
+  uint16_t* const* out_ptrs;    // or: per-group output base (row = token index inside the group)
+  int lo, hi;
+  int64_t row_bound;
+};
+
+template <int TT>
+struct Mx4Stage {
+  intx4 A[4];                   // packed fp4: one 32-value scale group per lane and tile
+  uint32_t S[4];                // the row's four scale bytes of this 128-K block
+  intx4 B[TT][4];               // tokens: 8 bf16 per step
+};
+
+__device__ __forceinline__ bf16x8 dequant8(uint32_t w, float scale) {
+  const bf16x2_t v0 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 0);
+  const bf16x2_t v1 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 1);
+  const bf16x2_t v2 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 2);
+  const bf16x2_t v3 = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(w, scale, 3);
+  return bf16x8{v0[0], v0[1], v1[0], v1[1], v2[0], v2[1], v3[0], v3[1]};
+}
+
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
+__global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g) {
+  constexpr int NT = 4;
+  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
+  const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles);
+  if (it.grp < 0) return;
+  const int grp = it.grp, cnt = it.cnt;
+  const int64_t row0 = g.cu[grp];
+  const int wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int r16 = lane & 15;
+  const int kq = lane >> 4;
+  const int K = g.k;
+  const int KB = K >> 7;
+  const int n0 = it.ntile * (FUSED ? 128 : 256);
+
+  const uint8_t* wb[2];
+  const uint8_t* sb[2];
+  wb[0] = g.w0.w_ptrs ? g.w0.w_ptrs[grp] : g.w0.w + (int64_t)grp * g.w0.w_group_stride;
+  sb[0] = g.w0.scale_ptrs ? g.w0.scale_ptrs[grp] : g.w0.scale + (int64_t)grp * g.w0.scale_group_stride;
+  if constexpr (FUSED) {
+    wb[1] = g.w1.w_ptrs ? g.w1.w_ptrs[grp] : g.w1.w + (int64_t)grp * g.w1.w_group_stride;
+    sb[1] = g.w1.scale_ptrs ? g.w1.scale_ptrs[grp] : g.w1.scale + (int64_t)grp * g.w1.scale_group_stride;
+  }
+  const uint8_t* wp[NT];
+  const uint8_t* sp[NT];
+  bool tv[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int nrow = FUSED ? n0 + 32 * wave + 16 * (t & 1) : n0 + 64 * wave + 16 * t;
+    tv[t] = nrow < g.n;
+    const int nr = min(nrow, g.n - 16);
+    const int mi = FUSED ? (t >> 1) : 0;
+    if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
+      wp[t] = wb[mi] + (int64_t)(nr + r16) * (K >> 1) + 16 * kq;
+      sp[t] = sb[mi] + (int64_t)(nr + r16) * (K >> 5);
+    } else {
+      wp[t] = wb[mi] + (int64_t)(nr >> 4) * KB * 1024 + lane * 16;
+      sp[t] = sb[mi] + (int64_t)(nr >> 4) * KB * 64 + r16 * 4;
+    }
+  }
+
+  const int t0 = it.chunk * 16 * TT;
+  uint16_t* const obase = g.out_ptrs ? g.out_ptrs[grp] : g.out + row0 * g.n;
+  const uint8_t* xp[TT];
+  bool xv[TT];
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) {
+    const int tok = t0 + 16 * tt + r16;
+    xv[tt] = tok < cnt;
+    xp[tt] = reinterpret_cast<const uint8_t*>(g.x + (row0 + (xv[tt] ? tok : 0)) * K) + 64 * kq;
+  }
+
+  floatx4 acc[TT][NT];
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  Mx4Stage<TT> st[NSTAGE];
+  auto load_stage = [&](Mx4Stage<TT>& s, int kb) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
+        s.A[t] = gload_x4_stream(wp[t] + (kb << 6));
+        s.S[t] = *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)(sp[t] + (kb << 2)));
+      } else {
+        s.A[t] = gload_x4_stream(wp[t] + ((int64_t)kb << 10));
+        s.S[t] = *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)(sp[t] + (kb << 6)));
+      }
+    }
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) s.B[tt][j] = gload_x4(xp[tt] + (kb << 8) + 16 * j);
+  };
+  auto compute = [&](const Mx4Stage<TT>& c) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const float sc = __uint_as_float(((c.S[t] >> (8 * kq)) & 0xffu) << 23);    // 2^(e8m0 - 127)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bf16x8 a = dequant8((uint32_t)c.A[t][j], sc);
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+          const bf16x8 b = __builtin_bit_cast(bf16x8, c.B[tt][j]);
+          acc[tt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[tt][t], 0, 0, 0);
+        }
+      }
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s) load_stage(st[s], min(s, KB - 1));
+  const int kb_main = KB - KB % NSTAGE;
+  for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
+#pragma unroll
+    for (int s = 0; s < NSTAGE; ++s) {
+      load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
+      compute(st[s]);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s)
+    if (kb_main + s < KB) compute(st[s]);
+
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) {
+    const int tok = t0 + 16 * tt + r16;
+    if (!xv[tt]) continue;
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float h[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) h[i] = silu_f32(acc[tt][j][i]) * acc[tt][j + 2][i];
+        uint2 o;
+        o.x = f32_to_bf16_bits(h[0]) | (f32_to_bf16_bits(h[1]) << 16);
+        o.y = f32_to_bf16_bits(h[2]) | (f32_to_bf16_bits(h[3]) << 16);
+        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = o;
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        if (!tv[t]) continue;
+        uint2 o;
+        o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
+        o.y = f32_to_bf16_bits(acc[tt][t][2]) | (f32_to_bf16_bits(acc[tt][t][3]) << 16);
+        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + 64 * wave + 16 * t + 4 * kq) = o;
+      }
+    }
+  }
+}
+
+// row-major -> tile-major for packed values (16-byte chunks) and scales (4-byte chunks)
+__global__ __launch_bounds__(256) void mxfp4_repack_kernel(const uint8_t* __restrict__ w, const uint8_t* __restrict__ s,
+                                                           uint8_t* __restrict__ wo, uint8_t* __restrict__ so,
+                                                           int64_t chunks, int n, int k) {
+  const int kb_n = k >> 7;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += stride) {
+    const int lane = (int)(c & 63);
+    const int64_t tile = c >> 6;                       // (group*n/16 + nt) * kb_n + kb
+    const int kb = (int)(tile % kb_n);
+    const int64_t nt_all = tile / kb_n;
+    const int r = lane & 15, q = lane >> 4;
+    const int64_t row = nt_all * 16 + r;
+    *reinterpret_cast<uint4*>(wo + c * 16) = *reinterpret_cast<const uint4*>(w + row * (k >> 1) + kb * 64 + 16 * q);
+    if (q == 0)
+      *reinterpret_cast<uint32_t*>(so + (tile * 16 + r) * 4) = *reinterpret_cast<const uint32_t*>(s + row * (k >> 5) + kb * 4);
+  }
+}
+
+int check_w(const char* what, const bgmoe_mxfp4_weight* w) {
+  BGMOE_REQUIRE(w != nullptr, "%s: null weight descriptor", what);
+  BGMOE_REQUIRE((w->w || w->w_ptrs) && (w->scale || w->scale_ptrs), "%s: null weight", what);
+  BGMOE_REQUIRE(w->layout == BGMOE_W_ROW_MAJOR || w->layout == BGMOE_W_TILE_MAJOR, "%s: unknown weight layout %d", what, w->layout);
+  BGMOE_REQUIRE(w->w_ptrs || ((uintptr_t)w->w % 16 == 0 && w->w_group_stride % 16 == 0), "%s: packed weights must be 16-byte aligned", what);
+  BGMOE_REQUIRE(w->scale_ptrs || ((uintptr_t)w->scale % 4 == 0 && w->scale_group_stride % 4 == 0), "%s: scales must be 4-byte aligned", what);
+  return BGMOE_OK;
+}
+
+int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
+  const int ntile = fused ? 128 : 256;
+  const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
+  const dim3 grid(bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 32)), block(256);
+  g.lo = 0; g.hi = 0x7fffffff;     // every group: more than 32 rows = more chunks (weights re-streamed)
+  const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
+  BgmoeProf prof(fused ? BGMOE_K_MXFP4_S1 : BGMOE_K_MXFP4_GEMM, st);
+  if (fused) {
+    if (tm) hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, true, 1>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, true, 0>), grid, block, 0, st, g);
+  } else {
+    if (tm) hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, false, 1>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, false, 0>), grid, block, 0, st, g);
+  }
+  return bgmoe_check_launch("mxfp4 grouped gemm");
+}
+
+int check_shape(const char* what, const uint16_t* x, const int32_t* seqlens, const int32_t* cu, int groups, int64_t m,
+                int n, int k, const uint16_t* out, uint16_t* const* out_ptrs) {
+  BGMOE_REQUIRE(groups >= 0 && groups <= 1024, "%s: groups=%d outside [0,1024]", what, groups);
+  BGMOE_REQUIRE(m >= 0, "%s: m < 0", what);
+  BGMOE_REQUIRE(k > 0 && k % 128 == 0, "%s: K=%d must be a positive multiple of 128", what, k);
+  BGMOE_REQUIRE(n > 0 && n % 128 == 0, "%s: N=%d must be a positive multiple of 128", what, n);
+  if (groups == 0 || m == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(x && seqlens && cu && (out || out_ptrs), "%s: null pointer", what);
+  BGMOE_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)out % 8 == 0, "%s: misaligned activations / output", what);
+  return BGMOE_OK;
+}
+
+}  // namespace
+
+extern "C" int bgmoe_mxfp4_grouped_gemm(const uint16_t* x, const bgmoe_mxfp4_weight* w, const int32_t* seqlens,
+                                        const int32_t* cu_seqlens, int groups, int64_t m, int n, int k,
+                                        uint16_t* out, uint16_t* const* out_ptrs, int64_t row_bound,
+                                        bgmoe_stream_t stream) {
+  int rc = check_shape("mxfp4_grouped_gemm", x, seqlens, cu_seqlens, groups, m, n, k, out, out_ptrs);
+  if (rc != BGMOE_OK) return rc;
+  if (groups == 0 || m == 0) return BGMOE_OK;
+  rc = check_w("mxfp4_grouped_gemm", w);
+  if (rc != BGMOE_OK) return rc;
+  Mx4Args g{};
+  g.x = x; g.w0 = *w; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups; g.n = n; g.k = k; g.out = out;
+  g.out_ptrs = out_ptrs; g.row_bound = row_bound;
+  return launch(false, g, m, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight* gate, const bgmoe_mxfp4_weight* up,
+                                    const int32_t* seqlens, const int32_t* cu_seqlens, int groups, int64_t m, int n,
+                                    int k, uint16_t* out, uint16_t* const* out_ptrs, int activation,
+                                    int64_t row_bound, bgmoe_stream_t stream) {
+  int rc = check_shape("mxfp4_fused_s1", x, seqlens, cu_seqlens, groups, m, n, k, out, out_ptrs);
+  if (rc != BGMOE_OK) return rc;
+  BGMOE_REQUIRE(activation == 0, "mxfp4_fused_s1: only SwiGLU (activation 0) is built");
+  if (groups == 0 || m == 0) return BGMOE_OK;
+  rc = check_w("mxfp4_fused_s1", gate);
+  if (rc != BGMOE_OK) return rc;
+  rc = check_w("mxfp4_fused_s1", up);
+  if (rc != BGMOE_OK) return rc;
+  BGMOE_REQUIRE(gate->layout == up->layout, "mxfp4_fused_s1: gate and up weights must use the same layout");
+  Mx4Args g{};
+  g.x = x; g.w0 = *gate; g.w1 = *up; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups; g.n = n; g.k = k;
+  g.out = out; g.out_ptrs = out_ptrs; g.row_bound = row_bound;
+  return launch(true, g, m, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_mxfp4_weight_repack(const uint8_t* w_packed, const uint8_t* scales, uint8_t* w_out,
+                                         uint8_t* scales_out, int groups, int n, int k, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(groups >= 0 && n > 0 && k > 0, "mxfp4_weight_repack: bad sizes");
+  BGMOE_REQUIRE(n % 16 == 0 && k % 128 == 0, "mxfp4_weight_repack: N=%d must be a multiple of 16 and K=%d of 128", n, k);
+  if (groups == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(w_packed && scales && w_out && scales_out && w_packed != w_out && scales != scales_out,
+                "mxfp4_weight_repack: needs distinct non-null buffers");
+  BGMOE_REQUIRE((uintptr_t)w_packed % 16 == 0 && (uintptr_t)w_out % 16 == 0 && (uintptr_t)scales % 4 == 0 &&
+                (uintptr_t)scales_out % 4 == 0, "mxfp4_weight_repack: misaligned buffers");
+  const int64_t chunks = (int64_t)groups * n * (k >> 1) / 16;
+  int64_t blocks = (chunks + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(mxfp4_repack_kernel, dim3((unsigned)blocks), dim3(256), 0, bgmoe_stream(stream), w_packed, scales,
+                     w_out, scales_out, chunks, n, k);
+  return bgmoe_check_launch("mxfp4_weight_repack");
+}

@@ -123,6 +123,58 @@ def make_fp8_weights(cfg: MoEConfig, device):
     return w, sh
 
 
+def quantize_mxfp4(w: torch.Tensor):
+    """w [..., K] fp32 -> (packed uint8 [..., K/2], e8m0 scale bytes [..., K/32]).  OCP MX closed form:
+    shared exponent floor(log2(amax)) - 2, elements rounded to nearest-even e2m1, saturating at 6
+    (torch restatement of oracle/mxfp4.py::quantize; equality is tested on the CPU)."""
+    *lead, k = w.shape
+    g = w.reshape(*lead, k // 32, 32)
+    amax = g.abs().amax(dim=-1)
+    e = torch.frexp(torch.where(amax > 0, amax, torch.ones_like(amax)))[1] - 1
+    byte = torch.clamp(e - 2 + 127, 1, 254)
+    byte = torch.where(amax > 0, byte, torch.full_like(byte, 127))
+    scale = torch.ldexp(torch.ones_like(amax), byte - 127)
+    a = (g / scale[..., None]).abs()
+    code = torch.zeros_like(a, dtype=torch.uint8)
+    for mid, tie_up in ((0.25, False), (0.75, True), (1.25, False), (1.75, True), (2.5, False), (3.5, True),
+                        (5.0, False)):
+        code += ((a >= mid) if tie_up else (a > mid)).to(torch.uint8)
+    code = code | (torch.signbit(g).to(torch.uint8) << 3)
+    code = code.reshape(*lead, k)
+    packed = code[..., 0::2] | (code[..., 1::2] << 4)
+    return packed.contiguous(), byte.to(torch.uint8).contiguous()
+
+
+def make_mxfp4_weights(cfg: MoEConfig, device):
+    """Local experts' MXFP4 weights (checkpoint layout) + a bf16 shared expert."""
+    dev = torch.device(device)
+    gen = torch.Generator(device=dev).manual_seed(cfg.seed + 1)
+    w = {}
+    for name, (n, k) in (("gate", (cfg.inter, cfg.hidden)), ("up", (cfg.inter, cfg.hidden)),
+                         ("down", (cfg.hidden, cfg.inter))):
+        p = torch.empty((cfg.e_local, n, k // 2), dtype=torch.uint8, device=dev)
+        s = torch.empty((cfg.e_local, n, k // 32), dtype=torch.uint8, device=dev)
+        for i in range(cfg.e_local):
+            p[i], s[i] = quantize_mxfp4(torch.randn((n, k), generator=gen, device=dev) * 0.02)
+        w[name + "_p"], w[name + "_s"] = p, s
+    sh = None
+    if cfg.shared_inter:
+        sh = {}
+        for name, (n, k) in (("gate", (cfg.shared_inter, cfg.hidden)), ("up", (cfg.shared_inter, cfg.hidden)),
+                             ("down", (cfg.hidden, cfg.shared_inter))):
+            sh[name] = (torch.randn((n, k), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    return w, sh
+
+
+def algorithmic_bytes_mxfp4(cfg: MoEConfig, active_experts: int, routed_rows: int) -> int:
+    h, i = cfg.hidden, cfg.inter
+    total = active_experts * (3 * h * i // 2 + 3 * h * i // 32)
+    if cfg.shared_inter:
+        total += 3 * h * cfg.shared_inter * 2
+    total += cfg.n_tokens * h * 2 * 2 + routed_rows * (2 * h + 2 * i) * 2
+    return int(total)
+
+
 def weights_to_numpy(w):
     """torch weight dict -> numpy (bytes as uint8) for the CPU oracle."""
     if w is None:

@@ -257,6 +257,50 @@ int bgmoe_fp8_fused_s1(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* gate,
                        int64_t out_scale_row_stride, int64_t out_scale_nb_stride,
                        bgmoe_stream_t stream);
 
+/* ------------------------------------------------------- MXFP4 (W4A16) GEMM */
+
+/* MXFP4 weights: e2m1 values packed two per byte (low nibble = even K), one e8m0 scale byte per 32
+ * consecutive K, scale = 2^(byte-127) (batchgen/moe/mxfp4_oracle_vector.py:48-115).
+ * ROW_MAJOR: packed [n, k/2], scales [n, k/32] (the checkpoint layout,
+ * batchgen/models/moonshotai/kimi_linear/k3/mxfp4_expert.py:239-285).
+ * TILE_MAJOR: per (16 rows x 128 K) tile, 1024 packed bytes in wave-lane order and 64 scale bytes
+ * [row][4]; produced by bgmoe_mxfp4_weight_repack.  It plays the role of the reference's Marlin
+ * repack (batchgen/moe/fused_moe_mxfp4_resident.py:13-15), whose NVIDIA register layout is not
+ * reproduced. */
+typedef struct bgmoe_mxfp4_weight {
+  const uint8_t* w;               /* [groups, ...] packed values                 */
+  int64_t w_group_stride;         /* bytes between groups (n*k/2)               */
+  const uint8_t* const* w_ptrs;   /* device table or NULL                       */
+  const uint8_t* scale;           /* [groups, ...] e8m0 bytes                   */
+  int64_t scale_group_stride;     /* bytes between groups (n*k/32)              */
+  const uint8_t* const* scale_ptrs;
+  int32_t layout;
+  int32_t reserved;
+} bgmoe_mxfp4_weight;
+
+int bgmoe_mxfp4_weight_repack(const uint8_t* w_packed, const uint8_t* scales, uint8_t* w_out,
+                              uint8_t* scales_out, int groups, int n, int k, bgmoe_stream_t stream);
+
+/* out[r, :] = bf16( x[r, :] (bf16) * dequant(W[g])^T ), fp32 accumulation, for rows of group g.
+ * Replaces `marlin_grouped_m16_mxfp4` (batchgen/moe/marlin_grouped_moe.py:476-543,
+ * batchgen_kernels/src/moe/marlin_grouped_gemm.cu).  row_bound: host-side upper bound on the live
+ * rows (0 = m); groups with more than 32 rows stream their weights once per 32-row chunk.
+ * Output: row r of x -> row r of `out`, or, when out_ptrs (device table, the reference's C_ptrs)
+ * is given, token t of group g -> out_ptrs[g] + t*n. */
+int bgmoe_mxfp4_grouped_gemm(const uint16_t* x, const bgmoe_mxfp4_weight* w, const int32_t* seqlens,
+                             const int32_t* cu_seqlens, int groups, int64_t m, int n, int k,
+                             uint16_t* out, uint16_t* const* out_ptrs, int64_t row_bound,
+                             bgmoe_stream_t stream);
+
+/* out = bf16( act(x Wg^T) * (x Wu^T) ).  Replaces `marlin_grouped_stage1_fused_mxfp4_situ`
+ * (batchgen/moe/marlin_grouped_moe.py:411-470).  activation 0 = SwiGLU (silu), the activation of
+ * the benchmark's Kimi-K3-shaped config; the reference model's SiTU epilogue is not built. */
+int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight* gate,
+                         const bgmoe_mxfp4_weight* up, const int32_t* seqlens,
+                         const int32_t* cu_seqlens, int groups, int64_t m, int n, int k, uint16_t* out,
+                         uint16_t* const* out_ptrs, int activation, int64_t row_bound,
+                         bgmoe_stream_t stream);
+
 /* ------------------------------------------------------------ whole layer */
 
 /* One FP8 MoE layer forward on one GPU's share of the experts:

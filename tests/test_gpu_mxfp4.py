@@ -1,0 +1,136 @@
+"""HIP MXFP4 (W4A16) grouped GEMMs vs the CPU oracle (dequantise with the frozen-vector-pinned codec, then
+fp32 matmul on bf16 operands)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as og
+from oracle import mxfp4 as mx
+from oracle import quant as oq
+from tests.util import rand_bf16, say
+
+pytestmark = pytest.mark.gpu
+
+
+def mg():
+    from batchgen_amd.kernels import load_extension
+    return load_extension("batchgen_kernels.moe._C_marlin_grouped_gemm")
+
+
+def _weights(seed, g, n, k):
+    rng = np.random.default_rng(seed)
+    return mx.quantize((0.02 * rng.standard_normal((g, n, k))).astype(np.float32))
+
+
+def _layout(counts, align=16):
+    counts = np.asarray(counts, dtype=np.int32)
+    cu = np.concatenate([[0], np.cumsum((counts + align - 1) // align * align)]).astype(np.int32)
+    return counts, cu
+
+
+def test_dequant_in_registers_is_exact(dev):
+    """One-hot activations read the dequantised weights back: every nibble code, scale bytes 112..134."""
+    n, k = 128, 256
+    rng = np.random.default_rng(0)
+    packed = rng.integers(0, 256, size=(1, n, k // 2), dtype=np.uint8)
+    scales = rng.integers(112, 135, size=(1, n, k // 32), dtype=np.uint8)
+    x = torch.eye(k, dtype=torch.bfloat16)                                  # token t = unit vector e_t
+    counts, cu = np.array([k], dtype=np.int32), np.array([0, k], dtype=np.int32)
+    out = mg().mxfp4_grouped_gemm(x.to(dev), torch.from_numpy(packed).to(dev), torch.from_numpy(scales).to(dev),
+                                  torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev))
+    w = mx.dequant(packed[0], scales[0])                                    # [n, k]
+    assert np.array_equal(out.float().cpu().numpy(), w.T)                   # exact: all values are bf16
+    # the reference's frozen vector through the kernel
+    vec = bytes([0xAB, 0x4C, 0x18, 0x65, 0x2C, 0x91, 0x04, 0x39, 0x48, 0x94, 0x58, 0x33, 0x94, 0xB5, 0x5B, 0x30])
+    packed[0, 0, :16] = np.frombuffer(vec, dtype=np.uint8)
+    scales[0, 0, 0] = 0x79
+    out = mg().mxfp4_grouped_gemm(x.to(dev), torch.from_numpy(packed).to(dev), torch.from_numpy(scales).to(dev),
+                                  torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev))
+    bits = out[:32, 0].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    expect = np.array([0xBCC0, 0xBC80, 0xBD00, 0x3D00, 0x8000, 0x3C00, 0x3D40, 0x3D80, 0xBD00, 0x3C80, 0x3C00, 0xBC00,
+                       0x3D00, 0x0000, 0xBC00, 0x3CC0, 0x8000, 0x3D00, 0x3D00, 0xBC00, 0x8000, 0x3D40, 0x3CC0, 0x3CC0,
+                       0x3D00, 0xBC00, 0x3D40, 0xBCC0, 0xBCC0, 0x3D40, 0x0000, 0x3CC0], dtype=np.uint16)
+    assert np.array_equal(bits & 0x7FFF, expect & 0x7FFF) and np.array_equal(bits[expect != 0x8000], expect[expect != 0x8000])
+
+
+@pytest.mark.parametrize("counts,n,k", [((0, 1, 15, 16, 17, 31, 32, 33, 64, 70), 256, 512), ((9,) * 4, 2048, 1024),
+                                        ((5, 0, 40), 384, 256)])
+@pytest.mark.parametrize("layout", ["row_major", "tile_major"])
+def test_grouped_gemm_and_fused_s1(dev, counts, n, k, layout):
+    say("mxfp4", counts, n, k, layout)
+    counts, cu = _layout(counts)
+    m = int(cu[-1])
+    g = torch.Generator().manual_seed(n + k)
+    x = rand_bf16(g, m, k)
+    (gp, gs), (up, us) = _weights(1, len(counts), n, k), _weights(2, len(counts), n, k)
+    d = lambda a: torch.from_numpy(a).to(dev)
+    gpd, gsd, upd, usd = d(gp), d(gs), d(up), d(us)
+    if layout == "tile_major":
+        gpd, gsd = mg().mxfp4_weight_repack(gpd, gsd)
+        upd, usd = mg().mxfp4_weight_repack(upd, usd)
+    cnt_d, cu_d = d(counts), d(cu)
+    live = np.zeros(m, dtype=bool)
+    for e, c in enumerate(counts):
+        live[cu[e]:cu[e] + c] = True
+    out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+    mg().mxfp4_grouped_gemm(x.to(dev), gpd, gsd, cnt_d, cu_d, out, weight_layout=layout)
+    ref = og.grouped_gemm_mxfp4(oq.as_f32(x), gp, gs, counts, cu, to_bf16=False)
+    o = out.float().cpu().numpy()
+    np.testing.assert_allclose(o[live], ref[live], rtol=1e-2, atol=2e-3)
+    assert og.rel_frobenius(o[live], ref[live]) < 3e-3 and np.all(o[~live] == 7.0)
+    h = mg().mxfp4_fused_s1(x.to(dev), gpd, gsd, upd, usd, cnt_d, cu_d, weight_layout=layout)
+    gate = og.grouped_gemm_mxfp4(oq.as_f32(x), gp, gs, counts, cu, to_bf16=False)
+    upv = og.grouped_gemm_mxfp4(oq.as_f32(x), up, us, counts, cu, to_bf16=False)
+    href = oq.silu_f32(gate) * upv
+    assert og.rel_frobenius(h.float().cpu().numpy()[live], href[live]) < 4e-3
+
+
+def test_reference_op_names_with_pointer_tables(dev):
+    counts, cu = _layout((7, 0, 20, 33))
+    m, n, k, e = int(cu[-1]), 256, 512, 4
+    g = torch.Generator().manual_seed(3)
+    x = rand_bf16(g, m, k).to(dev)
+    (gp, gs), (up, us) = _weights(4, e, n, k), _weights(5, e, n, k)
+    d = lambda a: torch.from_numpy(a).to(dev)
+    gpt, gst = mg().mxfp4_weight_repack(d(gp), d(gs))
+    upt, ust = mg().mxfp4_weight_repack(d(up), d(us))
+    tbl = lambda t: torch.tensor([t[i].data_ptr() for i in range(e)], dtype=torch.int64, device=dev)
+    cnt_d, cu_d = d(counts), d(cu[:e].copy())
+    c = torch.zeros((m, n), dtype=torch.bfloat16, device=dev)
+    c_ptrs = torch.tensor([c[int(cu[i])].data_ptr() for i in range(e)], dtype=torch.int64, device=dev)
+    mg().grouped_marlin_gemm_m16_s1_mxfp4_situ(x, tbl(gpt), tbl(upt), c_ptrs, tbl(gst), tbl(ust), cu_d, cnt_d, e, n, k,
+                                               None, n // 256, 4)
+    ref = mg().mxfp4_fused_s1(x, gpt, gst, upt, ust, cnt_d, d(cu), weight_layout="tile_major")
+    live = torch.zeros(m, dtype=torch.bool)
+    for i, cc in enumerate(counts):
+        live[cu[i]:cu[i] + cc] = True
+    assert torch.equal(c[live.to(dev)], ref[live.to(dev)])
+    c2 = torch.zeros((m, n), dtype=torch.bfloat16, device=dev)
+    c2_ptrs = torch.tensor([c2[int(cu[i])].data_ptr() for i in range(e)], dtype=torch.int64, device=dev)
+    mg().marlin_grouped_m16_mxfp4(x, tbl(gpt), c2_ptrs, tbl(gst), cu_d, cnt_d, e, n, k, None, 1, n // 256, 4)
+    ref2 = mg().mxfp4_grouped_gemm(x, gpt, gst, cnt_d, d(cu), weight_layout="tile_major")
+    assert torch.equal(c2[live.to(dev)], ref2[live.to(dev)])
+
+
+def test_mxfp4_layer_matches_oracle(dev):
+    from batchgen_amd import workloads as wl
+    from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
+    from oracle import layer as ol
+    cfg = wl.scaled(wl.CONFIGS[3], n_tokens=96, hidden=512, inter=256, shared_inter=256, n_experts=224, e_local=28,
+                    expert_start=56, max_tokens=96)
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_mxfp4_weights(cfg, "cpu")
+    layer = Mxfp4MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
+                          inp["bias"].to(dev))
+    out = layer(inp["x"].to(dev), inp["logits"].to(dev))
+    wn = {k: v.numpy() for k, v in w.items()}
+    shn = {k: v.float().numpy() for k, v in sh.items()}
+    ref = ol.moe_layer_mxfp4(inp["x"], inp["logits"].numpy(), inp["bias"].numpy(),
+                             dict(top_k=cfg.top_k, n_group=1, topk_group=1, rsf=cfg.rsf), wn, cfg.expert_start,
+                             cfg.e_local, layout="masked", max_tokens=cfg.max_tokens, shared_bf16=shn)
+    assert np.array_equal(layer.topk_ids.cpu().numpy(), ref["ids"])
+    assert np.array_equal(layer.topk_pos.cpu().numpy(), ref["pos"])
+    assert np.array_equal(layer.expert_counts.cpu().numpy(), ref["counts"])
+    err = og.rel_frobenius(out.float().cpu().numpy(), ref["out"])
+    say("   mxfp4 layer rel frobenius:", err)
+    assert err < 1e-2

@@ -140,3 +140,14 @@ def test_mxfp4_quantize_closed_form():
     t = np.array([[0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0] + [0.0] * 24], dtype=np.float32)
     pt, st = mx.quantize(t)
     assert st[0, 0] == 127 and mx.dequant(pt, st)[0, :8].tolist() == [0.0, 1.0, 1.0, 2.0, 2.0, 4.0, 4.0, 6.0]
+
+
+def test_torch_mxfp4_quantiser_of_the_workloads_equals_the_oracle():
+    from batchgen_amd.workloads import quantize_mxfp4
+    g = torch.Generator().manual_seed(5)
+    w = torch.randn(64, 256, generator=g) * 0.02
+    w[0, :32] = 0
+    w[1, 0] = 5.0 * 2.0 ** -7
+    p, s = quantize_mxfp4(w)
+    po, so = mx.quantize(w.numpy())
+    assert np.array_equal(p.numpy(), po) and np.array_equal(s.numpy(), so)
