@@ -301,14 +301,21 @@ static void launch_variant(bool fused, int layout, dim3 grid, const SkinnyArgs& 
 // Rows per group up to which the weight-streaming kernel is used (each 32-row chunk of a group
 // streams the group's weights once more, mostly from the last-level cache); groups with more
 // rows go to the LDS-tiled kernel.
+static int g_skinny_max_rows = -1;
+
 static int skinny_limit() {
-  static int v = -1;
-  if (v < 0) {
+  if (g_skinny_max_rows < 0) {
     const char* e = getenv("BGMOE_SKINNY_MAX_ROWS");
-    v = e ? atoi(e) : 256;
-    if (v < 0) v = 0;
+    g_skinny_max_rows = e ? atoi(e) : 256;
+    if (g_skinny_max_rows < 0) g_skinny_max_rows = 0;
   }
-  return v;
+  return g_skinny_max_rows;
+}
+
+extern "C" int bgmoe_set_skinny_max_rows(int rows) {
+  BGMOE_REQUIRE(rows >= 0, "set_skinny_max_rows: rows must be >= 0");
+  g_skinny_max_rows = rows;
+  return BGMOE_OK;
 }
 
 static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {

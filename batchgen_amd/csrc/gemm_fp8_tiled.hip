@@ -1,30 +1,39 @@
-// Block-scaled FP8 grouped GEMM for MANY rows per group (prefill, the shared
-// expert): an LDS-tiled MFMA kernel.
+// Block-scaled FP8 grouped GEMM for MANY rows per group (prefill): an LDS-tiled MFMA kernel.
 //
-// Macro tile: 128 tokens x 256 weight rows x 128 K per step (fused stage 1:
-// 128 gate + 128 up rows, so SwiGLU and the requant of one 128-column group
-// stay inside the block).  4 waves; wave w owns 64 weight rows (fused: 32 gate
-// + 32 up) for all 128 tokens = 8 x 4 MFMA 16x16x128 tiles, 128 accumulator
-// registers.  Global -> registers -> LDS double buffering, one barrier per K
-// step.  LDS rows are 128 B with the 16-byte chunk index XOR-swizzled by
-// (row & 7), which makes both the 16-byte stores and the MFMA operand reads
-// (16 rows x 16 B per quarter-wave) conflict free.
+// Macro tile: 128 tokens x 256 weight rows x 128 K per step (fused stage 1: 128 gate + 128 up rows, so
+// SwiGLU and the requant of one 128-column group stay inside the block).  4 waves; wave w owns 64
+// weight rows (fused: 32 gate + 32 up) for all 128 tokens = 8 x 4 MFMA 16x16x128 tiles, 128 fp32
+// accumulators per lane.
 //
-// Scheduling: a fixed grid of persistent blocks walks a device-built list of
-// (group, n-tile, m-tile) work items, m fastest, so the blocks of one XCD
-// (block b runs on XCD b % 8) work on neighbouring m-tiles of the same weight
-// tile and share it through that XCD's L2.  Groups with <= `lo` rows are left
-// to the weight-streaming kernel; empty groups cost nothing.
+// Operand staging: a 3-slot LDS ring filled by ASYNCHRONOUS global -> LDS loads
+// (global_load_lds_dwordx4: every lane supplies its own global address, the wave's 64 x 16 bytes land
+// contiguously at the LDS address in M0).  The lane -> address map is chosen so that each 1 KiB wave
+// load is half of an MFMA operand "tile image": lane l = q*16 + r carries row r, bytes 16q..16q+15 of
+// the 64-byte half-segment, which is exactly what lane l feeds to v_mfma_f32_16x16x128_f8f6f4 -- so
+// operand reads from LDS are plain lane*16 accesses (conflict free, no swizzle), for row-major tokens,
+// row-major weights and tile-major weights alike.  Two K-steps are always in flight behind the one
+// being computed; completion is tracked by hand with s_waitcnt vmcnt(N) (the loads are issued from
+// inline asm, which keeps the compiler from draining the whole queue before every LDS read) and one
+// s_barrier per K-step.
+//
+// Scheduling: a fixed grid of persistent blocks walks a device-built list of (group, n-tile, m-tile)
+// work items, m fastest, so the blocks of one XCD (block b runs on XCD b % 8) work on neighbouring
+// m-tiles of the same weight tile and share it through that XCD's L2.  Groups with <= `lo` rows are
+// left to the weight-streaming kernel; empty groups cost nothing.
 #include "bgmoe_common.h"
 
 namespace {
 
 constexpr int TM = 128;            // tokens per macro tile
 constexpr int TW = 256;            // weight rows per macro tile
+constexpr int NS = 3;              // LDS ring slots
 constexpr int kTokBytes = TM * 128;
 constexpr int kWBytes = TW * 128;
-constexpr int kBufBytes = kTokBytes + kWBytes + TM * 4;
+constexpr int kXsOff = kTokBytes + kWBytes;
+constexpr int kSlotBytes = kXsOff + TM * 4;
+constexpr int kLoadsPerStage = 13; // per wave: 4 token halves + 8 weight halves + 1 scale load
 constexpr int kMaxGroups = 1024;
+constexpr int kMaxKB = 256;        // K <= 32768
 
 struct TiledArgs {
   bgmoe_fp8_act a;
@@ -37,15 +46,28 @@ struct TiledArgs {
   float* out_s;
   int64_t os_row, os_nb;
   int lo;
-  int fused;
 };
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
+// 64 lanes x 16 bytes -> LDS [lds_base, lds_base + 1024); lds_base must be wave-uniform.  No
+// instruction offset is used: the hardware would add it to the LDS address as well as to the
+// global address.
+__device__ __forceinline__ void async_load16(const uint8_t* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :: "s"(lds_base), "v"(gptr) : "memory", "m0");
+}
+// 64 lanes x 4 bytes -> LDS [lds_base, lds_base + 256)
+__device__ __forceinline__ void async_load4(const float* gptr, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" :: "s"(lds_base), "v"(gptr) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+__device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 template <bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
-  extern __shared__ __align__(16) uint8_t smem[];
-  __shared__ int s_tiles[kMaxGroups + 1];       // exclusive prefix of m-tiles per group
+  extern __shared__ __align__(16) uint8_t smem[];      // NS slots
+  __shared__ int s_tiles[kMaxGroups + 1];              // exclusive prefix of m-tiles per group
+  __shared__ float s_ws[2][kMaxKB];                    // this item's weight scales along K
   __shared__ float s_amax[4][8][16];
 
   const int tid = threadIdx.x;
@@ -55,16 +77,23 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
   const int kq = lane >> 4;
   const int K = g.k;
   const int KB = K >> 7;
-  const int ncols = FUSED ? 128 : 256;           // output columns per macro tile
+  const int ncols = FUSED ? 128 : 256;                 // output columns per macro tile
   const int ntn = (g.n + ncols - 1) / ncols;
+  const uint32_t smem_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
+  const uint32_t wave_u = __builtin_amdgcn_readfirstlane((uint32_t)wave);
 
   // ---- work list: m-tiles per group, prefix-summed (every block computes the same list) ----
+  for (int e = tid; e < g.groups; e += 256) {
+    const int c = g.seqlens[e];
+    s_tiles[e + 1] = c > g.lo ? (c + TM - 1) / TM : 0;
+  }
+  __syncthreads();
   if (tid == 0) {
     int run = 0;
     for (int e = 0; e < g.groups; ++e) {
+      const int t = s_tiles[e + 1];
       s_tiles[e] = run;
-      const int c = g.seqlens[e];
-      run += c > g.lo ? (c + TM - 1) / TM : 0;
+      run += t;
     }
     s_tiles[g.groups] = run;
   }
@@ -78,17 +107,14 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
   const int bstep = (gridDim.x + nx - 1 - xcd) / nx;   // blocks living on this XCD
   const int bidx = blockIdx.x / nx;
 
-  for (int64_t it = (int64_t)bidx; it < per_x; it += bstep) {
-    const int64_t item = (int64_t)xcd * per_x + it;
+  for (int64_t itx = (int64_t)bidx; itx < per_x; itx += bstep) {
+    const int64_t item = (int64_t)xcd * per_x + itx;
     if (item >= total) break;
     // item -> (group, n-tile, m-tile): within a group, m fastest
     int lo_g = 0, hi_g = g.groups - 1;
-    {
-      // find group: largest e with s_tiles[e]*ntn <= item
-      while (lo_g < hi_g) {
-        const int mid = (lo_g + hi_g + 1) >> 1;
-        if ((int64_t)s_tiles[mid] * ntn <= item) lo_g = mid; else hi_g = mid - 1;
-      }
+    while (lo_g < hi_g) {
+      const int mid = (lo_g + hi_g + 1) >> 1;
+      if ((int64_t)s_tiles[mid] * ntn <= item) lo_g = mid; else hi_g = mid - 1;
     }
     const int grp = lo_g;
     const int mt_g = s_tiles[grp + 1] - s_tiles[grp];
@@ -110,65 +136,60 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
             (int64_t)(n0 >> 7) * g.w1.scale_nb_stride;
       ws0 += (int64_t)(n0 >> 7) * g.w0.scale_nb_stride;
     }
-    const float* wsw = nullptr;                    // non-fused: this wave's 128-row block
-    if constexpr (!FUSED) wsw = ws0 + (int64_t)(min(n0 + 64 * wave, g.n - 1) >> 7) * g.w0.scale_nb_stride;
 
-    // ---- global -> register staging: 4 token chunks + 8 weight chunks per thread per step ----
-    const int lrow = tid >> 3;                     // 0..31
-    const int chunk = tid & 7;
-    const uint8_t* tok_src[4];
+    __syncthreads();          // the previous item's reads of s_ws / s_amax / the LDS ring are done
+    // weight scales of this item along K -> LDS (fused: [0] gate, [1] up; else [0] cols 0..127, [1] cols 128..255)
+    for (int kb = tid; kb < KB; kb += 256) {
+      if constexpr (FUSED) {
+        s_ws[0][kb] = ws0[kb];
+        s_ws[1][kb] = ws1[kb];
+      } else {
+        const int nb0 = min(n0, g.n - 1) >> 7, nb1 = min(n0 + 128, g.n - 1) >> 7;
+        s_ws[0][kb] = ws0[(int64_t)nb0 * g.w0.scale_nb_stride + kb];
+        s_ws[1][kb] = ws0[(int64_t)nb1 * g.w0.scale_nb_stride + kb];
+      }
+    }
+
+    // ---- this wave's share of a stage: token tiles 2w, 2w+1; weight tiles 4w .. 4w+3; 64 token scales ----
+    const uint8_t* tok_src[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int tok = min(m0 + 16 * (2 * wave + i) + r16, cnt - 1);
+      tok_src[i] = g.a.x + (row0 + tok) * K + 16 * kq;
+    }
+    const uint8_t* w_src[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int tok = min(m0 + i * 32 + lrow, cnt - 1);
-      tok_src[i] = g.a.x + (row0 + tok) * K + chunk * 16;
+      const int lt = 4 * wave + i;                 // LDS weight tile 0..15 (16 rows each)
+      const int r = lt * 16;
+      const int nrow = FUSED ? min(n0 + (r & 127), g.n - 16) : min(n0 + r, g.n - 16);
+      const uint8_t* base = (FUSED && r >= 128) ? wb1 : wb0;
+      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) w_src[i] = base + (int64_t)(nrow + r16) * K + 16 * kq;
+      else w_src[i] = base + (int64_t)(nrow >> 4) * K * 16 + lane * 16;
     }
-    const uint8_t* w_src[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
-        const int r = i * 32 + lrow;               // LDS weight row 0..255
-        if constexpr (FUSED) {
-          const int nrow = min(n0 + (r & 127), g.n - 1);
-          w_src[i] = (r < 128 ? wb0 : wb1) + (int64_t)nrow * K + chunk * 16;
-        } else {
-          const int nrow = min(n0 + r, g.n - 1);
-          w_src[i] = wb0 + (int64_t)nrow * K + chunk * 16;
-        }
-      } else {
-        // tile-major source: LDS keeps the 2 KiB tile image; this thread moves 16 bytes of LDS tile
-        // 2*i + (tid >> 7) (16 weight rows each), a contiguous 2 KiB per 128 threads
-        const int lt = 2 * i + (tid >> 7);         // LDS tile 0..15
-        const int r = lt * 16;
-        const int nrow = FUSED ? min(n0 + (r & 127), g.n - 16) : min(n0 + r, g.n - 16);
-        w_src[i] = ((FUSED && r >= 128) ? wb1 : wb0) + (int64_t)(nrow >> 4) * K * 16 + (tid & 127) * 16;
-      }
-    }
-    const float* xs_src = nullptr;
-    if (tid < TM) xs_src = g.a.scale + (row0 + min(m0 + tid, cnt - 1)) * g.a.scale_row_stride;
+    const float* xs_src = g.a.scale + (row0 + min(m0 + 64 * (wave & 1) + lane, cnt - 1)) * g.a.scale_row_stride;
 
-    intx4 rt[4], rw[8];
-    float rxs = 0.0f;
-    auto gload = [&](int kb) {
+    auto issue = [&](int kb, int slot) {
+      const uint32_t sb = smem_base + (uint32_t)slot * kSlotBytes;
       const int ko = kb << 7;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) rt[i] = gload_x4(tok_src[i] + ko);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        rw[i] = gload_x4(w_src[i] + (LAYOUT == BGMOE_W_ROW_MAJOR ? (int64_t)ko : ((int64_t)kb << 11)));
-      if (tid < TM) rxs = xs_src[(int64_t)kb * g.a.scale_kb_stride];
-    };
-    auto lstore = [&](int buf) {
-      uint8_t* b = smem + buf * kBufBytes;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<intx4*>(b + swz(i * 32 + lrow, chunk)) = rt[i];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR)
-          *reinterpret_cast<intx4*>(b + kTokBytes + swz(i * 32 + lrow, chunk)) = rw[i];
-        else
-          *reinterpret_cast<intx4*>(b + kTokBytes + i * 4096 + tid * 16) = rw[i];
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t d = sb + (2 * wave_u + i) * 2048;
+        async_load16(tok_src[i] + ko, d);
+        async_load16(tok_src[i] + ko + 64, d + 1024);
       }
-      if (tid < TM) reinterpret_cast<float*>(b + kTokBytes + kWBytes)[tid] = rxs;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t d = sb + kTokBytes + (4 * wave_u + i) * 2048;
+        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
+          async_load16(w_src[i] + ko, d);
+          async_load16(w_src[i] + ko + 64, d + 1024);
+        } else {
+          async_load16(w_src[i] + ((int64_t)kb << 11), d);
+          async_load16(w_src[i] + ((int64_t)kb << 11) + 1024, d + 1024);
+        }
+      }
+      async_load4(xs_src + (int64_t)kb * g.a.scale_kb_stride, sb + kXsOff + (wave_u & 1) * 256);
     };
 
     floatx4 acc[8][4];
@@ -177,58 +198,53 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    __syncthreads();          // previous item's LDS reads are done
-    gload(0);
-    lstore(0);
-    __syncthreads();
+    // prologue: two K-steps in flight (a step past the end re-reads the last one; it is never computed)
+    issue(0, 0);
+    issue(min(1, KB - 1), 1);
+    __syncthreads();          // s_ws is visible (compiler-tracked stores)
 
     for (int kb = 0; kb < KB; ++kb) {
-      const int cur = kb & 1;
-      if (kb + 1 < KB) gload(kb + 1);
-      const uint8_t* b = smem + cur * kBufBytes;
+      const int slot = kb % NS;
+      wait_vm<kLoadsPerStage>();                 // this wave's loads of step kb have landed ...
+      block_barrier();                           // ... and everybody's; everybody is done with step kb-1
+      issue(min(kb + 2, KB - 1), (kb + 2) % NS); // refill the slot step kb-1 used
+
+      const uint8_t* b = smem + slot * kSlotBytes;
       const uint8_t* bw = b + kTokBytes;
-      const float* bxs = reinterpret_cast<const float*>(b + kTokBytes + kWBytes);
-      float wsc[2];
-      if constexpr (FUSED) { wsc[0] = ws0[kb]; wsc[1] = ws1[kb]; }
-      else { wsc[0] = wsw[kb]; wsc[1] = wsc[0]; }
+      const float* bxs = reinterpret_cast<const float*>(b + kXsOff);
+      const float wsc0 = s_ws[0][kb], wsc1 = s_ws[1][kb];
 
       intx8 A[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const int wr = FUSED ? ((t >> 1) * 128 + 32 * wave + 16 * (t & 1) + r16) : (64 * wave + 16 * t + r16);
-        intx4 lo, hi;
-        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
-          lo = *reinterpret_cast<const intx4*>(bw + swz(wr, kq));
-          hi = *reinterpret_cast<const intx4*>(bw + swz(wr, 4 + kq));
-        } else {
-          lo = *reinterpret_cast<const intx4*>(bw + (wr >> 4) * 2048 + lane * 16);
-          hi = *reinterpret_cast<const intx4*>(bw + (wr >> 4) * 2048 + 1024 + lane * 16);
-        }
+        const int lt = FUSED ? ((t >> 1) * 8 + 2 * wave + (t & 1)) : (4 * wave + t);
+        const intx4 lo = *reinterpret_cast<const intx4*>(bw + lt * 2048 + lane * 16);
+        const intx4 hi = *reinterpret_cast<const intx4*>(bw + lt * 2048 + 1024 + lane * 16);
         A[t] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
 #pragma unroll
       for (int tt = 0; tt < 8; ++tt) {
-        const int tr = 16 * tt + r16;
-        const intx4 lo = *reinterpret_cast<const intx4*>(b + swz(tr, kq));
-        const intx4 hi = *reinterpret_cast<const intx4*>(b + swz(tr, 4 + kq));
+        const intx4 lo = *reinterpret_cast<const intx4*>(b + tt * 2048 + lane * 16);
+        const intx4 hi = *reinterpret_cast<const intx4*>(b + tt * 2048 + 1024 + lane * 16);
         const intx8 B = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        const float xs = bxs[tr];
+        const float xs = bxs[16 * tt + r16];
+        const float sc0 = xs * wsc0;
+        const float sc1 = xs * (FUSED ? wsc1 : ((wave >= 2) ? wsc1 : wsc0));
+        const float sc_lo = FUSED ? sc0 : sc1;   // non-fused: all four tiles of a wave share one 128-column block
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
               A[t], B, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-          const float sc = xs * wsc[FUSED ? (t >> 1) : 0];
+          const float sc = FUSED ? ((t >> 1) ? sc1 : sc0) : sc_lo;
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[tt][t][i] = fmaf(p[i], sc, acc[tt][t][i]);
         }
       }
-      if (kb + 1 < KB) lstore(cur ^ 1);
-      __syncthreads();
     }
+    wait_vm<0>();             // drain the tail prefetches before the ring is reused
 
     // ---- epilogue ----------------------------------------------------------------
     if constexpr (FUSED) {
-      // h = bf16(silu(gate) * up), kept in acc[tt][0..1]
 #pragma unroll
       for (int tt = 0; tt < 8; ++tt) {
         float am = 0.0f;
@@ -308,10 +324,15 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
     bgmoe_set_error("fp8 tiled gemm: groups=%d exceeds %d", groups, kMaxGroups);
     return BGMOE_ERR_ARG;
   }
+  if ((k >> 7) > kMaxKB) {
+    bgmoe_set_error("fp8 tiled gemm: K=%d exceeds %d", k, kMaxKB * 128);
+    return BGMOE_ERR_ARG;
+  }
   TiledArgs g{};
   g.a = *a; g.w0 = *w0; if (w1) g.w1 = *w1;
   g.seqlens = seqlens; g.cu = cu; g.groups = groups; g.n = n; g.k = k;
   g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.lo = lo;
+  constexpr int kLds = NS * kSlotBytes;
   static bool attr_set = false;
   if (!attr_set) {
     hipDeviceProp_t prop;
@@ -327,11 +348,11 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
                           reinterpret_cast<const void*>(&fp8_tiled_kernel<true, 1>),
                           reinterpret_cast<const void*>(&fp8_tiled_kernel<false, 1>)};
     for (const void* f : fns) {
-      hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kBufBytes);
+      hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
       if (e != hipSuccess) e1 = e;
     }
     if (e1 != hipSuccess) {
-      bgmoe_set_error("fp8 tiled gemm: cannot reserve %d bytes of LDS", 2 * kBufBytes);
+      bgmoe_set_error("fp8 tiled gemm: cannot reserve %d bytes of LDS", kLds);
       return BGMOE_ERR_HIP;
     }
     attr_set = true;
@@ -347,11 +368,11 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   const dim3 grid((unsigned)blocks), block(256);
   const bool tm = w0->layout == BGMOE_W_TILE_MAJOR;
   if (w1) {
-    if (tm) hipLaunchKernelGGL((fp8_tiled_kernel<true, 1>), grid, block, 2 * kBufBytes, st, g);
-    else hipLaunchKernelGGL((fp8_tiled_kernel<true, 0>), grid, block, 2 * kBufBytes, st, g);
+    if (tm) hipLaunchKernelGGL((fp8_tiled_kernel<true, 1>), grid, block, kLds, st, g);
+    else hipLaunchKernelGGL((fp8_tiled_kernel<true, 0>), grid, block, kLds, st, g);
   } else {
-    if (tm) hipLaunchKernelGGL((fp8_tiled_kernel<false, 1>), grid, block, 2 * kBufBytes, st, g);
-    else hipLaunchKernelGGL((fp8_tiled_kernel<false, 0>), grid, block, 2 * kBufBytes, st, g);
+    if (tm) hipLaunchKernelGGL((fp8_tiled_kernel<false, 1>), grid, block, kLds, st, g);
+    else hipLaunchKernelGGL((fp8_tiled_kernel<false, 0>), grid, block, kLds, st, g);
   }
   return bgmoe_check_launch("fp8 grouped gemm (tiled)");
 }

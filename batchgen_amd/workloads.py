@@ -91,7 +91,7 @@ def zipf_logit_bias(cfg: MoEConfig, c: float, device) -> torch.Tensor:
     return (c * pmf.log()).to(device)
 
 
-ZIPF_C = 2.6   # chosen so that about 30% of the experts get no token and the hottest gets > 2000 (config 4)
+ZIPF_C = 0.67   # chosen so that about 30% of the experts get no token and the hottest gets > 2000 (config 4)
 
 
 def make_inputs(cfg: MoEConfig, device, n_tokens: Optional[int] = None):

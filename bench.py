@@ -31,7 +31,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 4])
+    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain copy kernel of known size (the weight re-layout kernel on a "
@@ -102,8 +102,14 @@ def main():
     torch.cuda.set_device(dev)
     cfg = wl.CONFIGS[a.config]
     inp = wl.make_inputs(cfg, dev)
-    w, sh = wl.make_fp8_weights(cfg, dev)
-    layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
+    mx4 = cfg.weight_format == "mxfp4"
+    if mx4:
+        from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
+        w, sh = wl.make_mxfp4_weights(cfg, dev)
+        layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"])
+    else:
+        w, sh = wl.make_fp8_weights(cfg, dev)
+        layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
     x, logits = inp["x"], inp["logits"]
 
     for _ in range(a.warmup):
@@ -125,7 +131,7 @@ def main():
     counts = layer.expert_counts[:cfg.e_local].cpu().numpy()
     active = int((counts > 0).sum())
     rows = int(counts.sum())
-    alg_bytes = wl.algorithmic_bytes_fp8(cfg, active, rows)
+    alg_bytes = wl.algorithmic_bytes_mxfp4(cfg, active, rows) if mx4 else wl.algorithmic_bytes_fp8(cfg, active, rows)
     flops = wl.flops_routed(cfg, rows) + (wl.flops_routed(cfg, cfg.n_tokens) * cfg.shared_inter // cfg.inter
                                           if cfg.shared_inter else 0)
     decode = cfg.layout == "masked"
@@ -140,7 +146,14 @@ def main():
     _lib.prof_enable(False)
     per_kernel = {k: v[0] / a.steps for k, v in prof.items()}          # ms per step
     h, i = cfg.hidden, cfg.inter
-    if decode:
+    if mx4:
+        dom = "mxfp4_s1"
+        dom_bytes = active * (2 * h * i // 2 + 2 * h * i // 32) + rows * (h + i) * 2
+        dom_ms = prof[dom][0] / max(prof[dom][1], 1)
+        roof = dict(bound="hbm", kernel="mxfp4_skinny_kernel<TT=2,NS=3,fused,tile_major>",
+                    achieved=dom_bytes / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None,
+                    bytes_per_launch=dom_bytes, avg_launch_us=dom_ms * 1e3)
+    elif decode:
         dom = "s1_skinny16"
         # one launch streams gate+up of every active routed expert and of the shared expert once
         # (algorithmic bytes: each weight byte once, each quantised row in, each requantised row out)
@@ -168,7 +181,7 @@ def main():
         "unit": "GB/s" if decode else "TFLOP/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp8_e4m3 (fp32 accumulate)", "data": "synthetic",
+        "dtype": "mxfp4 weights x bf16 (fp32 accumulate)" if mx4 else "fp8_e4m3 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": cfg.name, "tokens": cfg.n_tokens, "hidden": h, "moe_intermediate": i,
                    "experts": cfg.n_experts, "local_experts": cfg.e_local, "top_k": cfg.top_k,
                    "layout": cfg.layout, "shared_expert": bool(cfg.shared_inter)},
@@ -179,7 +192,7 @@ def main():
         "kernel_ms_per_step": per_kernel,
         "roofline": roof,
     }
-    if not a.no_cpu_baseline:
+    if not a.no_cpu_baseline and not mx4:
         ids = layer.topk_ids.cpu().numpy()
         wt = layer.topk_weights.cpu().numpy()
         t, threads, cores, sample, frac = cpu_baseline(cfg, inp, w, sh, ids, wt, alg_bytes, flops)

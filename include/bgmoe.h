@@ -243,6 +243,12 @@ int bgmoe_fp8_grouped_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* b,
                            const int32_t* seqlens, const int32_t* cu_seqlens, int groups,
                            int64_t m, int n, int k, uint16_t* out, bgmoe_stream_t stream);
 
+/* Tuning knob (no reference counterpart): groups with at most `rows` rows are served by the
+ * weight-streaming kernel, larger ones by the LDS-tiled kernel.  0 sends everything to the tiled
+ * kernel.  Default 256 (or the environment variable BGMOE_SKINNY_MAX_ROWS at first use).
+ * Results do not depend on it beyond fp32 summation order. */
+int bgmoe_set_skinny_max_rows(int rows);
+
 /* Fused stage 1: out = bf16( silu(X*Wg^T) * (X*Wu^T) ), fp32 gate and up.
  * Replaces `fp8_blockwise_fused_s1` / `_ptrs`
  * (grouped_fp8_blockwise_moe.py:423-560, fp8_blockwise_s1_kernel.cuh:425-607).

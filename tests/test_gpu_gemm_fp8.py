@@ -245,3 +245,43 @@ def test_tile_major_weights_equal_row_major(dev, counts, n, k):
     a = gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16)
     b = gm().fp8_blockwise_fused_s1(xq_d, gq_t, uq_t, cnt_d, cu_d, xs_t, gs_d, us_d, 16, weight_layout="tile_major")
     assert torch.equal(a[live], b[live])
+
+
+@pytest.mark.parametrize("limit", [0, 16, 256])
+@pytest.mark.parametrize("layout", ["row_major", "tile_major"])
+def test_kernel_choice_does_not_change_results_beyond_rounding(dev, limit, layout):
+    """The same problem through the LDS-tiled kernel only (limit 0), a mix, and the streaming kernel."""
+    from batchgen_amd._lib import check, lib
+    counts, n, k = (0, 1, 15, 16, 17, 127, 128, 129, 260, 5), 384, 640
+    counts, cu, m, xq, xs, ws = _make(400, counts, n, k, nmat=2)
+    (gq, gs), (uq, us) = ws
+    xq_d, xs_t, gq_d, gs_d = _dev(dev, xq, xs, gq, gs)
+    _, _, uq_d, us_d = _dev(dev, xq, xs, uq, us)
+    if layout == "tile_major":
+        gq_d, uq_d = gm().fp8_weight_repack(gq_d), gm().fp8_weight_repack(uq_d)
+    cnt_d, cu_d = torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev)
+    live = np.zeros(m, dtype=bool)
+    for e, c in enumerate(counts):
+        live[cu[e]:cu[e] + c] = True
+    check(lib().bgmoe_set_skinny_max_rows(limit))
+    try:
+        out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+        gm().fp8_blockwise_grouped_gemm(xq_d, gq_d, cnt_d, cu_d, xs_t, gs_d, 16, out, weight_layout=layout)
+        h = gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16, weight_layout=layout)
+        hq = torch.zeros((m, n), dtype=torch.uint8, device=dev)
+        hs = torch.zeros((n // 128, m), dtype=torch.float32, device=dev)
+        gm().fp8_blockwise_fused_s1_quant(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, hq, hs, weight_layout=layout)
+        hq2 = torch.zeros((m, n), dtype=torch.uint8, device=dev)
+        hs2 = torch.zeros((n // 128, m), dtype=torch.float32, device=dev)
+        qops().act_quant_ragged(h, cnt_d, cu_d, hq2, hs2, 1)
+    finally:
+        check(lib().bgmoe_set_skinny_max_rows(256))
+    ref = og.grouped_gemm_fp8(xq, xs, gq, gs, counts, cu, to_bf16=False)
+    o = out.float().cpu().numpy()
+    np.testing.assert_allclose(o[live], ref[live], rtol=2e-2, atol=5e-3)
+    assert og.rel_frobenius(o[live], ref[live]) < 3e-3 and np.all(o[~live] == 7.0)
+    up = og.grouped_gemm_fp8(xq, xs, uq, us, counts, cu, to_bf16=False)
+    href = oq.silu_f32(ref) * up
+    assert og.rel_frobenius(h.float().cpu().numpy()[live], href[live]) < 4e-3
+    lv = torch.from_numpy(live).to(dev)
+    assert torch.equal(hq[lv], hq2[lv]) and torch.equal(hs[:, lv], hs2[:, lv])
