@@ -1,20 +1,22 @@
 // Block-scaled FP8 grouped GEMM for MANY rows per group (prefill): an LDS-tiled MFMA kernel.
 //
-// Macro tile: 128 tokens x 256 weight rows x 128 K per step (fused stage 1: 128 gate + 128 up rows, so
-// SwiGLU and the requant of one 128-column group stay inside the block).  4 waves; wave w owns 64
-// weight rows (fused: 32 gate + 32 up) for all 128 tokens = 8 x 4 MFMA 16x16x128 tiles, 128 fp32
-// accumulators per lane.
+// Macro tile: 256 tokens x 256 weight rows x 128 K per step (fused stage 1: 128 gate + 128 up rows, so
+// SwiGLU and the requant of one 128-column group stay inside the block).  8 waves = 4 (weight rows) x
+// 2 (tokens); a wave owns 64 weight rows (fused: 32 gate + 32 up) x 128 tokens = 8 x 4 MFMA 16x16x128
+// tiles, 128 fp32 accumulators per lane.  Two waves share a SIMD, so the fp32 promotion
+// (acc += partial * token_scale * weight_scale, VALU) of one overlaps the MFMAs of the other, and with
+// <= 256 registers per lane the compiler emits the MFMAs with VGPR destinations (no AGPR copies).
 //
-// Operand staging: a 3-slot LDS ring filled by ASYNCHRONOUS global -> LDS loads
+// Operand staging: a 2-slot LDS ring (2 x 65 KB) filled by ASYNCHRONOUS global -> LDS loads
 // (global_load_lds_dwordx4: every lane supplies its own global address, the wave's 64 x 16 bytes land
 // contiguously at the LDS address in M0).  The lane -> address map is chosen so that each 1 KiB wave
 // load is half of an MFMA operand "tile image": lane l = q*16 + r carries row r, bytes 16q..16q+15 of
 // the 64-byte half-segment, which is exactly what lane l feeds to v_mfma_f32_16x16x128_f8f6f4 -- so
 // operand reads from LDS are plain lane*16 accesses (conflict free, no swizzle), for row-major tokens,
-// row-major weights and tile-major weights alike.  Two K-steps are always in flight behind the one
-// being computed; completion is tracked by hand with s_waitcnt vmcnt(N) (the loads are issued from
-// inline asm, which keeps the compiler from draining the whole queue before every LDS read) and one
-// s_barrier per K-step.
+// row-major weights and tile-major weights alike.  The next K-step is in flight while the current one
+// is computed; completion is tracked by hand with s_waitcnt vmcnt (the loads are issued from inline
+// asm, which keeps the compiler from draining the queue before every LDS read) and one s_barrier per
+// K-step.
 //
 // Scheduling: a fixed grid of persistent blocks walks a device-built list of (group, n-tile, m-tile)
 // work items, m fastest, so the blocks of one XCD (block b runs on XCD b % 8) work on neighbouring
@@ -24,14 +26,14 @@
 
 namespace {
 
-constexpr int TM = 128;            // tokens per macro tile
+constexpr int TM = 256;            // tokens per macro tile
 constexpr int TW = 256;            // weight rows per macro tile
-constexpr int NS = 3;              // LDS ring slots
+constexpr int NS = 2;              // LDS ring slots
+constexpr int NT = 512;            // threads per block
 constexpr int kTokBytes = TM * 128;
 constexpr int kWBytes = TW * 128;
 constexpr int kXsOff = kTokBytes + kWBytes;
 constexpr int kSlotBytes = kXsOff + TM * 4;
-constexpr int kLoadsPerStage = 13; // per wave: 4 token halves + 8 weight halves + 1 scale load
 constexpr int kMaxGroups = 1024;
 constexpr int kMaxKB = 256;        // K <= 32768
 
@@ -64,14 +66,16 @@ __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :
 __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 template <bool FUSED, int LAYOUT>
-__global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
+__global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
   extern __shared__ __align__(16) uint8_t smem[];      // NS slots
   __shared__ int s_tiles[kMaxGroups + 1];              // exclusive prefix of m-tiles per group
   __shared__ float s_ws[2][kMaxKB];                    // this item's weight scales along K
-  __shared__ float s_amax[4][8][16];
+  __shared__ float s_amax[2][4][8][16];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
+  const int wn = wave & 3;                             // which 64 weight rows
+  const int wm = wave >> 2;                            // which 128 tokens
   const int lane = tid & 63;
   const int r16 = lane & 15;
   const int kq = lane >> 4;
@@ -83,7 +87,7 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane((uint32_t)wave);
 
   // ---- work list: m-tiles per group, prefix-summed (every block computes the same list) ----
-  for (int e = tid; e < g.groups; e += 256) {
+  for (int e = tid; e < g.groups; e += NT) {
     const int c = g.seqlens[e];
     s_tiles[e + 1] = c > g.lo ? (c + TM - 1) / TM : 0;
   }
@@ -139,7 +143,7 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
 
     __syncthreads();          // the previous item's reads of s_ws / s_amax / the LDS ring are done
     // weight scales of this item along K -> LDS (fused: [0] gate, [1] up; else [0] cols 0..127, [1] cols 128..255)
-    for (int kb = tid; kb < KB; kb += 256) {
+    for (int kb = tid; kb < KB; kb += NT) {
       if constexpr (FUSED) {
         s_ws[0][kb] = ws0[kb];
         s_ws[1][kb] = ws1[kb];
@@ -150,24 +154,24 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
       }
     }
 
-    // ---- this wave's share of a stage: token tiles 2w, 2w+1; weight tiles 4w .. 4w+3; 64 token scales ----
+    // ---- this wave's share of a stage: token tiles 2w, 2w+1; weight tiles 2w, 2w+1; waves 0..3: 64 token scales ----
     const uint8_t* tok_src[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int tok = min(m0 + 16 * (2 * wave + i) + r16, cnt - 1);
       tok_src[i] = g.a.x + (row0 + tok) * K + 16 * kq;
     }
-    const uint8_t* w_src[4];
+    const uint8_t* w_src[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int lt = 4 * wave + i;                 // LDS weight tile 0..15 (16 rows each)
+    for (int i = 0; i < 2; ++i) {
+      const int lt = 2 * wave + i;                 // LDS weight tile 0..15 (16 rows each)
       const int r = lt * 16;
       const int nrow = FUSED ? min(n0 + (r & 127), g.n - 16) : min(n0 + r, g.n - 16);
       const uint8_t* base = (FUSED && r >= 128) ? wb1 : wb0;
       if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) w_src[i] = base + (int64_t)(nrow + r16) * K + 16 * kq;
       else w_src[i] = base + (int64_t)(nrow >> 4) * K * 16 + lane * 16;
     }
-    const float* xs_src = g.a.scale + (row0 + min(m0 + 64 * (wave & 1) + lane, cnt - 1)) * g.a.scale_row_stride;
+    const float* xs_src = g.a.scale + (row0 + min(m0 + 64 * wn + lane, cnt - 1)) * g.a.scale_row_stride;
 
     auto issue = [&](int kb, int slot) {
       const uint32_t sb = smem_base + (uint32_t)slot * kSlotBytes;
@@ -179,8 +183,8 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
         async_load16(tok_src[i] + ko + 64, d + 1024);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t d = sb + kTokBytes + (4 * wave_u + i) * 2048;
+      for (int i = 0; i < 2; ++i) {
+        const uint32_t d = sb + kTokBytes + (2 * wave_u + i) * 2048;
         if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
           async_load16(w_src[i] + ko, d);
           async_load16(w_src[i] + ko + 64, d + 1024);
@@ -189,7 +193,7 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
           async_load16(w_src[i] + ((int64_t)kb << 11) + 1024, d + 1024);
         }
       }
-      async_load4(xs_src + (int64_t)kb * g.a.scale_kb_stride, sb + kXsOff + (wave_u & 1) * 256);
+      if (wave_u < 4) async_load4(xs_src + (int64_t)kb * g.a.scale_kb_stride, sb + kXsOff + wave_u * 256);
     };
 
     floatx4 acc[8][4];
@@ -198,16 +202,14 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // prologue: two K-steps in flight (a step past the end re-reads the last one; it is never computed)
     issue(0, 0);
-    issue(min(1, KB - 1), 1);
     __syncthreads();          // s_ws is visible (compiler-tracked stores)
 
     for (int kb = 0; kb < KB; ++kb) {
-      const int slot = kb % NS;
-      wait_vm<kLoadsPerStage>();                 // this wave's loads of step kb have landed ...
+      const int slot = kb & 1;
+      wait_vm<0>();                              // this wave's loads of step kb have landed ...
       block_barrier();                           // ... and everybody's; everybody is done with step kb-1
-      issue(min(kb + 2, KB - 1), (kb + 2) % NS); // refill the slot step kb-1 used
+      if (kb + 1 < KB) issue(kb + 1, slot ^ 1);  // refill the slot step kb-1 used
 
       const uint8_t* b = smem + slot * kSlotBytes;
       const uint8_t* bw = b + kTokBytes;
@@ -217,19 +219,19 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
       intx8 A[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const int lt = FUSED ? ((t >> 1) * 8 + 2 * wave + (t & 1)) : (4 * wave + t);
+        const int lt = FUSED ? ((t >> 1) * 8 + 2 * wn + (t & 1)) : (4 * wn + t);
         const intx4 lo = *reinterpret_cast<const intx4*>(bw + lt * 2048 + lane * 16);
         const intx4 hi = *reinterpret_cast<const intx4*>(bw + lt * 2048 + 1024 + lane * 16);
         A[t] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
 #pragma unroll
       for (int tt = 0; tt < 8; ++tt) {
-        const intx4 lo = *reinterpret_cast<const intx4*>(b + tt * 2048 + lane * 16);
-        const intx4 hi = *reinterpret_cast<const intx4*>(b + tt * 2048 + 1024 + lane * 16);
+        const intx4 lo = *reinterpret_cast<const intx4*>(b + (8 * wm + tt) * 2048 + lane * 16);
+        const intx4 hi = *reinterpret_cast<const intx4*>(b + (8 * wm + tt) * 2048 + 1024 + lane * 16);
         const intx8 B = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        const float xs = bxs[16 * tt + r16];
+        const float xs = bxs[128 * wm + 16 * tt + r16];
         const float sc0 = xs * wsc0;
-        const float sc1 = xs * (FUSED ? wsc1 : ((wave >= 2) ? wsc1 : wsc0));
+        const float sc1 = xs * (FUSED ? wsc1 : ((wn >= 2) ? wsc1 : wsc0));
         const float sc_lo = FUSED ? sc0 : sc1;   // non-fused: all four tiles of a wave share one 128-column block
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -241,7 +243,6 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
         }
       }
     }
-    wait_vm<0>();             // drain the tail prefetches before the ring is reused
 
     // ---- epilogue ----------------------------------------------------------------
     if constexpr (FUSED) {
@@ -256,38 +257,38 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
             acc[tt][j][i] = h;
             am = fmaxf(am, fabsf(h));
           }
-        const int tok = m0 + 16 * tt + r16;
+        const int tok = m0 + 128 * wm + 16 * tt + r16;
         if (g.out != nullptr && tok < cnt) {
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
             uint2 o;
             o.x = f32_to_bf16_bits(acc[tt][j][0]) | (f32_to_bf16_bits(acc[tt][j][1]) << 16);
             o.y = f32_to_bf16_bits(acc[tt][j][2]) | (f32_to_bf16_bits(acc[tt][j][3]) << 16);
-            *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = o;
+            *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 32 * wn + 16 * j + 4 * kq) = o;
           }
         }
         if (g.out_q != nullptr) {
           am = fmaxf(am, __shfl_xor(am, 16, BGMOE_WAVE));
           am = fmaxf(am, __shfl_xor(am, 32, BGMOE_WAVE));
-          if (kq == 0) s_amax[wave][tt][r16] = am;
+          if (kq == 0) s_amax[wm][wn][tt][r16] = am;
         }
       }
       if (g.out_q != nullptr) {
         __syncthreads();
 #pragma unroll
         for (int tt = 0; tt < 8; ++tt) {
-          const float am = fmaxf(fmaxf(s_amax[0][tt][r16], s_amax[1][tt][r16]),
-                                 fmaxf(s_amax[2][tt][r16], s_amax[3][tt][r16]));
+          const float am = fmaxf(fmaxf(s_amax[wm][0][tt][r16], s_amax[wm][1][tt][r16]),
+                                 fmaxf(s_amax[wm][2][tt][r16], s_amax[wm][3][tt][r16]));
           const float sc = quant_scale_from_amax(am);
-          const int tok = m0 + 16 * tt + r16;
+          const int tok = m0 + 128 * wm + 16 * tt + r16;
           if (tok < cnt) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
               const uint32_t q = pack4_e4m3(clamp448(acc[tt][j][0] / sc), clamp448(acc[tt][j][1] / sc),
                                             clamp448(acc[tt][j][2] / sc), clamp448(acc[tt][j][3] / sc));
-              *reinterpret_cast<uint32_t*>(g.out_q + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = q;
+              *reinterpret_cast<uint32_t*>(g.out_q + (row0 + tok) * g.n + n0 + 32 * wn + 16 * j + 4 * kq) = q;
             }
-            if (wave == 0 && kq == 0)
+            if (wn == 0 && kq == 0)
               g.out_s[(row0 + tok) * g.os_row + (int64_t)(n0 >> 7) * g.os_nb] = sc;
           }
         }
@@ -295,11 +296,11 @@ __global__ __launch_bounds__(256) void fp8_tiled_kernel(TiledArgs g) {
     } else {
 #pragma unroll
       for (int tt = 0; tt < 8; ++tt) {
-        const int tok = m0 + 16 * tt + r16;
+        const int tok = m0 + 128 * wm + 16 * tt + r16;
         if (tok >= cnt) continue;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          const int col = n0 + 64 * wave + 16 * t + 4 * kq;
+          const int col = n0 + 64 * wn + 16 * t + 4 * kq;
           if (col >= g.n) continue;
           uint2 o;
           o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
@@ -365,7 +366,7 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   if (blocks > max_items) blocks = max_items;
   if (blocks < 8) blocks = 8;
   BgmoeProf prof(w1 ? BGMOE_K_S1_TILED : BGMOE_K_GEMM_TILED, st);
-  const dim3 grid((unsigned)blocks), block(256);
+  const dim3 grid((unsigned)blocks), block(NT);
   const bool tm = w0->layout == BGMOE_W_TILE_MAJOR;
   if (w1) {
     if (tm) hipLaunchKernelGGL((fp8_tiled_kernel<true, 1>), grid, block, kLds, st, g);
