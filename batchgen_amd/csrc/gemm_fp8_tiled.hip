@@ -34,6 +34,7 @@ constexpr int kTokBytes = TM * 128;
 constexpr int kWBytes = TW * 128;
 constexpr int kXsOff = kTokBytes + kWBytes;
 constexpr int kSlotBytes = kXsOff + TM * 4;
+constexpr int kPanel = 8;          // m-tiles per panel of the work-item order
 constexpr int kMaxGroups = 1024;
 constexpr int kMaxKB = 256;        // K <= 32768
 
@@ -53,13 +54,22 @@ struct TiledArgs {
 // 64 lanes x 16 bytes -> LDS [lds_base, lds_base + 1024); lds_base must be wave-uniform.  No
 // instruction offset is used: the hardware would add it to the LDS address as well as to the
 // global address.
-__device__ __forceinline__ void async_load16(const uint8_t* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-               :: "s"(lds_base), "v"(gptr) : "memory", "m0");
+// The global address is a wave-uniform base plus a 32-bit byte offset per lane.
+__device__ __forceinline__ void async_load16(const uint8_t* base, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_base), "v"(lane_off), "s"(base) : "memory", "m0");
 }
 // 64 lanes x 4 bytes -> LDS [lds_base, lds_base + 256)
-__device__ __forceinline__ void async_load4(const float* gptr, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" :: "s"(lds_base), "v"(gptr) : "memory", "m0");
+__device__ __forceinline__ void async_load4(const float* base, uint32_t lane_off, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :: "s"(lds_base), "v"(lane_off), "s"(base) : "memory", "m0");
+}
+template <typename T>
+__device__ __forceinline__ const T* uniform_ptr(const T* p) {   // tell the compiler a pointer is wave-uniform
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return reinterpret_cast<const T*>(((uint64_t)hi << 32) | lo);
 }
 template <int N>
 __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
@@ -114,17 +124,22 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
   for (int64_t itx = (int64_t)bidx; itx < per_x; itx += bstep) {
     const int64_t item = (int64_t)xcd * per_x + itx;
     if (item >= total) break;
-    // item -> (group, n-tile, m-tile): within a group, m fastest
+    // item -> (group, n-tile, m-tile)
     int lo_g = 0, hi_g = g.groups - 1;
     while (lo_g < hi_g) {
       const int mid = (lo_g + hi_g + 1) >> 1;
       if ((int64_t)s_tiles[mid] * ntn <= item) lo_g = mid; else hi_g = mid - 1;
     }
-    const int grp = lo_g;
-    const int mt_g = s_tiles[grp + 1] - s_tiles[grp];
-    const int64_t rel = item - (int64_t)s_tiles[grp] * ntn;
-    const int nt = (int)(rel / mt_g);
-    const int mt = (int)(rel - (int64_t)nt * mt_g);
+    const int grp = __builtin_amdgcn_readfirstlane(lo_g);   // (LDS reads look divergent to the compiler)
+    const int mt_g = __builtin_amdgcn_readfirstlane(s_tiles[grp + 1] - s_tiles[grp]);
+    const int64_t rel = item - (int64_t)__builtin_amdgcn_readfirstlane(s_tiles[grp]) * ntn;
+    // panels of kPanel m-tiles; inside a panel n-tiles advance with m fastest, so the 32 items an XCD works
+    // on at one time form a compact (m, n) patch: few distinct token and weight streams per L2
+    const int panel = (int)(rel / ((int64_t)kPanel * ntn));
+    const int pm = min(kPanel, mt_g - panel * kPanel);
+    const int r2 = (int)(rel - (int64_t)panel * kPanel * ntn);
+    const int nt = r2 / pm;
+    const int mt = panel * kPanel + (r2 - nt * pm);
     const int cnt = g.seqlens[grp];
     const int64_t row0 = g.cu[grp];
     const int m0 = mt * TM;
@@ -155,23 +170,32 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
     }
 
     // ---- this wave's share of a stage: token tiles 2w, 2w+1; weight tiles 2w, 2w+1; waves 0..3: 64 token scales ----
-    const uint8_t* tok_src[2];
+    // row-major sources: load j of a tile covers rows 8j..8j+7, lane p = (row p>>3, LDS chunk p&7) fetches
+    // the row's 16-byte chunk (p&7) ^ (p>>3): whole 128-byte lines per 8 lanes, XOR-swizzled in LDS
+    const int lrow = lane >> 3;
+    const int lchunk = ((lane & 7) ^ lrow) * 16;
+    const uint8_t* tok_base = uniform_ptr(g.a.x + (row0 + m0) * K);
+    uint32_t tok_off[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int tok = min(16 * (2 * wave + i) + 8 * j + lrow, cnt - 1 - m0);
+        tok_off[i][j] = (uint32_t)tok * (uint32_t)K + lchunk;
+      }
+    const uint8_t* w_base[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int tok = min(m0 + 16 * (2 * wave + i) + r16, cnt - 1);
-      tok_src[i] = g.a.x + (row0 + tok) * K + 16 * kq;
-    }
-    const uint8_t* w_src[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int lt = 2 * wave + i;                 // LDS weight tile 0..15 (16 rows each)
+      const int lt = 2 * wave_u + i;               // LDS weight tile 0..15 (16 rows each)
       const int r = lt * 16;
       const int nrow = FUSED ? min(n0 + (r & 127), g.n - 16) : min(n0 + r, g.n - 16);
       const uint8_t* base = (FUSED && r >= 128) ? wb1 : wb0;
-      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) w_src[i] = base + (int64_t)(nrow + r16) * K + 16 * kq;
-      else w_src[i] = base + (int64_t)(nrow >> 4) * K * 16 + lane * 16;
+      // row-major: row nrow; tile-major: tile nrow / 16 (16 x K bytes per row of tiles)
+      w_base[i] = uniform_ptr(base + (int64_t)(LAYOUT == BGMOE_W_ROW_MAJOR ? nrow : (nrow & ~15)) * K);
     }
-    const float* xs_src = g.a.scale + (row0 + min(m0 + 64 * wn + lane, cnt - 1)) * g.a.scale_row_stride;
+    const uint32_t w_off = LAYOUT == BGMOE_W_ROW_MAJOR ? (uint32_t)lrow * (uint32_t)K + lchunk : lane * 16;
+    const float* xs_base = uniform_ptr(g.a.scale + (row0 + m0) * g.a.scale_row_stride);
+    const uint32_t xs_off = (uint32_t)min(64 * wn + lane, cnt - 1 - m0) * (uint32_t)g.a.scale_row_stride * 4u;
 
     auto issue = [&](int kb, int slot) {
       const uint32_t sb = smem_base + (uint32_t)slot * kSlotBytes;
@@ -179,21 +203,22 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const uint32_t d = sb + (2 * wave_u + i) * 2048;
-        async_load16(tok_src[i] + ko, d);
-        async_load16(tok_src[i] + ko + 64, d + 1024);
+        async_load16(tok_base + ko, tok_off[i][0], d);
+        async_load16(tok_base + ko, tok_off[i][1], d + 1024);
       }
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const uint32_t d = sb + kTokBytes + (2 * wave_u + i) * 2048;
         if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
-          async_load16(w_src[i] + ko, d);
-          async_load16(w_src[i] + ko + 64, d + 1024);
+          async_load16(w_base[i] + ko, w_off, d);
+          async_load16(w_base[i] + ko + 8 * (int64_t)K, w_off, d + 1024);
         } else {
-          async_load16(w_src[i] + ((int64_t)kb << 11), d);
-          async_load16(w_src[i] + ((int64_t)kb << 11) + 1024, d + 1024);
+          async_load16(w_base[i] + ((int64_t)kb << 11), w_off, d);
+          async_load16(w_base[i] + ((int64_t)kb << 11) + 1024, w_off, d + 1024);
         }
       }
-      if (wave_u < 4) async_load4(xs_src + (int64_t)kb * g.a.scale_kb_stride, sb + kXsOff + wave_u * 256);
+      if (wave_u < 4)
+        async_load4(xs_base + (int64_t)kb * g.a.scale_kb_stride, xs_off, sb + kXsOff + wave_u * 256);
     };
 
     floatx4 acc[8][4];
@@ -216,30 +241,54 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
       const float* bxs = reinterpret_cast<const float*>(b + kXsOff);
       const float wsc0 = s_ws[0][kb], wsc1 = s_ws[1][kb];
 
+      // operand offsets inside a 2 KiB tile image: swizzled row-major (tokens, row-major weights) or lane order
+      const int sw_lo = r16 * 128 + ((kq ^ (r16 & 7)) * 16);
+      const int a_lo = LAYOUT == BGMOE_W_ROW_MAJOR ? sw_lo : lane * 16;
+      const int a_hi = LAYOUT == BGMOE_W_ROW_MAJOR ? (sw_lo ^ 64) : lane * 16 + 1024;
       intx8 A[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int lt = FUSED ? ((t >> 1) * 8 + 2 * wn + (t & 1)) : (4 * wn + t);
-        const intx4 lo = *reinterpret_cast<const intx4*>(bw + lt * 2048 + lane * 16);
-        const intx4 hi = *reinterpret_cast<const intx4*>(bw + lt * 2048 + 1024 + lane * 16);
+        const intx4 lo = *reinterpret_cast<const intx4*>(bw + lt * 2048 + a_lo);
+        const intx4 hi = *reinterpret_cast<const intx4*>(bw + lt * 2048 + a_hi);
         A[t] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
+      const uint8_t* bt = b + 8 * wm * 2048;
+      const float* bx = bxs + 128 * wm + r16;
+      auto load_b = [&](int tt) {
+        const intx4 lo = *reinterpret_cast<const intx4*>(bt + tt * 2048 + sw_lo);
+        const intx4 hi = *reinterpret_cast<const intx4*>(bt + tt * 2048 + (sw_lo ^ 64));
+        return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      };
+      // 32 MFMAs (token tile tt = idx/4, weight tile t = idx%4) in one software pipeline: token tile tt+1
+      // is fetched from LDS while tile tt is multiplied, and the promotion of product idx-2
+      // (acc += partial * scale, VALU) is issued behind MFMA idx
+      intx8 Bb[2];
+      float xb[2];
+      Bb[0] = load_b(0);
+      xb[0] = bx[0];
+      floatx4 P[3];
+      float psc[2][2];
 #pragma unroll
-      for (int tt = 0; tt < 8; ++tt) {
-        const intx4 lo = *reinterpret_cast<const intx4*>(b + (8 * wm + tt) * 2048 + lane * 16);
-        const intx4 hi = *reinterpret_cast<const intx4*>(b + (8 * wm + tt) * 2048 + 1024 + lane * 16);
-        const intx8 B = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        const float xs = bxs[128 * wm + 16 * tt + r16];
-        const float sc0 = xs * wsc0;
-        const float sc1 = xs * (FUSED ? wsc1 : ((wn >= 2) ? wsc1 : wsc0));
-        const float sc_lo = FUSED ? sc0 : sc1;   // non-fused: all four tiles of a wave share one 128-column block
+      for (int idx = 0; idx < 34; ++idx) {
+        if (idx < 32) {
+          const int tt = idx >> 2, t = idx & 3;
+          if (t == 0) {
+            if (tt < 7) {
+              Bb[(tt + 1) & 1] = load_b(tt + 1);
+              xb[(tt + 1) & 1] = bx[16 * (tt + 1)];
+            }
+            // fused: tiles 0,1 gate (scale 0), 2,3 up (scale 1); else all four tiles share one 128-column block
+            psc[tt & 1][0] = xb[tt & 1] * (FUSED ? wsc0 : ((wn >= 2) ? wsc1 : wsc0));
+            psc[tt & 1][1] = xb[tt & 1] * (FUSED ? wsc1 : ((wn >= 2) ? wsc1 : wsc0));
+          }
+          P[idx % 3] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+              A[t], Bb[tt & 1], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+        }
+        if (idx >= 2) {
+          const int j = idx - 2, tt = j >> 2, t = j & 3;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-              A[t], B, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-          const float sc = FUSED ? ((t >> 1) ? sc1 : sc0) : sc_lo;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[tt][t][i] = fmaf(p[i], sc, acc[tt][t][i]);
+          for (int i = 0; i < 4; ++i) acc[tt][t][i] = fmaf(P[j % 3][i], psc[tt & 1][t >> 1], acc[tt][t][i]);
         }
       }
     }
