@@ -2,6 +2,27 @@
 #pragma once
 #include "bgmoe_common.h"
 
+// Which kernel serves a group.  The weight-streaming kernel re-streams a group's weights once per
+// 32-row chunk; the LDS-tiled kernel works in 256-row tiles and needs enough of them to fill the chip.
+// Groups with at most small_rows rows always stream; groups with more than max_rows rows are always
+// tiled; groups in between are tiled only when all groups above small_rows together make at least
+// min_tiles 256-row tiles.  Both kernels evaluate this on the device from the same counts.
+struct BgmoeSplit { int small_rows, max_rows, min_tiles; };
+
+// Wave-uniform; every wave runs it redundantly.  Returns the row limit of the weight-streaming kernel.
+__device__ __forceinline__ int bgmoe_split_limit(const int32_t* seqlens, int groups, BgmoeSplit s) {
+  if (s.small_rows >= s.max_rows) return s.max_rows;
+  const int lane = threadIdx.x & 63;
+  int tiles = 0;
+  for (int g0 = lane; g0 < groups; g0 += 64) {
+    const int c = seqlens[g0];
+    tiles += c > s.small_rows ? (c + 255) >> 8 : 0;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) tiles += __shfl_xor(tiles, off, BGMOE_WAVE);
+  return tiles >= s.min_tiles ? s.small_rows : s.max_rows;
+}
+
 // Work items of one launch: every group with lo < count <= hi contributes ceil(count / chunk_rows)
 // items (ascending group, ascending chunk).  Returns the group of item `item` and its chunk index,
 // or -1 when there are fewer items.  Wave-uniform; every wave of the block runs it redundantly.
@@ -38,26 +59,38 @@ __device__ __forceinline__ int nth_active_item(const int32_t* seqlens, int group
 // chunks streams the same weight tile once per chunk; the map puts all chunks of one n-tile on the
 // SAME XCD in neighbouring blocks: block q of the group -> n-tile 8*(q / (8*chunks)) + q % 8,
 // chunk (q / 8) % chunks.  `ntiles_pad` = n-tile count rounded up to 8 so every group starts on XCD 0.
+// `block` is the virtual block index (blockIdx.x, or blockIdx.x + i * gridDim.x in a persistent kernel
+// whose grid is a multiple of 8, which keeps block % 8 == XCD).  grp == BGMOE_ITEM_END: `block` lies past
+// the last item (so do all larger ones); grp == BGMOE_ITEM_PAD: a padding n-tile, nothing to do.
 struct BgmoeItem { int grp, ntile, chunk, cnt; };
+constexpr int BGMOE_ITEM_PAD = -1;
+constexpr int BGMOE_ITEM_END = -2;
 
 __device__ __forceinline__ BgmoeItem bgmoe_decode_item(const int32_t* seqlens, int groups, int lo, int hi,
-                                                       int chunk_rows, int ntiles) {
+                                                       int chunk_rows, int ntiles, unsigned block) {
   BgmoeItem it;
   const int ntiles_pad = (ntiles + 7) & ~7;
   int crow = 0;
-  it.grp = nth_active_item(seqlens, groups, lo, hi, chunk_rows, blockIdx.x / ntiles_pad, &crow);
+  it.grp = nth_active_item(seqlens, groups, lo, hi, chunk_rows, (int)(block / ntiles_pad), &crow);
   it.ntile = it.chunk = it.cnt = 0;
-  if (it.grp < 0) return it;
+  if (it.grp < 0) {
+    it.grp = BGMOE_ITEM_END;
+    return it;
+  }
   it.cnt = seqlens[it.grp];
   const int chunks = (it.cnt + chunk_rows - 1) / chunk_rows;
-  const int q = crow * ntiles_pad + blockIdx.x % ntiles_pad;
+  const int q = crow * ntiles_pad + (int)(block % ntiles_pad);
   it.ntile = 8 * (q / (8 * chunks)) + (q & 7);
   it.chunk = (q >> 3) % chunks;
-  if (it.ntile >= ntiles) it.grp = -1;
+  if (it.ntile >= ntiles) it.grp = BGMOE_ITEM_PAD;
   return it;
 }
 
-static inline unsigned bgmoe_item_grid(int ntiles, int groups, int64_t row_bound, int chunk_rows) {
-  const int64_t items = groups + row_bound / chunk_rows;          // >= sum of ceil(count / chunk_rows)
+// Upper bound on the virtual blocks of a launch from host-side knowledge only: `row_bound` bounds the
+// total live rows, `max_rows` the rows of any group the launch serves.
+static inline unsigned bgmoe_item_grid(int ntiles, int groups, int64_t row_bound, int max_rows, int chunk_rows) {
+  int64_t items = groups + row_bound / chunk_rows;                 // >= sum of ceil(count / chunk_rows)
+  const int64_t per_group = (int64_t)groups * (((int64_t)max_rows + chunk_rows - 1) / chunk_rows);
+  if (per_group < items) items = per_group;
   return (unsigned)(((ntiles + 7) & ~7) * items);
 }

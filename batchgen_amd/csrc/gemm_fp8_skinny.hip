@@ -46,7 +46,7 @@ struct SkinnyArgs {
   uint8_t* out_q;
   float* out_s;
   int64_t os_row, os_nb;
-  int lo, hi;                 // this launch serves groups with lo < count <= hi
+  BgmoeSplit split;           // this launch serves groups with count <= bgmoe_split_limit(...)
   int64_t row_bound;          // host-side upper bound on the total live rows
 };
 
@@ -77,15 +77,11 @@ __device__ __forceinline__ intx8 load32_stream(const uint8_t* p) {
   return r;
 }
 
+// One work item: 16*TT rows of one group x one n-tile, streamed over K.
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
-__global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
+__device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const BgmoeItem& it, float (*s_amax)[TT][16]) {
   constexpr int NT = 4;                  // weight tiles per wave
   constexpr int NSC = FUSED ? 2 : 1;     // weight-scale streams per wave
-  __shared__ float s_amax[4][TT][16];
-
-  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
-  const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles);
-  if (it.grp < 0) return;                         // whole block: fewer items than the grid allows
   const int grp = it.grp, cnt = it.cnt, ntile = it.ntile, chunk = it.chunk;
   const int64_t row0 = g.cu[grp];
   const int wave = threadIdx.x >> 6;
@@ -259,6 +255,22 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g) {
   }
 }
 
+// Persistent grid: block b works on virtual blocks b, b + gridDim.x, ... until the item list ends, so
+// a launch sized from host-side bounds pays nothing for the (many) virtual blocks past the real work.
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
+__global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned vblocks) {
+  __shared__ float s_amax[4][TT][16];
+  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
+  const int hi = bgmoe_split_limit(g.seqlens, g.groups, g.split);
+  for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
+    const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, 0, hi, 16 * TT, ntiles, vb);
+    if (it.grp == BGMOE_ITEM_END) break;
+    if (it.grp == BGMOE_ITEM_PAD) continue;
+    fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT>(g, it, s_amax);
+    __syncthreads();                      // s_amax is reused by the next item
+  }
+}
+
 int check_common(const char* what, const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w, const int32_t* seqlens,
                  const int32_t* cu, int groups, int64_t m, int n, int k) {
   BGMOE_REQUIRE(a && w, "%s: null operand descriptor", what);
@@ -284,17 +296,40 @@ int check_common(const char* what, const bgmoe_fp8_act* a, const bgmoe_fp8_weigh
 int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                            const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                            uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
-                           int lo, hipStream_t st);
+                           BgmoeSplit split, hipStream_t st);
+
+// Blocks of `kernel` that are resident on the whole device at once (a multiple of 8, so that the
+// virtual block index keeps its XCD); queried once per kernel.
+template <typename K>
+static unsigned resident_blocks(K kernel, unsigned* cache) {
+  if (*cache == 0) {
+    int per_cu = 0, dev = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1) per_cu = 2;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+      cus = 256;
+    *cache = (unsigned)(per_cu * cus) & ~7u;
+    if (*cache == 0) *cache = 8;
+  }
+  return *cache;
+}
+
+template <int TT, int NS, bool FUSED, int LAYOUT>
+static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
+  static unsigned resident = 0;
+  const unsigned cap = resident_blocks(fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>, &resident);
+  const dim3 grid(vblocks < cap ? vblocks : cap), block(256);
+  hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks);
+}
 
 template <int TT, int NS>
-static void launch_variant(bool fused, int layout, dim3 grid, const SkinnyArgs& g, hipStream_t st) {
-  const dim3 block(256);
+static void launch_variant(bool fused, int layout, unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
   if (fused) {
-    if (layout == BGMOE_W_TILE_MAJOR) hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, true, BGMOE_W_TILE_MAJOR>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, true, BGMOE_W_ROW_MAJOR>), grid, block, 0, st, g);
+    if (layout == BGMOE_W_TILE_MAJOR) launch_one<TT, NS, true, BGMOE_W_TILE_MAJOR>(vblocks, g, st);
+    else launch_one<TT, NS, true, BGMOE_W_ROW_MAJOR>(vblocks, g, st);
   } else {
-    if (layout == BGMOE_W_TILE_MAJOR) hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, false, BGMOE_W_TILE_MAJOR>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, false, BGMOE_W_ROW_MAJOR>), grid, block, 0, st, g);
+    if (layout == BGMOE_W_TILE_MAJOR) launch_one<TT, NS, false, BGMOE_W_TILE_MAJOR>(vblocks, g, st);
+    else launch_one<TT, NS, false, BGMOE_W_ROW_MAJOR>(vblocks, g, st);
   }
 }
 
@@ -331,19 +366,23 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   }
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
   const int hi = skinny_limit();
+  const BgmoeSplit split{hi < 64 ? hi : 64, hi, 8};
   if (hi > 0) {
     static const int tt = getenv("BGMOE_SKINNY_TT") ? atoi(getenv("BGMOE_SKINNY_TT")) : 2;
-    const dim3 grid(bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 16 * tt));
-    g.lo = 0; g.hi = hi;
+    const unsigned grid = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, hi, 16 * tt);
+    g.split = split;
     BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
     if (tt == 4) launch_variant<4, 2>(fused, layout, grid, g, st);
     else launch_variant<2, 3>(fused, layout, grid, g, st);
     int rc = bgmoe_check_launch("fp8 grouped gemm (skinny)");
     if (rc != BGMOE_OK) return rc;
   }
-  if (bound <= hi) return BGMOE_OK;
+  // no group can reach the tiled kernel: too few rows in total for one group above small_rows, or for
+  // min_tiles tiles of them while none exceeds max_rows
+  if (bound <= split.small_rows || (bound <= hi && bound <= (int64_t)split.min_tiles * split.small_rows))
+    return BGMOE_OK;
   return bgmoe_launch_fp8_tiled(&g.a, &g.w0, fused ? &g.w1 : nullptr, g.seqlens, g.cu, g.groups, m, g.n,
-                                g.k, g.out, g.out_q, g.out_s, g.os_row, g.os_nb, hi, st);
+                                g.k, g.out, g.out_q, g.out_s, g.os_row, g.os_nb, split, st);
 }
 
 int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,

@@ -19,10 +19,11 @@
 // K-step.
 //
 // Scheduling: a fixed grid of persistent blocks walks a device-built list of (group, n-tile, m-tile)
-// work items, m fastest, so the blocks of one XCD (block b runs on XCD b % 8) work on neighbouring
-// m-tiles of the same weight tile and share it through that XCD's L2.  Groups with <= `lo` rows are
-// left to the weight-streaming kernel; empty groups cost nothing.
+// work items ordered so that the blocks of one XCD (block b runs on XCD b % 8) work on a compact patch
+// of m- and n-tiles and share their operands through that XCD's L2.  Groups at or below the row limit
+// of bgmoe_split_limit() are left to the weight-streaming kernel; empty groups cost nothing.
 #include "bgmoe_common.h"
+#include "bgmoe_sched.h"
 
 namespace {
 
@@ -48,7 +49,7 @@ struct TiledArgs {
   uint8_t* out_q;
   float* out_s;
   int64_t os_row, os_nb;
-  int lo;
+  BgmoeSplit split;
 };
 
 // 64 lanes x 16 bytes -> LDS [lds_base, lds_base + 1024); lds_base must be wave-uniform.  No
@@ -97,9 +98,10 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane((uint32_t)wave);
 
   // ---- work list: m-tiles per group, prefix-summed (every block computes the same list) ----
+  const int lo = bgmoe_split_limit(g.seqlens, g.groups, g.split);   // groups above this row count are ours
   for (int e = tid; e < g.groups; e += NT) {
     const int c = g.seqlens[e];
-    s_tiles[e + 1] = c > g.lo ? (c + TM - 1) / TM : 0;
+    s_tiles[e + 1] = c > lo ? (c + TM - 1) / TM : 0;
   }
   __syncthreads();
   if (tid == 0) {
@@ -368,7 +370,7 @@ int g_num_cu = 0;
 int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                            const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                            uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
-                           int lo, hipStream_t st) {
+                           BgmoeSplit split, hipStream_t st) {
   if (groups == 0 || m == 0) return BGMOE_OK;
   if (groups > kMaxGroups) {
     bgmoe_set_error("fp8 tiled gemm: groups=%d exceeds %d", groups, kMaxGroups);
@@ -381,7 +383,7 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   TiledArgs g{};
   g.a = *a; g.w0 = *w0; if (w1) g.w1 = *w1;
   g.seqlens = seqlens; g.cu = cu; g.groups = groups; g.n = n; g.k = k;
-  g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.lo = lo;
+  g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.split = split;
   constexpr int kLds = NS * kSlotBytes;
   static bool attr_set = false;
   if (!attr_set) {

@@ -56,7 +56,7 @@ template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g) {
   constexpr int NT = 4;
   const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
-  const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles);
+  const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, blockIdx.x);
   if (it.grp < 0) return;
   const int grp = it.grp, cnt = it.cnt;
   const int64_t row0 = g.cu[grp];
@@ -217,7 +217,7 @@ int check_w(const char* what, const bgmoe_mxfp4_weight* w) {
 int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
   const int ntile = fused ? 128 : 256;
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
-  const dim3 grid(bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 32)), block(256);
+  const dim3 grid(bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 32)), block(256);
   g.lo = 0; g.hi = 0x7fffffff;     // every group: more than 32 rows = more chunks (weights re-streamed)
   const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
   BgmoeProf prof(fused ? BGMOE_K_MXFP4_S1 : BGMOE_K_MXFP4_GEMM, st);

@@ -249,10 +249,15 @@ def test_tile_major_weights_equal_row_major(dev, counts, n, k):
 
 @pytest.mark.parametrize("limit", [0, 16, 256])
 @pytest.mark.parametrize("layout", ["row_major", "tile_major"])
-def test_kernel_choice_does_not_change_results_beyond_rounding(dev, limit, layout):
-    """The same problem through the LDS-tiled kernel only (limit 0), a mix, and the streaming kernel."""
+@pytest.mark.parametrize("counts", [
+    (0, 1, 15, 16, 17, 127, 128, 129, 260, 5),            # few rows above 64: they stay on the streaming kernel
+    (70, 100, 0, 129, 65, 90, 260, 33, 64, 200, 80),      # nine 256-row tiles above 64 rows: those groups are tiled
+], ids=["few_big", "many_big"])
+def test_kernel_choice_does_not_change_results_beyond_rounding(dev, limit, layout, counts):
+    """The same problem through the LDS-tiled kernel only (limit 0), a mix, and the streaming kernel
+    (limit 256: groups of 65..256 rows are tiled only when there are at least eight tiles of them)."""
     from batchgen_amd._lib import check, lib
-    counts, n, k = (0, 1, 15, 16, 17, 127, 128, 129, 260, 5), 384, 640
+    n, k = 384, 640
     counts, cu, m, xq, xs, ws = _make(400, counts, n, k, nmat=2)
     (gq, gs), (uq, us) = ws
     xq_d, xs_t, gq_d, gs_d = _dev(dev, xq, xs, gq, gs)
