@@ -1,12 +1,13 @@
 // Block-scaled FP8 grouped GEMM for FEW rows per group (decode): a
 // weight-streaming kernel bound by HBM bandwidth.
 //
-// Work split: block = (group, 128 gate + 128 up output columns) for the fused
-// stage 1, (group, 256 output columns) for a single GEMM; 4 waves, each owning
-// four 16-row weight tiles over the whole K.  Every weight byte is read from
-// HBM exactly once, straight into registers (no LDS: no other wave needs it),
-// with 16-byte loads and a multi-stage register prefetch so that each wave
-// keeps 16-24 KB of loads in flight.
+// Work split: item = (group, up to 32 or 64 rows, 128 gate + 128 up output columns) for the fused
+// stage 1, (group, rows, 256 output columns) for a single GEMM; 4 waves, each owning four 16-row
+// weight tiles over the whole K.  A weight byte is read from HBM once per item, straight into
+// registers (no LDS: no other wave needs it), with 16-byte loads and a multi-stage register prefetch
+// so that each wave keeps 16-24 KB of loads in flight.  The item's tokens are needed by all four
+// waves: they go through a small LDS ring filled by asynchronous global -> LDS loads, one copy per
+// block instead of one per wave (the per-CU request rate, not HBM, is what a second copy costs).
 //
 // MFMA: v_mfma_f32_16x16x128_f8f6f4 with the WEIGHT tile as the A operand
 // (16 output features x 128 K) and the TOKEN tile as B (128 K x 16 tokens):
@@ -33,6 +34,7 @@
 
 #include "bgmoe_common.h"
 #include "bgmoe_sched.h"
+#include "bgmoe_async.h"
 
 namespace {
 
@@ -50,22 +52,11 @@ struct SkinnyArgs {
   int64_t row_bound;          // host-side upper bound on the total live rows
 };
 
-template <int TT, int NSC>
+template <int NSC>
 struct Stage {
   intx8 A[4];
-  intx8 B[TT];
-  float xs[TT];
   float ws[NSC];
 };
-
-__device__ __forceinline__ intx8 load32(const uint8_t* p) {
-  const intx4 lo = gload_x4(p);
-  const intx4 hi = gload_x4(p + 64);
-  intx8 r;
-  r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
-  r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
-  return r;
-}
 
 template <int HI>
 __device__ __forceinline__ intx8 load32_stream(const uint8_t* p) {
@@ -77,14 +68,24 @@ __device__ __forceinline__ intx8 load32_stream(const uint8_t* p) {
   return r;
 }
 
-// One work item: 16*TT rows of one group x one n-tile, streamed over K.
+// LDS ring slot of one K-block of tokens: TT 2-KiB tile images + 64 token scales
+template <int TT>
+struct TokSlot {
+  static constexpr int kBytes = TT * 2048 + 256;
+};
+
+// One work item: up to 16*TT rows of one group x one n-tile, streamed over K.
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
-__device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const BgmoeItem& it, float (*s_amax)[TT][16]) {
+__device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const BgmoeItem& it, float (*s_amax)[TT][16],
+                                                const uint8_t* ring, uint32_t ring_lds) {
   constexpr int NT = 4;                  // weight tiles per wave
   constexpr int NSC = FUSED ? 2 : 1;     // weight-scale streams per wave
+  constexpr int kSlot = TokSlot<TT>::kBytes;
+  constexpr int LT = TT / 2;             // token half-tile loads per wave and K-block
   const int grp = it.grp, cnt = it.cnt, ntile = it.ntile, chunk = it.chunk;
   const int64_t row0 = g.cu[grp];
   const int wave = threadIdx.x >> 6;
+  const uint32_t wave_u = __builtin_amdgcn_readfirstlane((uint32_t)wave);
   const int lane = threadIdx.x & 63;
   const int r16 = lane & 15;
   const int kq = lane >> 4;
@@ -122,134 +123,166 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
     wsp[0] = wsb[0] + (int64_t)nb * g.w0.scale_nb_stride;
   }
 
-  {
-    const int t0 = chunk * 16 * TT;
-    const uint8_t* xp[TT];
-    const float* xsp[TT];
-    bool xv[TT];
+  const int t0 = chunk * 16 * TT;
+  const int live = cnt - t0;                              // >= 1 rows of this item
+  const int tiles = min(TT, (live + 15) >> 4);            // token tiles with at least one live row
+
+  // ---- tokens: the 4 waves share them through an LDS ring filled by asynchronous loads ----
+  // A load covers rows 8j..8j+7 of a tile: lane p = (row p>>3, LDS chunk p&7) fetches the row's 16-byte
+  // chunk (p&7) ^ (p>>3) -- whole 128-byte lines, XOR-swizzled so that the MFMA operand reads below are
+  // conflict free.  Wave w loads half-tiles w*LT .. w*LT+LT-1; rows past the count re-read the last row.
+  const uint8_t* tok_base = uniform_ptr(g.a.x + (row0 + t0) * K);
+  uint32_t tok_off[LT];
+  bool tok_on[LT];
+#pragma unroll
+  for (int i = 0; i < LT; ++i) {
+    const int h = (int)wave_u * LT + i;                   // half-tile 0 .. 2*TT-1
+    const int row = min(8 * h + (lane >> 3), live - 1);
+    tok_off[i] = (uint32_t)row * (uint32_t)K + (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
+    tok_on[i] = (h >> 1) < tiles;
+  }
+  const float* xs_base = uniform_ptr(g.a.scale + (row0 + t0) * g.a.scale_row_stride);
+  const uint32_t xs_off = (uint32_t)min(lane, live - 1) * (uint32_t)g.a.scale_row_stride * 4u;
+
+  auto issue_tokens = [&](int kb, int slot) {
+    const uint32_t sb = ring_lds + (uint32_t)slot * kSlot;
+#pragma unroll
+    for (int i = 0; i < LT; ++i)
+      if (tok_on[i]) async_load16(tok_base + (kb << 7), tok_off[i], sb + (wave_u * LT + i) * 1024);
+    if (wave_u == 0) async_load4(xs_base + (int64_t)kb * g.a.scale_kb_stride, xs_off, sb + TT * 2048);
+  };
+
+  floatx4 acc[TT][NT];
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- weights: straight from HBM into registers, NSTAGE-1 K-blocks ahead ----
+  Stage<NSC> st[NSTAGE];
+  auto load_stage = [&](Stage<NSC>& s, int kb) {
+#pragma unroll
+    for (int i = 0; i < NSC; ++i) s.ws[i] = gload_f32(wsp[i] + kb);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) s.A[t] = load32_stream<64>(wp[t] + (kb << 7));
+      else s.A[t] = load32_stream<1024>(wp[t] + ((int64_t)kb << 11));
+    }
+  };
+  const int sw_lo = r16 * 128 + ((kq ^ (r16 & 7)) * 16);
+  auto compute = [&](const Stage<NSC>& c, int slot) {
+    const uint8_t* b = ring + slot * kSlot;
+    const float* bxs = reinterpret_cast<const float*>(b + TT * 2048);
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
-      const int tok = t0 + 16 * tt + r16;
-      xv[tt] = tok < cnt;
-      const int64_t r = row0 + (xv[tt] ? tok : 0);     // cnt >= 1 here
-      xp[tt] = g.a.x + r * K + 16 * kq;
-      xsp[tt] = g.a.scale + r * g.a.scale_row_stride;
-    }
-
-    floatx4 acc[TT][NT];
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-      for (int t = 0; t < NT; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-    Stage<TT, NSC> st[NSTAGE];
-    // tokens past the count re-read the group's first row; their columns are never stored
-    auto load_stage = [&](Stage<TT, NSC>& s, int kb) {
-      const int ko = kb << 7;
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) s.A[t] = load32_stream<64>(wp[t] + ko);
-        else s.A[t] = load32_stream<1024>(wp[t] + ((int64_t)kb << 11));
-      }
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt) {
-        s.B[tt] = load32(xp[tt] + ko);
-        s.xs[tt] = gload_f32(xsp[tt] + (int64_t)kb * g.a.scale_kb_stride);
-      }
-#pragma unroll
-      for (int i = 0; i < NSC; ++i) s.ws[i] = gload_f32(wsp[i] + kb);
-    };
-    auto compute = [&](const Stage<TT, NSC>& c) {
-#pragma unroll
-      for (int tt = 0; tt < TT; ++tt) {
+      if (tt < tiles) {
+        const intx4 lo = *reinterpret_cast<const intx4*>(b + tt * 2048 + sw_lo);
+        const intx4 hi = *reinterpret_cast<const intx4*>(b + tt * 2048 + (sw_lo ^ 64));
+        const intx8 B = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const float xs = bxs[16 * tt + r16];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
           const floatx4 p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-              c.A[t], c.B[tt], floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-          const float sc = c.xs[tt] * c.ws[FUSED ? (t >> 1) : 0];
+              c.A[t], B, floatx4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+          const float sc = xs * c.ws[FUSED ? (t >> 1) : 0];
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[tt][t][i] = fmaf(p[i], sc, acc[tt][t][i]);
         }
       }
-    };
-
-    // software pipeline, NSTAGE-1 K-blocks ahead; prefetches past the end re-read the last block
-#pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s) load_stage(st[s], min(s, KB - 1));
-    const int kb_main = KB - KB % NSTAGE;
-    for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
-#pragma unroll
-      for (int s = 0; s < NSTAGE; ++s) {
-        load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
-        compute(st[s]);
-      }
     }
-#pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s)
-      if (kb_main + s < KB) compute(st[s]);
+  };
 
-    // ---- epilogue -------------------------------------------------------------
-    if constexpr (FUSED) {
-      float hv[TT][2][4];
+  // Software pipeline, NSTAGE-1 K-blocks ahead; prefetches past the end re-read the last block.  In an
+  // iteration the token loads are issued before the weight loads, and vector-memory loads complete in
+  // issue order: once at most the 8 weight loads of the youngest stage are outstanding, this wave's
+  // tokens and weights of the stage about to be computed have landed; the barrier extends that to the
+  // other waves' token loads and tells everybody that the slot refilled next is no longer being read.
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt) {
-        float am = 0.0f;
+  for (int s = 0; s < NSTAGE - 1; ++s) {
+    issue_tokens(min(s, KB - 1), s);
+    load_stage(st[s], min(s, KB - 1));
+  }
+  const int kb_main = KB - KB % NSTAGE;
+  for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+    for (int s = 0; s < NSTAGE; ++s) {
+      wait_vm<8>();
+      block_barrier();
+      issue_tokens(min(kb0 + s + NSTAGE - 1, KB - 1), (s + NSTAGE - 1) % NSTAGE);
+      load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
+      compute(st[s], s);
+    }
+  }
+  wait_vm<0>();           // the tail needs everything; no asynchronous write may outlive the item
+  block_barrier();
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            hv[tt][j][i] = bf16_round_f32(silu_f32(acc[tt][j][i]) * acc[tt][j + 2][i]);
-            am = fmaxf(am, fabsf(hv[tt][j][i]));
-          }
-        const int tok = t0 + 16 * tt + r16;
-        if (g.out != nullptr && xv[tt]) {
+  for (int s = 0; s < NSTAGE - 1; ++s)
+    if (kb_main + s < KB) compute(st[s], s);
+
+  // ---- epilogue -------------------------------------------------------------
+  bool xv[TT];
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            uint2 o;
-            o.x = f32_to_bf16_bits(hv[tt][j][0]) | (f32_to_bf16_bits(hv[tt][j][1]) << 16);
-            o.y = f32_to_bf16_bits(hv[tt][j][2]) | (f32_to_bf16_bits(hv[tt][j][3]) << 16);
-            *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = o;
-          }
+  for (int tt = 0; tt < TT; ++tt) xv[tt] = 16 * tt + r16 < live;
+  if constexpr (FUSED) {
+    float hv[TT][2][4];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      float am = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          hv[tt][j][i] = bf16_round_f32(silu_f32(acc[tt][j][i]) * acc[tt][j + 2][i]);
+          am = fmaxf(am, fabsf(hv[tt][j][i]));
         }
-        if (g.out_q != nullptr) {
-          am = fmaxf(am, __shfl_xor(am, 16, BGMOE_WAVE));
-          am = fmaxf(am, __shfl_xor(am, 32, BGMOE_WAVE));
-          if (kq == 0) s_amax[wave][tt][r16] = am;
+      const int tok = t0 + 16 * tt + r16;
+      if (g.out != nullptr && xv[tt]) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          uint2 o;
+          o.x = f32_to_bf16_bits(hv[tt][j][0]) | (f32_to_bf16_bits(hv[tt][j][1]) << 16);
+          o.y = f32_to_bf16_bits(hv[tt][j][2]) | (f32_to_bf16_bits(hv[tt][j][3]) << 16);
+          *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = o;
         }
       }
       if (g.out_q != nullptr) {
-        __syncthreads();
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-          const float am = fmaxf(fmaxf(s_amax[0][tt][r16], s_amax[1][tt][r16]),
-                                 fmaxf(s_amax[2][tt][r16], s_amax[3][tt][r16]));
-          const float sc = quant_scale_from_amax(am);
-          const int tok = t0 + 16 * tt + r16;
-          if (xv[tt]) {
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-              const uint32_t q = pack4_e4m3(clamp448(hv[tt][j][0] / sc), clamp448(hv[tt][j][1] / sc),
-                                            clamp448(hv[tt][j][2] / sc), clamp448(hv[tt][j][3] / sc));
-              *reinterpret_cast<uint32_t*>(g.out_q + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = q;
-            }
-            if (wave == 0 && kq == 0)
-              g.out_s[(row0 + tok) * g.os_row + (int64_t)(n0 >> 7) * g.os_nb] = sc;
-          }
-        }
+        am = fmaxf(am, __shfl_xor(am, 16, BGMOE_WAVE));
+        am = fmaxf(am, __shfl_xor(am, 32, BGMOE_WAVE));
+        if (kq == 0) s_amax[wave][tt][r16] = am;
       }
-    } else {
+    }
+    if (g.out_q != nullptr) {
+      __syncthreads();
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) {
+        const float am = fmaxf(fmaxf(s_amax[0][tt][r16], s_amax[1][tt][r16]),
+                               fmaxf(s_amax[2][tt][r16], s_amax[3][tt][r16]));
+        const float sc = quant_scale_from_amax(am);
         const int tok = t0 + 16 * tt + r16;
-        if (!xv[tt]) continue;
+        if (xv[tt]) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-          if (!tv[t]) continue;
-          uint2 o;
-          o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
-          o.y = f32_to_bf16_bits(acc[tt][t][2]) | (f32_to_bf16_bits(acc[tt][t][3]) << 16);
-          *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 64 * wave + 16 * t + 4 * kq) = o;
+          for (int j = 0; j < 2; ++j) {
+            const uint32_t q = pack4_e4m3(clamp448(hv[tt][j][0] / sc), clamp448(hv[tt][j][1] / sc),
+                                          clamp448(hv[tt][j][2] / sc), clamp448(hv[tt][j][3] / sc));
+            *reinterpret_cast<uint32_t*>(g.out_q + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = q;
+          }
+          if (wave == 0 && kq == 0)
+            g.out_s[(row0 + tok) * g.os_row + (int64_t)(n0 >> 7) * g.os_nb] = sc;
         }
+      }
+    }
+  } else {
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      const int tok = t0 + 16 * tt + r16;
+      if (!xv[tt]) continue;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        if (!tv[t]) continue;
+        uint2 o;
+        o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
+        o.y = f32_to_bf16_bits(acc[tt][t][2]) | (f32_to_bf16_bits(acc[tt][t][3]) << 16);
+        *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 64 * wave + 16 * t + 4 * kq) = o;
       }
     }
   }
@@ -260,14 +293,16 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned vblocks) {
   __shared__ float s_amax[4][TT][16];
+  __shared__ __align__(16) uint8_t s_ring[NSTAGE * TokSlot<TT>::kBytes];
+  const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
   const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
   const int hi = bgmoe_split_limit(g.seqlens, g.groups, g.split);
   for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
     const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, 0, hi, 16 * TT, ntiles, vb);
     if (it.grp == BGMOE_ITEM_END) break;
     if (it.grp == BGMOE_ITEM_PAD) continue;
-    fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT>(g, it, s_amax);
-    __syncthreads();                      // s_amax is reused by the next item
+    fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT>(g, it, s_amax, s_ring, ring_lds);
+    __syncthreads();                      // s_amax and the token ring are reused by the next item
   }
 }
 
@@ -322,14 +357,19 @@ static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
   hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks);
 }
 
-template <int TT, int NS>
-static void launch_variant(bool fused, int layout, unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
+// Stage 1 works on 32-row items (its epilogue keeps 16*TT x 8 fp32 results per lane alive next to the
+// prefetch stages); the plain GEMM on 64-row items, which halves the passes over the weights of groups
+// with more than 32 rows.
+static void launch_variant(bool fused, int layout, int n, int groups, int64_t bound, int hi, const SkinnyArgs& g,
+                           hipStream_t st) {
   if (fused) {
-    if (layout == BGMOE_W_TILE_MAJOR) launch_one<TT, NS, true, BGMOE_W_TILE_MAJOR>(vblocks, g, st);
-    else launch_one<TT, NS, true, BGMOE_W_ROW_MAJOR>(vblocks, g, st);
+    const unsigned vb = bgmoe_item_grid((n + 127) / 128, groups, bound, hi, 32);
+    if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 3, true, BGMOE_W_TILE_MAJOR>(vb, g, st);
+    else launch_one<2, 3, true, BGMOE_W_ROW_MAJOR>(vb, g, st);
   } else {
-    if (layout == BGMOE_W_TILE_MAJOR) launch_one<TT, NS, false, BGMOE_W_TILE_MAJOR>(vblocks, g, st);
-    else launch_one<TT, NS, false, BGMOE_W_ROW_MAJOR>(vblocks, g, st);
+    const unsigned vb = bgmoe_item_grid((n + 255) / 256, groups, bound, hi, 64);
+    if (layout == BGMOE_W_TILE_MAJOR) launch_one<4, 2, false, BGMOE_W_TILE_MAJOR>(vb, g, st);
+    else launch_one<4, 2, false, BGMOE_W_ROW_MAJOR>(vb, g, st);
   }
 }
 
@@ -354,7 +394,6 @@ extern "C" int bgmoe_set_skinny_max_rows(int rows) {
 }
 
 static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
-  const int ntile = fused ? 128 : 256;
   const int layout = g.w0.layout;
   if (fused && g.w1.layout != layout) {
     bgmoe_set_error("fp8_fused_s1: gate and up weights must use the same layout");
@@ -368,12 +407,9 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   const int hi = skinny_limit();
   const BgmoeSplit split{hi < 64 ? hi : 64, hi, 8};
   if (hi > 0) {
-    static const int tt = getenv("BGMOE_SKINNY_TT") ? atoi(getenv("BGMOE_SKINNY_TT")) : 2;
-    const unsigned grid = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, hi, 16 * tt);
     g.split = split;
     BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
-    if (tt == 4) launch_variant<4, 2>(fused, layout, grid, g, st);
-    else launch_variant<2, 3>(fused, layout, grid, g, st);
+    launch_variant(fused, layout, g.n, g.groups, bound, hi, g, st);
     int rc = bgmoe_check_launch("fp8 grouped gemm (skinny)");
     if (rc != BGMOE_OK) return rc;
   }
