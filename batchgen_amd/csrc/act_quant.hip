@@ -171,6 +171,55 @@ __global__ __launch_bounds__(256) void act_quant_kernel(QuantArgs a) {
   }
 }
 
+// Permute + quantise: a token row is quantised ONCE and its bytes and scales are written to every row it
+// is routed to (topk_pos, negative = not local) and to its identity row (extra rows: the shared expert).
+// One wave per (token, 512 columns): a single 16-byte load per lane, no loop-carried latency chain.
+__global__ __launch_bounds__(256) void scatter_quant_kernel(QuantArgs a, int steps, int extra_rows) {
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int k = a.k;
+  const int64_t njobs = a.jobs * steps;               // a.jobs = tokens here
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  for (int64_t job = (int64_t)blockIdx.x * 4 + wave; job < njobs; job += stride) {
+    const int64_t tok = job / steps;
+    const int c0 = (int)(job - tok * steps) * 512 + lane * 8;
+    const bool in = c0 < k;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+    if (in) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(a.x + tok * (int64_t)k + c0);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] = bf16_bits_to_f32(w[i] & 0xffffu);
+        v[2 * i + 1] = bf16_bits_to_f32(w[i] >> 16);
+      }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    amax = wave_max_xor<16>(amax);
+    const float sc = quant_scale_from_amax(amax);
+    uint2 o;
+    {
+      float q[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) q[i] = clamp448(v[i] / sc);
+      o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
+      o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
+    }
+    const bool lead = (lane & 15) == 0;
+    const int ndst = a.topk + (tok < extra_rows ? 1 : 0);
+    for (int j = 0; j < ndst; ++j) {
+      const int64_t dst = j < a.topk ? (int64_t)a.topk_pos[tok * a.topk + j] : a.extra_start + tok;
+      if (dst < 0 || !in) continue;
+      *reinterpret_cast<uint2*>(a.y + dst * (int64_t)k + c0) = o;
+      if (lead) a.scale[dst * a.srow + (int64_t)(c0 >> 7) * a.skb] = sc;
+    }
+  }
+}
+
 template <int MODE>
 int launch(const QuantArgs& a, hipStream_t st) {
   if (a.jobs <= 0 || a.k <= 0) return BGMOE_OK;
@@ -258,7 +307,16 @@ int bgmoe_internal_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int
   QuantArgs a{};
   a.x = x; a.y = y; a.scale = scale; a.pairs = (int64_t)n * k; a.jobs = a.pairs + extra_rows; a.k = h;
   a.srow = srow; a.skb = skb; a.topk_pos = topk_pos; a.topk = k; a.extra_start = extra_start;
-  return launch<kGather>(a, st);
+  const bool vec = h % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 8 == 0 && extra_rows <= n;
+  if (!vec) return launch<kGather>(a, st);          // odd shapes: one wave per destination row
+  if (n <= 0 || h <= 0) return BGMOE_OK;
+  a.jobs = n;
+  const int steps = (h + 511) / 512;
+  int64_t blocks = ((int64_t)n * steps + 3) / 4;
+  if (blocks > 65536) blocks = 65536;
+  BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
+  hipLaunchKernelGGL(scatter_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a, steps, extra_rows);
+  return bgmoe_check_launch("scatter_quant");
 }
 
 extern "C" int bgmoe_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h,

@@ -55,7 +55,7 @@ struct BgmoeProf {
 int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                             const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                             uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
-                            int64_t row_bound, hipStream_t st);
+                            int64_t row_bound, int64_t group_bound, hipStream_t st);
 
 static inline hipStream_t bgmoe_stream(bgmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -50,6 +50,7 @@ struct SkinnyArgs {
   int64_t os_row, os_nb;
   BgmoeSplit split;           // this launch serves groups with count <= bgmoe_split_limit(...)
   int64_t row_bound;          // host-side upper bound on the total live rows
+  int64_t group_bound;        // host-side upper bound on the rows of any one group (0 = unknown)
 };
 
 template <int NSC>
@@ -405,7 +406,11 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   }
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
   const int hi = skinny_limit();
-  const BgmoeSplit split{hi < 64 ? hi : 64, hi, 8};
+  // When the caller knows that no group can exceed max_rows (a decode batch: a group never has more rows
+  // than there are tokens), everything streams and the tiled launch is skipped; otherwise the device
+  // decides per launch from the counts.
+  const bool stream_only = g.group_bound > 0 && g.group_bound <= hi;
+  const BgmoeSplit split{stream_only || hi < 64 ? hi : 64, hi, 8};
   if (hi > 0) {
     g.split = split;
     BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
@@ -415,7 +420,8 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   }
   // no group can reach the tiled kernel: too few rows in total for one group above small_rows, or for
   // min_tiles tiles of them while none exceeds max_rows
-  if (bound <= split.small_rows || (bound <= hi && bound <= (int64_t)split.min_tiles * split.small_rows))
+  if (stream_only || bound <= split.small_rows ||
+      (bound <= hi && bound <= (int64_t)split.min_tiles * split.small_rows))
     return BGMOE_OK;
   return bgmoe_launch_fp8_tiled(&g.a, &g.w0, fused ? &g.w1 : nullptr, g.seqlens, g.cu, g.groups, m, g.n,
                                 g.k, g.out, g.out_q, g.out_s, g.os_row, g.os_nb, split, st);
@@ -424,11 +430,12 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
 int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                             const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                             uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
-                            int64_t row_bound, hipStream_t st) {
+                            int64_t row_bound, int64_t group_bound, hipStream_t st) {
   SkinnyArgs g{};
   g.a = *a; g.w0 = *w0; if (w1) g.w1 = *w1;
   g.seqlens = seqlens; g.cu = cu; g.groups = groups; g.n = n; g.k = k;
   g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.row_bound = row_bound;
+  g.group_bound = group_bound;
   return launch_skinny(w1 != nullptr, g, m, st);
 }
 

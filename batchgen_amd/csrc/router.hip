@@ -16,16 +16,48 @@ __device__ __forceinline__ float sigmoid_cr(float x) {
   return (float)(1.0 / (1.0 + exp(-(double)x)));
 }
 
-__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    const float ov = __shfl_xor(v, off, BGMOE_WAVE);
-    const int oi = __shfl_xor(idx, off, BGMOE_WAVE);
-    if (ov > v || (ov == v && oi < idx)) {
-      v = ov;
-      idx = oi;
-    }
+// Data-parallel-primitive lane exchanges inside a row of 16 lanes (a VALU modifier, no LDS round trip):
+// quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror.  Applied in this order with an
+// order-independent merge, all 16 lanes of a row end up with the row's result.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+
+__device__ __forceinline__ void argmax_merge(float& v, int& idx, float ov, int oi) {
+  if (ov > v || (ov == v && oi < idx)) {
+    v = ov;
+    idx = oi;
   }
+}
+
+// "larger value wins, equal values go to the lower index": a total order, so any reduction network gives
+// the same winner.  Rows of 16 lanes reduce with DPP; the four row results are combined from scalars.
+__device__ __forceinline__ void wave_argmax(float& v, int& idx) {
+  argmax_merge(v, idx, dpp_f32<kDppXor1>(v), dpp_i32<kDppXor1>(idx));
+  argmax_merge(v, idx, dpp_f32<kDppXor2>(v), dpp_i32<kDppXor2>(idx));
+  argmax_merge(v, idx, dpp_f32<kDppHalfMirror>(v), dpp_i32<kDppHalfMirror>(idx));
+  argmax_merge(v, idx, dpp_f32<kDppMirror>(v), dpp_i32<kDppMirror>(idx));
+  float rv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  int ri = __builtin_amdgcn_readlane(idx, 0);
+#pragma unroll
+  for (int row = 1; row < 4; ++row)
+    argmax_merge(rv, ri, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16 * row)),
+                 __builtin_amdgcn_readlane(idx, 16 * row));
+  v = rv;
+  idx = ri;
+}
+
+// two largest values (with multiplicity) of the union of two (m1 >= m2) pairs
+__device__ __forceinline__ void top2_merge(float& m1, float& m2, float o1, float o2) {
+  const float lo = fminf(m1, o1);
+  m1 = fmaxf(m1, o1);
+  m2 = fmaxf(lo, fmaxf(m2, o2));
 }
 
 struct RouterArgs {
@@ -107,28 +139,54 @@ __global__ __launch_bounds__(256) void router_kernel(RouterArgs a) {
   }
 
   if constexpr (GROUPED) {
-    // group score = sum of the group's two largest biased scores (strict '>' scan from -1e9)
-    float* s = s_lds + wave * a.e;
-#pragma unroll
-    for (int i = 0; i < VPL; ++i) {
-      const int ex = i * BGMOE_WAVE + lane;
-      if (ex < a.e) s[ex] = key[i] == kNegInf ? -1e9f : key[i];
-    }
-    // the slice is private to this wave: order its LDS writes before the reads below
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // group score = sum of the group's two largest biased scores (strict '>' scan from -1e9, i.e. the two
+    // largest values with multiplicity, -1e9 standing in for missing ones)
     const int epg = a.e / a.n_group;
     float gscore = kNegInf;
-    if (lane < a.n_group) {
-      float m1 = -1e9f, m2 = -1e9f;
-      for (int i = 0; i < epg; ++i) {
-        const float v = s[lane * epg + i];
-        if (v > m1) { m2 = m1; m1 = v; }
-        else if (v > m2) { m2 = v; }
+    if ((epg & (epg - 1)) == 0 && epg <= BGMOE_WAVE) {
+      // a group is an aligned run of epg lanes of one register slot: top-2 butterfly in registers
+      float gs[VPL];
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        float m1 = key[i] == kNegInf ? -1e9f : key[i], m2 = -1e9f;
+        if (epg >= 2) top2_merge(m1, m2, dpp_f32<kDppXor1>(m1), dpp_f32<kDppXor1>(m2));
+        if (epg >= 4) top2_merge(m1, m2, dpp_f32<kDppXor2>(m1), dpp_f32<kDppXor2>(m2));
+        if (epg >= 8) top2_merge(m1, m2, dpp_f32<kDppHalfMirror>(m1), dpp_f32<kDppHalfMirror>(m2));
+        if (epg >= 16) top2_merge(m1, m2, dpp_f32<kDppMirror>(m1), dpp_f32<kDppMirror>(m2));
+        if (epg >= 32) top2_merge(m1, m2, __shfl_xor(m1, 16, BGMOE_WAVE), __shfl_xor(m2, 16, BGMOE_WAVE));
+        if (epg >= 64) top2_merge(m1, m2, __shfl_xor(m1, 32, BGMOE_WAVE), __shfl_xor(m2, 32, BGMOE_WAVE));
+        gs[i] = m1 + m2;
       }
-      const float g = m1 + m2;
-      gscore = g > -1e9f ? g : kNegInf;
+      // lane g < n_group collects group g's score from its first expert g*epg = slot (g*epg)/64, lane (g*epg)%64
+      const int ex0 = lane < a.n_group ? lane * epg : 0;
+      float g = -1e9f;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const float t = __shfl(gs[i], ex0 & (BGMOE_WAVE - 1), BGMOE_WAVE);
+        if ((ex0 >> 6) == i) g = t;
+      }
+      if (lane < a.n_group) gscore = g > -1e9f ? g : kNegInf;
+    } else {
+      float* s = s_lds + wave * a.e;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        const int ex = i * BGMOE_WAVE + lane;
+        if (ex < a.e) s[ex] = key[i] == kNegInf ? -1e9f : key[i];
+      }
+      // the slice is private to this wave: order its LDS writes before the reads below
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if (lane < a.n_group) {
+        float m1 = -1e9f, m2 = -1e9f;
+        for (int i = 0; i < epg; ++i) {
+          const float v = s[lane * epg + i];
+          if (v > m1) { m2 = m1; m1 = v; }
+          else if (v > m2) { m2 = v; }
+        }
+        const float g = m1 + m2;
+        gscore = g > -1e9f ? g : kNegInf;
+      }
     }
     unsigned long long gmask = 0ull;
     for (int r = 0; r < a.topk_group; ++r) {
