@@ -57,7 +57,7 @@ template <bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
   extern __shared__ __align__(16) uint8_t smem[];      // NS slots
   __shared__ int s_tiles[kMaxGroups + 1];              // exclusive prefix of m-tiles per group
-  __shared__ float s_ws[2][kMaxKB];                    // this item's weight scales along K
+  __shared__ float s_ws[2][2][kMaxKB];                 // [buffer][row] weight scales along K of an item
   __shared__ float s_amax[2][4][8][16];
 
   const int tid = threadIdx.x;
@@ -100,10 +100,25 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
   const int bstep = (gridDim.x + nx - 1 - xcd) / nx;   // blocks living on this XCD
   const int bidx = blockIdx.x / nx;
 
-  for (int64_t itx = (int64_t)bidx; itx < per_x; itx += bstep) {
+  // ---- per-item state ----
+  struct Meta { int cnt, m0, n0; int64_t row0; };
+  const uint32_t ws_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)&s_ws[0][0][0]);
+  const int lrow = lane >> 3;
+  const int lchunk = ((lane & 7) ^ lrow) * 16;
+  // load sources of the item whose K-loop runs (or is about to run): wave-uniform bases + lane offsets
+  const uint8_t* tok_base = nullptr;
+  uint32_t tok_off[2][2] = {{0u, 0u}, {0u, 0u}};
+  const uint8_t* w_base[2] = {nullptr, nullptr};
+  const uint32_t w_off = LAYOUT == BGMOE_W_ROW_MAJOR ? (uint32_t)lrow * (uint32_t)K + lchunk : lane * 16;
+  const float* xs_base = nullptr;
+  uint32_t xs_off = 0u;
+  const float* ws_src = nullptr;                       // waves 0 and 1: the weight-scale row each stages
+
+  // item index of this block's walk -> (group, n-tile, m-tile) and its load sources
+  auto prepare = [&](int64_t itx, Meta& mt) -> bool {
+    if (itx >= per_x) return false;
     const int64_t item = (int64_t)xcd * per_x + itx;
-    if (item >= total) break;
-    // item -> (group, n-tile, m-tile)
+    if (item >= total) return false;
     int lo_g = 0, hi_g = g.groups - 1;
     while (lo_g < hi_g) {
       const int mid = (lo_g + hi_g + 1) >> 1;
@@ -118,43 +133,32 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
     const int pm = min(kPanel, mt_g - panel * kPanel);
     const int r2 = (int)(rel - (int64_t)panel * kPanel * ntn);
     const int nt = r2 / pm;
-    const int mt = panel * kPanel + (r2 - nt * pm);
+    const int mtile = panel * kPanel + (r2 - nt * pm);
     const int cnt = g.seqlens[grp];
     const int64_t row0 = g.cu[grp];
-    const int m0 = mt * TM;
+    const int m0 = mtile * TM;
     const int n0 = nt * ncols;
+    mt.cnt = cnt; mt.m0 = m0; mt.n0 = n0; mt.row0 = row0;
 
     const uint8_t* wb0 = g.w0.w_ptrs ? g.w0.w_ptrs[grp] : g.w0.w + (int64_t)grp * g.w0.w_group_stride;
     const float* ws0 = (g.w0.scale_ptrs ? g.w0.scale_ptrs[grp] : g.w0.scale + (int64_t)grp * g.w0.scale_group_stride);
     const uint8_t* wb1 = nullptr;
-    const float* ws1 = nullptr;
+    // weight scales along K: fused [0] gate, [1] up; else [0] columns 0..127, [1] columns 128..255 of the tile
     if constexpr (FUSED) {
       wb1 = g.w1.w_ptrs ? g.w1.w_ptrs[grp] : g.w1.w + (int64_t)grp * g.w1.w_group_stride;
-      ws1 = (g.w1.scale_ptrs ? g.w1.scale_ptrs[grp] : g.w1.scale + (int64_t)grp * g.w1.scale_group_stride) +
-            (int64_t)(n0 >> 7) * g.w1.scale_nb_stride;
+      const float* ws1 = (g.w1.scale_ptrs ? g.w1.scale_ptrs[grp] : g.w1.scale + (int64_t)grp * g.w1.scale_group_stride) +
+                         (int64_t)(n0 >> 7) * g.w1.scale_nb_stride;
       ws0 += (int64_t)(n0 >> 7) * g.w0.scale_nb_stride;
+      ws_src = uniform_ptr(wave_u == 0 ? ws0 : ws1);
+    } else {
+      const int nb = min(n0 + (wave_u == 0 ? 0 : 128), g.n - 1) >> 7;
+      ws_src = uniform_ptr(ws0 + (int64_t)nb * g.w0.scale_nb_stride);
     }
 
-    __syncthreads();          // the previous item's reads of s_ws / s_amax / the LDS ring are done
-    // weight scales of this item along K -> LDS (fused: [0] gate, [1] up; else [0] cols 0..127, [1] cols 128..255)
-    for (int kb = tid; kb < KB; kb += NT) {
-      if constexpr (FUSED) {
-        s_ws[0][kb] = ws0[kb];
-        s_ws[1][kb] = ws1[kb];
-      } else {
-        const int nb0 = min(n0, g.n - 1) >> 7, nb1 = min(n0 + 128, g.n - 1) >> 7;
-        s_ws[0][kb] = ws0[(int64_t)nb0 * g.w0.scale_nb_stride + kb];
-        s_ws[1][kb] = ws0[(int64_t)nb1 * g.w0.scale_nb_stride + kb];
-      }
-    }
-
-    // ---- this wave's share of a stage: token tiles 2w, 2w+1; weight tiles 2w, 2w+1; waves 0..3: 64 token scales ----
-    // row-major sources: load j of a tile covers rows 8j..8j+7, lane p = (row p>>3, LDS chunk p&7) fetches
+    // this wave's share of a stage: token tiles 2w, 2w+1; weight tiles 2w, 2w+1; waves 0..3: 64 token scales.
+    // Row-major sources: load j of a tile covers rows 8j..8j+7, lane p = (row p>>3, LDS chunk p&7) fetches
     // the row's 16-byte chunk (p&7) ^ (p>>3): whole 128-byte lines per 8 lanes, XOR-swizzled in LDS
-    const int lrow = lane >> 3;
-    const int lchunk = ((lane & 7) ^ lrow) * 16;
-    const uint8_t* tok_base = uniform_ptr(g.a.x + (row0 + m0) * K);
-    uint32_t tok_off[2][2];
+    tok_base = uniform_ptr(g.a.x + (row0 + m0) * K);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -162,7 +166,6 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
         const int tok = min(16 * (2 * wave + i) + 8 * j + lrow, cnt - 1 - m0);
         tok_off[i][j] = (uint32_t)tok * (uint32_t)K + lchunk;
       }
-    const uint8_t* w_base[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int lt = 2 * wave_u + i;               // LDS weight tile 0..15 (16 rows each)
@@ -172,45 +175,64 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
       // row-major: row nrow; tile-major: tile nrow / 16 (16 x K bytes per row of tiles)
       w_base[i] = uniform_ptr(base + (int64_t)(LAYOUT == BGMOE_W_ROW_MAJOR ? nrow : (nrow & ~15)) * K);
     }
-    const uint32_t w_off = LAYOUT == BGMOE_W_ROW_MAJOR ? (uint32_t)lrow * (uint32_t)K + lchunk : lane * 16;
-    const float* xs_base = uniform_ptr(g.a.scale + (row0 + m0) * g.a.scale_row_stride);
-    const uint32_t xs_off = (uint32_t)min(64 * wn + lane, cnt - 1 - m0) * (uint32_t)g.a.scale_row_stride * 4u;
+    xs_base = uniform_ptr(g.a.scale + (row0 + m0) * g.a.scale_row_stride);
+    xs_off = (uint32_t)min(64 * wn + lane, cnt - 1 - m0) * (uint32_t)g.a.scale_row_stride * 4u;
+    return true;
+  };
 
-    auto issue = [&](int kb, int slot) {
-      const uint32_t sb = smem_base + (uint32_t)slot * kSlotBytes;
-      const int ko = kb << 7;
+  auto issue = [&](int kb, int slot) {
+    const uint32_t sb = smem_base + (uint32_t)slot * kSlotBytes;
+    const int ko = kb << 7;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const uint32_t d = sb + (2 * wave_u + i) * 2048;
-        async_load16(tok_base + ko, tok_off[i][0], d);
-        async_load16(tok_base + ko, tok_off[i][1], d + 1024);
-      }
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t d = sb + (2 * wave_u + i) * 2048;
+      async_load16(tok_base + ko, tok_off[i][0], d);
+      async_load16(tok_base + ko, tok_off[i][1], d + 1024);
+    }
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const uint32_t d = sb + kTokBytes + (2 * wave_u + i) * 2048;
-        if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
-          async_load16(w_base[i] + ko, w_off, d);
-          async_load16(w_base[i] + ko + 8 * (int64_t)K, w_off, d + 1024);
-        } else {
-          async_load16(w_base[i] + ((int64_t)kb << 11), w_off, d);
-          async_load16(w_base[i] + ((int64_t)kb << 11) + 1024, w_off, d + 1024);
-        }
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t d = sb + kTokBytes + (2 * wave_u + i) * 2048;
+      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
+        async_load16(w_base[i] + ko, w_off, d);
+        async_load16(w_base[i] + ko + 8 * (int64_t)K, w_off, d + 1024);
+      } else {
+        async_load16(w_base[i] + ((int64_t)kb << 11), w_off, d);
+        async_load16(w_base[i] + ((int64_t)kb << 11) + 1024, w_off, d + 1024);
       }
-      if (wave_u < 4)
-        async_load4(xs_base + (int64_t)kb * g.a.scale_kb_stride, xs_off, sb + kXsOff + wave_u * 256);
-    };
+    }
+    if (wave_u < 4)
+      async_load4(xs_base + (int64_t)kb * g.a.scale_kb_stride, xs_off, sb + kXsOff + wave_u * 256);
+  };
+  // waves 0 and 1 stage the item's two weight-scale rows (KB floats each) into s_ws[buf]
+  auto issue_scales = [&](int buf) {
+    if (wave_u < 2) {
+      for (int c = 0; c < KB; c += 64)
+        async_load4(ws_src, (uint32_t)min(c + lane, KB - 1) * 4u,
+                    ws_lds + (uint32_t)(((buf * 2 + (int)wave_u) * kMaxKB + c) * 4));
+    }
+  };
 
+  // The walk is software-pipelined across items: the first K-step and the scales of the next item are
+  // requested before the epilogue of the current one, into the ring slot and scale buffer it no longer uses.
+  Meta cur{}, nxt{};
+  int64_t itx = bidx;
+  bool have = prepare(itx, cur);
+  int sbase = 0, buf = 0;
+  if (have) {
+    issue_scales(buf);
+    issue(0, sbase);
+  }
+  while (have) {
+    const int cnt = cur.cnt, m0 = cur.m0, n0 = cur.n0;
+    const int64_t row0 = cur.row0;
     floatx4 acc[8][4];
 #pragma unroll
     for (int tt = 0; tt < 8; ++tt)
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    issue(0, 0);
-    __syncthreads();          // s_ws is visible (compiler-tracked stores)
-
     for (int kb = 0; kb < KB; ++kb) {
-      const int slot = kb & 1;
+      const int slot = (sbase + kb) & 1;
       wait_vm<0>();                              // this wave's loads of step kb have landed ...
       block_barrier();                           // ... and everybody's; everybody is done with step kb-1
       if (kb + 1 < KB) issue(kb + 1, slot ^ 1);  // refill the slot step kb-1 used
@@ -218,7 +240,7 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
       const uint8_t* b = smem + slot * kSlotBytes;
       const uint8_t* bw = b + kTokBytes;
       const float* bxs = reinterpret_cast<const float*>(b + kXsOff);
-      const float wsc0 = s_ws[0][kb], wsc1 = s_ws[1][kb];
+      const float wsc0 = s_ws[buf][0][kb], wsc1 = s_ws[buf][1][kb];
 
       // operand offsets inside a 2 KiB tile image: swizzled row-major (tokens, row-major weights) or lane order
       const int sw_lo = r16 * 128 + ((kq ^ (r16 & 7)) * 16);
@@ -272,7 +294,16 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
       }
     }
 
-    // ---- epilogue ----------------------------------------------------------------
+    // ---- next item: sources, scales and first K-step (the slot used by step KB-2 is free) ----
+    itx += bstep;
+    const int nslot = (sbase + KB) & 1;
+    have = prepare(itx, nxt);
+    if (have) {
+      issue_scales(buf ^ 1);
+      issue(0, nslot);
+    }
+
+    // ---- epilogue of the current item -----------------------------------------------
     if constexpr (FUSED) {
 #pragma unroll
       for (int tt = 0; tt < 8; ++tt) {
@@ -337,6 +368,9 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
         }
       }
     }
+    cur = nxt;
+    sbase = nslot;
+    buf ^= 1;
   }
 }
 
