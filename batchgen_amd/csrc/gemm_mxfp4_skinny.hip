@@ -1,8 +1,9 @@
 // W4A16 grouped GEMM for MXFP4 weights (e2m1 values, one e8m0 scale per 32 along K) and bf16
 // activations: a weight-streaming kernel bound by HBM bandwidth (decode).
 //
-// Same work split and scheduling as the FP8 weight-streaming kernel: block = (group, 32-token chunk,
-// 128 gate + 128 up columns | 256 columns), 4 waves x four 16-row weight tiles, register prefetch.
+// Same work split and scheduling as the FP8 weight-streaming kernel: item = (group, 64-token chunk,
+// 128 gate + 128 up columns | 256 columns), 4 waves x four 16-row weight tiles, register prefetch,
+// tokens shared through an LDS ring, persistent grid.
 // Weights are dequantised IN REGISTERS: one lane's 16-byte load is one row's 32-value scale group;
 // v_cvt_scalef32_pk_bf16_fp4 turns a byte (low nibble = even K) into two bf16 already multiplied by
 // 2^(scale-127), exactly (a power-of-two times a 2-bit-mantissa value), so the MFMA consumes the
@@ -20,6 +21,7 @@
 
 #include "bgmoe_common.h"
 #include "bgmoe_sched.h"
+#include "bgmoe_async.h"
 
 namespace {
 
@@ -37,11 +39,9 @@ struct Mx4Args {
   int64_t row_bound;
 };
 
-template <int TT>
 struct Mx4Stage {
   intx4 A[4];                   // packed fp4: one 32-value scale group per lane and tile
   uint32_t S[4];                // the row's four scale bytes of this 128-K block
-  intx4 B[TT][4];               // tokens: 8 bf16 per step
 };
 
 __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float scale) {
@@ -52,15 +52,19 @@ __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float scale) {
   return bf16x8{v0[0], v0[1], v1[0], v1[1], v2[0], v2[1], v3[0], v3[1]};
 }
 
+// One work item: up to 16*TT rows of one group x one n-tile, streamed over K.  Weights go from HBM
+// straight into registers; the item's bf16 tokens (4x the bytes of the fp4 weights they meet) are shared by
+// the four waves through an LDS ring filled by asynchronous global -> LDS loads.  A token tile is 16 rows x
+// 256 bytes per K-block; a load covers 4 rows: lane p = (row p>>4, LDS chunk p&15) fetches the row's 16-byte
+// chunk (p&15) ^ row, so that the MFMA operand reads (16 rows, same chunk) hit 16 different bank groups.
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
-__global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g) {
+__device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it, const uint8_t* ring, uint32_t ring_lds) {
   constexpr int NT = 4;
-  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
-  const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, blockIdx.x);
-  if (it.grp < 0) return;
+  constexpr int kSlot = TT * 4096;
   const int grp = it.grp, cnt = it.cnt;
   const int64_t row0 = g.cu[grp];
   const int wave = threadIdx.x >> 6;
+  const uint32_t wave_u = __builtin_amdgcn_readfirstlane((uint32_t)wave);
   const int lane = threadIdx.x & 63;
   const int r16 = lane & 15;
   const int kq = lane >> 4;
@@ -95,15 +99,28 @@ __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g) {
   }
 
   const int t0 = it.chunk * 16 * TT;
+  const int live = cnt - t0;
+  const int tiles = min(TT, (live + 15) >> 4);
   uint16_t* const obase = g.out_ptrs ? g.out_ptrs[grp] : g.out + row0 * g.n;
-  const uint8_t* xp[TT];
-  bool xv[TT];
+
+  // tokens: wave w loads quarter-tiles w*TT .. w*TT+TT-1 (4 rows x 256 bytes each)
+  const uint8_t* tok_base = uniform_ptr(reinterpret_cast<const uint8_t*>(g.x + (row0 + t0) * K));
+  uint32_t tok_off[TT];
+  bool tok_on[TT];
 #pragma unroll
-  for (int tt = 0; tt < TT; ++tt) {
-    const int tok = t0 + 16 * tt + r16;
-    xv[tt] = tok < cnt;
-    xp[tt] = reinterpret_cast<const uint8_t*>(g.x + (row0 + (xv[tt] ? tok : 0)) * K) + 64 * kq;
+  for (int i = 0; i < TT; ++i) {
+    const int qt = (int)wave_u * TT + i;                  // quarter-tile 0 .. 4*TT-1
+    const int rt = 4 * (qt & 3) + (lane >> 4);            // row inside its tile
+    const int row = min(16 * (qt >> 2) + rt, live - 1);
+    tok_off[i] = (uint32_t)row * (uint32_t)(2 * K) + (uint32_t)((((lane & 15) ^ rt) & 15) * 16);
+    tok_on[i] = (qt >> 2) < tiles;
   }
+  auto issue_tokens = [&](int kb, int slot) {
+    const uint32_t sbs = ring_lds + (uint32_t)slot * kSlot;
+#pragma unroll
+    for (int i = 0; i < TT; ++i)
+      if (tok_on[i]) async_load16(tok_base + (kb << 8), tok_off[i], sbs + (wave_u * TT + i) * 1024);
+  };
 
   floatx4 acc[TT][NT];
 #pragma unroll
@@ -111,8 +128,8 @@ __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  Mx4Stage<TT> st[NSTAGE];
-  auto load_stage = [&](Mx4Stage<TT>& s, int kb) {
+  Mx4Stage st[NSTAGE];
+  auto load_stage = [&](Mx4Stage& s, int kb) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
@@ -123,45 +140,59 @@ __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g) {
         s.S[t] = *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)(sp[t] + (kb << 6)));
       }
     }
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) s.B[tt][j] = gload_x4(xp[tt] + (kb << 8) + 16 * j);
   };
-  auto compute = [&](const Mx4Stage<TT>& c) {
+  auto compute = [&](const Mx4Stage& c, int slot) {
+    const uint8_t* b = ring + slot * kSlot + r16 * 256;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const float sc = __uint_as_float(((c.S[t] >> (8 * kq)) & 0xffu) << 23);    // 2^(e8m0 - 127)
+    for (int j = 0; j < 4; ++j) {
+      const int boff = (((4 * kq + j) ^ r16) & 15) * 16;
+      bf16x8 a[NT];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const bf16x8 a = dequant8((uint32_t)c.A[t][j], sc);
+      for (int t = 0; t < NT; ++t) {
+        const float sc = __uint_as_float(((c.S[t] >> (8 * kq)) & 0xffu) << 23);    // 2^(e8m0 - 127)
+        a[t] = dequant8((uint32_t)c.A[t][j], sc);
+      }
 #pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-          const bf16x8 b = __builtin_bit_cast(bf16x8, c.B[tt][j]);
-          acc[tt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[tt][t], 0, 0, 0);
+      for (int tt = 0; tt < TT; ++tt) {
+        if (tt < tiles) {
+          const bf16x8 bv = __builtin_bit_cast(bf16x8, *reinterpret_cast<const intx4*>(b + tt * 4096 + boff));
+#pragma unroll
+          for (int t = 0; t < NT; ++t) acc[tt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], bv, acc[tt][t], 0, 0, 0);
         }
       }
     }
   };
 
+  // Same pipeline as the FP8 streaming kernel: tokens are requested before the weights of the same
+  // K-block, loads complete in issue order, so "at most the 8 weight loads of the youngest stage
+  // outstanding" means the stage about to be computed has landed for this wave; the barrier extends
+  // that to the other waves' token loads and frees the slot refilled next.
 #pragma unroll
-  for (int s = 0; s < NSTAGE - 1; ++s) load_stage(st[s], min(s, KB - 1));
+  for (int s = 0; s < NSTAGE - 1; ++s) {
+    issue_tokens(min(s, KB - 1), s);
+    load_stage(st[s], min(s, KB - 1));
+  }
   const int kb_main = KB - KB % NSTAGE;
   for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
+      wait_vm<8>();
+      block_barrier();
+      issue_tokens(min(kb0 + s + NSTAGE - 1, KB - 1), (s + NSTAGE - 1) % NSTAGE);
       load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
-      compute(st[s]);
+      compute(st[s], s);
     }
   }
+  wait_vm<0>();           // the tail needs everything; no asynchronous write may outlive the item
+  block_barrier();
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s)
-    if (kb_main + s < KB) compute(st[s]);
+    if (kb_main + s < KB) compute(st[s], s);
 
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) {
     const int tok = t0 + 16 * tt + r16;
-    if (!xv[tt]) continue;
+    if (16 * tt + r16 >= live) continue;
     if constexpr (FUSED) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -183,6 +214,21 @@ __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g) {
         *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + 64 * wave + 16 * t + 4 * kq) = o;
       }
     }
+  }
+}
+
+// Persistent grid: block b works on virtual blocks b, b + gridDim.x, ... until the item list ends.
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
+__global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned vblocks) {
+  __shared__ __align__(16) uint8_t s_ring[NSTAGE * TT * 4096];
+  const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
+  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
+  for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
+    const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, vb);
+    if (it.grp == BGMOE_ITEM_END) break;
+    if (it.grp == BGMOE_ITEM_PAD) continue;
+    mxfp4_item<TT, NSTAGE, FUSED, LAYOUT>(g, it, s_ring, ring_lds);
+    __syncthreads();                      // the token ring is reused by the next item
   }
 }
 
@@ -214,19 +260,37 @@ int check_w(const char* what, const bgmoe_mxfp4_weight* w) {
   return BGMOE_OK;
 }
 
+template <int TT, int NS, bool FUSED, int LAYOUT>
+void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
+  static unsigned resident = 0;       // blocks resident on the whole device at once, a multiple of 8
+  if (resident == 0) {
+    int per_cu = 0, dev = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>, 256, 0) != hipSuccess || per_cu < 1)
+      per_cu = 1;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+      cus = 256;
+    resident = (unsigned)(per_cu * cus) & ~7u;
+    if (resident == 0) resident = 8;
+  }
+  const dim3 grid(vblocks < resident ? vblocks : resident), block(256);
+  hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks);
+}
+
 int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
+  constexpr int TT = 4;            // 64-row items: every group is streamed once per 64 rows
   const int ntile = fused ? 128 : 256;
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
-  const dim3 grid(bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 32)), block(256);
-  g.lo = 0; g.hi = 0x7fffffff;     // every group: more than 32 rows = more chunks (weights re-streamed)
+  const unsigned vblocks = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 16 * TT);
+  g.lo = 0; g.hi = 0x7fffffff;     // every group: more rows = more chunks (weights re-streamed)
   const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
   BgmoeProf prof(fused ? BGMOE_K_MXFP4_S1 : BGMOE_K_MXFP4_GEMM, st);
   if (fused) {
-    if (tm) hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, true, 1>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, true, 0>), grid, block, 0, st, g);
+    if (tm) launch_one<TT, 3, true, 1>(vblocks, g, st);
+    else launch_one<TT, 3, true, 0>(vblocks, g, st);
   } else {
-    if (tm) hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, false, 1>), grid, block, 0, st, g);
-    else hipLaunchKernelGGL((mxfp4_skinny_kernel<2, 3, false, 0>), grid, block, 0, st, g);
+    if (tm) launch_one<TT, 3, false, 1>(vblocks, g, st);
+    else launch_one<TT, 3, false, 0>(vblocks, g, st);
   }
   return bgmoe_check_launch("mxfp4 grouped gemm");
 }
