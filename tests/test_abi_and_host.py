@@ -177,3 +177,20 @@ def test_ragged_capacity_formula():
 def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_config4_routing_has_the_skew_the_baseline_names():
+    """Config 4 is the skewed workload: Zipf-distributed expert popularity with roughly 30% of the experts
+    receiving no token and a hot expert with thousands of rows (the empty-group and long-group paths)."""
+    import numpy as np
+    from batchgen_amd import workloads as wl
+    from oracle import layer as ol
+    cfg = wl.CONFIGS[4]
+    inp = wl.make_inputs(cfg, "cpu")
+    ids, _ = ol.route(inp["logits"].numpy(), inp["bias"].numpy(),
+                      dict(top_k=cfg.top_k, n_group=cfg.n_group, topk_group=cfg.topk_group, rsf=cfg.rsf))
+    counts = np.bincount(ids.ravel(), minlength=cfg.n_experts)
+    empty = float((counts == 0).mean())
+    assert 0.2 <= empty <= 0.4, empty
+    assert counts.max() > 2000
+    assert counts.sum() == cfg.n_tokens * cfg.top_k
