@@ -73,7 +73,7 @@ __device__ __forceinline__ BgmoeItem bgmoe_decode_item(const int32_t* seqlens, i
   int crow = 0;
   it.grp = nth_active_item(seqlens, groups, lo, hi, chunk_rows, (int)(block / ntiles_pad), &crow);
   it.ntile = it.chunk = it.cnt = 0;
-  if (it.grp < 0) {
+  if (__builtin_amdgcn_readfirstlane(it.grp) < 0) {
     it.grp = BGMOE_ITEM_END;
     return it;
   }
@@ -83,6 +83,12 @@ __device__ __forceinline__ BgmoeItem bgmoe_decode_item(const int32_t* seqlens, i
   it.ntile = 8 * (q / (8 * chunks)) + (q & 7);
   it.chunk = (q >> 3) % chunks;
   if (it.ntile >= ntiles) it.grp = BGMOE_ITEM_PAD;
+  // the fields are wave-uniform by construction; say so, so that everything derived from them (pointers,
+  // loop bounds, branches) is scalar code
+  it.grp = __builtin_amdgcn_readfirstlane(it.grp);
+  it.ntile = __builtin_amdgcn_readfirstlane(it.ntile);
+  it.chunk = __builtin_amdgcn_readfirstlane(it.chunk);
+  it.cnt = __builtin_amdgcn_readfirstlane(it.cnt);
   return it;
 }
 

@@ -59,10 +59,18 @@ struct Stage {
   float ws[NSC];
 };
 
-template <int HI>
+// KEEP: the bytes will be read again soon (the group has more row chunks than this one), so they are
+// loaded with the default cache policy; otherwise as a non-temporal stream that does not displace them.
+template <int HI, bool KEEP>
 __device__ __forceinline__ intx8 load32_stream(const uint8_t* p) {
-  const intx4 lo = gload_x4_stream(p);
-  const intx4 hi = gload_x4_stream(p + HI);
+  intx4 lo, hi;
+  if constexpr (KEEP) {
+    lo = gload_x4(p);
+    hi = gload_x4(p + HI);
+  } else {
+    lo = gload_x4_stream(p);
+    hi = gload_x4_stream(p + HI);
+  }
   intx8 r;
   r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
   r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
@@ -76,7 +84,7 @@ struct TokSlot {
 };
 
 // One work item: up to 16*TT rows of one group x one n-tile, streamed over K.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP>
 __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const BgmoeItem& it, float (*s_amax)[TT][16],
                                                 const uint8_t* ring, uint32_t ring_lds) {
   constexpr int NT = 4;                  // weight tiles per wave
@@ -166,8 +174,8 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
     for (int i = 0; i < NSC; ++i) s.ws[i] = gload_f32(wsp[i] + kb);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) s.A[t] = load32_stream<64>(wp[t] + (kb << 7));
-      else s.A[t] = load32_stream<1024>(wp[t] + ((int64_t)kb << 11));
+      if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) s.A[t] = load32_stream<64, KEEP>(wp[t] + (kb << 7));
+      else s.A[t] = load32_stream<1024, KEEP>(wp[t] + ((int64_t)kb << 11));
     }
   };
   const int sw_lo = r16 * 128 + ((kq ^ (r16 & 7)) * 16);
@@ -302,7 +310,9 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned 
     const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, 0, hi, 16 * TT, ntiles, vb);
     if (it.grp == BGMOE_ITEM_END) break;
     if (it.grp == BGMOE_ITEM_PAD) continue;
-    fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT>(g, it, s_amax, s_ring, ring_lds);
+    // a group with several row chunks has its weights streamed once per chunk: keep them cacheable
+    if (it.cnt > 16 * TT) fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, true>(g, it, s_amax, s_ring, ring_lds);
+    else fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, false>(g, it, s_amax, s_ring, ring_lds);
     __syncthreads();                      // s_amax and the token ring are reused by the next item
   }
 }
