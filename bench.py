@@ -25,6 +25,16 @@ FP8_PEAK_TFLOPS = 5000.0        # MI355X published dense FP8 MFMA peak
 
 METRIC = "MoE layer TFLOP/s (FP8 prefill) & HBM GB/s (decode), % roofline, 1xMI355X"
 
+# HBM bytes per launch of each configuration's dominant kernel, measured with two `rocprofv3 --pmc` runs
+# (FETCH_SIZE, then WRITE_SIZE; each scaled by what the same counter reads for a plain 256 MiB copy kernel in
+# the same run: x2.000 and x1.000).  The summaries with the exact commands are profiles/fp8_decode_c1_rocprof.md
+# and profiles/fp8_prefill_c2_rocprof.md.  A configuration that was not measured reports null.
+MIB = 1024 * 1024
+MEASURED_TRAFFIC_BYTES = {
+    1: int((632.3 + 1.4) * MIB),      # fp8_skinny_kernel<2,3,fused,tile_major>, config 1
+    2: int((2269.4 + 82.1) * MIB),    # fp8_tiled_kernel<fused,tile_major>, config 2
+}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -82,6 +92,21 @@ def cpu_baseline(cfg, inp, w, sh, ids, wt, alg_bytes, flops):
     frac = n / cfg.n_tokens
     return t, threads, cores, f"{n} of {cfg.n_tokens} tokens of the workload, all experts they route to, " \
                               f"bf16 dequantised weights, 1 warm-up + median of {reps}", frac
+
+
+def cpu_baseline_mxfp4(cfg, inp, w, sh):
+    """The NumPy restatement of the MXFP4 layer (oracle.layer.moe_layer_mxfp4: dequantise, bf16-valued GEMMs,
+    SwiGLU, combine) on a few tokens; its cost is dominated by dequantising the experts those tokens use."""
+    from oracle import layer as ol
+    n = min(cfg.n_tokens, 8)
+    wn = {k: v.cpu().numpy() for k, v in w.items()}
+    shn = {k: v.float().cpu().numpy() for k, v in sh.items()} if sh else None
+    t0 = time.perf_counter()
+    ol.moe_layer_mxfp4(inp["x"][:n].cpu(), inp["logits"][:n].cpu().numpy(), inp["bias"].cpu().numpy(),
+                       dict(top_k=cfg.top_k, n_group=1, topk_group=1, rsf=cfg.rsf), wn, cfg.expert_start,
+                       cfg.e_local, layout="masked", max_tokens=cfg.max_tokens, shared_bf16=shn)
+    t = time.perf_counter() - t0
+    return t, n / cfg.n_tokens, f"{n} of {cfg.n_tokens} tokens of the workload and the experts they route to, one pass, NumPy"
 
 
 def main():
@@ -150,7 +175,7 @@ def main():
         dom = "mxfp4_s1"
         dom_bytes = active * (2 * h * i // 2 + 2 * h * i // 32) + rows * (h + i) * 2
         dom_ms = prof[dom][0] / max(prof[dom][1], 1)
-        roof = dict(bound="hbm", kernel="mxfp4_skinny_kernel<TT=2,NS=3,fused,tile_major>",
+        roof = dict(bound="hbm", kernel="mxfp4_skinny_kernel<TT=4,NS=3,fused,tile_major>",
                     achieved=dom_bytes / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None,
                     bytes_per_launch=dom_bytes, avg_launch_us=dom_ms * 1e3)
     elif decode:
@@ -167,13 +192,17 @@ def main():
                     avg_launch_us=dom_ms * 1e3)
     else:
         dom = "s1_tiled"
-        big = counts[counts > 64].sum()
+        # the device-side rule of the library: groups above 64 rows are tiled when they make >= 8 tiles of 256
+        allc = np.append(counts, cfg.n_tokens if cfg.shared_inter else 0)
+        lo = 64 if int(((allc[allc > 64] + 255) // 256).sum()) >= 8 else 256
+        big = counts[counts > lo].sum()
         dom_flops = int(big) * 4 * h * i + (cfg.n_tokens * 4 * h * cfg.shared_inter if cfg.shared_inter else 0)
         dom_ms = prof[dom][0] / max(prof[dom][1], 1)
-        roof = dict(bound="mfma", kernel="fp8_tiled_kernel<fused>", achieved=dom_flops / (dom_ms * 1e-3) / 1e12,
+        roof = dict(bound="mfma", kernel="fp8_tiled_kernel<fused,tile_major>", achieved=dom_flops / (dom_ms * 1e-3) / 1e12,
                     peak=FP8_PEAK_TFLOPS, unit="TFLOP/s", traffic=None, flops_per_launch=dom_flops,
                     avg_launch_us=dom_ms * 1e3)
     roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(a.config)
 
     out = {
         "metric": METRIC,
@@ -192,6 +221,11 @@ def main():
         "kernel_ms_per_step": per_kernel,
         "roofline": roof,
     }
+    if not a.no_cpu_baseline and mx4:
+        t, frac, sample = cpu_baseline_mxfp4(cfg, inp, w, sh)
+        out["cpu_baseline"] = {"value": alg_bytes * frac / t / 1e9, "unit": out["unit"], "cores": 1,
+                               "host_cores": os.cpu_count() or 1, "kind": "port", "sample": sample, "seconds": t,
+                               "tokens_per_s": cfg.n_tokens * frac / t}
     if not a.no_cpu_baseline and not mx4:
         ids = layer.topk_ids.cpu().numpy()
         wt = layer.topk_weights.cpu().numpy()
