@@ -223,8 +223,9 @@ def main():
     }
     if not a.no_cpu_baseline and mx4:
         t, frac, sample = cpu_baseline_mxfp4(cfg, inp, w, sh)
-        out["cpu_baseline"] = {"value": alg_bytes * frac / t / 1e9, "unit": out["unit"], "cores": 1,
-                               "host_cores": os.cpu_count() or 1, "kind": "port", "sample": sample, "seconds": t,
+        out["cpu_baseline"] = {"value": alg_bytes * frac / t / 1e9, "unit": out["unit"],
+                               "cores": min(os.cpu_count() or 1, 16), "host_cores": os.cpu_count() or 1,
+                               "kind": "port", "sample": sample + " (BLAS threads for the matrix products, one thread for the dequantisation)", "seconds": t,
                                "tokens_per_s": cfg.n_tokens * frac / t}
     if not a.no_cpu_baseline and not mx4:
         ids = layer.topk_ids.cpu().numpy()
