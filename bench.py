@@ -43,6 +43,8 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="time replays of one captured HIP graph of the layer instead of eager launches")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain copy kernel of known size (the weight re-layout kernel on a "
                          "256 MiB buffer: 256 MiB read, 256 MiB written) so that rocprofv3 --pmc FETCH_SIZE / "
@@ -145,10 +147,18 @@ def main():
         cal = torch.zeros((1, 32768, 8192), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
         repack_tile_major(cal)
         torch.cuda.synchronize()
+    step = lambda: layer(x, logits)
+    if a.graph:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            layer(x, logits)
+        step = graph.replay
+        step()
+        torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(a.steps):
-        layer(x, logits)
+        step()
     stop.record()
     torch.cuda.synchronize()
     ms = start.elapsed_time(stop) / a.steps
@@ -209,7 +219,7 @@ def main():
         "value": gbps if decode else tflops,
         "unit": "GB/s" if decode else "TFLOP/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "launch": "hip_graph" if a.graph else "eager",
         "dtype": "mxfp4 weights x bf16 (fp32 accumulate)" if mx4 else "fp8_e4m3 (fp32 accumulate)", "data": "synthetic",
         "config": {"workload": cfg.name, "tokens": cfg.n_tokens, "hidden": h, "moe_intermediate": i,
                    "experts": cfg.n_experts, "local_experts": cfg.e_local, "top_k": cfg.top_k,

@@ -130,3 +130,41 @@ def test_weight_layouts_give_identical_layers(dev, layout):
     a = mk("row_major")(inp["x"].to(dev), inp["logits"].to(dev)).clone()
     b = mk(layout)(inp["x"].to(dev), inp["logits"].to(dev)).clone()
     assert torch.equal(a, b)
+
+
+def test_layer_forward_replays_from_a_hip_graph(dev):
+    """One captured forward pass, replayed over changing inputs (the device-side counts change with them),
+    with eager work and synchronisations between the replays: every replay equals the eager result bit for
+    bit.  Launch geometry depends on host shapes only and the library allocates nothing, which is what makes
+    the capture legal."""
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = wl.scaled(wl.CONFIGS[1], hidden=1024, inter=512, shared_inter=512)
+    w, sh = wl.make_fp8_weights(cfg, dev)
+    bias = wl.make_inputs(cfg, dev)["bias"]
+    layer = Fp8MoELayer(cfg, w, sh, bias)
+    gen = torch.Generator(device="cpu").manual_seed(7)
+    xs = [torch.randn((cfg.n_tokens, cfg.hidden), generator=gen).to(torch.bfloat16).to(dev) for _ in range(3)]
+    ls = [(torch.randn((cfg.n_tokens, cfg.n_experts), generator=gen) * (1.0 + i)).to(dev) for i in range(3)]
+    eager = []
+    for x, lg in zip(xs, ls):
+        eager.append(layer(x, lg).clone())
+    torch.cuda.synchronize()
+    x_in, l_in = xs[0].clone(), ls[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer(x_in, l_in)                       # warm-up on the capture stream (first-launch attribute queries)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = layer(x_in, l_in)
+    for rnd in range(2):
+        for i in (2, 0, 1):
+            x_in.copy_(xs[i])
+            l_in.copy_(ls[i])
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out_static, eager[i]), f"replay of input {i} (round {rnd}) differs from eager"
+            scratch = layer(xs[(i + 1) % 3], ls[(i + 1) % 3])   # eager work between replays
+            assert torch.equal(scratch, eager[(i + 1) % 3])
