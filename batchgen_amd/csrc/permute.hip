@@ -174,6 +174,96 @@ __global__ __launch_bounds__(256) void perm_rank_kernel(PermArgs a) {
   }
 }
 
+// Decode-sized problems (nk <= 2048 pairs, <= 256 local experts) in ONE block of 16 waves: every lane reads
+// its two ids once, ranks inside a wave come from ballots, one pass over the 16 per-wave histograms turns
+// them into offsets, a single wave scans the experts.  Latency chain: one global load, ~10 LDS round trips.
+constexpr int kSmallLocal = 256;
+__global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
+  __shared__ int32_t whist[16][kSmallLocal];   // per-wave counts, then exclusive offsets over the waves
+  __shared__ int32_t s_cu[kSmallLocal + 1];
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int el = a.e_local;
+  int le[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) le[s] = local_id(a, (int64_t)wave * 128 + s * 64 + lane);
+  for (int e = threadIdx.x; e < 16 * el; e += 1024) whist[e / el][e % el] = 0;
+  __syncthreads();
+  int nbits = 0;
+  while ((1 << nbits) < el) ++nbits;
+  const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+  int off[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    unsigned long long peers = __ballot(le[s] >= 0);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = (le[s] >> b) & 1;
+      const unsigned long long m = __ballot(bit);
+      peers &= bit ? m : ~m;
+    }
+    off[s] = -1;
+    if (le[s] >= 0) off[s] = whist[wave][le[s]] + __popcll(peers & lt);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (le[s] >= 0 && (peers & lt) == 0ull) whist[wave][le[s]] += __popcll(peers);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < el; e += 1024) {
+    int run = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int t = whist[w][e];
+      whist[w][e] = run;
+      run += t;
+    }
+    const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
+    a.counts[e] = cnt;
+    if (a.counters) a.counters[e] = cnt;
+    s_cu[e + 1] = cnt;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    int64_t base = 0;
+    for (int g0 = 0; g0 < el; g0 += 64) {
+      const int g = g0 + lane;
+      const int cnt = g < el ? s_cu[g + 1] : 0;
+      const int64_t span = g < el ? (a.mtp > 0 ? (int64_t)a.mtp
+                                              : (((int64_t)cnt + a.row_align - 1) & ~(int64_t)(a.row_align - 1)))
+                                  : 0;
+      int64_t inc = span;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int64_t up = __shfl_up(inc, o, BGMOE_WAVE);
+        if (lane >= o) inc += up;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();          // everybody has read s_cu[g + 1] before s_cu[g] is overwritten
+      if (g < el) {
+        s_cu[g] = (int32_t)(base + inc - span);
+        if (a.cu) a.cu[g] = (int32_t)(base + inc - span);
+      }
+      base += __shfl(inc, 63, BGMOE_WAVE);
+    }
+    if (lane == 0) write_tail(a, base);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const int64_t i = (int64_t)wave * 128 + s * 64 + lane;
+    if (i < a.nk) {
+      int p = -1;
+      if (le[s] >= 0) {
+        const int slot = whist[wave][le[s]] + off[s];
+        if (a.mtp > 0) p = slot < a.mtp ? le[s] * a.mtp + slot : -1;
+        else p = s_cu[le[s]] + slot;
+      }
+      a.pos[i] = p;
+    }
+  }
+}
+
 // one wave per pair: act[pos] = x[token]
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x,
                                                           const int32_t* __restrict__ pos,
@@ -230,7 +320,8 @@ int run_index(PermArgs& a, void* workspace, size_t workspace_bytes, hipStream_t 
   if (a.nk <= kChunk) {
     a.nchunks = 1;
     BgmoeProf prof(BGMOE_K_PERM_RANK, st);
-    hipLaunchKernelGGL((perm_rank_kernel<true>), dim3(1), dim3(256), 0, st, a);
+    if (a.e_local <= kSmallLocal) hipLaunchKernelGGL(perm_small_kernel, dim3(1), dim3(1024), 0, st, a);
+    else hipLaunchKernelGGL((perm_rank_kernel<true>), dim3(1), dim3(256), 0, st, a);
     return bgmoe_check_launch("dispatch(single)");
   }
   a.nchunks = (int)((a.nk + kChunk - 1) / kChunk);
