@@ -116,3 +116,6 @@ __device__ __forceinline__ float wave_max_xor(float v) {
 }
 
 __device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-g)); }
+// same with the hardware reciprocal (1 ulp) instead of the correctly rounded division: for GEMM epilogues that
+// evaluate it 64 times per lane, where the accumulation order already moves the last bits
+__device__ __forceinline__ float silu_rcp_f32(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }

@@ -312,7 +312,7 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
         for (int j = 0; j < 2; ++j)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float h = bf16_round_f32(silu_f32(acc[tt][j][i]) * acc[tt][j + 2][i]);
+            const float h = bf16_round_f32(silu_rcp_f32(acc[tt][j][i]) * acc[tt][j + 2][i]);
             acc[tt][j][i] = h;
             am = fmaxf(am, fabsf(h));
           }
