@@ -231,12 +231,16 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) acc[tt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+    const bool wave_live = m0 + 128 * (int)(wave_u >> 2) < cnt;
     for (int kb = 0; kb < KB; ++kb) {
       const int slot = (sbase + kb) & 1;
       wait_vm<0>();                              // this wave's loads of step kb have landed ...
       block_barrier();                           // ... and everybody's; everybody is done with step kb-1
       if (kb + 1 < KB) issue(kb + 1, slot ^ 1);  // refill the slot step kb-1 used
 
+      // a wave whose 128 tokens all lie past the group's end (the last m-tile of a ragged group) only keeps
+      // the barriers and its share of the loads: the wave it shares a SIMD with gets the whole MFMA pipe
+      if (!wave_live) continue;
       const uint8_t* b = smem + slot * kSlotBytes;
       const uint8_t* bw = b + kTokBytes;
       const float* bxs = reinterpret_cast<const float*>(b + kXsOff);
