@@ -211,8 +211,12 @@ __global__ __launch_bounds__(256) void scatter_quant_kernel(QuantArgs a, int ste
     }
     const bool lead = (lane & 15) == 0;
     const int ndst = a.topk + (tok < extra_rows ? 1 : 0);
+    // all destinations of the token in one load (lane j holds destination j), not one dependent load per route
+    int64_t mine = -1;
+    if (lane < a.topk) mine = a.topk_pos[tok * a.topk + lane];
+    else if (lane == a.topk && tok < extra_rows) mine = a.extra_start + tok;
     for (int j = 0; j < ndst; ++j) {
-      const int64_t dst = j < a.topk ? (int64_t)a.topk_pos[tok * a.topk + j] : a.extra_start + tok;
+      const int64_t dst = __shfl(mine, j, BGMOE_WAVE);
       if (dst < 0 || !in) continue;
       *reinterpret_cast<uint2*>(a.y + dst * (int64_t)k + c0) = o;
       if (lead) a.scale[dst * a.srow + (int64_t)(c0 >> 7) * a.skb] = sc;
@@ -307,7 +311,7 @@ int bgmoe_internal_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int
   QuantArgs a{};
   a.x = x; a.y = y; a.scale = scale; a.pairs = (int64_t)n * k; a.jobs = a.pairs + extra_rows; a.k = h;
   a.srow = srow; a.skb = skb; a.topk_pos = topk_pos; a.topk = k; a.extra_start = extra_start;
-  const bool vec = h % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 8 == 0 && extra_rows <= n;
+  const bool vec = h % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 8 == 0 && extra_rows <= n && k < 64;
   if (!vec) return launch<kGather>(a, st);          // odd shapes: one wave per destination row
   if (n <= 0 || h <= 0) return BGMOE_OK;
   a.jobs = n;

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(
   __shared__ int32_t s_pos[kMaxK];
   __shared__ float s_w[kMaxK];
   const int token = blockIdx.y;
-  if (threadIdx.x == 0) {
+  if ((!VEC || MODE == 2) && threadIdx.x == 0) {
     const int64_t base = (int64_t)token * k;
     if constexpr (MODE == 2) {
       int32_t eid[kMaxK];
@@ -71,21 +71,56 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(
   float acc[W];
 #pragma unroll
   for (int i = 0; i < W; ++i) acc[i] = 0.0f;
-  for (int j = 0; j < k; ++j) {
-    const int p = s_pos[j];
-    if (p < 0) continue;
-    const float wj = s_w[j];
-    float v[W];
-    if constexpr (VEC) {
-      unpack8(*reinterpret_cast<const uint4*>(y + (int64_t)p * h + c0), v);
-    } else {
-      v[0] = bf16_bits_to_f32(y[(int64_t)p * h + c0]);
-    }
+  if constexpr (VEC && MODE != 2) {
+    // rows of up to 8 routes are requested together (a route that is not local costs nothing), then
+    // accumulated in route order: the loads overlap, the arithmetic keeps its order
+    const int64_t base = (int64_t)token * k;
+    for (int j0 = 0; j0 < k; j0 += 8) {
+      uint4 raw[8];
+      float wj[8];
+      bool on[8];
 #pragma unroll
-    for (int i = 0; i < W; ++i) {
-      const float prod = v[i] * wj;
-      if constexpr (MODE == 2) acc[i] = bf16_round_f32(acc[i] + bf16_round_f32(prod));
-      else acc[i] = acc[i] + prod;
+      for (int u = 0; u < 8; ++u) {
+        const int j = j0 + u;
+        const int p = j < k ? pos[base + j] : -1;        // wave-uniform: scalar loads
+        on[u] = p >= 0;
+        wj[u] = 0.0f;
+        raw[u] = uint4{0u, 0u, 0u, 0u};
+        if (on[u]) {
+          wj[u] = w[base + j];
+          raw[u] = *reinterpret_cast<const uint4*>(y + (int64_t)p * h + c0);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (on[u]) {
+          float v[8];
+          unpack8(raw[u], v);
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            const float prod = v[i] * wj[u];
+            acc[i] = acc[i] + prod;
+          }
+        }
+      }
+    }
+  } else {
+    for (int j = 0; j < k; ++j) {
+      const int p = s_pos[j];
+      if (p < 0) continue;
+      const float wj = s_w[j];
+      float v[W];
+      if constexpr (VEC) {
+        unpack8(*reinterpret_cast<const uint4*>(y + (int64_t)p * h + c0), v);
+      } else {
+        v[0] = bf16_bits_to_f32(y[(int64_t)p * h + c0]);
+      }
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        const float prod = v[i] * wj;
+        if constexpr (MODE == 2) acc[i] = bf16_round_f32(acc[i] + bf16_round_f32(prod));
+        else acc[i] = acc[i] + prod;
+      }
     }
   }
   const int64_t o = (int64_t)token * h + c0;
