@@ -250,6 +250,19 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
       const int sw_lo = r16 * 128 + ((kq ^ (r16 & 7)) * 16);
       const int a_lo = LAYOUT == BGMOE_W_ROW_MAJOR ? sw_lo : lane * 16;
       const int a_hi = LAYOUT == BGMOE_W_ROW_MAJOR ? (sw_lo ^ 64) : lane * 16 + 1024;
+      const uint8_t* bt = b + 8 * wm * 2048;
+      const float* bx = bxs + 128 * wm + r16;
+      auto load_b = [&](int tt) {
+        const intx4 lo = *reinterpret_cast<const intx4*>(bt + tt * 2048 + sw_lo);
+        const intx4 hi = *reinterpret_cast<const intx4*>(bt + tt * 2048 + (sw_lo ^ 64));
+        return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      };
+      // LDS returns data in request order: the first token tile and the first weight tile are requested
+      // first, so the first MFMA waits for 4 reads instead of 10
+      intx8 Bb[2];
+      float xb[2];
+      Bb[0] = load_b(0);
+      xb[0] = bx[0];
       intx8 A[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -258,20 +271,9 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
         const intx4 hi = *reinterpret_cast<const intx4*>(bw + lt * 2048 + a_hi);
         A[t] = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       }
-      const uint8_t* bt = b + 8 * wm * 2048;
-      const float* bx = bxs + 128 * wm + r16;
-      auto load_b = [&](int tt) {
-        const intx4 lo = *reinterpret_cast<const intx4*>(bt + tt * 2048 + sw_lo);
-        const intx4 hi = *reinterpret_cast<const intx4*>(bt + tt * 2048 + (sw_lo ^ 64));
-        return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      };
       // 32 MFMAs (token tile tt = idx/4, weight tile t = idx%4) in one software pipeline: token tile tt+1
       // is fetched from LDS while tile tt is multiplied, and the promotion of product idx-2
       // (acc += partial * scale, VALU) is issued behind MFMA idx
-      intx8 Bb[2];
-      float xb[2];
-      Bb[0] = load_b(0);
-      xb[0] = bx[0];
       floatx4 P[3];
       float psc[2][2];
 #pragma unroll
