@@ -26,6 +26,8 @@ def _ids(g, n, k, e_total, extra=None):
 CASES = [  # n, k, h, e_total, expert_start, e_local
     (1, 4, 256, 16, 0, 16), (64, 4, 1024, 16, 0, 16), (256, 8, 7168, 256, 0, 32), (256, 8, 512, 256, 64, 32),
     (100, 2, 131, 64, 32, 8), (700, 8, 256, 256, 0, 256), (4096, 8, 128, 256, 32, 32), (513, 16, 64, 896, 28, 28),
+    (200, 8, 128, 256, 0, 256),      # <= 2048 pairs, 256 local experts: the one-block kernel at its limit
+    (250, 8, 64, 600, 100, 300),     # <= 2048 pairs, more than 256 local experts: the four-wave one-launch kernel
 ]
 
 
