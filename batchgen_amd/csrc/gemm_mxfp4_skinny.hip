@@ -57,7 +57,9 @@ __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float scale) {
 // the four waves through an LDS ring filled by asynchronous global -> LDS loads.  A token tile is 16 rows x
 // 256 bytes per K-block; a load covers 4 rows: lane p = (row p>>4, LDS chunk p&15) fetches the row's 16-byte
 // chunk (p&15) ^ row, so that the MFMA operand reads (16 rows, same chunk) hit 16 different bank groups.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
+// KEEP: the group has more row chunks than this one, so its weights are loaded with the default cache
+// policy (the next chunk finds them in L2); otherwise as a non-temporal stream.
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP>
 __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it, const uint8_t* ring, uint32_t ring_lds) {
   constexpr int NT = 4;
   constexpr int kSlot = TT * 4096;
@@ -133,10 +135,10 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
-        s.A[t] = gload_x4_stream(wp[t] + (kb << 6));
+        s.A[t] = KEEP ? gload_x4(wp[t] + (kb << 6)) : gload_x4_stream(wp[t] + (kb << 6));
         s.S[t] = *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)(sp[t] + (kb << 2)));
       } else {
-        s.A[t] = gload_x4_stream(wp[t] + ((int64_t)kb << 10));
+        s.A[t] = KEEP ? gload_x4(wp[t] + ((int64_t)kb << 10)) : gload_x4_stream(wp[t] + ((int64_t)kb << 10));
         s.S[t] = *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)(sp[t] + (kb << 6)));
       }
     }
@@ -227,7 +229,8 @@ __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned v
     const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, vb);
     if (it.grp == BGMOE_ITEM_END) break;
     if (it.grp == BGMOE_ITEM_PAD) continue;
-    mxfp4_item<TT, NSTAGE, FUSED, LAYOUT>(g, it, s_ring, ring_lds);
+    if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true>(g, it, s_ring, ring_lds);
+    else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false>(g, it, s_ring, ring_lds);
     __syncthreads();                      // the token ring is reused by the next item
   }
 }
