@@ -31,8 +31,8 @@ METRIC = "MoE layer TFLOP/s (FP8 prefill) & HBM GB/s (decode), % roofline, 1xMI3
 # and profiles/fp8_prefill_c2_rocprof.md.  A configuration that was not measured reports null.
 MIB = 1024 * 1024
 MEASURED_TRAFFIC_BYTES = {
-    1: int((632.3 + 1.4) * MIB),      # fp8_skinny_kernel<2,3,fused,tile_major>, config 1
-    2: int((2269.4 + 82.1) * MIB),    # fp8_tiled_kernel<fused,tile_major>, config 2
+    1: int((630.5 + 1.4) * MIB),      # fp8_skinny_kernel<2,3,fused,tile_major>, config 1
+    2: int((3067.3 + 83.4) * MIB),    # fp8_tiled_kernel<fused,tile_major>, config 2
 }
 
 
