@@ -40,6 +40,7 @@ class Fp8Act(C.Structure):
 _SIGS = {
     "bgmoe_last_error": (C.c_char_p, []),
     "bgmoe_version": (i32, []),
+    "bgmoe_init": (i32, []),
     "bgmoe_prof_enable": (i32, [i32]),
     "bgmoe_prof_kernel_count": (i32, []),
     "bgmoe_prof_kernel_name": (C.c_char_p, [i32]),

@@ -361,9 +361,14 @@ static unsigned resident_blocks(K kernel, unsigned* cache) {
 }
 
 template <int TT, int NS, bool FUSED, int LAYOUT>
-static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
+static unsigned skinny_resident() {
   static unsigned resident = 0;
-  const unsigned cap = resident_blocks(fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>, &resident);
+  return resident_blocks(fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>, &resident);
+}
+
+template <int TT, int NS, bool FUSED, int LAYOUT>
+static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
+  const unsigned cap = skinny_resident<TT, NS, FUSED, LAYOUT>();
   const dim3 grid(vblocks < cap ? vblocks : cap), block(256);
   hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks);
 }
@@ -382,6 +387,15 @@ static void launch_variant(bool fused, int layout, int n, int groups, int64_t bo
     if (layout == BGMOE_W_TILE_MAJOR) launch_one<4, 2, false, BGMOE_W_TILE_MAJOR>(vb, g, st);
     else launch_one<4, 2, false, BGMOE_W_ROW_MAJOR>(vb, g, st);
   }
+}
+
+// first-launch queries of every variant, so that later launches are pure enqueues (graph capture)
+int bgmoe_internal_init_fp8_skinny() {
+  skinny_resident<2, 3, true, BGMOE_W_TILE_MAJOR>();
+  skinny_resident<2, 3, true, BGMOE_W_ROW_MAJOR>();
+  skinny_resident<4, 2, false, BGMOE_W_TILE_MAJOR>();
+  skinny_resident<4, 2, false, BGMOE_W_ROW_MAJOR>();
+  return BGMOE_OK;
 }
 
 // Rows per group up to which the weight-streaming kernel is used (each 32-row chunk of a group

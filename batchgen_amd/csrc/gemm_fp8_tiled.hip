@@ -384,6 +384,35 @@ int g_num_cu = 0;
 
 }  // namespace
 
+// device query and the dynamic-LDS opt-in of every variant, once
+int bgmoe_internal_init_fp8_tiled() {
+  static bool attr_set = false;
+  if (attr_set) return BGMOE_OK;
+  constexpr int kLds = NS * kSlotBytes;
+  hipDeviceProp_t prop;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+    bgmoe_set_error("fp8 tiled gemm: cannot query the device");
+    return BGMOE_ERR_HIP;
+  }
+  g_num_cu = prop.multiProcessorCount;
+  hipError_t e1 = hipSuccess;
+  const void* fns[4] = {reinterpret_cast<const void*>(&fp8_tiled_kernel<true, 0>),
+                        reinterpret_cast<const void*>(&fp8_tiled_kernel<false, 0>),
+                        reinterpret_cast<const void*>(&fp8_tiled_kernel<true, 1>),
+                        reinterpret_cast<const void*>(&fp8_tiled_kernel<false, 1>)};
+  for (const void* f : fns) {
+    hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+    if (e != hipSuccess) e1 = e;
+  }
+  if (e1 != hipSuccess) {
+    bgmoe_set_error("fp8 tiled gemm: cannot reserve %d bytes of LDS", kLds);
+    return BGMOE_ERR_HIP;
+  }
+  attr_set = true;
+  return BGMOE_OK;
+}
+
 int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                            const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                            uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
@@ -402,30 +431,8 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   g.seqlens = seqlens; g.cu = cu; g.groups = groups; g.n = n; g.k = k;
   g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.split = split;
   constexpr int kLds = NS * kSlotBytes;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipDeviceProp_t prop;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) {
-      bgmoe_set_error("fp8 tiled gemm: cannot query the device");
-      return BGMOE_ERR_HIP;
-    }
-    g_num_cu = prop.multiProcessorCount;
-    hipError_t e1 = hipSuccess;
-    const void* fns[4] = {reinterpret_cast<const void*>(&fp8_tiled_kernel<true, 0>),
-                          reinterpret_cast<const void*>(&fp8_tiled_kernel<false, 0>),
-                          reinterpret_cast<const void*>(&fp8_tiled_kernel<true, 1>),
-                          reinterpret_cast<const void*>(&fp8_tiled_kernel<false, 1>)};
-    for (const void* f : fns) {
-      hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-      if (e != hipSuccess) e1 = e;
-    }
-    if (e1 != hipSuccess) {
-      bgmoe_set_error("fp8 tiled gemm: cannot reserve %d bytes of LDS", kLds);
-      return BGMOE_ERR_HIP;
-    }
-    attr_set = true;
-  }
+  const int irc = bgmoe_internal_init_fp8_tiled();
+  if (irc != BGMOE_OK) return irc;
   // upper bound on work items from host shapes only
   const int ncols = w1 ? 128 : 256;
   const int64_t ntn = (n + ncols - 1) / ncols;

@@ -263,9 +263,10 @@ int check_w(const char* what, const bgmoe_mxfp4_weight* w) {
   return BGMOE_OK;
 }
 
+// blocks resident on the whole device at once, a multiple of 8 (queried once per kernel)
 template <int TT, int NS, bool FUSED, int LAYOUT>
-void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
-  static unsigned resident = 0;       // blocks resident on the whole device at once, a multiple of 8
+unsigned mx_resident() {
+  static unsigned resident = 0;
   if (resident == 0) {
     int per_cu = 0, dev = 0, cus = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>, 256, 0) != hipSuccess || per_cu < 1)
@@ -276,12 +277,20 @@ void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
     resident = (unsigned)(per_cu * cus) & ~7u;
     if (resident == 0) resident = 8;
   }
+  return resident;
+}
+
+template <int TT, int NS, bool FUSED, int LAYOUT>
+void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
+  const unsigned resident = mx_resident<TT, NS, FUSED, LAYOUT>();
   const dim3 grid(vblocks < resident ? vblocks : resident), block(256);
   hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks);
 }
 
+constexpr int kMxTT = 4;           // 64-row items: every group is streamed once per 64 rows
+
 int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
-  constexpr int TT = 4;            // 64-row items: every group is streamed once per 64 rows
+  constexpr int TT = kMxTT;
   const int ntile = fused ? 128 : 256;
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
   const unsigned vblocks = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 16 * TT);
@@ -311,6 +320,14 @@ int check_shape(const char* what, const uint16_t* x, const int32_t* seqlens, con
 }
 
 }  // namespace
+
+int bgmoe_internal_init_mxfp4() {
+  mx_resident<kMxTT, 3, true, 1>();
+  mx_resident<kMxTT, 3, true, 0>();
+  mx_resident<kMxTT, 3, false, 1>();
+  mx_resident<kMxTT, 3, false, 0>();
+  return BGMOE_OK;
+}
 
 extern "C" int bgmoe_mxfp4_grouped_gemm(const uint16_t* x, const bgmoe_mxfp4_weight* w, const int32_t* seqlens,
                                         const int32_t* cu_seqlens, int groups, int64_t m, int n, int k,

@@ -25,6 +25,13 @@ int bgmoe_check_launch(const char* what) {
 extern "C" const char* bgmoe_last_error(void) { return g_err; }
 extern "C" int bgmoe_version(void) { return 1; }
 
+extern "C" int bgmoe_init(void) {
+  int rc = bgmoe_internal_init_fp8_skinny();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_fp8_tiled();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_mxfp4();
+  return rc;
+}
+
 // ---- per-launch timing ------------------------------------------------------------
 // When enabled, every kernel launch of the library is bracketed by a pair of HIP
 // events on its own stream.  bgmoe_prof_collect() synchronises, sums the elapsed

@@ -76,6 +76,8 @@ class Fp8MoELayer:
                  shared_mode: str = "bf16_add", fold_shared: bool = True, weight_layout: str = "tile_major"):
         self.cfg = cfg
         dev = weights["gate_q"].device
+        with torch.cuda.device(dev):
+            check(lib().bgmoe_init())          # first-launch queries now, so that forward() is capturable at once
         if weight_layout not in ("tile_major", "row_major"):
             raise ValueError(f"unknown weight_layout {weight_layout!r}")
         self.layout = W_TILE_MAJOR if weight_layout == "tile_major" else W_ROW_MAJOR

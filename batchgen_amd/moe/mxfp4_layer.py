@@ -24,6 +24,8 @@ class Mxfp4MoELayer:
         self.cfg = cfg
         dev = weights["gate_p"].device
         self.device = dev
+        with torch.cuda.device(dev):
+            check(lib().bgmoe_init())
         mg = load_extension("batchgen_kernels.moe._C_marlin_grouped_gemm")
         self.w = {}
         for name in ("gate", "up", "down"):

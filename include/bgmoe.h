@@ -36,6 +36,13 @@ enum {
 const char* bgmoe_last_error(void);
 int bgmoe_version(void);
 
+/* Optional one-time set-up on the current device: the occupancy and device-property queries and the
+ * dynamic-LDS opt-in that the GEMM entry points otherwise perform at their first call.  After it (or after
+ * one eager call of each entry point) every call is a pure sequence of enqueues, which is what HIP-graph
+ * capture needs.  No counterpart in the reference (its TMA plans play this role,
+ * batchgen/moe/grouped_fp8_blockwise_moe.py, `fp8_blockwise_prepare_s1_s3_tma`). */
+int bgmoe_init(void);
+
 /* Per-launch timing for benchmarks.  bgmoe_prof_enable(1) brackets every kernel
  * launch with HIP events on its stream; bgmoe_prof_collect synchronises the
  * device and returns, per kernel id in [0, bgmoe_prof_kernel_count()), the total
