@@ -24,9 +24,11 @@
 // roofline (DRAM pages are opened once); ROW_MAJOR is supported for the op-level API and reads
 // 64-byte pieces of 16 rows per load.
 //
-// Scheduling: the grid is sized for every (group, n-tile) but block b serves the b-th ACTIVE item,
-// found with a ballot scan of seqlens, so the blocks that have work are consecutive block ids and
-// the hardware dispatcher spreads them evenly over the CUs whatever the pattern of empty groups.
+// Scheduling: a persistent grid (as many blocks as are resident at once) walks virtual block ids; virtual
+// block b is the b-th ACTIVE item, found with a ballot scan of seqlens, so empty groups and the host's
+// loose bound on the item count cost nothing and the work spreads evenly over the CUs.  Groups that are
+// streamed in several row chunks load their weights with the default cache policy (the next chunk,
+// placed on the same XCD, finds them in L2), single-chunk groups as a non-temporal stream.
 //
 // Algorithmic bytes per group: n*k weight bytes (+ n*k/16384*4 scale bytes)
 // per matrix; activations (rows*k) are re-read per block from L2.
