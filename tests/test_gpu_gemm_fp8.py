@@ -290,3 +290,39 @@ def test_kernel_choice_does_not_change_results_beyond_rounding(dev, limit, layou
     assert og.rel_frobenius(h.float().cpu().numpy()[live], href[live]) < 4e-3
     lv = torch.from_numpy(live).to(dev)
     assert torch.equal(hq[lv], hq2[lv]) and torch.equal(hs[:, lv], hs2[:, lv])
+
+
+@pytest.mark.parametrize("layout", ["row_major", "tile_major"])
+@pytest.mark.parametrize("n,k", [(128, 128), (256, 256), (640, 384)])
+def test_tiled_kernel_edge_shapes(dev, n, k, layout):
+    """The LDS-tiled kernel alone (row limit 0) on shapes at its edges: one and two K-steps, an output narrower
+    than its 256-column tile, groups of exactly one tile, one row more, one row, none, and two tiles."""
+    from batchgen_amd._lib import check, lib
+    counts = (256, 257, 1, 0, 512)
+    say("tiled edges", n, k, layout)
+    counts, cu, m, xq, xs, ws = _make(900 + n + k, counts, n, k, nmat=2)
+    (gq, gs), (uq, us) = ws
+    xq_d, xs_t, gq_d, gs_d = _dev(dev, xq, xs, gq, gs)
+    _, _, uq_d, us_d = _dev(dev, xq, xs, uq, us)
+    if layout == "tile_major":
+        gq_d, uq_d = gm().fp8_weight_repack(gq_d), gm().fp8_weight_repack(uq_d)
+    cnt_d, cu_d = torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev)
+    live = np.zeros(m, dtype=bool)
+    for e, c in enumerate(counts):
+        live[cu[e]:cu[e] + c] = True
+    check(lib().bgmoe_set_skinny_max_rows(0))
+    try:
+        out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+        gm().fp8_blockwise_grouped_gemm(xq_d, gq_d, cnt_d, cu_d, xs_t, gs_d, 16, out, weight_layout=layout)
+        h = torch.full((m, n), 5.0, dtype=torch.bfloat16, device=dev)
+        gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16, h, weight_layout=layout)
+    finally:
+        check(lib().bgmoe_set_skinny_max_rows(256))
+    ref = og.grouped_gemm_fp8(xq, xs, gq, gs, counts, cu, to_bf16=False)
+    o = out.float().cpu().numpy()
+    np.testing.assert_allclose(o[live], ref[live], rtol=2e-2, atol=5e-3)
+    assert np.all(o[~live] == 7.0)
+    up = og.grouped_gemm_fp8(xq, xs, uq, us, counts, cu, to_bf16=False)
+    href = oq.silu_f32(ref) * up
+    hh = h.float().cpu().numpy()
+    assert og.rel_frobenius(hh[live], href[live]) < 4e-3 and np.all(hh[~live] == 5.0)
