@@ -27,12 +27,14 @@ METRIC = "MoE layer TFLOP/s (FP8 prefill) & HBM GB/s (decode), % roofline, 1xMI3
 
 # HBM bytes per launch of each configuration's dominant kernel, measured with two `rocprofv3 --pmc` runs
 # (FETCH_SIZE, then WRITE_SIZE; each scaled by what the same counter reads for a plain 256 MiB copy kernel in
-# the same run: x2.000 and x1.000).  The summaries with the exact commands are profiles/fp8_decode_c1_rocprof.md
-# and profiles/fp8_prefill_c2_rocprof.md.  A configuration that was not measured reports null.
+# the same run: x2.000 and x1.000).  The summaries with the exact commands are under profiles/ (one file per
+# configuration).  A configuration that was not measured reports null.
 MIB = 1024 * 1024
 MEASURED_TRAFFIC_BYTES = {
     1: int((630.5 + 1.4) * MIB),      # fp8_skinny_kernel<2,3,fused,tile_major>, config 1
     2: int((3067.3 + 83.4) * MIB),    # fp8_tiled_kernel<fused,tile_major>, config 2
+    3: int((227.6 + 0.7) * MIB),      # mxfp4_skinny_kernel<4,3,fused,tile_major>, config 3
+    4: int((6054.0 + 154.9) * MIB),   # fp8_tiled_kernel<fused,tile_major>, config 4
 }
 
 
