@@ -23,6 +23,20 @@ __device__ __forceinline__ int bgmoe_split_limit(const int32_t* seqlens, int gro
   return tiles >= s.min_tiles ? s.small_rows : s.max_rows;
 }
 
+// Row chunks of all groups with lo < count <= hi (the number of items per n-tile).  Wave-uniform; every wave
+// runs it redundantly.
+__device__ __forceinline__ int bgmoe_total_chunks(const int32_t* seqlens, int groups, int lo, int hi, int chunk_rows) {
+  const int lane = threadIdx.x & 63;
+  int chunks = 0;
+  for (int g0 = lane; g0 < groups; g0 += 64) {
+    const int c = seqlens[g0];
+    chunks += (c > lo && c <= hi) ? (c + chunk_rows - 1) / chunk_rows : 0;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) chunks += __shfl_xor(chunks, off, BGMOE_WAVE);
+  return __builtin_amdgcn_readfirstlane(chunks);
+}
+
 // Work items of one launch: every group with lo < count <= hi contributes ceil(count / chunk_rows)
 // items (ascending group, ascending chunk).  Returns the group of item `item` and its chunk index,
 // or -1 when there are fewer items.  Wave-uniform; every wave of the block runs it redundantly.

@@ -59,9 +59,10 @@ __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float scale) {
 // chunk (p&15) ^ row, so that the MFMA operand reads (16 rows, same chunk) hit 16 different bank groups.
 // KEEP: the group has more row chunks than this one, so its weights are loaded with the default cache
 // policy (the next chunk finds them in L2); otherwise as a non-temporal stream.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP>
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP, int NT>
 __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it, const uint8_t* ring, uint32_t ring_lds) {
-  constexpr int NT = 4;
+  constexpr int NH = NT / 2;                      // fused: gate tiles (= up tiles) per wave
+  constexpr int NW = FUSED ? 16 * NH : 16 * NT;   // output columns per wave
   constexpr int kSlot = TT * 4096;
   const int grp = it.grp, cnt = it.cnt;
   const int64_t row0 = g.cu[grp];
@@ -72,7 +73,7 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
   const int kq = lane >> 4;
   const int K = g.k;
   const int KB = K >> 7;
-  const int n0 = it.ntile * (FUSED ? 128 : 256);
+  const int n0 = it.ntile * (4 * NW);
 
   const uint8_t* wb[2];
   const uint8_t* sb[2];
@@ -87,10 +88,10 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
   bool tv[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int nrow = FUSED ? n0 + 32 * wave + 16 * (t & 1) : n0 + 64 * wave + 16 * t;
+    const int nrow = FUSED ? n0 + NW * wave + 16 * (t % NH) : n0 + NW * wave + 16 * t;
     tv[t] = nrow < g.n;
     const int nr = min(nrow, g.n - 16);
-    const int mi = FUSED ? (t >> 1) : 0;
+    const int mi = FUSED ? (t / NH) : 0;
     if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
       wp[t] = wb[mi] + (int64_t)(nr + r16) * (K >> 1) + 16 * kq;
       sp[t] = sb[mi] + (int64_t)(nr + r16) * (K >> 5);
@@ -166,7 +167,7 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
   };
 
   // Same pipeline as the FP8 streaming kernel: tokens are requested before the weights of the same
-  // K-block, loads complete in issue order, so "at most the 8 weight loads of the youngest stage
+  // K-block, loads complete in issue order, so "at most the 2*NT weight loads of the youngest stage
   // outstanding" means the stage about to be computed has landed for this wave; the barrier extends
   // that to the other waves' token loads and frees the slot refilled next.
 #pragma unroll
@@ -178,7 +179,7 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
   for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
-      wait_vm<8>();
+      wait_vm<2 * NT>();
       block_barrier();
       issue_tokens(min(kb0 + s + NSTAGE - 1, KB - 1), (s + NSTAGE - 1) % NSTAGE);
       load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
@@ -197,14 +198,14 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
     if (16 * tt + r16 >= live) continue;
     if constexpr (FUSED) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NH; ++j) {
         float h[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) h[i] = silu_f32(acc[tt][j][i]) * acc[tt][j + 2][i];
+        for (int i = 0; i < 4; ++i) h[i] = silu_f32(acc[tt][j][i]) * acc[tt][j + NH][i];
         uint2 o;
         o.x = f32_to_bf16_bits(h[0]) | (f32_to_bf16_bits(h[1]) << 16);
         o.y = f32_to_bf16_bits(h[2]) | (f32_to_bf16_bits(h[3]) << 16);
-        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = o;
+        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * j + 4 * kq) = o;
       }
     } else {
 #pragma unroll
@@ -213,25 +214,43 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
         uint2 o;
         o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
         o.y = f32_to_bf16_bits(acc[tt][t][2]) | (f32_to_bf16_bits(acc[tt][t][3]) << 16);
-        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + 64 * wave + 16 * t + 4 * kq) = o;
+        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * t + 4 * kq) = o;
       }
     }
   }
 }
 
 // Persistent grid: block b works on virtual blocks b, b + gridDim.x, ... until the item list ends.
+// Item width is chosen per launch on the device: with 4 weight tiles per wave (128 fused / 256 plain output
+// columns per item) when that already gives every resident block an item, else with 2 tiles per wave --
+// fp4 weight stages are small, so with few items twice as many narrower ones keep more loads in flight.
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned vblocks) {
   __shared__ __align__(16) uint8_t s_ring[NSTAGE * TT * 4096];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
-  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
-  for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
-    const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, vb);
-    if (it.grp == BGMOE_ITEM_END) break;
-    if (it.grp == BGMOE_ITEM_PAD) continue;
-    if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true>(g, it, s_ring, ring_lds);
-    else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false>(g, it, s_ring, ring_lds);
-    __syncthreads();                      // the token ring is reused by the next item
+  const int wide_cols = FUSED ? 128 : 256;
+  const int ntiles_wide = (g.n + wide_cols - 1) / wide_cols;
+  const int chunks = bgmoe_total_chunks(g.seqlens, g.groups, g.lo, g.hi, 16 * TT);
+  const bool narrow = (int64_t)chunks * ((ntiles_wide + 7) & ~7) < (int64_t)gridDim.x;
+  if (narrow) {
+    const int ntiles = (g.n + wide_cols / 2 - 1) / (wide_cols / 2);
+    for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
+      const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, vb);
+      if (it.grp == BGMOE_ITEM_END) break;
+      if (it.grp == BGMOE_ITEM_PAD) continue;
+      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 2>(g, it, s_ring, ring_lds);
+      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 2>(g, it, s_ring, ring_lds);
+      __syncthreads();                    // the token ring is reused by the next item
+    }
+  } else {
+    for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
+      const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles_wide, vb);
+      if (it.grp == BGMOE_ITEM_END) break;
+      if (it.grp == BGMOE_ITEM_PAD) continue;
+      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 4>(g, it, s_ring, ring_lds);
+      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 4>(g, it, s_ring, ring_lds);
+      __syncthreads();
+    }
   }
 }
 
@@ -291,7 +310,7 @@ constexpr int kMxTT = 4;           // 64-row items: every group is streamed once
 
 int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
   constexpr int TT = kMxTT;
-  const int ntile = fused ? 128 : 256;
+  const int ntile = fused ? 64 : 128;      // the narrow item width bounds the virtual block count of both widths
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
   const unsigned vblocks = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 16 * TT);
   g.lo = 0; g.hi = 0x7fffffff;     // every group: more rows = more chunks (weights re-streamed)
