@@ -99,6 +99,17 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
   const int per_x = (int)((total + nx - 1) / nx);
   const int bstep = (gridDim.x + nx - 1 - xcd) / nx;   // blocks living on this XCD
   const int bidx = blockIdx.x / nx;
+  // Tail of the static walk: this XCD's items are dealt to its bstep blocks in rounds.  When the last round
+  // is at most half full, each of its items is split into two 128-token halves handled by different blocks
+  // (a half keeps one wave per SIMD busy and takes little more than half the time), so the kernel ends
+  // half a round earlier.
+  const int64_t first_x = (int64_t)xcd * per_x;
+  const int cnt_x = (int)max((int64_t)0, min((int64_t)per_x, total - first_x));
+  const int rounds_x = (cnt_x + bstep - 1) / bstep;
+  const int split_base = rounds_x > 0 ? (rounds_x - 1) * bstep : 0;
+  const int split_rem = cnt_x - split_base;
+  const bool split_tail = rounds_x > 0 && 2 * split_rem <= bstep;
+  const int walk_x = split_tail ? split_base + 2 * split_rem : cnt_x;      // virtual items of this XCD
 
   // ---- per-item state ----
   struct Meta { int cnt, m0, n0; int64_t row0; };
@@ -116,9 +127,13 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
 
   // item index of this block's walk -> (group, n-tile, m-tile) and its load sources
   auto prepare = [&](int64_t itx, Meta& mt) -> bool {
-    if (itx >= per_x) return false;
-    const int64_t item = (int64_t)xcd * per_x + itx;
-    if (item >= total) return false;
+    if (itx >= walk_x) return false;
+    int half = -1;                                         // -1: the whole 256-token tile
+    int64_t item = first_x + itx;
+    if (split_tail && itx >= split_base) {
+      item = first_x + split_base + ((itx - split_base) >> 1);
+      half = (int)((itx - split_base) & 1);
+    }
     int lo_g = 0, hi_g = g.groups - 1;
     while (lo_g < hi_g) {
       const int mid = (lo_g + hi_g + 1) >> 1;
@@ -134,9 +149,15 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
     const int r2 = (int)(rel - (int64_t)panel * kPanel * ntn);
     const int nt = r2 / pm;
     const int mtile = panel * kPanel + (r2 - nt * pm);
-    const int cnt = g.seqlens[grp];
+    int cnt = g.seqlens[grp];
     const int64_t row0 = g.cu[grp];
-    const int m0 = mtile * TM;
+    int m0 = mtile * TM;
+    if (half >= 0) {                                       // rows [m0 + 128*half, +128) of the tile
+      m0 += 128 * half;
+      if (m0 >= cnt) return false;                         // no live row in this half; a block has at most one
+                                                           // split item and it is its last, so it is done
+      cnt = min(cnt, m0 + 128);
+    }
     const int n0 = nt * ncols;
     mt.cnt = cnt; mt.m0 = m0; mt.n0 = n0; mt.row0 = row0;
 
