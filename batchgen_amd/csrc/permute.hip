@@ -67,34 +67,52 @@ __global__ __launch_bounds__(256) void perm_hist_kernel(PermArgs a) {
     a.chunk_hist[(int64_t)blockIdx.x * a.e_local + e] = hist[e];
 }
 
-// exclusive scan over chunks per expert (in place), then counts / cu_seqlens
+// exclusive scan over chunks per expert (in place), then counts / cu_seqlens.  One wave per expert (16 at a
+// time): lane = chunk, a shuffle scan per 64 chunks with a running carry.
 __global__ __launch_bounds__(1024) void perm_scan_kernel(PermArgs a) {
   __shared__ int32_t tot[kMaxLocal];
-  const int e = threadIdx.x;
-  if (e < a.e_local) {
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  for (int e = wave; e < a.e_local; e += 16) {
     int run = 0;
-    for (int c = 0; c < a.nchunks; ++c) {
+    for (int c0 = 0; c0 < a.nchunks; c0 += 64) {
+      const int c = c0 + lane;
       const int64_t o = (int64_t)c * a.e_local + e;
-      const int t = a.chunk_hist[o];
-      a.chunk_hist[o] = run;
-      run += t;
+      const int t = c < a.nchunks ? a.chunk_hist[o] : 0;
+      int inc = t;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(inc, off, BGMOE_WAVE);
+        if (lane >= off) inc += up;
+      }
+      if (c < a.nchunks) a.chunk_hist[o] = run + inc - t;
+      run += __shfl(inc, 63, BGMOE_WAVE);
     }
-    const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
-    tot[e] = cnt;
-    a.counts[e] = cnt;
-    if (a.counters) a.counters[e] = cnt;
+    if (lane == 0) {
+      const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
+      tot[e] = cnt;
+      a.counts[e] = cnt;
+      if (a.counters) a.counters[e] = cnt;
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0 && a.cu) {
-    int64_t off = 0;
-    for (int g = 0; g < a.e_local; ++g) {
-      a.cu[g] = (int32_t)off;
-      off += a.mtp > 0 ? (int64_t)a.mtp
-                       : (((int64_t)tot[g] + a.row_align - 1) & ~(int64_t)(a.row_align - 1));
+  if (wave == 0) {
+    int64_t base = 0;
+    for (int g0 = 0; g0 < a.e_local; g0 += 64) {
+      const int g = g0 + lane;
+      const int64_t span = g < a.e_local ? (a.mtp > 0 ? (int64_t)a.mtp
+                                                      : (((int64_t)tot[g] + a.row_align - 1) & ~(int64_t)(a.row_align - 1)))
+                                         : 0;
+      int64_t inc = span;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int64_t up = __shfl_up(inc, off, BGMOE_WAVE);
+        if (lane >= off) inc += up;
+      }
+      if (g < a.e_local && a.cu) a.cu[g] = (int32_t)(base + inc - span);
+      base += __shfl(inc, 63, BGMOE_WAVE);
     }
-    write_tail(a, off);
-  } else if (threadIdx.x == 0) {
-    write_tail(a, 0);
+    if (lane == 0) write_tail(a, a.cu ? base : 0);
   }
 }
 
