@@ -1,8 +1,8 @@
 // Sigmoid + bias-corrected top-k routers for gfx950: ONE wave64 per token.
 // A token's experts live in registers (expert id = i*64 + lane, VPL values per
-// lane); every arg-max round is a lane-local scan plus a 6-step butterfly with
-// the rule "larger value wins, equal values go to the lower expert id", which
-// gives a unique winner whatever the reduction tree.
+// lane); every arg-max round is a lane-local scan plus a 6-step DPP reduction
+// with the rule "larger value wins, equal values go to the lower expert id",
+// which gives a unique winner whatever the reduction tree.
 #include <math.h>
 
 #include "bgmoe_common.h"
@@ -28,29 +28,38 @@ __device__ __forceinline__ int dpp_i32(int v) {
   return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
 }
 constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+constexpr int kDppBcast15 = 0x142, kDppBcast31 = 0x143;
 
+// branch-free on purpose: three compares, two mask operations, two selects (a short-circuit `if` turns into
+// exec-mask juggling that costs more than the reduction itself)
 __device__ __forceinline__ void argmax_merge(float& v, int& idx, float ov, int oi) {
-  if (ov > v || (ov == v && oi < idx)) {
-    v = ov;
-    idx = oi;
-  }
+  const bool gt = ov > v;
+  const bool eq = ov == v;
+  const bool lower = oi < idx;
+  const bool take = gt | (eq & lower);
+  v = take ? ov : v;
+  idx = take ? oi : idx;
 }
 
 // "larger value wins, equal values go to the lower index": a total order, so any reduction network gives
-// the same winner.  Rows of 16 lanes reduce with DPP; the four row results are combined from scalars.
+// the same winner.  Rows of 16 lanes reduce with DPP butterflies (every lane of a row then holds the row's
+// result); row_bcast15 folds rows 0/2 into rows 1/3, row_bcast31 folds row 1 into row 3, and lane 63 holds
+// the wave's winner.  Rows left out by a row mask receive their own value, for which the merge is a no-op.
+template <int CTRL, int ROWS>
+__device__ __forceinline__ int dpp_rows_i32(int v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, ROWS, 0xf, false);
+}
 __device__ __forceinline__ void wave_argmax(float& v, int& idx) {
   argmax_merge(v, idx, dpp_f32<kDppXor1>(v), dpp_i32<kDppXor1>(idx));
   argmax_merge(v, idx, dpp_f32<kDppXor2>(v), dpp_i32<kDppXor2>(idx));
   argmax_merge(v, idx, dpp_f32<kDppHalfMirror>(v), dpp_i32<kDppHalfMirror>(idx));
   argmax_merge(v, idx, dpp_f32<kDppMirror>(v), dpp_i32<kDppMirror>(idx));
-  float rv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-  int ri = __builtin_amdgcn_readlane(idx, 0);
-#pragma unroll
-  for (int row = 1; row < 4; ++row)
-    argmax_merge(rv, ri, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16 * row)),
-                 __builtin_amdgcn_readlane(idx, 16 * row));
-  v = rv;
-  idx = ri;
+  argmax_merge(v, idx, __int_as_float(dpp_rows_i32<kDppBcast15, 0xa>(__float_as_int(v))),
+               dpp_rows_i32<kDppBcast15, 0xa>(idx));
+  argmax_merge(v, idx, __int_as_float(dpp_rows_i32<kDppBcast31, 0xc>(__float_as_int(v))),
+               dpp_rows_i32<kDppBcast31, 0xc>(idx));
+  v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+  idx = __builtin_amdgcn_readlane(idx, 63);
 }
 
 // two largest values (with multiplicity) of the union of two (m1 >= m2) pairs
@@ -166,6 +175,27 @@ __global__ __launch_bounds__(256) void router_kernel(RouterArgs a) {
         if ((ex0 >> 6) == i) g = t;
       }
       if (lane < a.n_group) gscore = g > -1e9f ? g : kNegInf;
+    } else if (epg % BGMOE_WAVE == 0) {
+      // a group is a run of epg/64 whole register slots: per-lane top-2 over the run, then a wave butterfly
+      const int spg = epg >> 6;
+      float m1 = -1e9f, m2 = -1e9f;
+#pragma unroll
+      for (int i = 0; i < VPL; ++i) {
+        if (i * BGMOE_WAVE < a.e) {
+          top2_merge(m1, m2, key[i] == kNegInf ? -1e9f : key[i], -1e9f);
+          if ((i + 1) % spg == 0) {
+            top2_merge(m1, m2, dpp_f32<kDppXor1>(m1), dpp_f32<kDppXor1>(m2));
+            top2_merge(m1, m2, dpp_f32<kDppXor2>(m1), dpp_f32<kDppXor2>(m2));
+            top2_merge(m1, m2, dpp_f32<kDppHalfMirror>(m1), dpp_f32<kDppHalfMirror>(m2));
+            top2_merge(m1, m2, dpp_f32<kDppMirror>(m1), dpp_f32<kDppMirror>(m2));
+            top2_merge(m1, m2, __shfl_xor(m1, 16, BGMOE_WAVE), __shfl_xor(m2, 16, BGMOE_WAVE));
+            top2_merge(m1, m2, __shfl_xor(m1, 32, BGMOE_WAVE), __shfl_xor(m2, 32, BGMOE_WAVE));
+            const float g = m1 + m2;
+            if (lane == i / spg) gscore = g > -1e9f ? g : kNegInf;
+            m1 = m2 = -1e9f;
+          }
+        }
+      }
     } else {
       float* s = s_lds + wave * a.e;
 #pragma unroll
@@ -234,7 +264,7 @@ __global__ __launch_bounds__(256) void router_kernel(RouterArgs a) {
           if (lane == owner) key[i] = kNegInf;
         }
       }
-      rv = __shfl(mine, owner, BGMOE_WAVE);
+      rv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), owner));   // owner is wave-uniform
     }
     total = total + rv;                        // route order, from 0.0f
     if (lane == r) {

@@ -26,6 +26,11 @@ GROUPED = [  # n, e, n_group, topk_group, top_k, rsf
     (37, 64, 4, 2, 2, 1.5),
     (19, 128, 8, 4, 6, 2.0),
     (5, 512, 8, 4, 8, 1.0),
+    (40, 96, 4, 2, 4, 1.0),      # 24 experts per group: not a power of two, the LDS scan
+    (20, 256, 1, 1, 8, 2.5),     # one group of 256: whole register slots per group
+    (9, 384, 2, 1, 4, 1.0),      # 192 per group
+    (12, 512, 2, 2, 8, 1.0),
+    (6, 1024, 4, 3, 16, 1.0),
 ]
 
 
