@@ -40,7 +40,7 @@ enum BgmoeKernelId {
   BGMOE_K_ACT_QUANT, BGMOE_K_COMBINE, BGMOE_K_COMPACT,
   BGMOE_K_S1_SKINNY16, BGMOE_K_S1_SKINNY64, BGMOE_K_S1_TILED,
   BGMOE_K_GEMM_SKINNY16, BGMOE_K_GEMM_SKINNY64, BGMOE_K_GEMM_TILED,
-  BGMOE_K_MXFP4_S1, BGMOE_K_MXFP4_GEMM, BGMOE_K_BF16_GEMM,
+  BGMOE_K_MXFP4_S1, BGMOE_K_MXFP4_GEMM, BGMOE_K_BF16_GEMM, BGMOE_K_ROUTER_GEMM, BGMOE_K_ROUTER_GEMM_REDUCE,
   BGMOE_K_COUNT
 };
 extern bool g_bgmoe_prof_on;
@@ -59,6 +59,10 @@ int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, 
                             const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                             uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
                             int64_t row_bound, int64_t group_bound, hipStream_t st);
+
+// router-GEMM logits as [*nplanes_out][n][e] fp32 planes for a consumer that adds them in plane order
+int bgmoe_internal_router_gemm_planes(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,
+                                      float* planes, size_t planes_bytes, int* nplanes_out, hipStream_t st);
 
 static inline hipStream_t bgmoe_stream(bgmoe_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 

@@ -72,6 +72,8 @@ __device__ __forceinline__ void top2_merge(float& m1, float& m2, float o1, float
 struct RouterArgs {
   const float* in;        // scores or logits, row stride `stride`
   int64_t stride;
+  int nsplit;             // > 0: `in` holds nsplit partial planes, plane_stride apart; the logit is their
+  int64_t plane_stride;   //      sum in plane order starting from 0.0f (the router GEMM's split-K output)
   const float* bias;
   int n, e, top_k;
   float rsf;
@@ -125,12 +127,42 @@ __global__ __launch_bounds__(256) void router_kernel(RouterArgs a) {
   const float* row = a.in + (int64_t)token * a.stride;
   float raw[VPL], key[VPL];
   const float floor_v = GROUPED ? -1e9f : -3.402823466e+38f;
+  float xin[VPL];
+  if (a.nsplit > 0) {
+    // split-K planes: logit = (((0 + p_0) + p_1) + ...); the VPL loads of a plane are in flight together
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) xin[i] = 0.0f;
+    constexpr int kBatch = VPL <= 4 ? 4 : 2;   // planes requested together
+    for (int sp = 0; sp < a.nsplit; sp += kBatch) {
+      float part[kBatch][VPL];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const float* prow = row + min(sp + b, a.nsplit - 1) * a.plane_stride;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+          const int ex = i * BGMOE_WAVE + lane;
+          part[b][i] = ex < a.e ? prow[ex] : 0.0f;
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b)
+        if (sp + b < a.nsplit) {
+#pragma unroll
+          for (int i = 0; i < VPL; ++i) xin[i] += part[b][i];
+        }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int ex = i * BGMOE_WAVE + lane;
+      xin[i] = ex < a.e ? row[ex] : 0.0f;
+    }
+  }
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int ex = i * BGMOE_WAVE + lane;
     if (ex < a.e) {
-      const float x = row[ex];
-      raw[i] = a.apply_sigmoid ? sigmoid_cr(x) : x;
+      raw[i] = a.apply_sigmoid ? sigmoid_cr(xin[i]) : xin[i];
       const float s = raw[i] + a.bias[ex];
       key[i] = s > floor_v ? s : kNegInf;     // NaN and <= floor are never candidates
     } else {
@@ -308,12 +340,7 @@ int launch_router(const RouterArgs& a, hipStream_t st) {
   return bgmoe_check_launch("router");
 }
 
-}  // namespace
-
-extern "C" int bgmoe_fused_gate(const float* scores, const float* bias, int n, int e, int n_group,
-                                int topk_group, int top_k, float routed_scaling_factor,
-                                int apply_sigmoid, int32_t* topk_ids, float* topk_weights,
-                                bgmoe_stream_t stream) {
+int check_fused_gate(int n, int e, int n_group, int topk_group, int top_k) {
   BGMOE_REQUIRE(n >= 0, "fused_gate: n < 0");
   BGMOE_REQUIRE(e >= 1 && e <= 1024, "fused_gate: n_routed_experts=%d outside [1,1024]", e);
   BGMOE_REQUIRE(n_group >= 1 && n_group <= 64, "fused_gate: n_group=%d outside [1,64]", n_group);
@@ -322,6 +349,28 @@ extern "C" int bgmoe_fused_gate(const float* scores, const float* bias, int n, i
   BGMOE_REQUIRE(topk_group >= 1 && topk_group <= n_group, "fused_gate: topk_group=%d outside [1,%d]",
                 topk_group, n_group);
   BGMOE_REQUIRE(top_k >= 1 && top_k <= 32 && top_k <= e, "fused_gate: unsupported top_k=%d", top_k);
+  return BGMOE_OK;
+}
+
+int check_gate_sigmoid_topk(int n, int e, int k, const int32_t* num_valid_tokens,
+                            const int64_t* rank_token_counts, int rows_per_rank) {
+  BGMOE_REQUIRE(n >= 0, "gate_sigmoid_topk: n < 0");
+  BGMOE_REQUIRE(e >= 1 && e <= 1024, "gate_sigmoid_topk: E=%d exceeds MAX_EXPERTS=1024", e);
+  BGMOE_REQUIRE(k == 2 || k == 4 || k == 8 || k == 16, "gate_sigmoid_topk: Unsupported k=%d. Supported: 2, 4, 8, 16", k);
+  BGMOE_REQUIRE(e >= k, "gate_sigmoid_topk: E=%d must be at least k=%d", e, k);
+  BGMOE_REQUIRE(!(num_valid_tokens && rank_token_counts),
+                "gate_sigmoid_topk: num_valid_tokens and rank_token_counts are mutually exclusive");
+  BGMOE_REQUIRE(!rank_token_counts || rows_per_rank > 0, "gate_sigmoid_topk: rows_per_rank must be positive");
+  return BGMOE_OK;
+}
+
+}  // namespace
+
+extern "C" int bgmoe_fused_gate(const float* scores, const float* bias, int n, int e, int n_group,
+                                int topk_group, int top_k, float routed_scaling_factor,
+                                int apply_sigmoid, int32_t* topk_ids, float* topk_weights,
+                                bgmoe_stream_t stream) {
+  if (int rc = check_fused_gate(n, e, n_group, topk_group, top_k)) return rc;
   if (n == 0) return BGMOE_OK;
   BGMOE_REQUIRE(scores && bias && topk_ids && topk_weights, "fused_gate: null pointer");
   RouterArgs a{};
@@ -338,14 +387,8 @@ extern "C" int bgmoe_gate_sigmoid_topk(const float* logits, int64_t logits_strid
                                        const int64_t* rank_token_counts, int rows_per_rank,
                                        uint16_t* latent_out, int latent_offset, int latent_size,
                                        bgmoe_stream_t stream) {
-  BGMOE_REQUIRE(n >= 0, "gate_sigmoid_topk: n < 0");
-  BGMOE_REQUIRE(e >= 1 && e <= 1024, "gate_sigmoid_topk: E=%d exceeds MAX_EXPERTS=1024", e);
-  BGMOE_REQUIRE(k == 2 || k == 4 || k == 8 || k == 16, "gate_sigmoid_topk: Unsupported k=%d. Supported: 2, 4, 8, 16", k);
-  BGMOE_REQUIRE(e >= k, "gate_sigmoid_topk: E=%d must be at least k=%d", e, k);
+  if (int rc = check_gate_sigmoid_topk(n, e, k, num_valid_tokens, rank_token_counts, rows_per_rank)) return rc;
   BGMOE_REQUIRE(logits_stride >= e, "gate_sigmoid_topk: row stride %lld < E=%d", (long long)logits_stride, e);
-  BGMOE_REQUIRE(!(num_valid_tokens && rank_token_counts),
-                "gate_sigmoid_topk: num_valid_tokens and rank_token_counts are mutually exclusive");
-  BGMOE_REQUIRE(!rank_token_counts || rows_per_rank > 0, "gate_sigmoid_topk: rows_per_rank must be positive");
   if (latent_out) {
     BGMOE_REQUIRE(latent_offset >= e, "gate_sigmoid_topk: latent_offset=%d must start at or after the %d router columns", latent_offset, e);
     BGMOE_REQUIRE((int64_t)latent_offset + latent_size <= logits_stride,
@@ -361,4 +404,37 @@ extern "C" int bgmoe_gate_sigmoid_topk(const float* logits, int64_t logits_strid
   a.rows_per_rank = rows_per_rank; a.latent_out = latent_out; a.latent_offset = latent_offset;
   a.latent_size = latent_size;
   return launch_router<false>(a, bgmoe_stream(stream));
+}
+
+// hidden -> logits -> routes without the logits round trip: the GEMM leaves its split-K planes in the
+// workspace and the router kernel adds them, in plane order, while it loads a token's row.
+extern "C" int bgmoe_router_gemm_gate(const uint16_t* hidden, const uint16_t* weight, const float* bias,
+                                      int n, int h, int e, int n_group, int topk_group, int top_k,
+                                      float routed_scaling_factor, int32_t* topk_ids, float* topk_weights,
+                                      const int64_t* rank_token_counts, int rows_per_rank, void* workspace,
+                                      size_t workspace_bytes, bgmoe_stream_t stream) {
+  const bool grouped = n_group > 0;
+  if (grouped) {
+    if (int rc = check_fused_gate(n, e, n_group, topk_group, top_k)) return rc;
+    BGMOE_REQUIRE(!rank_token_counts, "router_gemm_gate: the grouped router has no padding rows");
+  } else {
+    if (int rc = check_gate_sigmoid_topk(n, e, top_k, nullptr, rank_token_counts, rows_per_rank)) return rc;
+  }
+  if (n == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(hidden && weight && bias && topk_ids && topk_weights, "router_gemm_gate: null pointer");
+  hipStream_t st = bgmoe_stream(stream);
+  int nseg = 0;
+  if (int rc = bgmoe_internal_router_gemm_planes(hidden, weight, n, h, e, static_cast<float*>(workspace),
+                                                 workspace_bytes, &nseg, st))
+    return rc;
+  RouterArgs a{};
+  a.in = static_cast<const float*>(workspace); a.stride = e; a.nsplit = nseg; a.plane_stride = (int64_t)n * e;
+  a.bias = bias; a.n = n; a.e = e; a.top_k = top_k; a.rsf = routed_scaling_factor; a.apply_sigmoid = 1;
+  a.ids32 = topk_ids; a.w = topk_weights;
+  if (grouped) {
+    a.n_group = n_group; a.topk_group = topk_group;
+    return launch_router<true>(a, st);
+  }
+  a.rank_counts = rank_token_counts; a.rows_per_rank = rows_per_rank;
+  return launch_router<false>(a, st);
 }

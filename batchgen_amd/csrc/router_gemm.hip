@@ -1,0 +1,378 @@
+// Router GEMM for gfx950: logits[n,e] (fp32) = hidden[n,h] (bf16) x router_weight[e,h]^T (bf16).
+//
+// The value of one logit is a fixed function of its token row and its expert row -- whatever the
+// number of tokens in the call, the tile the token falls in, or the launch shape picked for the size:
+//   * K is cut into segments of 512 elements; a segment's partial sum is one chain of
+//     v_mfma_f32_16x16x32_bf16 over its 64-element steps in ascending order (fp32 accumulation inside);
+//   * the logit is (((0 + p_0) + p_1) + ...) over the segments in ascending order, in fp32.
+// Two launch shapes compute exactly that: "whole" (a block walks every segment and folds as it goes; used
+// when the token count alone fills the chip) and "split" (one block per segment writes its partial plane to
+// the workspace; a reduce pass -- or the router kernel itself -- adds the planes in order).
+//
+// Operands go from global memory straight to MFMA registers: lane (r, q) of a 16-row tile reads the 32
+// contiguous bytes [q*16, q*16+16) elements of row r in a 64-element step, so the four lanes of a row fetch
+// one whole 128-byte line; tokens and experts use the same K permutation, which a dot product does not see.
+// Experts are the MFMA's row operand, so a lane ends up with 4 consecutive experts of one token: 16-byte
+// stores.
+#include "bgmoe_common.h"
+
+namespace {
+
+constexpr int kSeg = 512;        // K elements per segment
+constexpr int kStep = 64;        // K elements per load step (two MFMAs)
+constexpr int kStepsPerSeg = kSeg / kStep;
+
+struct RouterGemmArgs {
+  const uint16_t* x;             // [n,h] bf16
+  const uint16_t* w;             // [e,h] bf16
+  float* out;                    // whole: logits [n,e]; split: planes [nseg][n][e]
+  const int64_t* rank_counts;    // whole only: rows past a rank's count get 0
+  int bucket, world;
+  int n, h, e, nseg;
+  int ttiles, eblocks;           // split: token tiles and expert blocks of the launch (1-D grid decode)
+};
+
+template <int TM, int NE>
+struct Stage {
+  intx4 a[NE][2];                // NE expert tiles x two 16-byte halves of the lane's 32 bytes
+  intx4 b[TM][2];                // TM token tiles
+};
+
+__device__ __forceinline__ bool row_is_padding(const RouterGemmArgs& a, int row) {
+  if (!a.rank_counts) return false;
+  const int rank = row / a.bucket;
+  if (rank >= a.world) return true;
+  return (int64_t)(row - rank * a.bucket) >= a.rank_counts[rank];
+}
+
+// A block is WAVES waves; a wave owns NE 16-expert tiles x TM 16-token tiles, the block WAVES*16*NE experts.
+template <int TM, int NE, int DEPTH, bool SPLIT, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void router_gemm_kernel(RouterGemmArgs a) {
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int r = lane & 15, q = lane >> 4;
+  // Split shape: a unit = (K segment, expert block); all token tiles of a unit run on ONE XCD (hardware
+  // deals consecutive block ids round-robin over the 8 XCDs), so an XCD's L2 fetches only its units'
+  // slices of the weights and of the tokens instead of every XCD fetching everything.
+  int bx = blockIdx.x, by = blockIdx.y, seg_lo = 0;
+  if constexpr (SPLIT) {
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int ul = j / a.ttiles;
+    const int unit = ul * 8 + xcd;
+    if (unit >= a.nseg * a.eblocks) return;
+    bx = j - ul * a.ttiles;
+    seg_lo = unit / a.eblocks;
+    by = unit - seg_lo * a.eblocks;
+  }
+  const int t0 = bx * (16 * TM);
+  const int e0 = (by * WAVES + wave) * (16 * NE);
+  if (e0 >= a.e) return;         // whole wave; the kernel uses no block-level barrier
+
+  // rows past the end are clamped for the loads and never stored
+  const uint8_t* wp[NE];
+  const uint8_t* xp[TM];
+#pragma unroll
+  for (int tn = 0; tn < NE; ++tn) {
+    const int er = min(e0 + tn * 16 + r, a.e - 1);
+    wp[tn] = reinterpret_cast<const uint8_t*>(a.w) + ((int64_t)er * a.h + q * 16) * 2;
+  }
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int tr = min(t0 + tm * 16 + r, a.n - 1);
+    xp[tm] = reinterpret_cast<const uint8_t*>(a.x) + ((int64_t)tr * a.h + q * 16) * 2;
+  }
+
+  const int seg_hi = SPLIT ? seg_lo + 1 : a.nseg;
+  const int k_lo = seg_lo * kSeg;
+  const int k_hi = min(seg_hi * kSeg, a.h);
+  const int full = (k_hi - k_lo) / kStep;          // whole 64-element steps (uniform)
+  const int tail = (k_hi - k_lo) - full * kStep;   // 0, or a multiple of 8 below 64
+
+  floatx4 acc[TM][NE], tot[TM][NE];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < NE; ++tn) {
+      acc[tm][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+      tot[tm][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+
+  auto load = [&](Stage<TM, NE>& s, int step) {
+    const int64_t off = (int64_t)(k_lo + step * kStep) * 2;
+#pragma unroll
+    for (int tn = 0; tn < NE; ++tn) {
+      s.a[tn][0] = gload_x4(wp[tn] + off);
+      s.a[tn][1] = gload_x4(wp[tn] + off + 16);
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      s.b[tm][0] = gload_x4(xp[tm] + off);
+      s.b[tm][1] = gload_x4(xp[tm] + off + 16);
+    }
+  };
+  auto compute = [&](const Stage<TM, NE>& s) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < NE; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, s.a[tn][j]),
+                                                                __builtin_bit_cast(bf16x8, s.b[tm][j]),
+                                                                acc[tm][tn], 0, 0, 0);
+  };
+  auto fold = [&]() {            // end of a segment
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < NE; ++tn) {
+        tot[tm][tn] += acc[tm][tn];
+        acc[tm][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+  };
+
+  Stage<TM, NE> ring[DEPTH];
+  if (SPLIT && full == kStepsPerSeg) {
+    // a whole segment (all but possibly the last): every load is unconditional, so the compiler keeps
+    // DEPTH steps in flight and waits for exactly the step it is about to use
+    // (the scheduling barriers keep the compiler from sinking the prefetches down to their uses, which
+    // it otherwise does to save registers -- and which leaves one step in flight instead of DEPTH)
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) load(ring[d], d);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int step = 0; step < kStepsPerSeg; ++step) {
+      compute(ring[step % DEPTH]);
+      if (step + DEPTH < kStepsPerSeg) load(ring[step % DEPTH], step + DEPTH);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (d < full) load(ring[d], d);
+    __builtin_amdgcn_sched_barrier(0);
+    int base = 0;
+    if constexpr (!SPLIT) {
+      // steady state, one segment per trip: every step and every prefetch is in range, so nothing is
+      // conditional and the waits are exact; the guarded loop below finishes the last steps
+      static_assert(kStepsPerSeg % DEPTH == 0, "ring slots must line up with segment starts");
+      for (; base + kStepsPerSeg + DEPTH <= full; base += kStepsPerSeg) {
+#pragma unroll
+        for (int step = 0; step < kStepsPerSeg; ++step) {
+          compute(ring[step % DEPTH]);
+          load(ring[step % DEPTH], base + step + DEPTH);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        fold();
+      }
+    }
+    for (int s = base; s < full; s += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int step = s + d;
+        if (step < full) {
+          compute(ring[d]);
+          if (step + DEPTH < full) load(ring[d], step + DEPTH);
+          if constexpr (!SPLIT)
+            if ((step & (kStepsPerSeg - 1)) == kStepsPerSeg - 1) fold();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  if (tail) {
+    // the last, partial step of the last segment: 16-byte pieces past the end of K count as zeros
+    Stage<TM, NE> s;
+    const int kbase = k_lo + full * kStep + q * 16;
+    const int64_t off = (int64_t)(k_lo + full * kStep) * 2;
+    const intx4 zero = intx4{0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const bool live = kbase + j * 8 < k_hi;
+#pragma unroll
+      for (int tn = 0; tn < NE; ++tn) s.a[tn][j] = live ? gload_x4(wp[tn] + off + j * 16) : zero;
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) s.b[tm][j] = live ? gload_x4(xp[tm] + off + j * 16) : zero;
+    }
+    compute(s);
+  }
+  // a segment still open (the split shape's only segment, or a last one shorter than 512): fold it
+  if (SPLIT || tail || (full & (kStepsPerSeg - 1)) != 0) fold();
+
+  float* plane = a.out + (SPLIT ? (int64_t)seg_lo * a.n * a.e : 0);
+  const bool vec = (a.e & 3) == 0;
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int token = t0 + tm * 16 + r;
+    if (token >= a.n) continue;
+    bool pad = false;
+    if constexpr (!SPLIT) pad = row_is_padding(a, token);
+#pragma unroll
+    for (int tn = 0; tn < NE; ++tn) {
+      const int ex = e0 + tn * 16 + q * 4;
+      floatx4 v = pad ? floatx4{0.f, 0.f, 0.f, 0.f} : tot[tm][tn];
+      float* dst = plane + (int64_t)token * a.e + ex;
+      if (vec) {
+        if (ex < a.e) *reinterpret_cast<floatx4*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (ex + i < a.e) dst[i] = v[i];
+      }
+    }
+  }
+}
+
+// logits = (((0 + p_0) + p_1) + ...) over the planes; rows past a rank's count get 0
+__global__ __launch_bounds__(256) void router_gemm_reduce_kernel(RouterGemmArgs a, const float* planes) {
+  const int64_t total = (int64_t)a.n * a.e;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int row = (int)(i / a.e);
+  float v = 0.0f;
+  if (!row_is_padding(a, row))
+    for (int s = 0; s < a.nseg; ++s) v += planes[(int64_t)s * total + i];
+  a.out[i] = v;
+}
+
+int g_plan_tm = -1, g_plan_split = -1;
+
+struct Plan { int tm; int ne; int waves; bool split; };
+
+// Launch shape from the sizes alone (results do not depend on it).
+// A CU sustains only ~35-60 GB/s of load requests whatever hits in cache, so what matters for few tokens
+// is (a) every CU busy and (b) few requested bytes per CU: one-wave blocks with the largest wave tile
+// (64 tokens x 64 experts: 128 rows requested per 4096 outputs), one K segment each.
+Plan make_plan(int n, int h, int e) {
+  const int nseg = (h + kSeg - 1) / kSeg;
+  const int64_t ey4 = (e + 255) / 256;
+  Plan p;
+  p.ne = 4;
+  p.waves = 4;
+  // split-K while the partial planes stay small next to the operands (<= 64 MiB) and the whole-K shape
+  // would leave CUs idle or starved
+  const bool planes_small = (int64_t)n * e * nseg <= (int64_t)16 << 20;
+  if (nseg == 1 || !planes_small || ((int64_t)(n + 63) / 64) * ey4 >= 192) {
+    p.split = false;
+    p.tm = n > 2048 ? 4 : n > 512 ? 2 : 1;
+  } else {
+    p.split = true;
+    p.waves = 1;
+    p.tm = n > 32 ? 4 : n > 16 ? 2 : 1;
+  }
+  if (g_plan_tm == 1 || g_plan_tm == 2 || g_plan_tm == 4) p.tm = g_plan_tm;
+  if (g_plan_split == 0) { p.split = false; p.waves = 4; }
+  if (g_plan_split == 1) { p.split = true; p.waves = 4; }
+  if (g_plan_split == 2) { p.split = true; p.waves = 1; }
+  return p;
+}
+
+template <bool SPLIT>
+void launch_gemm(const RouterGemmArgs& a0, const Plan& p, hipStream_t st) {
+  RouterGemmArgs a = a0;
+  const dim3 block(64 * p.waves);
+  a.ttiles = (a.n + 16 * p.tm - 1) / (16 * p.tm);
+  a.eblocks = (a.e + 16 * p.ne * p.waves - 1) / (16 * p.ne * p.waves);
+  dim3 grid(a.ttiles, a.eblocks, 1);
+  if (SPLIT) grid = dim3((unsigned)(8 * ((a.nseg * a.eblocks + 7) / 8) * a.ttiles), 1, 1);
+  if (p.waves == 1) {
+    if (p.tm == 4) hipLaunchKernelGGL((router_gemm_kernel<4, 4, 4, SPLIT, 1>), grid, block, 0, st, a);
+    else if (p.tm == 2) hipLaunchKernelGGL((router_gemm_kernel<2, 4, 4, SPLIT, 1>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((router_gemm_kernel<1, 4, 4, SPLIT, 1>), grid, block, 0, st, a);
+  } else {
+    if (p.tm == 4) hipLaunchKernelGGL((router_gemm_kernel<4, 4, 2, SPLIT, 4>), grid, block, 0, st, a);
+    else if (p.tm == 2) hipLaunchKernelGGL((router_gemm_kernel<2, 4, 4, SPLIT, 4>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((router_gemm_kernel<1, 4, 4, SPLIT, 4>), grid, block, 0, st, a);
+  }
+}
+
+int check_shapes(int n, int h, int e) {
+  BGMOE_REQUIRE(n >= 0 && h >= 8 && e >= 1, "router_gemm: bad sizes n=%d h=%d e=%d", n, h, e);
+  BGMOE_REQUIRE(h % 8 == 0, "router_gemm: hidden size %d must be a multiple of 8 (16-byte row pieces)", h);
+  return BGMOE_OK;
+}
+
+}  // namespace
+
+extern "C" int bgmoe_set_router_gemm_plan(int token_tiles, int split) {
+  BGMOE_REQUIRE(token_tiles == -1 || token_tiles == 1 || token_tiles == 2 || token_tiles == 4,
+                "set_router_gemm_plan: token_tiles must be -1, 1, 2 or 4");
+  BGMOE_REQUIRE(split >= -1 && split <= 2, "set_router_gemm_plan: split must be -1, 0, 1 or 2");
+  g_plan_tm = token_tiles;
+  g_plan_split = split;
+  return BGMOE_OK;
+}
+
+extern "C" size_t bgmoe_router_gemm_workspace_bytes(int n, int h, int e) {
+  if (n <= 0 || h <= 0 || e <= 0) return 0;
+  const Plan p = make_plan(n, h, e);
+  const int nseg = (h + kSeg - 1) / kSeg;
+  return (size_t)(p.split ? nseg : 1) * (size_t)n * (size_t)e * sizeof(float);
+}
+
+// For the fused router: the logits as planes to be added in order, [*nplanes_out][n][e] fp32 -- the split-K
+// planes, or one plane of finished logits when the whole-K shape is the one for these sizes.
+int bgmoe_internal_router_gemm_planes(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,
+                                      float* planes, size_t planes_bytes, int* nplanes_out, hipStream_t st) {
+  if (int rc = check_shapes(n, h, e)) return rc;
+  RouterGemmArgs a{};
+  a.x = hidden; a.w = weight; a.out = planes; a.n = n; a.h = h; a.e = e;
+  a.nseg = (h + kSeg - 1) / kSeg;
+  const Plan p = make_plan(n, h, e);
+  *nplanes_out = p.split ? a.nseg : 1;
+  if (n == 0) return BGMOE_OK;
+  if (planes_bytes < bgmoe_router_gemm_workspace_bytes(n, h, e) || !planes) {
+    bgmoe_set_error("router_gemm: workspace of %zu bytes is smaller than the %zu needed", planes_bytes,
+                    bgmoe_router_gemm_workspace_bytes(n, h, e));
+    return BGMOE_ERR_WORKSPACE;
+  }
+  BgmoeProf prof(BGMOE_K_ROUTER_GEMM, st);
+  if (p.split) launch_gemm<true>(a, p, st);
+  else launch_gemm<false>(a, p, st);
+  return bgmoe_check_launch("router_gemm");
+}
+
+extern "C" int bgmoe_router_gemm(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,
+                                 const int64_t* rank_token_counts, int bucket_size, int world_size,
+                                 float* logits, void* workspace, size_t workspace_bytes,
+                                 bgmoe_stream_t stream) {
+  if (int rc = check_shapes(n, h, e)) return rc;
+  if (rank_token_counts) {
+    BGMOE_REQUIRE(world_size > 0, "router_gemm: world_size must be positive when rank_token_counts is provided");
+    BGMOE_REQUIRE(bucket_size > 0, "router_gemm: bucket_size must be positive when rank_token_counts is provided");
+  }
+  if (n == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(hidden && weight && logits, "router_gemm: null pointer");
+  hipStream_t st = bgmoe_stream(stream);
+  RouterGemmArgs a{};
+  a.x = hidden; a.w = weight; a.n = n; a.h = h; a.e = e;
+  a.rank_counts = rank_token_counts; a.bucket = bucket_size; a.world = world_size;
+  a.nseg = (h + kSeg - 1) / kSeg;
+  Plan p = make_plan(n, h, e);
+  // without a workspace the whole-K shape is the only one possible (slower for few tokens, same bits)
+  if (p.split && (!workspace || workspace_bytes < bgmoe_router_gemm_workspace_bytes(n, h, e))) {
+    BGMOE_REQUIRE(g_plan_split < 1, "router_gemm: the split shape was forced but the workspace is too small");
+    p.split = false;
+    p.waves = 4;
+  }
+  if (!p.split) {
+    a.out = logits;
+    BgmoeProf prof(BGMOE_K_ROUTER_GEMM, st);
+    launch_gemm<false>(a, p, st);
+    return bgmoe_check_launch("router_gemm");
+  }
+  {
+    RouterGemmArgs g = a;
+    g.out = static_cast<float*>(workspace);
+    g.rank_counts = nullptr;
+    BgmoeProf prof(BGMOE_K_ROUTER_GEMM, st);
+    launch_gemm<true>(g, p, st);
+    if (int rc = bgmoe_check_launch("router_gemm")) return rc;
+  }
+  a.out = logits;
+  const int64_t total = (int64_t)n * e;
+  BgmoeProf prof(BGMOE_K_ROUTER_GEMM_REDUCE, st);
+  hipLaunchKernelGGL(router_gemm_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a,
+                     static_cast<const float*>(workspace));
+  return bgmoe_check_launch("router_gemm_reduce");
+}

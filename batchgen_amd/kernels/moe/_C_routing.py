@@ -1,9 +1,11 @@
 """gfx950 implementation of the reference extension ``batchgen_kernels.moe._C_routing``
 (bindings: batchgen_kernels/src/moe/routing/routing_extension.cc:12-105).
 
-Exports gate_sigmoid_topk, gate_sigmoid_topk_warp, dispatch_count_gather,
-reduce_weighted_scatter.  The softmax router, the router GEMM and the bias
-epilogue of that extension are not part of this build.
+Exports gate_sigmoid_topk, gate_sigmoid_topk_warp, glm5_router_gemm,
+dispatch_count_gather, reduce_weighted_scatter, and router_gemm_gate (GEMM +
+top-k without the logits round trip; no counterpart in the reference).  The
+softmax router and the bias epilogue of that extension are not part of this
+build.
 """
 from __future__ import annotations
 
@@ -11,7 +13,7 @@ import torch
 
 from ..._lib import check, lib, ptr, stream
 from .. import _checks as ck
-from .._workspace import dispatch_workspace
+from .._workspace import dispatch_workspace, router_gemm_workspace
 
 
 def _padding(n, logits, num_valid_tokens, rank_token_counts, rows_per_rank):
@@ -97,6 +99,97 @@ def gate_sigmoid_topk_warp(router_logits, e_score_correction, k, routed_scaling_
         ck.fail("gate_sigmoid_topk_warp needs caller-owned topk_indices and topk_weights")
     return _gate(router_logits, e_score_correction, k, routed_scaling_factor, topk_indices, topk_weights,
                  num_valid_tokens, None, None, rank_token_counts, rows_per_rank, 256, True)
+
+
+def _router_gemm_operands(hidden_states, router_weight):
+    """The reference binding's operand checks (glm5_router_gemm.cu:116-133)."""
+    ck.gpu(hidden_states, "hidden_states")
+    ck.gpu(router_weight, "router_weight")
+    if hidden_states.dtype != torch.bfloat16:
+        ck.fail("hidden_states must be BF16")
+    if router_weight.dtype != torch.bfloat16:
+        ck.fail("router_weight must be BF16")
+    if hidden_states.dim() != 2:
+        ck.fail("hidden_states must be rank-2 [N, H]")
+    if router_weight.dim() != 2:
+        ck.fail("router_weight must be rank-2 [E, H]")
+    ck.contiguous(hidden_states, "hidden_states")
+    ck.contiguous(router_weight, "router_weight")
+    ck.same_device(hidden_states, router_weight, "router_weight")
+    n, h = hidden_states.shape
+    e = router_weight.size(0)
+    if router_weight.size(1) != h:
+        ck.fail(f"router_weight hidden dim mismatch: got {router_weight.size(1)}, expected {h}")
+    return n, h, e
+
+
+def glm5_router_gemm(hidden_states, router_weight, rank_token_counts, output, bucket_size, world_size):
+    """logits [N,E] fp32 = hidden [N,H] bf16 x router_weight [E,H]^T bf16 with a per-row summation order
+    that does not depend on N; rows past their rank's count are zeroed (glm5_router_gemm.cu:107-180)."""
+    n, h, e = _router_gemm_operands(hidden_states, router_weight)
+    dev = hidden_states.device
+    if output is None or output.numel() == 0:
+        output = torch.empty((n, e), dtype=torch.float32, device=dev)
+    ck.gpu(output, "output")
+    if output.dtype != torch.float32:
+        ck.fail("output must be FP32")
+    if output.dim() != 2:
+        ck.fail("output must be rank-2 [N, E]")
+    if tuple(output.shape) != (n, e):
+        ck.fail(f"output shape mismatch: got [{output.size(0)}, {output.size(1)}], expected [{n}, {e}]")
+    ck.contiguous(output, "output")
+    rc = None
+    if rank_token_counts is not None and rank_token_counts.numel() > 0:
+        ck.gpu(rank_token_counts, "rank_token_counts")
+        if rank_token_counts.dtype != torch.int64:
+            ck.fail("rank_token_counts must be int64")
+        ck.contiguous(rank_token_counts, "rank_token_counts")
+        if int(world_size) <= 0:
+            ck.fail("world_size must be positive when rank_token_counts is provided")
+        if rank_token_counts.numel() < int(world_size):
+            ck.fail(f"rank_token_counts length {rank_token_counts.numel()} is smaller than world_size {world_size}")
+        if int(bucket_size) <= 0:
+            ck.fail("bucket_size must be positive when rank_token_counts is provided")
+        rc = rank_token_counts
+    if n == 0 or e == 0:
+        return output
+    ws, ws_bytes = router_gemm_workspace(dev, n, h, e)
+    with torch.cuda.device(dev):
+        check(lib().bgmoe_router_gemm(ptr(hidden_states), ptr(router_weight), n, h, e, ptr(rc), int(bucket_size),
+                                      int(world_size), ptr(output), ptr(ws), ws_bytes, stream()))
+    return output
+
+
+def router_gemm_gate(hidden_states, router_weight, e_score_correction, k, routed_scaling_factor, topk_indices,
+                     topk_weights, n_group=0, topk_group=0, rank_token_counts=None, rows_per_rank=None):
+    """glm5_router_gemm followed by gate_sigmoid_topk (n_group == 0) or by the grouped gate on sigmoided
+    logits (n_group >= 1), identical ids and weights, without writing the logits: the GEMM's split-K
+    planes are summed by the router kernel.  Returns [topk_indices, topk_weights]."""
+    n, h, e = _router_gemm_operands(hidden_states, router_weight)
+    dev = hidden_states.device
+    ck.cuda_tensor(hidden_states, e_score_correction, torch.float32, "e_score_correction")
+    if e_score_correction.numel() != e:
+        ck.fail("e_score_correction must have E elements")
+    if topk_indices is None or topk_indices.numel() == 0:
+        topk_indices = torch.empty((n, k), dtype=torch.int32, device=dev)
+    if topk_weights is None or topk_weights.numel() == 0:
+        topk_weights = torch.empty((n, k), dtype=torch.float32, device=dev)
+    ck.cuda_tensor(hidden_states, topk_indices, torch.int32, "topk_indices")
+    ck.cuda_tensor(hidden_states, topk_weights, torch.float32, "topk_weights")
+    if tuple(topk_indices.shape) != (n, k) or tuple(topk_weights.shape) != (n, k):
+        ck.fail(f"topk_indices / topk_weights must be contiguous [{n}, {k}] tensors")
+    rc, rpr = None, 0
+    if rank_token_counts is not None and rank_token_counts.numel() > 0:
+        _, rc, rpr = _padding(n, hidden_states, None, rank_token_counts, rows_per_rank)
+    if n == 0:
+        return [topk_indices, topk_weights]
+    ws, ws_bytes = router_gemm_workspace(dev, n, h, e)
+    with torch.cuda.device(dev):
+        check(lib().bgmoe_router_gemm_gate(ptr(hidden_states), ptr(router_weight), ptr(e_score_correction), n, h,
+                                           e, int(n_group), int(topk_group), int(k), float(routed_scaling_factor),
+                                           ptr(topk_indices), ptr(topk_weights), ptr(rc), rpr, ptr(ws), ws_bytes,
+                                           stream()))
+    return [topk_indices, topk_weights]
 
 
 def dispatch_count_gather(x, topk_indices, expert_start, num_local_experts, expert_counts, expert_offsets,

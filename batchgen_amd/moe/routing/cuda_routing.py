@@ -93,6 +93,55 @@ def gate_sigmoid_topk_warp_cuda(router_logits, e_score_correction, k=8, routed_s
     return r[0], r[1]
 
 
+def glm5_router_gemm_cuda(hidden_states, router_weight, router_logits=None, rank_token_counts=None,
+                          bucket_size=0, world_size=1):
+    """``hidden_states @ router_weight.T`` as fp32 logits from bf16 operands, graph-safe: with
+    ``rank_token_counts`` the rows are rank-major ``[world_size, bucket_size]`` and padding rows are zeroed
+    on the device (cuda_routing.py:318-366)."""
+    if hidden_states.dtype != torch.bfloat16:
+        hidden_states = hidden_states.to(torch.bfloat16)
+    if router_weight.dtype != torch.bfloat16:
+        router_weight = router_weight.to(torch.bfloat16)
+    if not hidden_states.is_contiguous():
+        hidden_states = hidden_states.contiguous()
+    if not router_weight.is_contiguous():
+        router_weight = router_weight.contiguous()
+    n = hidden_states.shape[0]
+    e = router_weight.shape[0]
+    dev = hidden_states.device
+    if router_logits is None:
+        router_logits = torch.empty(n, e, dtype=torch.float32, device=dev)
+    elif not router_logits.is_contiguous():
+        raise ValueError("router_logits must be contiguous")
+    if rank_token_counts is None:
+        rank_token_counts = torch.empty(0, dtype=torch.int64, device=dev)
+    else:
+        if rank_token_counts.dtype != torch.int64:
+            rank_token_counts = rank_token_counts.to(torch.int64)
+        if not rank_token_counts.is_contiguous():
+            rank_token_counts = rank_token_counts.contiguous()
+    return _get_ext().glm5_router_gemm(hidden_states, router_weight, rank_token_counts, router_logits,
+                                       int(bucket_size), int(world_size))
+
+
+def router_gemm_gate_sigmoid_topk(hidden_states, router_weight, e_score_correction, k=8,
+                                  routed_scaling_factor=2.5, topk_indices=None, topk_weights=None,
+                                  n_group=0, topk_group=0, rank_token_counts=None, rows_per_rank=None):
+    """``glm5_router_gemm_cuda`` then ``gate_sigmoid_topk_cuda`` (or, with ``n_group >= 1``, the
+    group-limited gate on the sigmoided logits) as one call that never writes the logits; ids and weights
+    are identical to the two-call sequence.  No counterpart in the reference, which runs the two ops back
+    to back (batchgen/models/glm5/model.py:1119-1161)."""
+    _check_gate_padding_args(None, rank_token_counts, rows_per_rank)
+    if hidden_states.dtype != torch.bfloat16:
+        hidden_states = hidden_states.to(torch.bfloat16)
+    if router_weight.dtype != torch.bfloat16:
+        router_weight = router_weight.to(torch.bfloat16)
+    r = _get_ext().router_gemm_gate(hidden_states.contiguous(), router_weight.contiguous(), e_score_correction,
+                                    k, routed_scaling_factor, topk_indices, topk_weights, n_group, topk_group,
+                                    rank_token_counts, rows_per_rank)
+    return r[0], r[1]
+
+
 def dispatch_count_gather_cuda(x, topk_indices, expert_start, num_local_experts, expert_counts=None,
                                expert_offsets=None, expert_counters=None, dispatched_x=None, topk_pos=None,
                                num_valid_tokens=-1):

@@ -86,6 +86,45 @@ int bgmoe_gate_sigmoid_topk(const float* logits, int64_t logits_stride, const fl
                             int rows_per_rank, uint16_t* latent_out, int latent_offset,
                             int latent_size, bgmoe_stream_t stream);
 
+/* ------------------------------------------------------------ router GEMM */
+
+/* Bytes of device workspace for the router GEMM at these sizes: the split-K planes
+ * (ceil(h/512) * n * e * 4) when few tokens make split-K the launch shape, else n * e * 4.  Without it
+ * bgmoe_router_gemm still works (one block walks all of K: the same bits, slower when n is small);
+ * bgmoe_router_gemm_gate needs it. */
+size_t bgmoe_router_gemm_workspace_bytes(int n, int h, int e);
+
+/* logits[n,e] fp32 = hidden[n,h] bf16 x router_weight[e,h]^T bf16, fp32 accumulation.
+ * Replaces `glm5_router_gemm_cuda` (batchgen/moe/routing/cuda_routing.py:318-366,
+ * batchgen_kernels/src/moe/routing/glm5_router_gemm.cu:35-180) and its contract: a row's logits do not
+ * depend on the number of rows in the call (batchgen/models/glm5/model.py:1135-1140), and with
+ * rank_token_counts (device int64 [world_size]) row i is padding when
+ * i % bucket_size >= rank_token_counts[i / bucket_size]: its logits are 0 and its hidden row may hold
+ * anything (NaN included).  The summation order differs from the reference kernel's (MFMA chains per
+ * 512-element K segment, segments added in order), so the fp32 bits differ in the last places; the order
+ * is fixed, so results are reproducible and equal between this entry point and
+ * bgmoe_router_gemm_gate.  h % 8 == 0.  rank_token_counts may be NULL. */
+int bgmoe_router_gemm(const uint16_t* hidden, const uint16_t* router_weight, int n, int h, int e,
+                      const int64_t* rank_token_counts, int bucket_size, int world_size, float* logits,
+                      void* workspace, size_t workspace_bytes, bgmoe_stream_t stream);
+
+/* Router GEMM + top-k in two launches without materialising the logits: identical ids and weights to
+ * bgmoe_router_gemm followed by bgmoe_fused_gate(apply_sigmoid=1) (n_group >= 1) or by
+ * bgmoe_gate_sigmoid_topk (n_group == 0; rank_token_counts / rows_per_rank as there).  The reference
+ * runs the GEMM and the gate as separate ops (batchgen/models/glm5/model.py:1119-1161); fusing them is
+ * this build's choice.  workspace: bgmoe_router_gemm_workspace_bytes(n,h,e). */
+int bgmoe_router_gemm_gate(const uint16_t* hidden, const uint16_t* router_weight, const float* bias,
+                           int n, int h, int e, int n_group, int topk_group, int top_k,
+                           float routed_scaling_factor, int32_t* topk_ids, float* topk_weights,
+                           const int64_t* rank_token_counts, int rows_per_rank, void* workspace,
+                           size_t workspace_bytes, bgmoe_stream_t stream);
+
+/* Tuning/test knob (no reference counterpart): force the router GEMM's launch shape.  token_tiles in
+ * {1,2,4} = 16-token tiles per wave; split 0 = one block walks all of K, 1 = one block per 512-element
+ * K segment, 2 = the same with one-wave blocks (the shape for few tokens); -1 = choose from the sizes.
+ * Results do not depend on it, bit for bit. */
+int bgmoe_set_router_gemm_plan(int token_tiles, int split);
+
 /* --------------------------------------------------------- FP8 act quant */
 
 /* Per-row, per-128 e4m3fn quantisation of plain rows:
