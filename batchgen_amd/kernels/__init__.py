@@ -20,6 +20,7 @@ AVAILABLE = (
     "moe._C_fp8_blockwise_ops",
     "moe._C_fp8_blockwise_gemm",
     "moe._C_marlin_grouped_gemm",
+    "attention._C_add_rmsnorm_fp8_quant",
 )
 
 

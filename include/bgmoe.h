@@ -125,6 +125,31 @@ int bgmoe_router_gemm_gate(const uint16_t* hidden, const uint16_t* router_weight
  * Results do not depend on it, bit for bit. */
 int bgmoe_set_router_gemm_plan(int token_tiles, int split);
 
+/* ------------------------------------------- producer: add + RMSNorm + FP8 */
+
+/* residual += hidden (bf16, in place); normed = RMSNorm(residual) * weight (bf16); and, when quant_out is
+ * not NULL, the per-token 128-block e4m3fn cast of `normed` in the same pass, so that the MoE layer's FP8
+ * activation never makes a second trip through memory.
+ * Replaces `cuda_add_rmsnorm_fp8_quant` (batchgen_kernels/attention/add_rmsnorm_fp8_quant.py:33-83,
+ * batchgen_kernels/src/attention/csrc/add_rmsnorm_fp8_quant.cu:242-541) with its thread partition and
+ * reduction tree (8 columns per thread, fma chain, 32-lane trees), its gates and its contract: `normed`
+ * and `residual` equal the unfused add+RMSNorm, and (quant_out, quant_scale) equal the standalone 1-D
+ * quantiser applied to the bf16 `normed` (batchgen_kernels/triton/fp8_quantize.py:252-331: amax floored
+ * at 2^-16, scale = max(amax/448, 1e-12)), bit for bit -- which for blocks with amax >= 2^-16 is also
+ * bgmoe_act_quant_rows(normed).  The CUDA kernel's rsqrtf and div.full.f32 are approximate instructions;
+ * here both are correctly rounded, so `normed` can differ from the CUDA bytes in the last bf16 place.
+ * h: a multiple of 128 up to 8192 (the reference is compiled for 6144 only).  Scale element (r,kb) at
+ * quant_scale[r*scale_row_stride + kb*scale_kb_stride]: (h/128, 1) is the contiguous form,
+ * (1, align4(rows)) the MN-major one.  Gates (device int32 scalars / bf16 [rows], any may be NULL):
+ * rows >= *norm_num_valid_tokens are not touched by the norm; rows >= *quant_num_valid_tokens get bytes 0
+ * and scales 1e-12; row_valid_mask[r] == 0 drops hidden row r from the sum (a predicate: NaN rows are
+ * safe).  norm_num_valid_tokens must be the same pointer as quant_num_valid_tokens when quantising. */
+int bgmoe_add_rmsnorm_fp8_quant(uint16_t* residual, const uint16_t* hidden, const uint16_t* weight,
+                                int64_t rows, int h, float eps, uint16_t* normed_out, uint8_t* quant_out,
+                                float* quant_scale, int64_t scale_row_stride, int64_t scale_kb_stride,
+                                const int32_t* norm_num_valid_tokens, const int32_t* quant_num_valid_tokens,
+                                const uint16_t* row_valid_mask, bgmoe_stream_t stream);
+
 /* --------------------------------------------------------- FP8 act quant */
 
 /* Per-row, per-128 e4m3fn quantisation of plain rows:

@@ -71,7 +71,11 @@ def act_quant(x, form: str = "C"):
         amax = np.fmax(amax, F32(2.0 ** -16))
         s = np.fmax(amax * INV448, EPS)
         q = xb / s[:, :, None]
-        q = np.where(np.isfinite(q), q, F32(0.0))
+        # clamp first, then |q| < 1e30 else 0 (fp8_quantize.py:321-325): with min/max that drop a NaN
+        # operand the guard never fires (NaN and +-inf have become +-448 by then)
+        with np.errstate(invalid="ignore"):
+            q = np.fmax(np.fmin(q.astype(F32), F32(448.0)), F32(-448.0))
+        q = np.where(np.abs(q) < F32(1e30), q, F32(0.0))
     elif form == "B":
         s = np.fmax(amax, EPS) / F32(448.0)
         q = xb * (F32(1.0) / s)[:, :, None]
