@@ -224,6 +224,40 @@ __global__ __launch_bounds__(256) void scatter_quant_kernel(QuantArgs a, int ste
   }
 }
 
+// Permute rows that are ALREADY quantised (a producer upstream wrote the bytes and scales): a token's bytes
+// and scales are copied to every row it is routed to and to its identity row.  One wave per (token, 1024
+// bytes = 8 scale blocks); source scale (t,kb) at xs[t*xs_row + kb*xs_kb].
+__global__ __launch_bounds__(256) void scatter_fp8_kernel(const uint8_t* xq, const float* xs, int64_t xs_row,
+                                                          int64_t xs_kb, QuantArgs a, int steps, int extra_rows) {
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int k = a.k;
+  const int64_t njobs = a.jobs * steps;               // a.jobs = tokens here
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  for (int64_t job = (int64_t)blockIdx.x * 4 + wave; job < njobs; job += stride) {
+    const int64_t tok = job / steps;
+    const int step = (int)(job - tok * steps);
+    const int c0 = step * 1024 + lane * 16;
+    const bool in = c0 < k;
+    const int kb = step * 8 + lane;                    // lanes 0..7 carry the step's scales
+    const bool has_scale = lane < 8 && kb * 128 < k;
+    uint4 bytes = make_uint4(0u, 0u, 0u, 0u);
+    float sc = 0.0f;
+    if (in) bytes = *reinterpret_cast<const uint4*>(xq + tok * (int64_t)k + c0);
+    if (has_scale) sc = xs[tok * xs_row + (int64_t)kb * xs_kb];
+    const int ndst = a.topk + (tok < extra_rows ? 1 : 0);
+    int64_t mine = -1;
+    if (lane < a.topk) mine = a.topk_pos[tok * a.topk + lane];
+    else if (lane == a.topk && tok < extra_rows) mine = a.extra_start + tok;
+    for (int j = 0; j < ndst; ++j) {
+      const int64_t dst = __shfl(mine, j, BGMOE_WAVE);
+      if (dst < 0) continue;
+      if (in) *reinterpret_cast<uint4*>(a.y + dst * (int64_t)k + c0) = bytes;
+      if (has_scale) a.scale[dst * a.srow + (int64_t)kb * a.skb] = sc;
+    }
+  }
+}
+
 template <int MODE>
 int launch(const QuantArgs& a, hipStream_t st) {
   if (a.jobs <= 0 || a.k <= 0) return BGMOE_OK;
@@ -331,4 +365,34 @@ extern "C" int bgmoe_scatter_quant(const uint16_t* x, const int32_t* topk_pos, i
   BGMOE_REQUIRE(x && y && scale && topk_pos, "scatter_quant: null pointer");
   return bgmoe_internal_scatter_quant(x, topk_pos, n, k, h, y, scale, scale_row_stride, scale_kb_stride, 0, 0,
                                       bgmoe_stream(stream));
+}
+
+int bgmoe_internal_scatter_fp8(const uint8_t* xq, const float* xs, int64_t xs_row, int64_t xs_kb,
+                               const int32_t* topk_pos, int n, int k, int h, uint8_t* y, float* scale,
+                               int64_t srow, int64_t skb, int extra_rows, int64_t extra_start, hipStream_t st) {
+  BGMOE_REQUIRE(h % 16 == 0 && (uintptr_t)xq % 16 == 0 && (uintptr_t)y % 16 == 0,
+                "scatter_fp8_rows: h must be a multiple of 16 and the byte buffers 16-byte aligned");
+  BGMOE_REQUIRE(k < 64 && extra_rows <= n, "scatter_fp8_rows: top_k must be below 64");
+  if (n <= 0 || h <= 0) return BGMOE_OK;
+  QuantArgs a{};
+  a.y = y; a.scale = scale; a.jobs = n; a.k = h; a.srow = srow; a.skb = skb;
+  a.topk_pos = topk_pos; a.topk = k; a.extra_start = extra_start;
+  const int steps = (h + 1023) / 1024;
+  int64_t blocks = ((int64_t)n * steps + 3) / 4;
+  if (blocks > 65536) blocks = 65536;
+  BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
+  hipLaunchKernelGGL(scatter_fp8_kernel, dim3((unsigned)blocks), dim3(256), 0, st, xq, xs, xs_row, xs_kb, a, steps,
+                     extra_rows);
+  return bgmoe_check_launch("scatter_fp8_rows");
+}
+
+extern "C" int bgmoe_scatter_fp8_rows(const uint8_t* xq, const float* xs, int64_t xs_row_stride,
+                                      int64_t xs_kb_stride, const int32_t* topk_pos, int n, int k, int h,
+                                      uint8_t* y, float* scale, int64_t scale_row_stride,
+                                      int64_t scale_kb_stride, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n >= 0 && k > 0 && h >= 0, "scatter_fp8_rows: bad size");
+  if (n == 0 || h == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(xq && xs && y && scale && topk_pos, "scatter_fp8_rows: null pointer");
+  return bgmoe_internal_scatter_fp8(xq, xs, xs_row_stride, xs_kb_stride, topk_pos, n, k, h, y, scale,
+                                    scale_row_stride, scale_kb_stride, 0, 0, bgmoe_stream(stream));
 }

@@ -34,6 +34,10 @@ int bgmoe_internal_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int
                                  float* scale, int64_t srow, int64_t skb, int extra_rows, int64_t extra_start,
                                  hipStream_t st);
 
+int bgmoe_internal_scatter_fp8(const uint8_t* xq, const float* xs, int64_t xs_row, int64_t xs_kb,
+                               const int32_t* topk_pos, int n, int k, int h, uint8_t* y, float* scale,
+                               int64_t srow, int64_t skb, int extra_rows, int64_t extra_start, hipStream_t st);
+
 // ---- optional per-launch timing (off by default; see bgmoe_prof_enable) -----------
 enum BgmoeKernelId {
   BGMOE_K_ROUTER = 0, BGMOE_K_PERM_HIST, BGMOE_K_PERM_SCAN, BGMOE_K_PERM_RANK, BGMOE_K_GATHER_ROWS,

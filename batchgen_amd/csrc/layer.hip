@@ -24,7 +24,13 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
                 (long long)L->cap_rows, (long long)need_rows);
   BGMOE_REQUIRE(L->cap_rows + n <= 2147483647LL, "moe_fp8_layer_forward: row space exceeds int32");
   if (n == 0) return BGMOE_OK;
-  BGMOE_REQUIRE(L->x && L->logits && L->bias && L->out, "moe_fp8_layer_forward: null input/output");
+  const bool pre_quant = L->x_fp8 != nullptr;
+  const bool own_logits = L->logits == nullptr;
+  BGMOE_REQUIRE(L->bias && L->out, "moe_fp8_layer_forward: null input/output");
+  BGMOE_REQUIRE(pre_quant ? L->x_scale != nullptr : L->x != nullptr,
+                "moe_fp8_layer_forward: needs x, or x_fp8 together with x_scale");
+  BGMOE_REQUIRE(!own_logits || (L->router_weight && (L->router_hidden || L->x)),
+                "moe_fp8_layer_forward: without logits the layer needs router_weight and bf16 hidden states");
   BGMOE_REQUIRE(L->topk_ids && L->topk_weights && L->expert_counts && L->cu_seqlens && L->topk_pos &&
                 L->xq && L->xs && L->hq && L->hs && L->y, "moe_fp8_layer_forward: null buffer");
   const bool shared = L->has_shared != 0;
@@ -36,13 +42,20 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
   hipStream_t st = bgmoe_stream(stream);
   int rc;
 
-  // 1. router
-  if (L->n_group > 1)
+  // 1. router (from logits, or from the hidden states through the router GEMM)
+  if (own_logits) {
+    const bool grouped = L->n_group > 1;
+    rc = bgmoe_router_gemm_gate(L->router_hidden ? L->router_hidden : L->x, L->router_weight, L->bias, n, h,
+                                L->e_total, grouped ? L->n_group : 0, grouped ? L->topk_group : 0, k,
+                                L->routed_scaling_factor, L->topk_ids, L->topk_weights, nullptr, 0,
+                                L->router_workspace, L->router_workspace_bytes, stream);
+  } else if (L->n_group > 1) {
     rc = bgmoe_fused_gate(L->logits, L->bias, n, L->e_total, L->n_group, L->topk_group, k,
                           L->routed_scaling_factor, 1, L->topk_ids, L->topk_weights, stream);
-  else
+  } else {
     rc = bgmoe_gate_sigmoid_topk(L->logits, L->e_total, L->bias, n, L->e_total, k, L->routed_scaling_factor,
                                  L->topk_ids, 0, L->topk_weights, nullptr, nullptr, 0, nullptr, 0, 0, stream);
+  }
   if (rc != BGMOE_OK) return rc;
 
   // 2. stable counting sort -> counts, cu_seqlens (+ the shared expert as one more group), topk_pos
@@ -54,8 +67,12 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
 
   // 3. quantise while scattering; the shared expert's rows are the tokens themselves
   const int hb = h / 128, ib = inter / 128;
-  rc = bgmoe_internal_scatter_quant(L->x, L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0,
-                                    L->cap_rows, st);
+  if (pre_quant)
+    rc = bgmoe_internal_scatter_fp8(L->x_fp8, L->x_scale, L->x_scale_row_stride, L->x_scale_kb_stride,
+                                    L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0, L->cap_rows, st);
+  else
+    rc = bgmoe_internal_scatter_quant(L->x, L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0,
+                                      L->cap_rows, st);
   if (rc != BGMOE_OK) return rc;
 
   // 4/5. gate_up + SwiGLU + requant, then down

@@ -36,6 +36,8 @@ class LayerStruct(C.Structure):
         ("topk_ids", vp), ("topk_weights", vp), ("expert_counts", vp), ("cu_seqlens", vp), ("topk_pos", vp),
         ("xq", vp), ("xs", vp), ("hq", vp), ("hs", vp), ("shq", vp), ("shs", vp), ("y", vp),
         ("workspace", vp), ("workspace_bytes", sz), ("out", vp),
+        ("x_fp8", vp), ("x_scale", vp), ("x_scale_row_stride", i64), ("x_scale_kb_stride", i64),
+        ("router_weight", vp), ("router_hidden", vp), ("router_workspace", vp), ("router_workspace_bytes", sz),
     ]
 
 
@@ -73,7 +75,8 @@ class Fp8MoELayer:
     """
 
     def __init__(self, cfg: MoEConfig, weights, shared, bias: torch.Tensor, max_tokens_in: Optional[int] = None,
-                 shared_mode: str = "bf16_add", fold_shared: bool = True, weight_layout: str = "tile_major"):
+                 shared_mode: str = "bf16_add", fold_shared: bool = True, weight_layout: str = "tile_major",
+                 router_weight: Optional[torch.Tensor] = None):
         self.cfg = cfg
         dev = weights["gate_q"].device
         with torch.cuda.device(dev):
@@ -150,23 +153,62 @@ class Fp8MoELayer:
         L.xq, L.xs, L.hq, L.hs, L.y = ptr(self.xq), ptr(self.xs), ptr(self.hq), ptr(self.hs), ptr(self.y)
         L.workspace, L.workspace_bytes = ptr(self.workspace), self.workspace.numel()
         L.out = ptr(self.out)
+        self.router_weight = None
+        if router_weight is not None:
+            # the layer then routes from the hidden states: router GEMM + gate, no logits tensor
+            if router_weight.dtype != torch.bfloat16 or tuple(router_weight.shape) != (cfg.n_experts, h):
+                raise RuntimeError(f"router_weight must be BF16 [{cfg.n_experts}, {h}]")
+            self.router_weight = router_weight.contiguous()
+            rb = int(lib().bgmoe_router_gemm_workspace_bytes(n, h, cfg.n_experts))
+            self.router_workspace = torch.empty(max(rb, 16), dtype=e8, device=dev)
+            L.router_weight = ptr(self.router_weight)
+            L.router_workspace, L.router_workspace_bytes = ptr(self.router_workspace), self.router_workspace.numel()
         self._L = L
         self._fn = lib().bgmoe_moe_fp8_layer_forward
 
-    def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
+    def forward(self, hidden_states: torch.Tensor, router_logits: Optional[torch.Tensor] = None,
+                x_fp8: Optional[torch.Tensor] = None, x_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``router_logits=None`` routes from ``hidden_states`` through the layer's ``router_weight``.
+        ``x_fp8``/``x_scale`` (``[N,H]`` e4m3fn or uint8, ``[N,H/128]`` fp32 of any strides) are the tokens
+        already quantised by the producer upstream (``cuda_add_rmsnorm_fp8_quant``); both or neither, as in
+        the reference's hand-down (batchgen/models/glm/glm5/wrappers.py:416-447)."""
         cfg = self.cfg
         if hidden_states.dtype != torch.bfloat16 or hidden_states.dim() != 2 or hidden_states.size(1) != cfg.hidden:
             raise RuntimeError(f"hidden_states must be BF16 [N, {cfg.hidden}]")
         n = hidden_states.size(0)
         if n > self.n_max:
             raise RuntimeError(f"{n} tokens exceed the {self.n_max} this layer's buffers were sized for")
-        if router_logits.dtype != torch.float32 or tuple(router_logits.shape) != (n, cfg.n_experts):
-            raise RuntimeError(f"router_logits must be FP32 [{n}, {cfg.n_experts}]")
-        if not (hidden_states.is_contiguous() and router_logits.is_contiguous()):
-            raise RuntimeError("hidden_states and router_logits must be contiguous")
+        if not hidden_states.is_contiguous():
+            raise RuntimeError("hidden_states must be contiguous")
         L = self._L
+        if router_logits is None:
+            if self.router_weight is None:
+                raise RuntimeError("router_logits=None needs a layer built with router_weight")
+            L.logits = None
+        else:
+            if router_logits.dtype != torch.float32 or tuple(router_logits.shape) != (n, cfg.n_experts):
+                raise RuntimeError(f"router_logits must be FP32 [{n}, {cfg.n_experts}]")
+            if not router_logits.is_contiguous():
+                raise RuntimeError("router_logits must be contiguous")
+            L.logits = ptr(router_logits)
+        if (x_fp8 is None) != (x_scale is None):
+            raise RuntimeError("x_fp8 and x_scale must be given together; got "
+                               f"{'x_scale' if x_fp8 is None else 'x_fp8'} alone")
+        if x_fp8 is not None:
+            blocks = cfg.hidden // 128
+            if x_fp8.dtype not in (torch.float8_e4m3fn, torch.uint8) or tuple(x_fp8.shape) != (n, cfg.hidden):
+                raise RuntimeError(f"x_fp8 must be float8_e4m3fn ({n}, {cfg.hidden}), got {x_fp8.dtype} "
+                                   f"{tuple(x_fp8.shape)}")
+            if not x_fp8.is_contiguous():
+                raise RuntimeError("x_fp8 must be contiguous")
+            if x_scale.dtype != torch.float32 or tuple(x_scale.shape) != (n, blocks):
+                raise RuntimeError(f"x_scale must be fp32 ({n}, {blocks}), got {x_scale.dtype} {tuple(x_scale.shape)}")
+            L.x_fp8, L.x_scale = ptr(x_fp8), ptr(x_scale)
+            L.x_scale_row_stride, L.x_scale_kb_stride = x_scale.stride(0), x_scale.stride(1)
+        else:
+            L.x_fp8 = L.x_scale = None
         L.n = n
-        L.x, L.logits = ptr(hidden_states), ptr(router_logits)
+        L.x = ptr(hidden_states)
         check(self._fn(C.byref(L), stream()))
         return self.out[:n]
 

@@ -233,6 +233,14 @@ int bgmoe_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k
                         uint8_t* y, float* scale, int64_t scale_row_stride,
                         int64_t scale_kb_stride, bgmoe_stream_t stream);
 
+/* The same permutation for tokens that arrive ALREADY quantised (bgmoe_add_rmsnorm_fp8_quant upstream):
+ * bytes xq [n,h] and scales (t,kb) at xs[t*xs_row_stride + kb*xs_kb_stride] are copied to every row the
+ * token is routed to.  Replaces the hand-down of `x_fp8`/`x_scale` into the expert chain
+ * (batchgen/models/glm/glm5/wrappers.py:409-447).  h % 16 == 0, k < 64. */
+int bgmoe_scatter_fp8_rows(const uint8_t* xq, const float* xs, int64_t xs_row_stride, int64_t xs_kb_stride,
+                           const int32_t* topk_pos, int n, int k, int h, uint8_t* y, float* scale,
+                           int64_t scale_row_stride, int64_t scale_kb_stride, bgmoe_stream_t stream);
+
 /* out[t] = bf16(sum_k float(y[pos[t,k]])*w[t,k]), k ascending, pos<0 skipped.
  * Replaces `reduce_weighted_scatter` (dispatch_scatter_3d.cu:365-395, 527-556;
  * batchgen_kernels/src/moe/routing/reduce_weighted_scatter.cu:26-131).
@@ -427,6 +435,19 @@ typedef struct bgmoe_moe_fp8_layer {
   void* workspace;            /* bgmoe_dispatch_workspace_bytes(n*top_k, e_local) */
   size_t workspace_bytes;
   uint16_t* out;              /* [n,h] bf16            */
+  /* Optional upstream fusions; all NULL/0 = the plain layer above.
+   * x_fp8/x_scale: the tokens already quantised (bgmoe_add_rmsnorm_fp8_quant): step 3 copies them instead
+   * of quantising x (x may then be NULL).  Scale (t,kb) at x_scale[t*x_scale_row_stride + kb*x_scale_kb_stride].
+   * router_weight: bf16 [e_total,h]; with logits == NULL the layer computes them itself from
+   * router_hidden (bf16 [n,h]; NULL = x) with bgmoe_router_gemm_gate, and needs router_workspace of
+   * bgmoe_router_gemm_workspace_bytes(n,h,e_total) bytes. */
+  const uint8_t* x_fp8;
+  const float* x_scale;
+  int64_t x_scale_row_stride, x_scale_kb_stride;
+  const uint16_t* router_weight;
+  const uint16_t* router_hidden;
+  void* router_workspace;
+  size_t router_workspace_bytes;
 } bgmoe_moe_fp8_layer;
 
 int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* layer, bgmoe_stream_t stream);

@@ -168,3 +168,37 @@ def test_layer_forward_replays_from_a_hip_graph(dev):
             assert torch.equal(out_static, eager[i]), f"replay of input {i} (round {rnd}) differs from eager"
             scratch = layer(xs[(i + 1) % 3], ls[(i + 1) % 3])   # eager work between replays
             assert torch.equal(scratch, eager[(i + 1) % 3])
+
+
+@pytest.mark.parametrize("name", ["c1_small", "c2_small", "ungrouped_fp8"])
+def test_layer_fed_by_the_fused_producer_and_its_own_router_gemm(dev, name):
+    """residual + hidden -> add + RMSNorm + FP8 cast -> (normed, x_fp8, x_scale) -> layer with router_weight.
+    The same layer fed the bf16 `normed` and the logits of the standalone router GEMM gives the same bits:
+    the producer's cast is the layer's own quantiser, and the fused router sums the same planes."""
+    from batchgen_amd.attention import cuda_add_rmsnorm_fp8_quant
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    from batchgen_amd.moe.routing import glm5_router_gemm_cuda
+    cfg = SMALL[name]
+    g = torch.Generator().manual_seed(31)
+    n, h = cfg.n_tokens, cfg.hidden
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    wd = {k: v.to(dev) for k, v in w.items()}
+    shd = {k: v.to(dev) for k, v in sh.items()} if sh else None
+    rw = (torch.randn(cfg.n_experts, h, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    residual = (torch.randn(n, h, generator=g) * 0.9).to(torch.bfloat16).to(dev)
+    hidden = (torch.randn(n, h, generator=g) * 0.4).to(torch.bfloat16).to(dev)
+    gamma = (torch.randn(h, generator=g) * 0.3 + 1.0).to(torch.bfloat16).to(dev)
+    normed, _, x_fp8, x_scale = cuda_add_rmsnorm_fp8_quant(residual, hidden, gamma, 1e-5, scale_tma_aligned=True)
+    layer = Fp8MoELayer(cfg, wd, shd, inp["bias"].to(dev), router_weight=rw)
+    fused = layer(normed, None, x_fp8=x_fp8, x_scale=x_scale).clone()
+    ids_f, xq_f = layer.topk_ids.clone(), layer.xq.clone()
+    logits = glm5_router_gemm_cuda(normed, rw)
+    plain = layer(normed, logits).clone()
+    assert torch.equal(layer.topk_ids, ids_f)
+    assert torch.equal(layer.xq, xq_f)
+    assert torch.equal(fused, plain)
+    with pytest.raises(RuntimeError, match="together"):
+        layer(normed, logits, x_fp8=x_fp8)
+    with pytest.raises(RuntimeError, match="router_weight"):
+        Fp8MoELayer(cfg, wd, shd, inp["bias"].to(dev))(normed, None)

@@ -127,6 +127,33 @@ def test_scatter_quant_equals_scatter_then_quant(dev):
     assert np.array_equal(s.cpu().numpy(), op_.gather_rows(sq, pos_o, k, rows))
 
 
+@pytest.mark.parametrize("h,mn_major", [(1024, False), (7168, True), (400 * 16, False), (144, True)])
+def test_scatter_of_prequantised_rows_equals_scatter_quant(dev, h, mn_major):
+    from batchgen_amd._lib import check, lib, ptr, stream
+    g = torch.Generator().manual_seed(h)
+    n, k, el = 70, 8, 32
+    ids = _ids(g, n, k, 64, extra=[-1, 70])
+    x = rand_bf16(g, n, h)
+    counts_o, cu_o, pos_o = op_.dispatch_ragged(ids.numpy(), 0, el, 16)
+    rows = int(cu_o[-1])
+    pos = torch.from_numpy(pos_o).to(dev)
+    kb = (h + 127) // 128
+    yq, sq = act_quant(x)
+    xq_d = torch.from_numpy(yq).to(dev)
+    xs_d = torch.from_numpy(sq).to(dev)
+    if mn_major:                                      # [kb, align4(n)] storage viewed as [n, kb]
+        store = torch.zeros((kb, (n + 3) // 4 * 4), dtype=torch.float32, device=dev)
+        store[:, :n] = xs_d.t()
+        xs_d = store.t()[:n]
+    y = torch.zeros((rows, h), dtype=torch.uint8, device=dev)
+    s = torch.zeros((rows, kb), dtype=torch.float32, device=dev)
+    check(lib().bgmoe_scatter_fp8_rows(ptr(xq_d), ptr(xs_d), xs_d.stride(0), xs_d.stride(1), ptr(pos), n, k, h,
+                                       ptr(y), ptr(s), kb, 1, stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), op_.gather_rows(yq, pos_o, k, rows))
+    assert np.array_equal(s.cpu().numpy(), op_.gather_rows(sq, pos_o, k, rows))
+
+
 @pytest.mark.parametrize("n,k,h", [(1, 2, 256), (64, 4, 1024), (256, 8, 7168), (33, 8, 131), (17, 4, 2880)])
 def test_reduce_weighted_scatter(dev, n, k, h):
     say("reduce", n, k, h)
