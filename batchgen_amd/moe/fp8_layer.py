@@ -47,9 +47,18 @@ _lib.register("bgmoe_moe_fp8_layer_forward", i32, [C.POINTER(LayerStruct), vp])
 W_ROW_MAJOR, W_TILE_MAJOR = 0, 1
 
 
-def _stack_desc(q: torch.Tensor, s: torch.Tensor, layout: int = W_ROW_MAJOR) -> Fp8Weight:
+def _check_stack(q: torch.Tensor, s: torch.Tensor):
+    """Stacks may be views (one half of a fused gate/up block, scales with a padded trailing axis): each
+    expert's [N, K] bytes must be dense and its scale rows unit-stride."""
     e, n, k = q.shape
-    return Fp8Weight(ptr(q), n * k, None, ptr(s), s.size(1) * s.size(2), s.size(2), None, layout, 0)
+    if q.stride(2) != 1 or q.stride(1) != k or s.stride(2) != 1:
+        raise RuntimeError(f"expert weights must be dense [N, K] per expert with unit-stride scale rows; got "
+                           f"strides {q.stride()} / {s.stride()}")
+
+
+def _stack_desc(q: torch.Tensor, s: torch.Tensor, layout: int = W_ROW_MAJOR) -> Fp8Weight:
+    _check_stack(q, s)
+    return Fp8Weight(ptr(q), q.stride(0), None, ptr(s), s.stride(0), s.stride(1), None, layout, 0)
 
 
 def repack_tile_major(q: torch.Tensor) -> torch.Tensor:
@@ -57,12 +66,16 @@ def repack_tile_major(q: torch.Tensor) -> torch.Tensor:
     include/bgmoe.h).  One-time, at weight load."""
     if q.dim() == 2:
         q = q.unsqueeze(0)
-    if not q.is_contiguous():
-        raise RuntimeError("weights must be contiguous")
     e, n, k = q.shape
-    out = torch.empty_like(q)
+    out = torch.empty((e, n, k), dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
-        check(lib().bgmoe_fp8_weight_repack(ptr(q), ptr(out), e, n, k, stream()))
+        if q.is_contiguous():
+            check(lib().bgmoe_fp8_weight_repack(ptr(q), ptr(out), e, n, k, stream()))
+        else:                                        # a strided stack of dense experts: one expert at a time
+            if q.stride(2) != 1 or q.stride(1) != k:
+                raise RuntimeError("each expert's weight must be a dense [N, K] block")
+            for i in range(e):
+                check(lib().bgmoe_fp8_weight_repack(ptr(q[i]), ptr(out[i]), 1, n, k, stream()))
     return out
 
 
@@ -140,7 +153,10 @@ class Fp8MoELayer:
                 tw = torch.tensor(wp, dtype=torch.int64, device=dev)
                 ts = torch.tensor(sp, dtype=torch.int64, device=dev)
                 self._tables[name] = (tw, ts)
-                setattr(L, name, Fp8Weight(None, 0, ptr(tw), None, 0, s.size(2), ptr(ts), self.layout, 0))
+                _check_stack(q, s)
+                if sq.stride(1) != q.size(2) or ss.stride(1) != s.stride(1):
+                    raise RuntimeError("a folded shared expert must use the routed experts' scale row stride")
+                setattr(L, name, Fp8Weight(None, 0, ptr(tw), None, 0, s.stride(1), ptr(ts), self.layout, 0))
         else:
             for name in ("gate", "up", "down"):
                 setattr(L, name, _stack_desc(weights[name + "_q"], weights[name + "_s"], self.layout))

@@ -202,3 +202,38 @@ def test_layer_fed_by_the_fused_producer_and_its_own_router_gemm(dev, name):
         layer(normed, logits, x_fp8=x_fp8)
     with pytest.raises(RuntimeError, match="router_weight"):
         Fp8MoELayer(cfg, wd, shd, inp["bias"].to(dev))(normed, None)
+
+
+@pytest.mark.parametrize("weight_layout", ["tile_major", "row_major"])
+@pytest.mark.parametrize("name,fold", [("c1_small", True), ("c1_unfolded_shared", False)])
+def test_layer_built_from_a_checkpoint(dev, tmp_path, name, fold, weight_layout):
+    """Per-expert checkpoint tensors (safetensors, HF names) -> loader (scale axis padded to 4, gate/up in one
+    fused block) -> layer.  Same bits as the layer built from the original stacks."""
+    from safetensors.torch import save_file
+    from batchgen_amd.moe import weight_loader as wld
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = SMALL[name]
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    g = torch.Generator().manual_seed(9)
+    rw = (torch.randn(cfg.n_experts, cfg.hidden, generator=g) * 0.05).to(torch.bfloat16)
+    prefix = "model.layers.5.mlp."
+    ck = wld.export_fp8_moe_layer(prefix, {k: v.view(torch.uint8) if v.dtype != torch.float32 else v for k, v in w.items()},
+                                  {k: v.view(torch.uint8) if v.dtype != torch.float32 else v for k, v in sh.items()},
+                                  inp["bias"], rw, expert_start=cfg.expert_start)
+    path = str(tmp_path / "layer.safetensors")
+    save_file(ck, path)
+    src = wld.SafetensorsSource(path)
+    experts = wld.stack_fp8_experts(src, prefix, range(cfg.expert_start, cfg.expert_start + cfg.e_local), cfg.hidden,
+                                    cfg.inter, dev, scale_pad4=True, fuse_gate_up=True)
+    shared = wld.stack_fp8_experts(src, prefix, [0], cfg.hidden, cfg.shared_inter, dev, scale_pad4=fold,
+                                   expert_fmt="shared_experts.")
+    bias = src[prefix + "gate.e_score_correction_bias"].to(dev)
+    a = Fp8MoELayer(cfg, experts, shared, bias, fold_shared=fold, weight_layout=weight_layout,
+                    router_weight=src[prefix + "gate.weight"].to(dev))
+    b = Fp8MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
+                    inp["bias"].to(dev), fold_shared=fold, weight_layout=weight_layout, router_weight=rw.to(dev))
+    assert a.folded == fold
+    x = inp["x"].to(dev)
+    assert torch.equal(a(x, None), b(x, None))
+    assert torch.equal(a(x, inp["logits"].to(dev)), b(x, inp["logits"].to(dev)))
