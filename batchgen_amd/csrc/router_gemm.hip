@@ -14,6 +14,7 @@
 // one whole 128-byte line; tokens and experts use the same K permutation, which a dot product does not see.
 // Experts are the MFMA's row operand, so a lane ends up with 4 consecutive experts of one token: 16-byte
 // stores.
+#include "bgmoe_async.h"
 #include "bgmoe_common.h"
 
 namespace {
@@ -223,6 +224,156 @@ __global__ __launch_bounds__(64 * WAVES) void router_gemm_kernel(RouterGemmArgs 
   }
 }
 
+// ---- many tokens: operands shared through LDS ------------------------------------------------------
+// A CU sustains only ~35-60 GB/s of load requests, so with many tokens the time goes where the requested
+// bytes go.  Four waves that each fetch their own 64 + 64 rows request twice what the block needs; here the
+// block's 128 experts + 128 tokens of a 64-element K step (256 rows x 128 B = 32 KB) are fetched ONCE, by
+// asynchronous global->LDS loads into a 4-slot ring, and every wave reads its share of the tile from LDS.
+// A row's eight 16-byte pieces land XOR-swizzled by (row & 7) -- done by choosing which piece each lane
+// fetches -- so that the 16-row operand reads hit all banks.  Lane (r, q) reads pieces 2q and 2q+1 of row
+// r: the same K assignment, MFMA order and segment folds as the register kernel above, hence the same bits.
+constexpr int kLdsStages = 4;
+constexpr int kLdsStageBytes = 256 * 128;
+constexpr int kLdsBytes = kLdsStages * kLdsStageBytes;
+
+// 8 waves = 2 expert halves x 4 token quarters (wave tile 64 experts x 32 tokens): two waves per SIMD, which
+// a single wave's MFMA issue rate needs (one wave alone issues a 16x16x32 MFMA every ~28 cycles, two
+// interleaved reach ~20 per SIMD -- measured), and which lets one wave's LDS reads hide behind the other's
+// MFMAs.
+constexpr int kLdsWaves = 8;
+constexpr int kLdsTM = 128 / (kLdsWaves / 2) / 16;      // 16-token tiles per wave
+
+template <bool SPLIT>
+__global__ __launch_bounds__(64 * kLdsWaves) void router_gemm_lds_kernel(RouterGemmArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  constexpr int TM = kLdsTM;
+  const uint32_t smem_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int lane = lane_id();
+  const int r16 = lane & 15, q = lane >> 4;
+  // consecutive block ids go round-robin over the 8 XCDs: the expert blocks of one token tile stay on one
+  // XCD (its L2 then serves the tile's second reader), token tiles are dealt over the XCDs
+  // (split shape: a unit = (K segment, expert block) with all its token tiles on one XCD, as in the register
+  // kernel)
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  int bx, by, seg = 0;
+  if constexpr (SPLIT) {
+    const int ul = j / a.ttiles;
+    const int unit = ul * 8 + xcd;
+    if (unit >= a.nseg * a.eblocks) return;
+    bx = j - ul * a.ttiles;
+    seg = unit / a.eblocks;
+    by = unit - seg * a.eblocks;
+  } else {
+    const int tl = j / a.eblocks;
+    by = j - tl * a.eblocks;
+    bx = tl * 8 + xcd;
+    if (bx >= a.ttiles) return;            // whole block, before any barrier
+  }
+  const int t0 = bx * 128, e0 = by * 128;
+  const int we = wave & 1, wt = wave >> 1;  // this wave's expert half and token share of the block tile
+
+  // loader: the first half of the waves fetches the 128 expert rows, the second half the 128 token rows;
+  // one issue = 8 rows x 128 B, lane p -> row p>>3, LDS piece p&7 <- global piece (p&7) ^ (row&7)
+  constexpr int kHalf = kLdsWaves / 2;
+  constexpr int kIssues = 16 / kHalf;       // issues per wave and step
+  const bool load_tokens = wave >= kHalf;
+  const int lrow0 = (wave % kHalf) * (8 * kIssues);
+  const uint8_t* src = load_tokens ? reinterpret_cast<const uint8_t*>(a.x) + (int64_t)t0 * a.h * 2
+                                   : reinterpret_cast<const uint8_t*>(a.w) + (int64_t)e0 * a.h * 2;
+  src = uniform_ptr(src);
+  const int row_lim = (load_tokens ? a.n - t0 : a.e - e0) - 1;      // clamp: rows past the end re-read the last
+  uint32_t loff[kIssues];
+#pragma unroll
+  for (int i = 0; i < kIssues; ++i) {
+    const int row = lrow0 + i * 8 + (lane >> 3);
+    const int piece = (lane & 7) ^ (row & 7);
+    loff[i] = (uint32_t)min(row, row_lim) * (uint32_t)a.h * 2u + (uint32_t)piece * 16u;
+  }
+  const uint32_t ldst = smem_base + (load_tokens ? 16384u : 0u) + (uint32_t)lrow0 * 128u;
+  auto issue = [&](int step) {
+    const uint32_t d = ldst + (uint32_t)(step & (kLdsStages - 1)) * kLdsStageBytes;
+    const uint8_t* p = src + (int64_t)step * (kStep * 2);
+#pragma unroll
+    for (int i = 0; i < kIssues; ++i) async_load16(p, loff[i], d + i * 1024);
+  };
+
+  floatx4 acc[TM][4], tot[TM][4];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+      acc[tm][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+      tot[tm][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+  // the host sends only h % 64 == 0 here; the split shape walks one segment's steps
+  const int step0 = SPLIT ? seg * kStepsPerSeg : 0;
+  const int nsteps = SPLIT ? min(kStepsPerSeg, a.h / kStep - step0) : a.h / kStep;
+  src += (int64_t)step0 * (kStep * 2);
+  const int rd_a = (we * 64 + r16) * 128, rd_b = 16384 + (wt * (16 * TM) + r16) * 128;
+  const int sw = r16 & 7;
+
+#pragma unroll
+  for (int s = 0; s < kLdsStages - 1; ++s)
+    if (s < nsteps) issue(s);
+  for (int s = 0; s < nsteps; ++s) {
+    // the step's loads have landed once at most the younger steps' loads are outstanding
+    const int younger = min(kLdsStages - 2, nsteps - 1 - s);      // steps requested after this one
+    if (younger >= 2) wait_vm<2 * kIssues>();
+    else if (younger == 1) wait_vm<kIssues>();
+    else wait_vm<0>();
+    block_barrier();                       // everyone's loads of step s are in; everyone is done with step s-1
+    if (s + kLdsStages - 1 < nsteps) issue(s + kLdsStages - 1);   // into the slot step s-1 just freed
+    const uint8_t* sb = smem + (s & (kLdsStages - 1)) * kLdsStageBytes;
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const int piece = ((2 * q + jj) ^ sw) * 16;
+      intx4 av[4], bv[TM];
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) av[tn] = *reinterpret_cast<const intx4*>(sb + rd_a + tn * 2048 + piece);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) bv[tm] = *reinterpret_cast<const intx4*>(sb + rd_b + tm * 2048 + piece);
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av[tn]),
+                                                                __builtin_bit_cast(bf16x8, bv[tm]),
+                                                                acc[tm][tn], 0, 0, 0);
+    }
+    if ((s & (kStepsPerSeg - 1)) == kStepsPerSeg - 1 || s == nsteps - 1) {   // end of a segment
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < 4; ++tn) {
+          tot[tm][tn] += acc[tm][tn];
+          acc[tm][tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+  }
+
+  const bool vec = (a.e & 3) == 0;
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int token = t0 + wt * (16 * TM) + tm * 16 + r16;
+    if (token >= a.n) continue;
+    const bool pad = SPLIT ? false : row_is_padding(a, token);
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+      const int ex = e0 + we * 64 + tn * 16 + q * 4;
+      const floatx4 v = pad ? floatx4{0.f, 0.f, 0.f, 0.f} : tot[tm][tn];
+      float* dst = a.out + (SPLIT ? (int64_t)seg * a.n * a.e : 0) + (int64_t)token * a.e + ex;
+      if (vec) {
+        if (ex < a.e) *reinterpret_cast<floatx4*>(dst) = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (ex + i < a.e) dst[i] = v[i];
+      }
+    }
+  }
+}
+
 // logits = (((0 + p_0) + p_1) + ...) over the planes; rows past a rank's count get 0
 __global__ __launch_bounds__(256) void router_gemm_reduce_kernel(RouterGemmArgs a, const float* planes) {
   const int64_t total = (int64_t)a.n * a.e;
@@ -236,8 +387,9 @@ __global__ __launch_bounds__(256) void router_gemm_reduce_kernel(RouterGemmArgs 
 }
 
 int g_plan_tm = -1, g_plan_split = -1;
+bool g_lds_ready = false;            // the LDS kernel's 128 KB opt-in succeeded on this process's device
 
-struct Plan { int tm; int ne; int waves; bool split; };
+struct Plan { int tm; int ne; int waves; bool split; bool lds; };
 
 // Launch shape from the sizes alone (results do not depend on it).
 // A CU sustains only ~35-60 GB/s of load requests whatever hits in cache, so what matters for few tokens
@@ -249,10 +401,22 @@ Plan make_plan(int n, int h, int e) {
   Plan p;
   p.ne = 4;
   p.waves = 4;
-  // split-K while the partial planes stay small next to the operands (<= 64 MiB) and the whole-K shape
-  // would leave CUs idle or starved
-  const bool planes_small = (int64_t)n * e * nseg <= (int64_t)16 << 20;
-  if (nseg == 1 || !planes_small || ((int64_t)(n + 63) / 64) * ey4 >= 192) {
+  // Measured on MI355X (h = 7168): an LDS block needs ~0.6 us per K step whatever else runs, so the whole-K LDS
+  // shape costs ~67 us per round of 256 tiles; one block per segment fills the chip from ~1K tokens on at the
+  // price of the planes (write + reduce); below that the one-wave register blocks win.
+  const bool planes_small = (int64_t)n * e * nseg <= (int64_t)16 << 20;      // <= 64 MiB of partial planes
+  const bool lds_ok = h % kStep == 0 && g_lds_ready;
+  const int64_t tiles128 = ((int64_t)(n + 127) / 128) * ((e + 127) / 128);
+  p.lds = false;
+  if (lds_ok && (tiles128 >= 96 || (nseg == 1 && tiles128 >= 16))) {
+    p.split = false;
+    p.lds = true;
+    p.tm = 4;
+  } else if (lds_ok && nseg > 1 && planes_small && tiles128 * nseg >= 128) {
+    p.split = true;
+    p.lds = true;
+    p.tm = 4;
+  } else if (nseg == 1 || !planes_small || ((int64_t)(n + 63) / 64) * ey4 >= 192) {
     p.split = false;
     p.tm = n > 2048 ? 4 : n > 512 ? 2 : 1;
   } else {
@@ -261,15 +425,25 @@ Plan make_plan(int n, int h, int e) {
     p.tm = n > 32 ? 4 : n > 16 ? 2 : 1;
   }
   if (g_plan_tm == 1 || g_plan_tm == 2 || g_plan_tm == 4) p.tm = g_plan_tm;
-  if (g_plan_split == 0) { p.split = false; p.waves = 4; }
-  if (g_plan_split == 1) { p.split = true; p.waves = 4; }
-  if (g_plan_split == 2) { p.split = true; p.waves = 1; }
+  if (g_plan_split == 0) { p.split = false; p.waves = 4; p.lds = false; }
+  if (g_plan_split == 3) { p.split = false; p.waves = 4; p.lds = h % kStep == 0 && g_lds_ready; }
+  if (g_plan_split == 4) { p.split = true; p.waves = 4; p.lds = h % kStep == 0 && g_lds_ready; }
+  if (g_plan_split == 1) { p.split = true; p.waves = 4; p.lds = false; }
+  if (g_plan_split == 2) { p.split = true; p.waves = 1; p.lds = false; }
   return p;
 }
 
 template <bool SPLIT>
 void launch_gemm(const RouterGemmArgs& a0, const Plan& p, hipStream_t st) {
   RouterGemmArgs a = a0;
+  if (p.lds) {
+    a.ttiles = (a.n + 127) / 128;
+    a.eblocks = (a.e + 127) / 128;
+    const unsigned blocks = SPLIT ? (unsigned)(8 * ((a.nseg * a.eblocks + 7) / 8) * a.ttiles)
+                                  : (unsigned)(8 * ((a.ttiles + 7) / 8) * a.eblocks);
+    hipLaunchKernelGGL(router_gemm_lds_kernel<SPLIT>, dim3(blocks), dim3(64 * kLdsWaves), kLdsBytes, st, a);
+    return;
+  }
   const dim3 block(64 * p.waves);
   a.ttiles = (a.n + 16 * p.tm - 1) / (16 * p.tm);
   a.eblocks = (a.e + 16 * p.ne * p.waves - 1) / (16 * p.ne * p.waves);
@@ -294,10 +468,26 @@ int check_shapes(int n, int h, int e) {
 
 }  // namespace
 
+// one-time: the LDS kernel needs more than the default 64 KB of dynamic LDS
+int bgmoe_internal_init_router_gemm() {
+  static int state = 0;                // 0 = not tried, 1 = ready, -1 = failed (the register kernels serve)
+  if (state == 0) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_gemm_lds_kernel<false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(router_gemm_lds_kernel<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    state = e == hipSuccess ? 1 : -1;
+    if (e != hipSuccess) (void)hipGetLastError();
+    g_lds_ready = state == 1;
+  }
+  return BGMOE_OK;
+}
+
 extern "C" int bgmoe_set_router_gemm_plan(int token_tiles, int split) {
   BGMOE_REQUIRE(token_tiles == -1 || token_tiles == 1 || token_tiles == 2 || token_tiles == 4,
                 "set_router_gemm_plan: token_tiles must be -1, 1, 2 or 4");
-  BGMOE_REQUIRE(split >= -1 && split <= 2, "set_router_gemm_plan: split must be -1, 0, 1 or 2");
+  BGMOE_REQUIRE(split >= -1 && split <= 4, "set_router_gemm_plan: split must be -1 ... 4");
   g_plan_tm = token_tiles;
   g_plan_split = split;
   return BGMOE_OK;
@@ -305,6 +495,7 @@ extern "C" int bgmoe_set_router_gemm_plan(int token_tiles, int split) {
 
 extern "C" size_t bgmoe_router_gemm_workspace_bytes(int n, int h, int e) {
   if (n <= 0 || h <= 0 || e <= 0) return 0;
+  bgmoe_internal_init_router_gemm();
   const Plan p = make_plan(n, h, e);
   const int nseg = (h + kSeg - 1) / kSeg;
   return (size_t)(p.split ? nseg : 1) * (size_t)n * (size_t)e * sizeof(float);
@@ -315,6 +506,7 @@ extern "C" size_t bgmoe_router_gemm_workspace_bytes(int n, int h, int e) {
 int bgmoe_internal_router_gemm_planes(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,
                                       float* planes, size_t planes_bytes, int* nplanes_out, hipStream_t st) {
   if (int rc = check_shapes(n, h, e)) return rc;
+  bgmoe_internal_init_router_gemm();
   RouterGemmArgs a{};
   a.x = hidden; a.w = weight; a.out = planes; a.n = n; a.h = h; a.e = e;
   a.nseg = (h + kSeg - 1) / kSeg;
@@ -343,6 +535,7 @@ extern "C" int bgmoe_router_gemm(const uint16_t* hidden, const uint16_t* weight,
   }
   if (n == 0) return BGMOE_OK;
   BGMOE_REQUIRE(hidden && weight && logits, "router_gemm: null pointer");
+  bgmoe_internal_init_router_gemm();
   hipStream_t st = bgmoe_stream(stream);
   RouterGemmArgs a{};
   a.x = hidden; a.w = weight; a.n = n; a.h = h; a.e = e;

@@ -8,6 +8,10 @@ requant GEMM -> down GEMM -> combine + shared expert) over one batch of syntheti
 tokens, with weights and inputs already resident in HBM.  Default workload is
 config 1 of BASELINE.json (DeepSeek-V3-shaped FP8 decode, 256 tokens, 32 of 256
 experts local, masked layout).  Prints ONE JSON line.
+
+`--op router_gemm` and `--op norm_quant` time the two producers that sit in front of the layer on the same
+configuration's shapes (hidden states -> logits -> routes in two launches; residual add + RMSNorm + FP8
+cast in one) and print the same kind of line for them.
 """
 from __future__ import annotations
 
@@ -22,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0          # MI355X published HBM3E bandwidth
 FP8_PEAK_TFLOPS = 5000.0        # MI355X published dense FP8 MFMA peak
+BF16_PEAK_TFLOPS = 2500.0       # MI355X published dense BF16 MFMA peak
 
 METRIC = "MoE layer TFLOP/s (FP8 prefill) & HBM GB/s (decode), % roofline, 1xMI355X"
 
@@ -44,6 +49,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
+    ap.add_argument("--op", default="layer", choices=["layer", "router_gemm", "norm_quant"],
+                    help="what one step is: the MoE layer (default), or one of its two producers")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of one captured HIP graph of the layer instead of eager launches")
@@ -113,12 +120,136 @@ def cpu_baseline_mxfp4(cfg, inp, w, sh):
     return t, n / cfg.n_tokens, f"{n} of {cfg.n_tokens} tokens of the workload and the experts they route to, one pass, NumPy"
 
 
+def _time(step, steps, warmup, torch):
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def bench_producer(a):
+    """One step = the router GEMM + top-k, or the add + RMSNorm + FP8 cast, on the configuration's shapes."""
+    import numpy as np
+    import torch
+    from batchgen_amd import _lib, workloads as wl
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = wl.CONFIGS[a.config]
+    n, h, e, k = cfg.n_tokens, cfg.hidden, cfg.n_experts, cfg.top_k
+    g = torch.Generator(device=dev).manual_seed(cfg.seed + 7)
+    base = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "launch": "eager", "data": "synthetic"}
+    if a.op == "router_gemm":
+        from batchgen_amd.moe.routing import router_gemm_gate_sigmoid_topk
+        from oracle import router as orr
+        from oracle import router_gemm as org
+        x = (torch.randn(n, h, generator=g, device=dev) * 0.1).to(torch.bfloat16)
+        w = (torch.randn(e, h, generator=g, device=dev) * 0.1).to(torch.bfloat16)
+        bias = torch.zeros(e, device=dev)
+        ids = torch.empty((n, k), dtype=torch.int32, device=dev)
+        wt = torch.empty((n, k), dtype=torch.float32, device=dev)
+        grouped = cfg.n_group > 1
+        step = lambda: router_gemm_gate_sigmoid_topk(x, w, bias, k, cfg.rsf, ids, wt,
+                                                     n_group=cfg.n_group if grouped else 0,
+                                                     topk_group=cfg.topk_group if grouped else 0)
+        ms = _time(step, a.steps, a.warmup, torch)
+        _lib.prof_enable(True)
+        for _ in range(a.steps):
+            step()
+        prof = _lib.prof_collect()
+        _lib.prof_enable(False)
+        gemm_ms = prof["router_gemm"][0] / prof["router_gemm"][1]
+        flops = 2.0 * n * h * e
+        alg_bytes = (n + e) * h * 2 + n * k * 8
+        mfma = flops / (BF16_PEAK_TFLOPS * 1e12) > alg_bytes / (HBM_PEAK_GBPS * 1e9)
+        if mfma:
+            roof = dict(bound="mfma", kernel="router_gemm_kernel", achieved=flops / (gemm_ms * 1e-3) / 1e12,
+                        peak=BF16_PEAK_TFLOPS, unit="TFLOP/s", traffic=None, flops_per_launch=flops,
+                        avg_launch_us=gemm_ms * 1e3)
+        else:
+            gb = (n + e) * h * 2
+            roof = dict(bound="hbm", kernel="router_gemm_kernel", achieved=gb / (gemm_ms * 1e-3) / 1e9,
+                        peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=gb,
+                        avg_launch_us=gemm_ms * 1e3)
+        roof["frac"] = roof["achieved"] / roof["peak"]
+        out = dict(base, metric="router GEMM + top-k: TFLOP/s (prefill) or HBM GB/s (decode), 1xMI355X",
+                   value=(flops / (ms * 1e-3) / 1e12) if mfma else (alg_bytes / (ms * 1e-3) / 1e9),
+                   unit="TFLOP/s" if mfma else "GB/s", ms_per_step=ms, dtype="bf16 (fp32 accumulate)",
+                   config={"workload": cfg.name + " / router", "tokens": n, "hidden": h, "experts": e, "top_k": k},
+                   tokens_per_s=n / (ms * 1e-3), kernel_ms_per_step={kk: v[0] / a.steps for kk, v in prof.items()},
+                   roofline=roof)
+        if not a.no_cpu_baseline:
+            m = min(n, 512)
+            xs, wc = x[:m].cpu(), w.cpu()
+            t0 = time.perf_counter()
+            logits = org.router_gemm_exact(xs, wc)
+            if grouped:
+                orr.grouped_router(logits, bias.cpu().numpy(), cfg.n_group, cfg.topk_group, k, cfg.rsf)
+            else:
+                orr.gate_sigmoid_topk(logits, bias.cpu().numpy(), k, cfg.rsf)
+            t = time.perf_counter() - t0
+            frac = m / n
+            out["cpu_baseline"] = {"value": (flops * frac / t / 1e12) if mfma else (alg_bytes * frac / t / 1e9),
+                                   "unit": out["unit"], "cores": min(os.cpu_count() or 1, 16), "kind": "port",
+                                   "sample": f"{m} of {n} tokens, float64 BLAS product + NumPy router", "seconds": t}
+        print(json.dumps(out))
+        return
+    from batchgen_amd.attention import cuda_add_rmsnorm_fp8_quant
+    from oracle import norm_quant as onq
+    res = (torch.randn(n, h, generator=g, device=dev) * 0.9).to(torch.bfloat16)
+    hid = (torch.randn(n, h, generator=g, device=dev) * 0.4).to(torch.bfloat16)
+    gamma = (torch.randn(h, generator=g, device=dev) * 0.3 + 1.0).to(torch.bfloat16)
+    res0 = res.clone()
+    from batchgen_amd._lib import check, lib, ptr, stream
+    normed = torch.empty_like(res)
+    q = torch.empty((n, h), dtype=torch.uint8, device=dev)
+    sc = torch.empty((n, h // 128), dtype=torch.float32, device=dev)
+    # the residual is updated in place; its growth over the timed steps does not change the work done
+    step = lambda: check(lib().bgmoe_add_rmsnorm_fp8_quant(ptr(res), ptr(hid), ptr(gamma), n, h, 1e-5, ptr(normed),
+                                                           ptr(q), ptr(sc), h // 128, 1, None, None, None, stream()))
+    ms = _time(step, a.steps, a.warmup, torch)
+    _lib.prof_enable(True)
+    for _ in range(a.steps):
+        step()
+    prof = _lib.prof_collect()
+    _lib.prof_enable(False)
+    k_ms = prof["norm_quant"][0] / prof["norm_quant"][1]
+    alg_bytes = n * h * 9 + n * (h // 128) * 4 + h * 2
+    roof = dict(bound="hbm", kernel="add_rmsnorm_fp8_quant_kernel", achieved=alg_bytes / (k_ms * 1e-3) / 1e9,
+                peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=alg_bytes, avg_launch_us=k_ms * 1e3)
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    out = dict(base, metric="add + RMSNorm + FP8 cast: HBM GB/s, 1xMI355X", value=alg_bytes / (ms * 1e-3) / 1e9,
+               unit="GB/s", ms_per_step=ms, dtype="bf16 in, fp32 arithmetic, e4m3 + fp32 scales out",
+               config={"workload": cfg.name + " / add_rmsnorm_fp8_quant", "rows": n, "hidden": h},
+               tokens_per_s=n / (ms * 1e-3), roofline=roof)
+    if not a.no_cpu_baseline:
+        m = min(n, 256)
+        t0 = time.perf_counter()
+        onq.add_rmsnorm_fp8_quant(res0[:m].cpu(), hid[:m].cpu(), gamma.cpu(), 1e-5)
+        t = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": alg_bytes * (m / n) / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": f"{m} of {n} rows, NumPy oracle, one thread", "seconds": t}
+    print(json.dumps(out))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
         print("bench.py measures one GPU's expert-parallel share; this build has no multi-GPU path "
               "(run with --gpus 1).", file=sys.stderr)
         sys.exit(2)
+    if a.op != "layer":
+        import torch
+        if not torch.cuda.is_available():
+            print("bench.py needs a GPU", file=sys.stderr)
+            sys.exit(2)
+        return bench_producer(a)
     import numpy as np
     import torch
     from batchgen_amd import _lib, workloads as wl

@@ -108,7 +108,7 @@ def test_production_graph_envelope_rank_counts(dev, world, bucket):
     assert torch.equal(out[~pad], compact)
 
 
-@pytest.mark.parametrize("n,h,e", [(50, 7168, 256), (200, 1096, 72), (1, 512, 256), (130, 64, 16)])
+@pytest.mark.parametrize("n,h,e", [(50, 7168, 256), (200, 1096, 72), (1, 512, 256), (130, 64, 16), (300, 1088, 200)])
 def test_every_launch_shape_gives_the_same_bits(dev, n, h, e):
     """Whole-K and split-K, 1/2/4 token tiles and 2/4 expert tiles per wave: one summation order, so one
     result."""
@@ -119,7 +119,7 @@ def test_every_launch_shape_gives_the_same_bits(dev, n, h, e):
     outs = {}
     try:
         for tm in (1, 2, 4):
-            for split in (0, 1, 2):
+            for split in (0, 1, 2, 3, 4):
                 check(lib().bgmoe_set_router_gemm_plan(tm, split))
                 outs[(tm, split)] = glm5_router_gemm_cuda(xd, wd).clone()
     finally:
