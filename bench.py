@@ -43,6 +43,15 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+# the same for the two producers (`--op`), keyed by (op, config); summaries under profiles/ as well
+MEASURED_TRAFFIC_PRODUCER = {
+    ("router_gemm", 1): int((17.7 + 3.5) * MIB),      # router_gemm_kernel<4,4,4,split,1 wave>, 256 tokens
+    ("router_gemm", 2): int((252.3 + 16.1) * MIB),    # router_gemm_lds_kernel<whole K>, 16384 tokens
+    ("norm_quant", 1): int((7.2 + 8.8) * MIB),        # add_rmsnorm_fp8_quant_kernel, 256 rows
+    ("norm_quant", 2): int((448.1 + 563.5) * MIB),    # add_rmsnorm_fp8_quant_kernel, 16384 rows
+}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -145,6 +154,10 @@ def bench_producer(a):
     g = torch.Generator(device=dev).manual_seed(cfg.seed + 7)
     base = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "launch": "eager", "data": "synthetic"}
+    if a.copy_calibration:
+        from batchgen_amd.moe.fp8_layer import repack_tile_major
+        repack_tile_major(torch.zeros((1, 32768, 8192), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn))
+        torch.cuda.synchronize()
     if a.op == "router_gemm":
         from batchgen_amd.moe.routing import router_gemm_gate_sigmoid_topk
         from oracle import router as orr
@@ -178,6 +191,7 @@ def bench_producer(a):
                         peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=gb,
                         avg_launch_us=gemm_ms * 1e3)
         roof["frac"] = roof["achieved"] / roof["peak"]
+        roof["traffic"] = MEASURED_TRAFFIC_PRODUCER.get((a.op, a.config))
         out = dict(base, metric="router GEMM + top-k: TFLOP/s (prefill) or HBM GB/s (decode), 1xMI355X",
                    value=(flops / (ms * 1e-3) / 1e12) if mfma else (alg_bytes / (ms * 1e-3) / 1e9),
                    unit="TFLOP/s" if mfma else "GB/s", ms_per_step=ms, dtype="bf16 (fp32 accumulate)",
@@ -224,6 +238,7 @@ def bench_producer(a):
     roof = dict(bound="hbm", kernel="add_rmsnorm_fp8_quant_kernel", achieved=alg_bytes / (k_ms * 1e-3) / 1e9,
                 peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=alg_bytes, avg_launch_us=k_ms * 1e3)
     roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["traffic"] = MEASURED_TRAFFIC_PRODUCER.get((a.op, a.config))
     out = dict(base, metric="add + RMSNorm + FP8 cast: HBM GB/s, 1xMI355X", value=alg_bytes / (ms * 1e-3) / 1e9,
                unit="GB/s", ms_per_step=ms, dtype="bf16 in, fp32 arithmetic, e4m3 + fp32 scales out",
                config={"workload": cfg.name + " / add_rmsnorm_fp8_quant", "rows": n, "hidden": h},
