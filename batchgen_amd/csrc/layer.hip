@@ -107,3 +107,37 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
   return bgmoe_reduce_weighted_scatter(L->y, L->topk_pos, L->topk_weights, n, h, k, L->out, -1,
                                        shared ? L->y + L->cap_rows * h : nullptr, L->shared_mode, stream);
 }
+
+extern "C" int bgmoe_moe_mxfp4_layer_forward(const bgmoe_moe_mxfp4_layer* L, int stages, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(L != nullptr, "moe_mxfp4_layer_forward: null layer");
+  BGMOE_REQUIRE(stages >= 1 && stages <= 3, "moe_mxfp4_layer_forward: stages must be ROUTED, COMBINE or both");
+  const int n = L->n, h = L->h, inter = L->inter, el = L->e_local, k = L->top_k;
+  BGMOE_REQUIRE(n >= 0 && h > 0 && inter > 0 && el > 0 && k > 0 && L->max_tokens > 0,
+                "moe_mxfp4_layer_forward: bad sizes");
+  if (n == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(L->topk_weights && L->topk_pos && L->y && L->out, "moe_mxfp4_layer_forward: null buffer");
+  const int64_t rows = (int64_t)el * L->max_tokens;
+  int rc;
+  if (stages & BGMOE_MXFP4_ROUTED) {
+    BGMOE_REQUIRE(L->x && L->logits && L->bias && L->topk_ids && L->expert_counts && L->expert_counters &&
+                  L->cu_seqlens && L->act && L->hmid, "moe_mxfp4_layer_forward: null input or buffer");
+    rc = bgmoe_gate_sigmoid_topk(L->logits, L->e_total, L->bias, n, L->e_total, k, L->routed_scaling_factor,
+                                 L->topk_ids, 0, L->topk_weights, nullptr, nullptr, 0, nullptr, 0, 0, stream);
+    if (rc != BGMOE_OK) return rc;
+    rc = bgmoe_dispatch_scatter_3d(L->x, L->topk_ids, n, k, h, L->act, L->expert_start, el, L->max_tokens,
+                                   L->expert_counts, L->expert_counters, L->topk_pos, L->workspace,
+                                   L->workspace_bytes, stream);
+    if (rc != BGMOE_OK) return rc;
+    const int64_t bound = (int64_t)n * k;
+    rc = bgmoe_mxfp4_fused_s1(L->act, &L->gate, &L->up, L->expert_counts, L->cu_seqlens, el, rows, inter, h,
+                              L->hmid, nullptr, 0, bound, stream);
+    if (rc != BGMOE_OK) return rc;
+    rc = bgmoe_mxfp4_grouped_gemm(L->hmid, &L->down, L->expert_counts, L->cu_seqlens, el, rows, h, inter, L->y,
+                                  nullptr, bound, stream);
+    if (rc != BGMOE_OK) return rc;
+  }
+  if (stages & BGMOE_MXFP4_COMBINE)
+    return bgmoe_reduce_weighted_scatter(L->y, L->topk_pos, L->topk_weights, n, h, k, L->out, -1, L->shared_out,
+                                         L->shared_mode, stream);
+  return BGMOE_OK;
+}

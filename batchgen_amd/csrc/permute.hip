@@ -192,27 +192,30 @@ __global__ __launch_bounds__(256) void perm_rank_kernel(PermArgs a) {
   }
 }
 
-// Decode-sized problems (nk <= 2048 pairs, <= 256 local experts) in ONE block of 16 waves: every lane reads
-// its two ids once, ranks inside a wave come from ballots, one pass over the 16 per-wave histograms turns
-// them into offsets, a single wave scans the experts.  Latency chain: one global load, ~10 LDS round trips.
+// Decode-sized problems (nk <= 64*16*S pairs, <= 256 local experts) in ONE block of 16 waves: every lane reads
+// its S ids once (S = 2: up to 2048 pairs, S = 8: up to 8192), ranks inside a wave come from ballots, one pass
+// over the 16 per-wave histograms turns them into offsets, a single wave scans the experts.  Latency chain:
+// one global load, a few LDS round trips per sub-step.
 constexpr int kSmallLocal = 256;
+constexpr int kSmallPairsMax = 64 * 16 * 8;
+template <int S>
 __global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
   __shared__ int32_t whist[16][kSmallLocal];   // per-wave counts, then exclusive offsets over the waves
   __shared__ int32_t s_cu[kSmallLocal + 1];
   const int wave = threadIdx.x >> 6;
   const int lane = lane_id();
   const int el = a.e_local;
-  int le[2];
+  int le[S];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) le[s] = local_id(a, (int64_t)wave * 128 + s * 64 + lane);
+  for (int s = 0; s < S; ++s) le[s] = local_id(a, (int64_t)wave * (64 * S) + s * 64 + lane);
   for (int e = threadIdx.x; e < 16 * el; e += 1024) whist[e / el][e % el] = 0;
   __syncthreads();
   int nbits = 0;
   while ((1 << nbits) < el) ++nbits;
   const unsigned long long lt = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-  int off[2];
+  int off[S];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
+  for (int s = 0; s < S; ++s) {
     unsigned long long peers = __ballot(le[s] >= 0);
     for (int b = 0; b < nbits; ++b) {
       const bool bit = (le[s] >> b) & 1;
@@ -268,8 +271,8 @@ __global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
   }
   __syncthreads();
 #pragma unroll
-  for (int s = 0; s < 2; ++s) {
-    const int64_t i = (int64_t)wave * 128 + s * 64 + lane;
+  for (int s = 0; s < S; ++s) {
+    const int64_t i = (int64_t)wave * (64 * S) + s * 64 + lane;
     if (i < a.nk) {
       int p = -1;
       if (le[s] >= 0) {
@@ -335,10 +338,11 @@ __global__ __launch_bounds__(64) void compact_kernel(const int32_t* __restrict__
 }
 
 int run_index(PermArgs& a, void* workspace, size_t workspace_bytes, hipStream_t st) {
-  if (a.nk <= kChunk) {
+  if (a.nk <= kChunk || (a.nk <= kSmallPairsMax && a.e_local <= kSmallLocal)) {
     a.nchunks = 1;
     BgmoeProf prof(BGMOE_K_PERM_RANK, st);
-    if (a.e_local <= kSmallLocal) hipLaunchKernelGGL(perm_small_kernel, dim3(1), dim3(1024), 0, st, a);
+    if (a.e_local <= kSmallLocal && a.nk <= kChunk) hipLaunchKernelGGL(perm_small_kernel<2>, dim3(1), dim3(1024), 0, st, a);
+    else if (a.e_local <= kSmallLocal) hipLaunchKernelGGL(perm_small_kernel<8>, dim3(1), dim3(1024), 0, st, a);
     else hipLaunchKernelGGL((perm_rank_kernel<true>), dim3(1), dim3(256), 0, st, a);
     return bgmoe_check_launch("dispatch(single)");
   }
@@ -382,6 +386,7 @@ int bgmoe_internal_dispatch_index(const int32_t* ids, int64_t nk, int expert_sta
 
 extern "C" size_t bgmoe_dispatch_workspace_bytes(int64_t nk, int num_local_experts) {
   if (nk <= kChunk || num_local_experts <= 0) return 0;
+  if (nk <= kSmallPairsMax && num_local_experts <= kSmallLocal) return 0;
   return (size_t)((nk + kChunk - 1) / kChunk) * (size_t)num_local_experts * sizeof(int32_t);
 }
 

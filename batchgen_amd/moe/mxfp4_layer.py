@@ -9,14 +9,37 @@ The shared expert is a plain dense bf16 MLP and runs on the library GEMM (hipBLA
 """
 from __future__ import annotations
 
+import os
+
 import ctypes as C
 
 import torch
 import torch.nn.functional as F
 
+from .. import _lib
 from .._lib import Mxfp4Weight, check, lib, ptr, stream
 from ..kernels import load_extension
 from ..workloads import MoEConfig
+
+
+i32, i64, f32, vp, sz = C.c_int32, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
+
+
+class Mxfp4LayerStruct(C.Structure):
+    """bgmoe_moe_mxfp4_layer (include/bgmoe.h)"""
+    _fields_ = [
+        ("n", i32), ("h", i32), ("inter", i32), ("e_total", i32), ("e_local", i32), ("expert_start", i32),
+        ("top_k", i32), ("max_tokens", i32), ("rsf", f32), ("shared_mode", i32),
+        ("x", vp), ("logits", vp), ("bias", vp),
+        ("gate", Mxfp4Weight), ("up", Mxfp4Weight), ("down", Mxfp4Weight),
+        ("topk_ids", vp), ("topk_weights", vp), ("expert_counts", vp), ("expert_counters", vp), ("cu_seqlens", vp),
+        ("topk_pos", vp), ("act", vp), ("hmid", vp), ("y", vp), ("workspace", vp), ("workspace_bytes", sz),
+        ("shared_out", vp), ("out", vp),
+    ]
+
+
+_lib.register("bgmoe_moe_mxfp4_layer_forward", i32, [C.POINTER(Mxfp4LayerStruct), i32, vp])
+ROUTED, COMBINE = 1, 2
 
 
 class Mxfp4MoELayer:
@@ -33,6 +56,12 @@ class Mxfp4MoELayer:
             self.w[name] = (p, s, Mxfp4Weight(ptr(p), p.size(1) * p.size(2), None, ptr(s), s.size(1) * s.size(2),
                                               None, 1, 0))
         self.shared = shared_bf16
+        self.overlap_shared = os.environ.get("BGMOE_MXFP4_OVERLAP_SHARED", "1") != "0"
+        if shared_bf16 is not None:
+            # gate and up as one [2I, H] matrix: one GEMM instead of two
+            self._shared_gate_up = torch.cat([shared_bf16["gate"], shared_bf16["up"]], dim=0).contiguous()
+            self._side = torch.cuda.Stream(device=dev)
+            self._fork, self._join = torch.cuda.Event(), torch.cuda.Event()
         self.bias = bias.to(dev, torch.float32).contiguous()
         n, h, inter, el, k = cfg.n_tokens, cfg.hidden, cfg.inter, cfg.e_local, cfg.top_k
         if cfg.layout != "masked":
@@ -50,33 +79,55 @@ class Mxfp4MoELayer:
         self.y = torch.zeros((self.rows, h), dtype=b2, device=dev)
         self.out = torch.empty((n, h), dtype=b2, device=dev)
         self.shared_mode = {"bf16_add": 0, "fp32_add": 1}[shared_mode]
-        self._routing = load_extension("batchgen_kernels.moe._C_routing")
-        self._dispatch = load_extension("batchgen_kernels.moe._C_dispatch_scatter_3d")
+        ws_bytes = int(lib().bgmoe_dispatch_workspace_bytes(n * k, el))
+        self.workspace = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+        L = Mxfp4LayerStruct()
+        L.h, L.inter, L.e_total, L.e_local, L.expert_start = h, inter, cfg.n_experts, el, cfg.expert_start
+        L.top_k, L.max_tokens, L.rsf, L.shared_mode = k, cfg.max_tokens, cfg.rsf, self.shared_mode
+        L.bias = ptr(self.bias)
+        L.gate, L.up, L.down = self.w["gate"][2], self.w["up"][2], self.w["down"][2]
+        L.topk_ids, L.topk_weights = ptr(self.topk_ids), ptr(self.topk_weights)
+        L.expert_counts, L.expert_counters, L.cu_seqlens = ptr(self.expert_counts), ptr(self.expert_counters), ptr(self.cu)
+        L.topk_pos, L.act, L.hmid, L.y = ptr(self.topk_pos), ptr(self.act), ptr(self.hmid), ptr(self.y)
+        L.workspace, L.workspace_bytes = ptr(self.workspace), self.workspace.numel()
+        L.out = ptr(self.out)
+        self._L = L
+        self._fn = lib().bgmoe_moe_mxfp4_layer_forward
 
     def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
         cfg = self.cfg
         n = hidden_states.size(0)
         if hidden_states.dtype != torch.bfloat16 or tuple(hidden_states.shape) != (n, cfg.hidden) or n > cfg.n_tokens:
             raise RuntimeError(f"hidden_states must be BF16 [N <= {cfg.n_tokens}, {cfg.hidden}]")
-        ids, wts, pos = self.topk_ids[:n], self.topk_weights[:n], self.topk_pos[:n * cfg.top_k]
-        self._routing.gate_sigmoid_topk(router_logits, self.bias, cfg.top_k, cfg.rsf, ids, wts)
-        self._dispatch.dispatch_scatter_3d(hidden_states, ids, self.act, cfg.expert_start, cfg.e_local, cfg.max_tokens,
-                                           self.expert_counts, self.expert_counters, pos)
-        bound = n * cfg.top_k
-        st = stream()
-        check(lib().bgmoe_mxfp4_fused_s1(ptr(self.act), C.byref(self.w["gate"][2]), C.byref(self.w["up"][2]),
-                                         ptr(self.expert_counts), ptr(self.cu), cfg.e_local, self.rows, cfg.inter,
-                                         cfg.hidden, ptr(self.hmid), None, 0, bound, st))
-        check(lib().bgmoe_mxfp4_grouped_gemm(ptr(self.hmid), C.byref(self.w["down"][2]), ptr(self.expert_counts),
-                                             ptr(self.cu), cfg.e_local, self.rows, cfg.hidden, cfg.inter, ptr(self.y),
-                                             None, bound, st))
+        if router_logits.dtype != torch.float32 or tuple(router_logits.shape) != (n, cfg.n_experts) or \
+                not router_logits.is_contiguous() or not hidden_states.is_contiguous():
+            raise RuntimeError(f"router_logits must be contiguous FP32 [{n}, {cfg.n_experts}] and hidden_states contiguous")
         sh = None
         if self.shared is not None:
-            g = F.linear(hidden_states, self.shared["gate"])
-            u = F.linear(hidden_states, self.shared["up"])
-            sh = F.linear(F.silu(g) * u, self.shared["down"])
-        check(lib().bgmoe_reduce_weighted_scatter(ptr(self.y), ptr(pos), ptr(wts), n, cfg.hidden, cfg.top_k,
-                                                  ptr(self.out), -1, ptr(sh), self.shared_mode, st))
+            # the dense bf16 shared expert (vendor GEMMs) runs beside the routed experts on a second stream of
+            # the same priority: its GEMMs are MFMA-bound, the routed kernels stream weights from HBM
+            cur = torch.cuda.current_stream(self.device)
+            side = self._side if self.overlap_shared else cur
+            if side is not cur:
+                self._fork.record(cur)
+                side.wait_event(self._fork)
+            with torch.cuda.stream(side):
+                gu = F.linear(hidden_states, self._shared_gate_up)
+                si = gu.size(1) // 2
+                sh = F.linear(F.silu(gu[:, :si]) * gu[:, si:], self.shared["down"])
+                if side is not cur:
+                    self._join.record(side)
+                    sh.record_stream(cur)
+        L = self._L
+        L.n, L.x, L.logits = n, ptr(hidden_states), ptr(router_logits)
+        L.shared_out = ptr(sh)
+        st = stream()
+        if sh is not None and self.overlap_shared:
+            check(self._fn(C.byref(L), ROUTED, st))
+            torch.cuda.current_stream(self.device).wait_event(self._join)
+            check(self._fn(C.byref(L), COMBINE, st))
+        else:
+            check(self._fn(C.byref(L), ROUTED | COMBINE, st))
         return self.out[:n]
 
     __call__ = forward

@@ -454,6 +454,40 @@ typedef struct bgmoe_moe_fp8_layer {
 
 int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* layer, bgmoe_stream_t stream);
 
+/* One MXFP4 (W4A16) MoE layer forward on one GPU's share of the experts, masked layout:
+ *   ungrouped sigmoid top-k -> masked dispatch of bf16 rows -> MXFP4 gate_up + SwiGLU -> MXFP4 down ->
+ *   weighted combine (+ the shared expert's output, computed by the caller: a dense bf16 MLP).
+ * Mirrors `ResidentEPMXFP4MoELayer._expert_path` / `forward`
+ * (batchgen/moe/fused_moe_mxfp4_resident.py:709-944) without its collectives and latent projections.
+ * stages: BGMOE_MXFP4_ROUTED runs everything up to the down projection, BGMOE_MXFP4_COMBINE the combine,
+ * their sum both -- so that a caller can run the shared expert on another stream beside the routed part
+ * and join before the combine.  All buffers caller-owned; capturable. */
+enum { BGMOE_MXFP4_ROUTED = 1, BGMOE_MXFP4_COMBINE = 2 };
+typedef struct bgmoe_moe_mxfp4_layer {
+  int32_t n, h, inter, e_total, e_local, expert_start, top_k, max_tokens;
+  float routed_scaling_factor;
+  int32_t shared_mode;            /* as bgmoe_reduce_weighted_scatter                        */
+  const uint16_t* x;              /* [n,h] bf16                                               */
+  const float* logits;            /* [n,e_total] fp32                                         */
+  const float* bias;              /* [e_total] fp32                                           */
+  bgmoe_mxfp4_weight gate, up, down;
+  int32_t* topk_ids;              /* [n,top_k]                                                */
+  float* topk_weights;            /* [n,top_k]                                                */
+  int32_t* expert_counts;         /* [e_local]                                                */
+  int32_t* expert_counters;       /* [e_local]                                                */
+  const int32_t* cu_seqlens;      /* [e_local+1], cu[e] = e*max_tokens (filled by the caller) */
+  int32_t* topk_pos;              /* [n*top_k]                                                */
+  uint16_t* act;                  /* [e_local*max_tokens, h] bf16                             */
+  uint16_t* hmid;                 /* [e_local*max_tokens, inter] bf16                         */
+  uint16_t* y;                    /* [e_local*max_tokens, h] bf16                             */
+  void* workspace;                /* bgmoe_dispatch_workspace_bytes(n*top_k, e_local)         */
+  size_t workspace_bytes;
+  const uint16_t* shared_out;     /* [n,h] bf16 or NULL                                       */
+  uint16_t* out;                  /* [n,h] bf16                                               */
+} bgmoe_moe_mxfp4_layer;
+
+int bgmoe_moe_mxfp4_layer_forward(const bgmoe_moe_mxfp4_layer* layer, int stages, bgmoe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

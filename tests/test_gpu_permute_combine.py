@@ -28,6 +28,8 @@ CASES = [  # n, k, h, e_total, expert_start, e_local
     (100, 2, 131, 64, 32, 8), (700, 8, 256, 256, 0, 256), (4096, 8, 128, 256, 32, 32), (513, 16, 64, 896, 28, 28),
     (200, 8, 128, 256, 0, 256),      # <= 2048 pairs, 256 local experts: the one-block kernel at its limit
     (250, 8, 64, 600, 100, 300),     # <= 2048 pairs, more than 256 local experts: the four-wave one-launch kernel
+    (512, 16, 64, 896, 28, 28),      # 8192 pairs: the one-block kernel's eight sub-steps, at its limit
+    (1000, 8, 64, 256, 0, 256),      # 8000 pairs, 256 local experts
 ]
 
 
