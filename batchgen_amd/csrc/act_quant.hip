@@ -87,10 +87,10 @@ __device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64
           }
           if (hr) {
             uint4 o;
-            o.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
-            o.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
-            o.z = f32_to_bf16_bits(v[4]) | (f32_to_bf16_bits(v[5]) << 16);
-            o.w = f32_to_bf16_bits(v[6]) | (f32_to_bf16_bits(v[7]) << 16);
+            o.x = pack2_bf16(v[0], v[1]);
+            o.y = pack2_bf16(v[2], v[3]);
+            o.z = pack2_bf16(v[4], v[5]);
+            o.w = pack2_bf16(v[6], v[7]);
             *reinterpret_cast<uint4*>(hr + c0) = o;
           }
         }

@@ -75,13 +75,15 @@ static inline hipStream_t bgmoe_stream(bgmoe_stream_t s) { return reinterpret_ca
 // ---- bf16 <-> fp32 -----------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
-// round-to-nearest-even; NaN stays NaN (quiet)
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+// round-to-nearest-even with the hardware convert (v_cvt_pk_bf16_f32: two values per instruction); NaN stays
+// a quiet NaN
+typedef __bf16 bgmoe_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float bgmoe_floatx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+  const bgmoe_floatx2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bgmoe_bf16x2));
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack2_bf16(f, 0.0f) & 0xffffu; }
 
 __device__ __forceinline__ float bf16_round_f32(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 

@@ -251,8 +251,8 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           uint2 o;
-          o.x = f32_to_bf16_bits(hv[tt][j][0]) | (f32_to_bf16_bits(hv[tt][j][1]) << 16);
-          o.y = f32_to_bf16_bits(hv[tt][j][2]) | (f32_to_bf16_bits(hv[tt][j][3]) << 16);
+          o.x = pack2_bf16(hv[tt][j][0], hv[tt][j][1]);
+          o.y = pack2_bf16(hv[tt][j][2], hv[tt][j][3]);
           *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = o;
         }
       }
@@ -291,8 +291,8 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
       for (int t = 0; t < NT; ++t) {
         if (!tv[t]) continue;
         uint2 o;
-        o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
-        o.y = f32_to_bf16_bits(acc[tt][t][2]) | (f32_to_bf16_bits(acc[tt][t][3]) << 16);
+        o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
+        o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
         *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 64 * wave + 16 * t + 4 * kq) = o;
       }
     }

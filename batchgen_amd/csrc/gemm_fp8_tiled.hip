@@ -348,8 +348,8 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
             uint2 o;
-            o.x = f32_to_bf16_bits(acc[tt][j][0]) | (f32_to_bf16_bits(acc[tt][j][1]) << 16);
-            o.y = f32_to_bf16_bits(acc[tt][j][2]) | (f32_to_bf16_bits(acc[tt][j][3]) << 16);
+            o.x = pack2_bf16(acc[tt][j][0], acc[tt][j][1]);
+            o.y = pack2_bf16(acc[tt][j][2], acc[tt][j][3]);
             *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 32 * wn + 16 * j + 4 * kq) = o;
           }
         }
@@ -389,8 +389,8 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
           const int col = n0 + 64 * wn + 16 * t + 4 * kq;
           if (col >= g.n) continue;
           uint2 o;
-          o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
-          o.y = f32_to_bf16_bits(acc[tt][t][2]) | (f32_to_bf16_bits(acc[tt][t][3]) << 16);
+          o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
+          o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
           *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + col) = o;
         }
       }

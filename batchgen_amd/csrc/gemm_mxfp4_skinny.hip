@@ -203,8 +203,8 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
 #pragma unroll
         for (int i = 0; i < 4; ++i) h[i] = silu_f32(acc[tt][j][i]) * acc[tt][j + NH][i];
         uint2 o;
-        o.x = f32_to_bf16_bits(h[0]) | (f32_to_bf16_bits(h[1]) << 16);
-        o.y = f32_to_bf16_bits(h[2]) | (f32_to_bf16_bits(h[3]) << 16);
+        o.x = pack2_bf16(h[0], h[1]);
+        o.y = pack2_bf16(h[2], h[3]);
         *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * j + 4 * kq) = o;
       }
     } else {
@@ -212,8 +212,8 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
       for (int t = 0; t < NT; ++t) {
         if (!tv[t]) continue;
         uint2 o;
-        o.x = f32_to_bf16_bits(acc[tt][t][0]) | (f32_to_bf16_bits(acc[tt][t][1]) << 16);
-        o.y = f32_to_bf16_bits(acc[tt][t][2]) | (f32_to_bf16_bits(acc[tt][t][3]) << 16);
+        o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
+        o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
         *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * t + 4 * kq) = o;
       }
     }

@@ -60,19 +60,23 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_fp8_quant_kernel(NormQuantAr
     const uint4 hh = *reinterpret_cast<const uint4*>(a.hidden + base);
     const uint32_t rw[4] = {rr.x, rr.y, rr.z, rr.w};
     const uint32_t hw[4] = {hh.x, hh.y, hh.z, hh.w};
-    uint32_t ob[8];
+    float sum[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t rb = (i & 1) ? rw[i >> 1] >> 16 : rw[i >> 1] & 0xffffu;
       const uint32_t hb = (i & 1) ? hw[i >> 1] >> 16 : hw[i >> 1] & 0xffffu;
       const float hv = row_valid ? bf16_bits_to_f32(hb) : 0.0f;   // a predicate, never a factor
-      const float sum = bf16_bits_to_f32(rb) + hv;
-      ob[i] = f32_to_bf16_bits(sum);
-      rounded[i] = bf16_bits_to_f32(ob[i]);
-      sum_sq = __builtin_fmaf(sum, sum, sum_sq);
+      sum[i] = bf16_bits_to_f32(rb) + hv;
+      sum_sq = __builtin_fmaf(sum[i], sum[i], sum_sq);
     }
-    *reinterpret_cast<uint4*>(a.residual + base) =
-        make_uint4(ob[0] | (ob[1] << 16), ob[2] | (ob[3] << 16), ob[4] | (ob[5] << 16), ob[6] | (ob[7] << 16));
+    uint32_t ow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ow[i] = pack2_bf16(sum[2 * i], sum[2 * i + 1]);
+      rounded[2 * i] = __uint_as_float(ow[i] << 16);
+      rounded[2 * i + 1] = __uint_as_float(ow[i] & 0xffff0000u);
+    }
+    *reinterpret_cast<uint4*>(a.residual + base) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
   }
   // the reference's tree: 32-lane sums (one per half wave), then those sums through the same tree
   const float wsum = half_wave_sum(sum_sq);
@@ -93,16 +97,16 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_fp8_quant_kernel(NormQuantAr
   const uint4 ww = *reinterpret_cast<const uint4*>(a.weight + (int64_t)t * 8);
   const uint32_t wv[4] = {ww.x, ww.y, ww.z, ww.w};
   float nv[8];
-  uint32_t nb[8];
+  uint32_t nw[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint32_t wb = (i & 1) ? wv[i >> 1] >> 16 : wv[i >> 1] & 0xffffu;
-    const float val = rounded[i] * inv;
-    nb[i] = f32_to_bf16_bits(val * bf16_bits_to_f32(wb));
-    nv[i] = bf16_bits_to_f32(nb[i]);        // the cast sees what a reader of `normed` would see
+  for (int i = 0; i < 4; ++i) {
+    const float w0 = bf16_bits_to_f32(wv[i] & 0xffffu), w1 = __uint_as_float(wv[i] & 0xffff0000u);
+    const float v0 = rounded[2 * i] * inv, v1 = rounded[2 * i + 1] * inv;
+    nw[i] = pack2_bf16(v0 * w0, v1 * w1);
+    nv[2 * i] = __uint_as_float(nw[i] << 16);            // the cast sees what a reader of `normed` would see
+    nv[2 * i + 1] = __uint_as_float(nw[i] & 0xffff0000u);
   }
-  *reinterpret_cast<uint4*>(a.normed + base) =
-      make_uint4(nb[0] | (nb[1] << 16), nb[2] | (nb[3] << 16), nb[4] | (nb[5] << 16), nb[6] | (nb[7] << 16));
+  *reinterpret_cast<uint4*>(a.normed + base) = make_uint4(nw[0], nw[1], nw[2], nw[3]);
   if (quant_skip || !a.q) return;
 
   // 16 consecutive threads share a 128-block; the xor offsets 1..8 stay inside that group
