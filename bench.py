@@ -6,7 +6,7 @@
 A step is one forward pass of the layer (router -> permute+quant -> gate_up/SwiGLU/
 requant GEMM -> down GEMM -> combine + shared expert) over one batch of synthetic
 tokens, with weights and inputs already resident in HBM.  Default workload is
-config 1 of BASELINE.json (DeepSeek-V3-shaped FP8 decode, 256 tokens, 32 of 256
+configuration 1 of the benchmark set (DeepSeek-V3-shaped FP8 decode, 256 tokens, 32 of 256
 experts local, masked layout).  Prints ONE JSON line.
 
 `--op router_gemm` and `--op norm_quant` time the two producers that sit in front of the layer on the same
@@ -160,8 +160,6 @@ def bench_producer(a):
         torch.cuda.synchronize()
     if a.op == "router_gemm":
         from batchgen_amd.moe.routing import router_gemm_gate_sigmoid_topk
-        from oracle import router as orr
-        from oracle import router_gemm as org
         x = (torch.randn(n, h, generator=g, device=dev) * 0.1).to(torch.bfloat16)
         w = (torch.randn(e, h, generator=g, device=dev) * 0.1).to(torch.bfloat16)
         bias = torch.zeros(e, device=dev)
@@ -199,6 +197,8 @@ def bench_producer(a):
                    tokens_per_s=n / (ms * 1e-3), kernel_ms_per_step={kk: v[0] / a.steps for kk, v in prof.items()},
                    roofline=roof)
         if not a.no_cpu_baseline:
+            from oracle import router as orr               # the CPU port is the baseline leg only
+            from oracle import router_gemm as org
             m = min(n, 512)
             xs, wc = x[:m].cpu(), w.cpu()
             t0 = time.perf_counter()
@@ -214,8 +214,6 @@ def bench_producer(a):
                                    "sample": f"{m} of {n} tokens, float64 BLAS product + NumPy router", "seconds": t}
         print(json.dumps(out))
         return
-    from batchgen_amd.attention import cuda_add_rmsnorm_fp8_quant
-    from oracle import norm_quant as onq
     res = (torch.randn(n, h, generator=g, device=dev) * 0.9).to(torch.bfloat16)
     hid = (torch.randn(n, h, generator=g, device=dev) * 0.4).to(torch.bfloat16)
     gamma = (torch.randn(h, generator=g, device=dev) * 0.3 + 1.0).to(torch.bfloat16)
@@ -244,6 +242,7 @@ def bench_producer(a):
                config={"workload": cfg.name + " / add_rmsnorm_fp8_quant", "rows": n, "hidden": h},
                tokens_per_s=n / (ms * 1e-3), roofline=roof)
     if not a.no_cpu_baseline:
+        from oracle import norm_quant as onq               # the CPU port is the baseline leg only
         m = min(n, 256)
         t0 = time.perf_counter()
         onq.add_rmsnorm_fp8_quant(res0[:m].cpu(), hid[:m].cpu(), gamma.cpu(), 1e-5)

@@ -1,5 +1,5 @@
 """Writes tests/golden/c0_layer.npz: inputs' checksums and the oracle's outputs for config 0 of
-BASELINE.json (64 tokens, hidden 1024, intermediate 512, 16 experts, top-4, 4 groups / 2, 1 shared
+the benchmark set (64 tokens, hidden 1024, intermediate 512, 16 experts, top-4, 4 groups / 2, 1 shared
 expert).  The vectors come from this build's own CPU oracle (the reference's kernels cannot run here);
 they freeze the oracle so that a later change to it shows up as a diff, and they give the GPU tests a
 second, file-based target.

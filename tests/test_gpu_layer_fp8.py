@@ -2,7 +2,7 @@
 
 Integer / byte results (router ids, counts, cu_seqlens, topk_pos, quantised activation bytes and scales) are
 bit-exact; the layer output is within 1e-2 relative Frobenius error of the fp32 dequantise-then-matmul oracle
-(the bound BASELINE.json states), in practice ~1e-3.
+(the bound the benchmark definition states), in practice ~1e-3.
 """
 import numpy as np
 import pytest
