@@ -237,3 +237,50 @@ def test_layer_built_from_a_checkpoint(dev, tmp_path, name, fold, weight_layout)
     x = inp["x"].to(dev)
     assert torch.equal(a(x, None), b(x, None))
     assert torch.equal(a(x, inp["logits"].to(dev)), b(x, inp["logits"].to(dev)))
+
+
+def test_producer_chain_replays_from_a_hip_graph(dev):
+    """add + RMSNorm + FP8 cast -> layer (router GEMM + gate inside, pre-quantised tokens) captured as one graph
+    and replayed over changing inputs, eager work in between: every replay equals the eager chain bit for bit."""
+    from batchgen_amd._lib import check, lib, ptr, stream
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = wl.scaled(wl.CONFIGS[1], hidden=1024, inter=512, shared_inter=512)
+    n, h = cfg.n_tokens, cfg.hidden
+    w, sh = wl.make_fp8_weights(cfg, dev)
+    bias = wl.make_inputs(cfg, dev)["bias"]
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    rw = (torch.randn(cfg.n_experts, h, generator=gen) * 0.05).to(torch.bfloat16).to(dev)
+    gamma = (torch.randn(h, generator=gen) * 0.3 + 1.0).to(torch.bfloat16).to(dev)
+    layer = Fp8MoELayer(cfg, w, sh, bias, router_weight=rw)
+    res = [(torch.randn(n, h, generator=gen) * (0.5 + i)).to(torch.bfloat16).to(dev) for i in range(3)]
+    hid = [(torch.randn(n, h, generator=gen) * 0.4).to(torch.bfloat16).to(dev) for _ in range(3)]
+    normed = torch.empty((n, h), dtype=torch.bfloat16, device=dev)
+    xq = torch.empty((n, h), dtype=torch.uint8, device=dev)
+    xs = torch.empty((n, h // 128), dtype=torch.float32, device=dev)
+    r_in, h_in = res[0].clone(), hid[0].clone()
+
+    def chain(r, hd):
+        check(lib().bgmoe_add_rmsnorm_fp8_quant(ptr(r), ptr(hd), ptr(gamma), n, h, 1e-5, ptr(normed), ptr(xq),
+                                                ptr(xs), h // 128, 1, None, None, None, stream()))
+        return layer(normed, None, x_fp8=xq, x_scale=xs)
+
+    eager = [chain(res[i].clone(), hid[i]).clone() for i in range(3)]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain(r_in.clone(), h_in)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = chain(r_in, h_in)
+    for rnd in range(2):
+        for i in (1, 2, 0):
+            r_in.copy_(res[i])                   # the captured kernel updates the residual in place
+            h_in.copy_(hid[i])
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out_static, eager[i]), f"replay of input {i} (round {rnd}) differs from eager"
+            j = (i + 1) % 3
+            assert torch.equal(chain(res[j].clone(), hid[j]), eager[j])      # eager work between replays
