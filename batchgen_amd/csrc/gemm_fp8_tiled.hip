@@ -58,7 +58,11 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
   extern __shared__ __align__(16) uint8_t smem[];      // NS slots
   __shared__ int s_tiles[kMaxGroups + 1];              // exclusive prefix of m-tiles per group
   __shared__ float s_ws[2][2][kMaxKB];                 // [buffer][row] weight scales along K of an item
-  __shared__ float s_amax[2][4][8][16];
+  // the fused epilogue's amax exchange [2][4][8][16] floats, or the plain epilogue's per-wave transpose
+  // patches (16 token rows x 144 B each): never both
+  constexpr int kEpiPitch = 144;
+  __shared__ __align__(16) uint8_t s_scratch[NT / 64 * 16 * kEpiPitch];
+  float (*s_amax)[4][8][16] = reinterpret_cast<float (*)[4][8][16]>(s_scratch);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -380,18 +384,43 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
         }
       }
     } else {
+      // A lane holds 4 consecutive output columns of one token: stored as they are, a store instruction
+      // would touch 16 token rows with 32 bytes each.  Each 16-token tile goes through a per-wave LDS patch
+      // instead (written 8 B per lane, read back 16 B per lane with 8 lanes per token row), so that a store
+      // instruction writes 8 whole 128-byte row segments.  LDS operations of one wave execute in order: no
+      // barrier is needed between the patch's write, its read and the next tile's write.
+      uint8_t* const patch = s_scratch + wave * (16 * kEpiPitch);
+      const int col0 = n0 + 64 * wn;                       // this wave's 64 columns: all inside or all outside N
+      const bool wide = ((uintptr_t)g.out & 15) == 0;
 #pragma unroll
       for (int tt = 0; tt < 8; ++tt) {
-        const int tok = m0 + 128 * wm + 16 * tt + r16;
-        if (tok >= cnt) continue;
+        const int tok0 = m0 + 128 * wm + 16 * tt;
+        if (tok0 >= cnt || col0 >= g.n) continue;          // wave-uniform
+        if (wide) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int col = n0 + 64 * wn + 16 * t + 4 * kq;
-          if (col >= g.n) continue;
-          uint2 o;
-          o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
-          o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
-          *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + col) = o;
+          for (int t = 0; t < 4; ++t) {
+            uint2 o;
+            o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
+            o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
+            *reinterpret_cast<uint2*>(patch + r16 * kEpiPitch + (16 * t + 4 * kq) * 2) = o;
+          }
+#pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            const int row = (lane >> 3) + 8 * i;
+            const uint4 v = *reinterpret_cast<const uint4*>(patch + row * kEpiPitch + (lane & 7) * 16);
+            if (tok0 + row < cnt)
+              *reinterpret_cast<uint4*>(g.out + (row0 + tok0 + row) * g.n + col0 + (lane & 7) * 8) = v;
+          }
+        } else {
+          const int tok = tok0 + r16;
+          if (tok >= cnt) continue;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            uint2 o;
+            o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
+            o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
+            *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + col0 + 16 * t + 4 * kq) = o;
+          }
         }
       }
     }
