@@ -45,7 +45,7 @@ enum BgmoeKernelId {
   BGMOE_K_S1_SKINNY16, BGMOE_K_S1_SKINNY64, BGMOE_K_S1_TILED,
   BGMOE_K_GEMM_SKINNY16, BGMOE_K_GEMM_SKINNY64, BGMOE_K_GEMM_TILED,
   BGMOE_K_MXFP4_S1, BGMOE_K_MXFP4_GEMM, BGMOE_K_BF16_GEMM, BGMOE_K_ROUTER_GEMM, BGMOE_K_ROUTER_GEMM_REDUCE,
-  BGMOE_K_NORM_QUANT,
+  BGMOE_K_NORM_QUANT, BGMOE_K_SITU,
   BGMOE_K_COUNT
 };
 extern bool g_bgmoe_prof_on;
@@ -134,3 +134,14 @@ __device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-
 // same with the hardware reciprocal (1 ulp) instead of the correctly rounded division: for GEMM epilogues that
 // evaluate it 64 times per lane, where the accumulation order already moves the last bits
 __device__ __forceinline__ float silu_rcp_f32(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }
+
+// SiTU-and-multiply (Kimi-K3): beta * tanh(g / beta) * sigmoid(g), times u or, with a linear beta,
+// lbeta * tanh(u / lbeta).  fp32 throughout, the library tanhf / expf and an IEEE division; the divisions by
+// beta are multiplications by the rounded reciprocal, as in the reference kernels
+// (batchgen_kernels/src/moe/marlin_grouped_gemm.cu:243-256, kimi_linear/situ_triton.py:41-45).
+__device__ __forceinline__ float situ_gate_f32(float g, float beta, float inv_beta) {
+  return beta * tanhf(g * inv_beta) * (1.0f / (1.0f + expf(-g)));
+}
+__device__ __forceinline__ float situ_linear_f32(float u, float lbeta, float inv_lbeta) {
+  return lbeta * tanhf(u * inv_lbeta);
+}

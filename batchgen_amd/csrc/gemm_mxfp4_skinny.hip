@@ -37,6 +37,7 @@ struct Mx4Args {
   uint16_t* const* out_ptrs;    // or: per-group output base (row = token index inside the group)
   int lo, hi;
   int64_t row_bound;
+  int activation;               // fused stage 1: BGMOE_ACT_SWIGLU or BGMOE_ACT_SITU
 };
 
 struct Mx4Stage {
@@ -201,7 +202,15 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
       for (int j = 0; j < NH; ++j) {
         float h[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) h[i] = silu_f32(acc[tt][j][i]) * acc[tt][j + NH][i];
+        for (int i = 0; i < 4; ++i) {
+          if (g.activation == BGMOE_ACT_SITU) {
+            // both branches are rounded to bf16 first (marlin_grouped_gemm.cu:1055-1069); beta 4, linear beta 25
+            const float gg = bf16_round_f32(acc[tt][j][i]), uu = bf16_round_f32(acc[tt][j + NH][i]);
+            h[i] = situ_gate_f32(gg, 4.0f, 0.25f) * situ_linear_f32(uu, 25.0f, 0.04f);
+          } else {
+            h[i] = silu_f32(acc[tt][j][i]) * acc[tt][j + NH][i];
+          }
+        }
         uint2 o;
         o.x = pack2_bf16(h[0], h[1]);
         o.y = pack2_bf16(h[2], h[3]);
@@ -369,7 +378,8 @@ extern "C" int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight*
                                     int64_t row_bound, bgmoe_stream_t stream) {
   int rc = check_shape("mxfp4_fused_s1", x, seqlens, cu_seqlens, groups, m, n, k, out, out_ptrs);
   if (rc != BGMOE_OK) return rc;
-  BGMOE_REQUIRE(activation == 0, "mxfp4_fused_s1: only SwiGLU (activation 0) is built");
+  BGMOE_REQUIRE(activation == BGMOE_ACT_SWIGLU || activation == BGMOE_ACT_SITU,
+                "mxfp4_fused_s1: activation must be BGMOE_ACT_SWIGLU (0) or BGMOE_ACT_SITU (1)");
   if (groups == 0 || m == 0) return BGMOE_OK;
   rc = check_w("mxfp4_fused_s1", gate);
   if (rc != BGMOE_OK) return rc;
@@ -378,7 +388,7 @@ extern "C" int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight*
   BGMOE_REQUIRE(gate->layout == up->layout, "mxfp4_fused_s1: gate and up weights must use the same layout");
   Mx4Args g{};
   g.x = x; g.w0 = *gate; g.w1 = *up; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups; g.n = n; g.k = k;
-  g.out = out; g.out_ptrs = out_ptrs; g.row_bound = row_bound;
+  g.out = out; g.out_ptrs = out_ptrs; g.row_bound = row_bound; g.activation = activation;
   return launch(true, g, m, bgmoe_stream(stream));
 }
 

@@ -130,7 +130,7 @@ extern "C" int bgmoe_moe_mxfp4_layer_forward(const bgmoe_moe_mxfp4_layer* L, int
     if (rc != BGMOE_OK) return rc;
     const int64_t bound = (int64_t)n * k;
     rc = bgmoe_mxfp4_fused_s1(L->act, &L->gate, &L->up, L->expert_counts, L->cu_seqlens, el, rows, inter, h,
-                              L->hmid, nullptr, 0, bound, stream);
+                              L->hmid, nullptr, L->activation, bound, stream);
     if (rc != BGMOE_OK) return rc;
     rc = bgmoe_mxfp4_grouped_gemm(L->hmid, &L->down, L->expert_counts, L->cu_seqlens, el, rows, h, inter, L->y,
                                   nullptr, bound, stream);

@@ -14,7 +14,7 @@
 namespace {
 
 struct NormQuantArgs {
-  uint16_t* residual;          // [rows,h] bf16, updated in place
+  uint16_t* residual;          // [rows,h] bf16, updated in place; nullptr: plain RMSNorm of `hidden`
   const uint16_t* hidden;      // [rows,h] bf16
   const uint16_t* weight;      // [h] bf16
   uint16_t* normed;            // [rows,h] bf16
@@ -56,8 +56,8 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_fp8_quant_kernel(NormQuantAr
   float rounded[8];
   float sum_sq = 0.0f;
   if (live) {
-    const uint4 rr = *reinterpret_cast<const uint4*>(a.residual + base);
     const uint4 hh = *reinterpret_cast<const uint4*>(a.hidden + base);
+    const uint4 rr = a.residual ? *reinterpret_cast<const uint4*>(a.residual + base) : hh;
     const uint32_t rw[4] = {rr.x, rr.y, rr.z, rr.w};
     const uint32_t hw[4] = {hh.x, hh.y, hh.z, hh.w};
     float sum[8];
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_fp8_quant_kernel(NormQuantAr
       const uint32_t rb = (i & 1) ? rw[i >> 1] >> 16 : rw[i >> 1] & 0xffffu;
       const uint32_t hb = (i & 1) ? hw[i >> 1] >> 16 : hw[i >> 1] & 0xffffu;
       const float hv = row_valid ? bf16_bits_to_f32(hb) : 0.0f;   // a predicate, never a factor
-      sum[i] = bf16_bits_to_f32(rb) + hv;
+      sum[i] = a.residual ? bf16_bits_to_f32(rb) + hv : hv;
       sum_sq = __builtin_fmaf(sum[i], sum[i], sum_sq);
     }
     uint32_t ow[4];
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_fp8_quant_kernel(NormQuantAr
       rounded[2 * i] = __uint_as_float(ow[i] << 16);
       rounded[2 * i + 1] = __uint_as_float(ow[i] & 0xffff0000u);
     }
-    *reinterpret_cast<uint4*>(a.residual + base) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    if (a.residual) *reinterpret_cast<uint4*>(a.residual + base) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
   }
   // the reference's tree: 32-lane sums (one per half wave), then those sums through the same tree
   const float wsum = half_wave_sum(sum_sq);
@@ -158,4 +158,22 @@ extern "C" int bgmoe_add_rmsnorm_fp8_quant(uint16_t* residual, const uint16_t* h
   BgmoeProf prof(BGMOE_K_NORM_QUANT, st);
   hipLaunchKernelGGL(add_rmsnorm_fp8_quant_kernel, dim3((unsigned)rows), dim3(threads), 0, st, a);
   return bgmoe_check_launch("add_rmsnorm_fp8_quant");
+}
+
+// Plain RMSNorm: the kernel above without a residual (the row itself is what gets normalised, and nothing is
+// written back), so the sum of squares, the reciprocal square root and the rounding are the fused op's.
+extern "C" int bgmoe_rmsnorm(const uint16_t* x, const uint16_t* weight, int64_t rows, int h, float eps,
+                             uint16_t* out, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(rows >= 0 && rows <= 0x7fffffffLL, "rmsnorm: bad row count %lld", (long long)rows);
+  BGMOE_REQUIRE(h >= 8 && h <= 8192 && h % 8 == 0, "rmsnorm: hidden size %d must be a multiple of 8 in [8, 8192]", h);
+  if (rows == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(x && weight && out, "rmsnorm: null pointer");
+  BGMOE_REQUIRE(((uintptr_t)x | (uintptr_t)weight | (uintptr_t)out) % 16 == 0, "rmsnorm: operands must be 16-byte aligned");
+  NormQuantArgs a{};
+  a.hidden = x; a.weight = weight; a.normed = out; a.eps = eps; a.h = h;
+  hipStream_t st = bgmoe_stream(stream);
+  const int threads = ((h / 8) + BGMOE_WAVE - 1) / BGMOE_WAVE * BGMOE_WAVE;
+  BgmoeProf prof(BGMOE_K_NORM_QUANT, st);
+  hipLaunchKernelGGL(add_rmsnorm_fp8_quant_kernel, dim3((unsigned)rows), dim3(threads), 0, st, a);
+  return bgmoe_check_launch("rmsnorm");
 }

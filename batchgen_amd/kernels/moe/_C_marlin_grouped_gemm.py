@@ -6,8 +6,11 @@ The op names and positional argument orders are the reference's.  The pointer ta
 in THIS build's resident layout (tile-major by default, made by ``mxfp4_weight_repack`` from the
 checkpoint layout packed ``[N, K/2]`` + scales ``[N, K/32]``); the reference's Marlin register layout is
 an NVIDIA ``ldmatrix`` / ``mma.m16n8k16`` artefact and is not reproduced.  ``workspace``, ``n_tiles``
-and ``max_m_tiles`` are accepted and ignored.  The stage-1 activation is SwiGLU (the benchmark's config);
-the reference model's SiTU is not built.  INT4 ops of that extension are out of scope.
+and ``max_m_tiles`` are accepted and ignored.  ``grouped_marlin_gemm_m16_s1_mxfp4_situ`` applies the
+reference op's activation, SiTU with beta 4 / linear beta 25 on the bf16-rounded branches
+(batchgen_kernels/src/moe/marlin_grouped_gemm.cu:243-256, :1055-1069); the stacked-weight form
+``mxfp4_fused_s1`` takes ``activation="swiglu"`` (the benchmark's config) or ``"situ"``.  INT4 ops of that
+extension are out of scope.
 """
 from __future__ import annotations
 
@@ -19,6 +22,7 @@ from ..._lib import Mxfp4Weight, check, lib, ptr, stream
 from .. import _checks as ck
 
 _LAYOUT = {"row_major": 0, "tile_major": 1}
+ACTIVATIONS = {"swiglu": 0, "situ": 1}      # BGMOE_ACT_SWIGLU, BGMOE_ACT_SITU
 
 
 def mxfp4_weight_repack(w_packed, scales):
@@ -53,7 +57,7 @@ def _counts(expert_starts, expert_counts, e):
 def grouped_marlin_gemm_m16_s1_mxfp4_situ(x, gate_B_ptrs, up_B_ptrs, C_ptrs, gate_scales_ptrs, up_scales_ptrs,
                                           expert_starts, expert_counts, E, N, K, workspace=None, n_tiles=None,
                                           max_m_tiles=None, weight_layout="tile_major"):
-    """Fused gate + up + activation, bf16 result written through C_ptrs[e] (token t of expert e at
+    """Fused gate + up + SiTU, bf16 result written through C_ptrs[e] (token t of expert e at
     C_ptrs[e] + t*N).  Zero-count experts are skipped on the device; the caller must not filter them."""
     ck.cuda_tensor(None, x, torch.bfloat16, "x")
     if x.dim() != 2 or x.size(1) != K:
@@ -67,7 +71,8 @@ def grouped_marlin_gemm_m16_s1_mxfp4_situ(x, gate_B_ptrs, up_B_ptrs, C_ptrs, gat
     wu = _tbl(up_B_ptrs, up_scales_ptrs, E, weight_layout)
     with torch.cuda.device(x.device):
         check(lib().bgmoe_mxfp4_fused_s1(ptr(x), C.byref(wg), C.byref(wu), ptr(expert_counts), ptr(expert_starts),
-                                         int(E), x.size(0), int(N), int(K), None, ptr(C_ptrs), 0, 0, stream()))
+                                         int(E), x.size(0), int(N), int(K), None, ptr(C_ptrs), ACTIVATIONS["situ"],
+                                         0, stream()))
     return None
 
 
@@ -97,9 +102,11 @@ def _stack(wp, sc, layout):
 
 
 def mxfp4_fused_s1(x, gate_p, gate_s, up_p, up_s, seqlens, cu_seqlens, output=None, weight_layout="row_major",
-                   row_bound=0):
+                   row_bound=0, activation="swiglu"):
     """Stacked-weight form: x [M,K] bf16; gate/up packed [G,N,K/2] + scales [G,N,K/32]; out [M,N] bf16,
     rows [cu[g], cu[g]+seqlens[g]) of group g."""
+    if activation not in ACTIVATIONS:
+        ck.fail(f"activation must be one of {sorted(ACTIVATIONS)}")
     ck.cuda_tensor(None, x, torch.bfloat16, "x")
     for t, name in ((gate_p, "gate_p"), (gate_s, "gate_s"), (up_p, "up_p"), (up_s, "up_s")):
         ck.cuda_tensor(x, t, torch.uint8, name)
@@ -114,7 +121,7 @@ def mxfp4_fused_s1(x, gate_p, gate_s, up_p, up_s, seqlens, cu_seqlens, output=No
     wg, wu = _stack(gate_p, gate_s, weight_layout), _stack(up_p, up_s, weight_layout)
     with torch.cuda.device(x.device):
         check(lib().bgmoe_mxfp4_fused_s1(ptr(x), C.byref(wg), C.byref(wu), ptr(seqlens), ptr(cu_seqlens), g, m, n, k,
-                                         ptr(output), None, 0, int(row_bound), stream()))
+                                         ptr(output), None, ACTIVATIONS[activation], int(row_bound), stream()))
     return output
 
 

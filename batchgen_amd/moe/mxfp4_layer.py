@@ -1,11 +1,18 @@
 """MXFP4 (W4A16) MoE layer forward on one GPU's share of the experts.
 
 Host-side counterpart of ``ResidentEPMXFP4MoELayer._expert_path`` / ``forward``
-(batchgen/moe/fused_moe_mxfp4_resident.py:709-944) without the latent projections and collectives:
-ungrouped sigmoid top-k router -> masked dispatch of bf16 rows -> grouped MXFP4 gate_up + SwiGLU ->
+(batchgen/moe/fused_moe_mxfp4_resident.py:709-944) without the collectives:
+ungrouped sigmoid top-k router -> masked dispatch of bf16 rows -> grouped MXFP4 gate_up + activation ->
 grouped MXFP4 down -> fp32 weighted combine + shared expert.  Weights are repacked once into the
 tile-major resident layout (the reference repacks to Marlin at the same point, :13-15).
 The shared expert is a plain dense bf16 MLP and runs on the library GEMM (hipBLASLt through torch).
+
+With ``latent`` weights the layer is the Kimi-K3 latent MoE (:922-944, kimi_linear/model.py:585-603): the
+router sees the hidden rows, ``down_proj`` takes them to the latent width once per token, the experts and
+the combine work on latent rows, then RMSNorm (optional) and ``up_proj`` bring the result back, and the
+shared expert's output is added.  The two projections are plain bf16 GEMMs and run on the library GEMM, as
+``nn.Linear`` does in the reference.  ``activation="situ"`` selects the K3 activation for the routed experts
+(fused into the stage-1 GEMM) and the shared expert (``situ_and_mul``).
 """
 from __future__ import annotations
 
@@ -19,6 +26,7 @@ import torch.nn.functional as F
 from .. import _lib
 from .._lib import Mxfp4Weight, check, lib, ptr, stream
 from ..kernels import load_extension
+from .latent import rmsnorm, situ_and_mul
 from ..workloads import MoEConfig
 
 
@@ -34,19 +42,34 @@ class Mxfp4LayerStruct(C.Structure):
         ("gate", Mxfp4Weight), ("up", Mxfp4Weight), ("down", Mxfp4Weight),
         ("topk_ids", vp), ("topk_weights", vp), ("expert_counts", vp), ("expert_counters", vp), ("cu_seqlens", vp),
         ("topk_pos", vp), ("act", vp), ("hmid", vp), ("y", vp), ("workspace", vp), ("workspace_bytes", sz),
-        ("shared_out", vp), ("out", vp),
+        ("shared_out", vp), ("out", vp), ("activation", i32),
     ]
 
 
 _lib.register("bgmoe_moe_mxfp4_layer_forward", i32, [C.POINTER(Mxfp4LayerStruct), i32, vp])
 ROUTED, COMBINE = 1, 2
+ACTIVATIONS = {"swiglu": 0, "situ": 1}
+K3_SITU_BETA, K3_SITU_LINEAR_BETA = 4.0, 25.0   # the constants the fused stage-1 epilogue compiles in
 
 
 class Mxfp4MoELayer:
-    def __init__(self, cfg: MoEConfig, weights, shared_bf16, bias: torch.Tensor, shared_mode: str = "bf16_add"):
+    def __init__(self, cfg: MoEConfig, weights, shared_bf16, bias: torch.Tensor, shared_mode: str = "bf16_add",
+                 latent=None):
         self.cfg = cfg
         dev = weights["gate_p"].device
         self.device = dev
+        if cfg.activation not in ACTIVATIONS:
+            raise ValueError(f"activation must be one of {sorted(ACTIVATIONS)}, got {cfg.activation!r}")
+        if bool(cfg.latent) != (latent is not None):
+            raise ValueError("latent weights are needed exactly when cfg.latent is set")
+        self.latent = latent
+        if latent is not None:
+            for name, shape in (("down_proj", (cfg.latent, cfg.hidden)), ("up_proj", (cfg.hidden, cfg.latent))):
+                t = latent[name]
+                if t.dtype != torch.bfloat16 or tuple(t.shape) != shape or not t.is_contiguous():
+                    raise ValueError(f"latent[{name!r}] must be contiguous BF16 {shape}")
+            if cfg.latent_norm != (latent.get("norm_weight") is not None):
+                raise ValueError("latent['norm_weight'] is needed exactly when cfg.latent_norm is set")
         with torch.cuda.device(dev):
             check(lib().bgmoe_init())
         mg = load_extension("batchgen_kernels.moe._C_marlin_grouped_gemm")
@@ -63,7 +86,7 @@ class Mxfp4MoELayer:
             self._side = torch.cuda.Stream(device=dev)
             self._fork, self._join = torch.cuda.Event(), torch.cuda.Event()
         self.bias = bias.to(dev, torch.float32).contiguous()
-        n, h, inter, el, k = cfg.n_tokens, cfg.hidden, cfg.inter, cfg.e_local, cfg.top_k
+        n, h, inter, el, k = cfg.n_tokens, cfg.expert_hidden, cfg.inter, cfg.e_local, cfg.top_k
         if cfg.layout != "masked":
             raise ValueError("the MXFP4 layer uses the masked layout")
         self.rows = el * cfg.max_tokens
@@ -91,6 +114,7 @@ class Mxfp4MoELayer:
         L.topk_pos, L.act, L.hmid, L.y = ptr(self.topk_pos), ptr(self.act), ptr(self.hmid), ptr(self.y)
         L.workspace, L.workspace_bytes = ptr(self.workspace), self.workspace.numel()
         L.out = ptr(self.out)
+        L.activation = ACTIVATIONS[cfg.activation]
         self._L = L
         self._fn = lib().bgmoe_moe_mxfp4_layer_forward
 
@@ -103,10 +127,10 @@ class Mxfp4MoELayer:
                 not router_logits.is_contiguous() or not hidden_states.is_contiguous():
             raise RuntimeError(f"router_logits must be contiguous FP32 [{n}, {cfg.n_experts}] and hidden_states contiguous")
         sh = None
+        cur = torch.cuda.current_stream(self.device)
         if self.shared is not None:
             # the dense bf16 shared expert (vendor GEMMs) runs beside the routed experts on a second stream of
             # the same priority: its GEMMs are MFMA-bound, the routed kernels stream weights from HBM
-            cur = torch.cuda.current_stream(self.device)
             side = self._side if self.overlap_shared else cur
             if side is not cur:
                 self._fork.record(cur)
@@ -114,20 +138,40 @@ class Mxfp4MoELayer:
             with torch.cuda.stream(side):
                 gu = F.linear(hidden_states, self._shared_gate_up)
                 si = gu.size(1) // 2
-                sh = F.linear(F.silu(gu[:, :si]) * gu[:, si:], self.shared["down"])
+                if cfg.activation == "situ":
+                    hh = situ_and_mul(gu, K3_SITU_BETA, K3_SITU_LINEAR_BETA)
+                else:
+                    hh = F.silu(gu[:, :si]) * gu[:, si:]
+                sh = F.linear(hh, self.shared["down"])
                 if side is not cur:
                     self._join.record(side)
                     sh.record_stream(cur)
+        x_exp = hidden_states
+        if self.latent is not None:
+            x_exp = F.linear(hidden_states, self.latent["down_proj"])      # hidden -> latent, once per token
         L = self._L
-        L.n, L.x, L.logits = n, ptr(hidden_states), ptr(router_logits)
-        L.shared_out = ptr(sh)
+        L.n, L.x, L.logits = n, ptr(x_exp), ptr(router_logits)
+        # latent: the shared expert's rows are hidden-sized and join after the latent -> hidden projection
+        L.shared_out = ptr(sh) if self.latent is None else None
         st = stream()
-        if sh is not None and self.overlap_shared:
+        joined = False
+        if sh is not None and self.overlap_shared and self.latent is None:
             check(self._fn(C.byref(L), ROUTED, st))
-            torch.cuda.current_stream(self.device).wait_event(self._join)
+            cur.wait_event(self._join)
+            joined = True
             check(self._fn(C.byref(L), COMBINE, st))
         else:
             check(self._fn(C.byref(L), ROUTED | COMBINE, st))
-        return self.out[:n]
+        if self.latent is None:
+            return self.out[:n]
+        y = self.out[:n]
+        if self.latent.get("norm_weight") is not None:
+            y = rmsnorm(y, self.latent["norm_weight"], self.latent["eps"])
+        y = F.linear(y, self.latent["up_proj"])                            # latent -> hidden
+        if sh is not None:
+            if self.overlap_shared and not joined:
+                cur.wait_event(self._join)
+            y = y + sh
+        return y
 
     __call__ = forward

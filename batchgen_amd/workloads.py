@@ -38,10 +38,17 @@ class MoEConfig:
     row_align: int        # ragged
     weight_format: str    # "fp8" | "mxfp4"
     zipf_s: float = 0.0
+    latent: int = 0       # > 0: routed experts work on rows of this width (hidden -> latent -> hidden projections)
+    activation: str = "swiglu"   # "swiglu" | "situ"
+    latent_norm: bool = False    # RMSNorm between the combined latent rows and the latent -> hidden projection
 
     @property
     def seed(self) -> int:
         return SEED0 + self.index
+
+    @property
+    def expert_hidden(self) -> int:
+        return self.latent or self.hidden
 
 
 CONFIGS = {
@@ -55,6 +62,13 @@ CONFIGS = {
     4: MoEConfig("c4_dsv3_fp8_zipf_8k_all_experts", 4, 8192, 7168, 2048, 256, 256, 0, 8, 8, 4, 2.5, 2048,
                  "ragged", 0, 128, "fp8", zipf_s=1.2),
 }
+
+# The Kimi-K3 model's own MoE layer (config 3 is its benchmark stand-in with SwiGLU and no latent seam):
+# hidden 7168 -> latent 3584 once per token, 896 MXFP4 experts of intermediate size 3072 with the SiTU
+# activation on latent rows, fp32 combine, RMSNorm, latent -> hidden, plus one bf16 SiTU shared expert on the
+# hidden rows (batchgen/models/moonshotai/kimi_linear/model.py:520-603, k3/mxfp4_expert.py:291-313).
+K3_LATENT = MoEConfig("k3_latent_mxfp4_decode_512tok_ep32", 5, 512, 7168, 3072, 896, 28, 0, 16, 1, 1, 1.0, 3072,
+                      "masked", 512, 16, "mxfp4", latent=3584, activation="situ", latent_norm=True)
 
 
 def scaled(cfg: MoEConfig, **kw) -> MoEConfig:
@@ -150,8 +164,8 @@ def make_mxfp4_weights(cfg: MoEConfig, device):
     dev = torch.device(device)
     gen = torch.Generator(device=dev).manual_seed(cfg.seed + 1)
     w = {}
-    for name, (n, k) in (("gate", (cfg.inter, cfg.hidden)), ("up", (cfg.inter, cfg.hidden)),
-                         ("down", (cfg.hidden, cfg.inter))):
+    eh = cfg.expert_hidden
+    for name, (n, k) in (("gate", (cfg.inter, eh)), ("up", (cfg.inter, eh)), ("down", (eh, cfg.inter))):
         p = torch.empty((cfg.e_local, n, k // 2), dtype=torch.uint8, device=dev)
         s = torch.empty((cfg.e_local, n, k // 32), dtype=torch.uint8, device=dev)
         for i in range(cfg.e_local):
@@ -166,12 +180,27 @@ def make_mxfp4_weights(cfg: MoEConfig, device):
     return w, sh
 
 
+def make_latent_weights(cfg: MoEConfig, device):
+    """The latent seam's bf16 tensors: down_proj [latent, hidden], up_proj [hidden, latent], norm weight [latent]
+    (None without ``latent_norm``)."""
+    dev = torch.device(device)
+    gen = torch.Generator(device=dev).manual_seed(cfg.seed + 2)
+    down = (torch.randn((cfg.latent, cfg.hidden), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    up = (torch.randn((cfg.hidden, cfg.latent), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+    norm = None
+    if cfg.latent_norm:
+        norm = (torch.randn(cfg.latent, generator=gen, device=dev) * 0.2 + 1.0).to(torch.bfloat16)
+    return dict(down_proj=down, up_proj=up, norm_weight=norm, eps=1e-5)
+
+
 def algorithmic_bytes_mxfp4(cfg: MoEConfig, active_experts: int, routed_rows: int) -> int:
-    h, i = cfg.hidden, cfg.inter
-    total = active_experts * (3 * h * i // 2 + 3 * h * i // 32)
+    h, i, eh = cfg.hidden, cfg.inter, cfg.expert_hidden
+    total = active_experts * (3 * eh * i // 2 + 3 * eh * i // 32)
     if cfg.shared_inter:
         total += 3 * h * cfg.shared_inter * 2
-    total += cfg.n_tokens * h * 2 * 2 + routed_rows * (2 * h + 2 * i) * 2
+    total += cfg.n_tokens * h * 2 * 2 + routed_rows * (2 * eh + 2 * i) * 2
+    if cfg.latent:     # the two projections' weights, and the latent rows written and read around the experts
+        total += 2 * h * eh * 2 + cfg.n_tokens * eh * 2 * 4
     return int(total)
 
 

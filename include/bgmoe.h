@@ -379,14 +379,39 @@ int bgmoe_mxfp4_grouped_gemm(const uint16_t* x, const bgmoe_mxfp4_weight* w, con
                              uint16_t* out, uint16_t* const* out_ptrs, int64_t row_bound,
                              bgmoe_stream_t stream);
 
-/* out = bf16( act(x Wg^T) * (x Wu^T) ).  Replaces `marlin_grouped_stage1_fused_mxfp4_situ`
- * (batchgen/moe/marlin_grouped_moe.py:411-470).  activation 0 = SwiGLU (silu), the activation of
- * the benchmark's Kimi-K3-shaped config; the reference model's SiTU epilogue is not built. */
+/* Stage-1 activations.  SWIGLU: out = bf16( silu(g) * u ) on the fp32 accumulators (the benchmark's
+ * Kimi-K3-shaped config).  SITU: the Kimi-K3 model's own activation, with the constants the reference
+ * kernel compiles in (batchgen_kernels/src/moe/marlin_grouped_gemm.cu:243-256; asserted against the
+ * config at kimi_linear/k3/mxfp4_expert.py:302-312): g and u are rounded to bf16 first (:1055-1069), then
+ *   out = bf16( 4*tanh(g/4)*sigmoid(g) * 25*tanh(u/25) )   in fp32. */
+enum { BGMOE_ACT_SWIGLU = 0, BGMOE_ACT_SITU = 1 };
+
+/* out = act(x Wg^T, x Wu^T).  Replaces `marlin_grouped_stage1_fused_mxfp4_situ`
+ * (batchgen/moe/marlin_grouped_moe.py:411-470) with activation = BGMOE_ACT_SITU. */
 int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight* gate,
                          const bgmoe_mxfp4_weight* up, const int32_t* seqlens,
                          const int32_t* cu_seqlens, int groups, int64_t m, int n, int k, uint16_t* out,
                          uint16_t* const* out_ptrs, int activation, int64_t row_bound,
                          bgmoe_stream_t stream);
+
+/* ------------------------------------------------- Kimi-K3 latent-MoE seam */
+
+/* out[r, c] = bf16( beta*tanh(g/beta)*sigmoid(g) * u' ),  g = x[r, c], u = x[r, d + c] (bf16 -> fp32),
+ * u' = linear_beta*tanh(u/linear_beta) when linear_beta > 0, else u.  One rounding, to bf16.
+ * Replaces `situ_and_mul_triton` (batchgen/models/moonshotai/kimi_linear/situ_triton.py:55-77), the
+ * activation of the Kimi-K3 shared expert and dense MLP (`SituAndMul`, kimi_linear/model.py:84-115).
+ * x is [rows, 2d] with row stride x_row_stride (elements), out [rows, d] with out_row_stride. */
+int bgmoe_situ_and_mul(const uint16_t* x, int64_t rows, int d, int64_t x_row_stride, float beta,
+                       float linear_beta, uint16_t* out, int64_t out_row_stride, bgmoe_stream_t stream);
+
+/* out[r, :] = bf16( x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight ): fp32 math, one rounding.
+ * Replaces `triton_rmsnorm` / `cuda_rmsnorm` as used by `KimiRMSNorm.forward`
+ * (batchgen/models/moonshotai/kimi_linear/rmsnorm_triton.py:24-44, kimi_linear/model.py:192-205): the norm
+ * between the combined latent rows and the latent -> hidden projection.  The sum of squares follows the
+ * same fixed tree as bgmoe_add_rmsnorm_fp8_quant and the reciprocal square root is the correctly rounded
+ * one.  h a multiple of 8, at most 8192; x, weight and out bf16, 16-byte aligned; out may alias x. */
+int bgmoe_rmsnorm(const uint16_t* x, const uint16_t* weight, int64_t rows, int h, float eps, uint16_t* out,
+                  bgmoe_stream_t stream);
 
 /* ------------------------------------------------------------ whole layer */
 
@@ -484,6 +509,7 @@ typedef struct bgmoe_moe_mxfp4_layer {
   size_t workspace_bytes;
   const uint16_t* shared_out;     /* [n,h] bf16 or NULL                                       */
   uint16_t* out;                  /* [n,h] bf16                                               */
+  int32_t activation;             /* BGMOE_ACT_SWIGLU or BGMOE_ACT_SITU                       */
 } bgmoe_moe_mxfp4_layer;
 
 int bgmoe_moe_mxfp4_layer_forward(const bgmoe_moe_mxfp4_layer* layer, int stages, bgmoe_stream_t stream);

@@ -17,6 +17,7 @@ import torch
 
 from .quant import act_dequant, act_quant, bf16_round, swiglu_bf16, weight_block_dequant
 from . import mxfp4 as _mx
+from . import situ as _situ
 
 F32 = np.float32
 
@@ -100,11 +101,12 @@ def grouped_gemm_mxfp4(x_bf16, w_packed, w_scales, seqlens, cu_seqlens, to_bf16=
     return bf16_round(out) if to_bf16 else out
 
 
-def expert_mlp_mxfp4(x, gate_p, gate_s, up_p, up_s, down_p, down_s, seqlens, cu_seqlens):
-    """bf16 activations, MXFP4 weights, SwiGLU with a bf16 intermediate."""
+def expert_mlp_mxfp4(x, gate_p, gate_s, up_p, up_s, down_p, down_s, seqlens, cu_seqlens, activation="swiglu"):
+    """bf16 activations, MXFP4 weights, a bf16 intermediate: SwiGLU on the fp32 products, or SiTU on the
+    bf16-rounded ones (``oracle.situ.situ_fused``)."""
     g = grouped_gemm_mxfp4(x, gate_p, gate_s, seqlens, cu_seqlens, to_bf16=False)
     u = grouped_gemm_mxfp4(x, up_p, up_s, seqlens, cu_seqlens, to_bf16=False)
-    h = swiglu_bf16(g, u)
+    h = _situ.situ_fused(g, u) if activation == "situ" else swiglu_bf16(g, u)
     y = grouped_gemm_mxfp4(h, down_p, down_s, seqlens, cu_seqlens, to_bf16=True)
     return y, h
 

@@ -27,6 +27,7 @@ from . import mxfp4 as _mx
 from . import permute as _pm
 from . import quant as _q
 from . import router as _rt
+from . import situ as _situ
 
 F32 = np.float32
 
@@ -82,26 +83,47 @@ def moe_layer_fp8(x, logits, bias, rcfg, w, expert_start, num_local,
 
 def moe_layer_mxfp4(x, logits, bias, rcfg, w, expert_start, num_local,
                     layout="masked", max_tokens=0, row_align=16, shared_bf16=None,
-                    shared_mode="bf16_add"):
+                    shared_mode="bf16_add", activation="swiglu", latent=None):
     """bf16 activations, MXFP4 routed experts (w = dict(gate_p,gate_s,up_p,up_s,
-    down_p,down_s)), bf16 shared expert (dict(gate,up,down) float32 holding bf16)."""
+    down_p,down_s)), bf16 shared expert (dict(gate,up,down) float32 holding bf16).
+
+    ``latent`` = dict(down_proj [L,H], up_proj [H,L], norm_weight [L] or None, eps) selects the Kimi-K3
+    latent-MoE data flow (kimi_linear/model.py:585-603, fused_moe_mxfp4_resident.py:922-944): the router sees
+    the hidden rows, the experts the rows of bf16(x @ down_proj^T); their fp32-combined output is rounded to
+    bf16, normalised, projected back with up_proj (bf16), and the shared expert's bf16 output -- computed from
+    the hidden rows with the same activation -- is added in bf16."""
     x = _q.as_f32(x)
     n, h = x.shape
     ids, wt = route(logits, bias, rcfg)
     k = ids.shape[1]
     counts, cu, pos, rows = _permute(ids, expert_start, num_local, layout, max_tokens, row_align)
-    xr = _pm.gather_rows(x, pos, k, max(rows, 1))
+    x_exp = x if latent is None else _q.bf16_round(_gm._mm(x, _q.as_f32(latent["down_proj"])))
+    xr = _pm.gather_rows(x_exp, pos, k, max(rows, 1))
     y, hmid = _gm.expert_mlp_mxfp4(xr, w["gate_p"], w["gate_s"], w["up_p"], w["up_s"],
-                                   w["down_p"], w["down_s"], counts, cu)
+                                   w["down_p"], w["down_s"], counts, cu, activation=activation)
     y_sh = None
     if shared_bf16 is not None:
         g = _gm._mm(x, shared_bf16["gate"])
         u = _gm._mm(x, shared_bf16["up"])
-        hh = _q.swiglu_bf16(g, u)
+        if activation == "situ":       # the module form: bf16 [gate | up] -> SituAndMul -> bf16
+            hh = _situ.situ_and_mul(np.concatenate([_q.bf16_round(g), _q.bf16_round(u)], axis=-1),
+                                    _situ.K3_BETA, _situ.K3_LINEAR_BETA)
+        else:
+            hh = _q.swiglu_bf16(g, u)
         y_sh = _q.bf16_round(_gm._mm(hh, shared_bf16["down"]))
-    out = _cb.reduce_weighted_scatter(y, pos, wt, n, k, shared=y_sh, shared_mode=shared_mode)
+    if latent is None:
+        out = _cb.reduce_weighted_scatter(y, pos, wt, n, k, shared=y_sh, shared_mode=shared_mode)
+        y_lat = None
+    else:
+        y_lat = _cb.reduce_weighted_scatter(y, pos, wt, n, k)
+        z = y_lat
+        if latent.get("norm_weight") is not None:
+            z = _situ.rmsnorm(z, latent["norm_weight"], latent["eps"])
+        out = _q.bf16_round(_gm._mm(z, _q.as_f32(latent["up_proj"])))
+        if y_sh is not None:
+            out = _q.bf16_round(out + y_sh)
     return dict(out=out, ids=ids, weights=wt, counts=counts, cu=cu, pos=pos, x_rows=xr, h=hmid,
-                y=y, y_shared=y_sh)
+                y=y, y_shared=y_sh, y_latent=y_lat, x_latent=x_exp if latent is not None else None)
 
 
 def moe_layer_dense_bruteforce(x, ids, wt, expert_fn, n_experts_start, num_local):

@@ -100,7 +100,7 @@ def test_reference_op_names_with_pointer_tables(dev):
     c_ptrs = torch.tensor([c[int(cu[i])].data_ptr() for i in range(e)], dtype=torch.int64, device=dev)
     mg().grouped_marlin_gemm_m16_s1_mxfp4_situ(x, tbl(gpt), tbl(upt), c_ptrs, tbl(gst), tbl(ust), cu_d, cnt_d, e, n, k,
                                                None, n // 256, 4)
-    ref = mg().mxfp4_fused_s1(x, gpt, gst, upt, ust, cnt_d, d(cu), weight_layout="tile_major")
+    ref = mg().mxfp4_fused_s1(x, gpt, gst, upt, ust, cnt_d, d(cu), weight_layout="tile_major", activation="situ")
     live = torch.zeros(m, dtype=torch.bool)
     for i, cc in enumerate(counts):
         live[cu[i]:cu[i] + cc] = True
