@@ -229,4 +229,4 @@ def algorithmic_bytes_fp8(cfg: MoEConfig, active_experts: int, routed_rows: int)
 
 
 def flops_routed(cfg: MoEConfig, routed_rows: int) -> int:
-    return int(routed_rows) * 6 * cfg.hidden * cfg.inter
+    return int(routed_rows) * 6 * cfg.expert_hidden * cfg.inter

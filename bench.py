@@ -40,6 +40,7 @@ MEASURED_TRAFFIC_BYTES = {
     2: int((3093.6 + 83.5) * MIB),    # fp8_tiled_kernel<fused,tile_major>, config 2
     3: int((227.5 + 0.7) * MIB),      # mxfp4_skinny_kernel<4,3,fused,tile_major>, config 3
     4: int((6065.8 + 154.8) * MIB),   # fp8_tiled_kernel<fused,tile_major>, config 4
+    5: int((186.7 + 1.9) * MIB),      # mxfp4_skinny_kernel<4,3,fused,tile_major>, Kimi-K3 latent layer
 }
 
 
@@ -57,7 +58,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4])
+    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4, 5],
+                    help="0-4: the benchmark set's configurations; 5: the Kimi-K3 latent MoE layer at its real shape")
     ap.add_argument("--op", default="layer", choices=["layer", "router_gemm", "norm_quant"],
                     help="what one step is: the MoE layer (default), or one of its two producers")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -114,9 +116,10 @@ def cpu_baseline(cfg, inp, w, sh, ids, wt, alg_bytes, flops):
                               f"bf16 dequantised weights, 1 warm-up + median of {reps}", frac
 
 
-def cpu_baseline_mxfp4(cfg, inp, w, sh):
+def cpu_baseline_mxfp4(cfg, inp, w, sh, lat=None):
     """The NumPy restatement of the MXFP4 layer (oracle.layer.moe_layer_mxfp4: dequantise, bf16-valued GEMMs,
     SwiGLU, combine) on a few tokens; its cost is dominated by dequantising the experts those tokens use."""
+    import torch
     from oracle import layer as ol
     n = min(cfg.n_tokens, 8)
     wn = {k: v.cpu().numpy() for k, v in w.items()}
@@ -124,7 +127,9 @@ def cpu_baseline_mxfp4(cfg, inp, w, sh):
     t0 = time.perf_counter()
     ol.moe_layer_mxfp4(inp["x"][:n].cpu(), inp["logits"][:n].cpu().numpy(), inp["bias"].cpu().numpy(),
                        dict(top_k=cfg.top_k, n_group=1, topk_group=1, rsf=cfg.rsf), wn, cfg.expert_start,
-                       cfg.e_local, layout="masked", max_tokens=cfg.max_tokens, shared_bf16=shn)
+                       cfg.e_local, layout="masked", max_tokens=cfg.max_tokens, shared_bf16=shn,
+                       activation=cfg.activation,
+                       latent=None if lat is None else {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in lat.items()})
     t = time.perf_counter() - t0
     return t, n / cfg.n_tokens, f"{n} of {cfg.n_tokens} tokens of the workload and the experts they route to, one pass, NumPy"
 
@@ -274,13 +279,15 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    cfg = wl.CONFIGS[a.config]
+    cfg = wl.K3_LATENT if a.config == 5 else wl.CONFIGS[a.config]
     inp = wl.make_inputs(cfg, dev)
     mx4 = cfg.weight_format == "mxfp4"
+    lat = None
     if mx4:
         from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
         w, sh = wl.make_mxfp4_weights(cfg, dev)
-        layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"])
+        lat = wl.make_latent_weights(cfg, dev) if cfg.latent else None
+        layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat)
     else:
         w, sh = wl.make_fp8_weights(cfg, dev)
         layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
@@ -314,8 +321,9 @@ def main():
     active = int((counts > 0).sum())
     rows = int(counts.sum())
     alg_bytes = wl.algorithmic_bytes_mxfp4(cfg, active, rows) if mx4 else wl.algorithmic_bytes_fp8(cfg, active, rows)
-    flops = wl.flops_routed(cfg, rows) + (wl.flops_routed(cfg, cfg.n_tokens) * cfg.shared_inter // cfg.inter
-                                          if cfg.shared_inter else 0)
+    flops = wl.flops_routed(cfg, rows) + (cfg.n_tokens * 6 * cfg.hidden * cfg.shared_inter if cfg.shared_inter else 0)
+    if cfg.latent:
+        flops += cfg.n_tokens * 4 * cfg.hidden * cfg.latent
     decode = cfg.layout == "masked"
     gbps = alg_bytes / (ms * 1e-3) / 1e9
     tflops = flops / (ms * 1e-3) / 1e12
@@ -330,7 +338,8 @@ def main():
     h, i = cfg.hidden, cfg.inter
     if mx4:
         dom = "mxfp4_s1"
-        dom_bytes = active * (2 * h * i // 2 + 2 * h * i // 32) + rows * (h + i) * 2
+        eh = cfg.expert_hidden
+        dom_bytes = active * (2 * eh * i // 2 + 2 * eh * i // 32) + rows * (eh + i) * 2
         dom_ms = prof[dom][0] / max(prof[dom][1], 1)
         roof = dict(bound="hbm", kernel="mxfp4_skinny_kernel<TT=4,NS=3,fused,tile_major>",
                     achieved=dom_bytes / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None,
@@ -368,7 +377,8 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "launch": "hip_graph" if a.graph else "eager",
         "dtype": "mxfp4 weights x bf16 (fp32 accumulate)" if mx4 else "fp8_e4m3 (fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": cfg.name, "tokens": cfg.n_tokens, "hidden": h, "moe_intermediate": i,
+        "config": {"workload": cfg.name, "tokens": cfg.n_tokens, "hidden": h, "latent": cfg.latent or None,
+                   "activation": cfg.activation, "moe_intermediate": i,
                    "experts": cfg.n_experts, "local_experts": cfg.e_local, "top_k": cfg.top_k,
                    "layout": cfg.layout, "shared_expert": bool(cfg.shared_inter)},
         "tokens_per_s": cfg.n_tokens / (ms * 1e-3),
@@ -379,7 +389,7 @@ def main():
         "roofline": roof,
     }
     if not a.no_cpu_baseline and mx4:
-        t, frac, sample = cpu_baseline_mxfp4(cfg, inp, w, sh)
+        t, frac, sample = cpu_baseline_mxfp4(cfg, inp, w, sh, lat)
         out["cpu_baseline"] = {"value": alg_bytes * frac / t / 1e9, "unit": out["unit"],
                                "cores": min(os.cpu_count() or 1, 16), "host_cores": os.cpu_count() or 1,
                                "kind": "port", "sample": sample + " (BLAS threads for the matrix products, one thread for the dequantisation)", "seconds": t,
