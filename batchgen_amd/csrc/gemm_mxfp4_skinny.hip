@@ -234,13 +234,13 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
 // columns per item) when that already gives every resident block an item, else with 2 tiles per wave --
 // fp4 weight stages are small, so with few items twice as many narrower ones keep more loads in flight.
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
-__global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned vblocks) {
+__global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned vblocks, unsigned slots) {
   __shared__ __align__(16) uint8_t s_ring[NSTAGE * TT * 4096];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
   const int wide_cols = FUSED ? 128 : 256;
   const int ntiles_wide = (g.n + wide_cols - 1) / wide_cols;
   const int chunks = bgmoe_total_chunks(g.seqlens, g.groups, g.lo, g.hi, 16 * TT);
-  const bool narrow = (int64_t)chunks * ((ntiles_wide + 7) & ~7) < (int64_t)gridDim.x;
+  const bool narrow = (int64_t)chunks * ((ntiles_wide + 7) & ~7) < (int64_t)slots;   // slots: blocks resident at once
   if (narrow) {
     const int ntiles = (g.n + wide_cols / 2 - 1) / (wide_cols / 2);
     for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
@@ -310,9 +310,14 @@ unsigned mx_resident() {
 
 template <int TT, int NS, bool FUSED, int LAYOUT>
 void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
-  const unsigned resident = mx_resident<TT, NS, FUSED, LAYOUT>();
-  const dim3 grid(vblocks < resident ? vblocks : resident), block(256);
-  hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks);
+  // Twice as many blocks as fit at once: with up to two rounds of items every block has one item and the
+  // hardware hands the second round out as blocks finish, which evens out items of unequal length (a 64-row
+  // item takes 1.7x a 16-row one); beyond that the blocks stride.  Measured: skewed counts 14% faster,
+  // uniform ones 3% slower (the late blocks' start-up).
+  const unsigned slots = mx_resident<TT, NS, FUSED, LAYOUT>();
+  const dim3 grid(vblocks < 2 * slots ? vblocks : 2 * slots), block(256);
+  hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks,
+                     vblocks < slots ? vblocks : slots);
 }
 
 constexpr int kMxTT = 4;           // 64-row items: every group is streamed once per 64 rows
