@@ -394,6 +394,19 @@ int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight* gate,
                          uint16_t* const* out_ptrs, int activation, int64_t row_bound,
                          bgmoe_stream_t stream);
 
+/* ---------------------------------------------------------------- self-check */
+
+/* The routers' sigmoid is the correctly rounded fp32 one (fp64 evaluation rounded once: the reference
+ * compiles its gate with fast-math, batchgen_kernels/setup.py:245, so its own `1/(1+expf(-x))`,
+ * gate_sigmoid_topk.cu:88, is not a reproducible function).  The kernels take a short fp64 evaluation when
+ * it provably rounds the same way and the library evaluation otherwise; this call runs both on the `count`
+ * float bit patterns starting at `first_bits` and adds the number of inputs whose results differ in any bit
+ * to *mismatches (device memory, caller-zeroed; 0 is the only acceptable value) and, when fallbacks is not
+ * NULL, the number of inputs the short evaluation hands to the library one to *fallbacks.  No counterpart
+ * in the reference. */
+int bgmoe_selfcheck_sigmoid(uint32_t first_bits, uint64_t count, uint64_t* mismatches, uint64_t* fallbacks,
+                            bgmoe_stream_t stream);
+
 /* ------------------------------------------------- Kimi-K3 latent-MoE seam */
 
 /* out[r, c] = bf16( beta*tanh(g/beta)*sigmoid(g) * u' ),  g = x[r, c], u = x[r, d + c] (bf16 -> fp32),
