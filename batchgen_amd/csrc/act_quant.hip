@@ -103,8 +103,7 @@ __device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64
       const float sc = quant_scale_from_amax(amax);
       if (in) {
         float q[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = clamp448(v[i] / sc);
+        quant_div_clamp(v, sc, q);
         uint2 o;
         o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
         o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
@@ -133,7 +132,9 @@ __device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64
       float amax = fmaxf(fabsf(v[0]), fabsf(v[1]));
       amax = wave_max_xor<64>(amax);
       const float sc = quant_scale_from_amax(amax);
-      const uint32_t p = pack4_e4m3(clamp448(v[0] / sc), clamp448(v[1] / sc), 0.0f, 0.0f);
+      float q2[2];
+      quant_div_clamp(v, sc, q2);
+      const uint32_t p = pack4_e4m3(q2[0], q2[1], 0.0f, 0.0f);
       if (c0 < k) yr[c0] = (uint8_t)(p & 0xff);
       if (c0 + 1 < k) yr[c0 + 1] = (uint8_t)((p >> 8) & 0xff);
       if (lane == 0) sr[(int64_t)b * a.skb] = sc;
@@ -204,22 +205,25 @@ __global__ __launch_bounds__(256) void scatter_quant_kernel(QuantArgs a, int ste
     uint2 o;
     {
       float q[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) q[i] = clamp448(v[i] / sc);
+      quant_div_clamp(v, sc, q);
       o.x = pack4_e4m3(q[0], q[1], q[2], q[3]);
       o.y = pack4_e4m3(q[4], q[5], q[6], q[7]);
     }
     const bool lead = (lane & 15) == 0;
-    const int ndst = a.topk + (tok < extra_rows ? 1 : 0);
-    // all destinations of the token in one load (lane j holds destination j), not one dependent load per route
-    int64_t mine = -1;
+    // all destinations of the token in one load (lane j holds destination j), not one dependent load per
+    // route; only the live ones (local routes, the identity row) are visited
+    int mine = -1;
     if (lane < a.topk) mine = a.topk_pos[tok * a.topk + lane];
-    else if (lane == a.topk && tok < extra_rows) mine = a.extra_start + tok;
-    for (int j = 0; j < ndst; ++j) {
-      const int64_t dst = __shfl(mine, j, BGMOE_WAVE);
-      if (dst < 0 || !in) continue;
-      *reinterpret_cast<uint2*>(a.y + dst * (int64_t)k + c0) = o;
-      if (lead) a.scale[dst * a.srow + (int64_t)(c0 >> 7) * a.skb] = sc;
+    else if (lane == a.topk && tok < extra_rows) mine = (int)(a.extra_start + tok);
+    unsigned long long live = __ballot(mine >= 0);
+    while (live) {
+      const int j = __ffsll((long long)live) - 1;
+      live &= live - 1;
+      const int64_t dst = __builtin_amdgcn_readlane(mine, j);
+      if (in) {
+        *reinterpret_cast<uint2*>(a.y + dst * (int64_t)k + c0) = o;
+        if (lead) a.scale[dst * a.srow + (int64_t)(c0 >> 7) * a.skb] = sc;
+      }
     }
   }
 }
@@ -245,13 +249,14 @@ __global__ __launch_bounds__(256) void scatter_fp8_kernel(const uint8_t* xq, con
     float sc = 0.0f;
     if (in) bytes = *reinterpret_cast<const uint4*>(xq + tok * (int64_t)k + c0);
     if (has_scale) sc = xs[tok * xs_row + (int64_t)kb * xs_kb];
-    const int ndst = a.topk + (tok < extra_rows ? 1 : 0);
-    int64_t mine = -1;
+    int mine = -1;
     if (lane < a.topk) mine = a.topk_pos[tok * a.topk + lane];
-    else if (lane == a.topk && tok < extra_rows) mine = a.extra_start + tok;
-    for (int j = 0; j < ndst; ++j) {
-      const int64_t dst = __shfl(mine, j, BGMOE_WAVE);
-      if (dst < 0) continue;
+    else if (lane == a.topk && tok < extra_rows) mine = (int)(a.extra_start + tok);
+    unsigned long long live = __ballot(mine >= 0);
+    while (live) {
+      const int j = __ffsll((long long)live) - 1;
+      live &= live - 1;
+      const int64_t dst = __builtin_amdgcn_readlane(mine, j);
       if (in) *reinterpret_cast<uint4*>(a.y + dst * (int64_t)k + c0) = bytes;
       if (has_scale) a.scale[dst * a.srow + (int64_t)kb * a.skb] = sc;
     }
@@ -395,4 +400,56 @@ extern "C" int bgmoe_scatter_fp8_rows(const uint8_t* xq, const float* xs, int64_
   BGMOE_REQUIRE(xq && xs && y && scale && topk_pos, "scatter_fp8_rows: null pointer");
   return bgmoe_internal_scatter_fp8(xq, xs, xs_row_stride, xs_kb_stride, topk_pos, n, k, h, y, scale,
                                     scale_row_stride, scale_kb_stride, 0, 0, bgmoe_stream(stream));
+}
+
+namespace {
+__device__ __forceinline__ uint32_t mix32(uint64_t v) {
+  v ^= v >> 33; v *= 0xff51afd7ed558ccdULL; v ^= v >> 33; v *= 0xc4ceb9fe1a85ec53ULL; v ^= v >> 33;
+  return (uint32_t)v;
+}
+// Pseudo-random (s, x) pairs from the quantisers' domain: s anywhere in (1e-30, 1e30), |x| <= 448.5 * s, x
+// either a full fp32 value or rounded down to bf16 (what the quantisers are fed).  Counts the pairs whose
+// short division differs from the IEEE one in the e4m3 byte, and in any bit of a normal-range quotient.
+__global__ __launch_bounds__(256) void scale_division_selfcheck_kernel(uint64_t seed, uint64_t count,
+                                                                       unsigned long long* byte_mismatches,
+                                                                       unsigned long long* bit_mismatches) {
+  unsigned long long bad_byte = 0, bad_bits = 0;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint32_t h0 = mix32(seed + 2 * i), h1 = mix32(seed + 2 * i + 1);
+    const int ex = 28 + (int)(h0 >> 23) % 199;                               // biased exponent 28 .. 226
+    const float s = __uint_as_float(((uint32_t)ex << 23) | (h0 & 0x7fffffu));
+    if (!scale_div_ok(s)) continue;
+    const float t = (float)(h1 >> 8) * (1.0f / 16777216.0f) * 448.5f;        // [0, 448.5)
+    float x = t * s;
+    if (h1 & 1u) x = __uint_as_float(__float_as_uint(x) & 0xffff0000u);      // a bf16 value
+    if (h1 & 2u) x = -x;
+    if ((h1 & 0xfcu) == 0) x = (h1 & 2u) ? -0.0f : 0.0f;                     // signed zeros now and then
+    const float r = 1.0f / s;
+    const float a = div_by_scale(x, s, r), b = x / s;
+    const uint32_t pa = pack4_e4m3(clamp448(a), 0.0f, 0.0f, 0.0f) & 0xffu;
+    const uint32_t pb = pack4_e4m3(clamp448(b), 0.0f, 0.0f, 0.0f) & 0xffu;
+    bad_byte += pa != pb;
+    bad_bits += fabsf(b) >= 1.17549435e-38f && __float_as_uint(a) != __float_as_uint(b);
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    bad_byte += __shfl_xor(bad_byte, off, BGMOE_WAVE);
+    bad_bits += __shfl_xor(bad_bits, off, BGMOE_WAVE);
+  }
+  if (lane_id() == 0) {
+    if (bad_byte) atomicAdd(byte_mismatches, bad_byte);
+    if (bad_bits) atomicAdd(bit_mismatches, bad_bits);
+  }
+}
+}  // namespace
+
+extern "C" int bgmoe_selfcheck_scale_division(uint64_t seed, uint64_t count, uint64_t* byte_mismatches,
+                                              uint64_t* bit_mismatches, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(byte_mismatches && bit_mismatches, "selfcheck_scale_division: null counter");
+  if (count == 0) return BGMOE_OK;
+  uint64_t blocks = (count + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  hipLaunchKernelGGL(scale_division_selfcheck_kernel, dim3((unsigned)blocks), dim3(256), 0, bgmoe_stream(stream), seed,
+                     count, reinterpret_cast<unsigned long long*>(byte_mismatches),
+                     reinterpret_cast<unsigned long long*>(bit_mismatches));
+  return bgmoe_check_launch("selfcheck_scale_division");
 }

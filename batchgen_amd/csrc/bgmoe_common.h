@@ -98,6 +98,32 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 // clamp as fmaxf(fminf(q, 448), -448): a NaN q becomes +448, as in the reference quantiser
 __device__ __forceinline__ float clamp448(float q) { return fmaxf(fminf(q, 448.0f), -448.0f); }
 
+// x / s for many x and one s, bit for bit the IEEE quotient at a third of its instructions: with r = RN(1/s),
+// q0 = RN(x*r) is within one ulp of x/s, e = x - q0*s is exact in an fma, and RN(q0 + e*r) is the correctly
+// rounded quotient (Markstein's division step).  Valid while nothing over- or underflows: callers use it for
+// s in (1e-30, 1e30) and |x/s| of order 448 at most (s comes from the block's amax), and take the IEEE
+// division otherwise.  An exact quotient (e == 0, which includes x = +-0) is returned as it is, so a zero keeps
+// its sign; quotients below 2^-126 may differ from the IEEE denormal in the last place and round to the same
+// signed zero in e4m3.  bgmoe_selfcheck_scale_division compares the two on the device.
+__device__ __forceinline__ bool scale_div_ok(float s) { return s > 1e-30f && s < 1e30f; }
+__device__ __forceinline__ float div_by_scale(float x, float s, float r) {
+  const float q0 = x * r;
+  const float e = __builtin_fmaf(-q0, s, x);
+  return e == 0.0f ? q0 : __builtin_fmaf(e, r, q0);
+}
+// q[i] = clamp(x[i] / s, +-448) for the N values of a lane that share the scale s
+template <int N>
+__device__ __forceinline__ void quant_div_clamp(const float (&x)[N], float s, float (&q)[N]) {
+  if (scale_div_ok(s)) {
+    const float r = 1.0f / s;
+#pragma unroll
+    for (int i = 0; i < N; ++i) q[i] = fmaxf(fminf(div_by_scale(x[i], s, r), 448.0f), -448.0f);
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; ++i) q[i] = fmaxf(fminf(x[i] / s, 448.0f), -448.0f);
+  }
+}
+
 // scale of one 128-block from its amax: fmaxf(amax, 1e-12f) * (1.0f / 448.0f)
 __device__ __forceinline__ float quant_scale_from_amax(float amax) {
   constexpr float kInv448 = 1.0f / 448.0f;

@@ -273,8 +273,9 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
         if (xv[tt]) {
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            const uint32_t q = pack4_e4m3(clamp448(hv[tt][j][0] / sc), clamp448(hv[tt][j][1] / sc),
-                                          clamp448(hv[tt][j][2] / sc), clamp448(hv[tt][j][3] / sc));
+            float qv[4];
+            quant_div_clamp(hv[tt][j], sc, qv);
+            const uint32_t q = pack4_e4m3(qv[0], qv[1], qv[2], qv[3]);
             *reinterpret_cast<uint32_t*>(g.out_q + (row0 + tok) * g.n + n0 + 32 * wave + 16 * j + 4 * kq) = q;
           }
           if (wave == 0 && kq == 0)

@@ -374,8 +374,10 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
           if (tok < cnt) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-              const uint32_t q = pack4_e4m3(clamp448(acc[tt][j][0] / sc), clamp448(acc[tt][j][1] / sc),
-                                            clamp448(acc[tt][j][2] / sc), clamp448(acc[tt][j][3] / sc));
+              const float hv[4] = {acc[tt][j][0], acc[tt][j][1], acc[tt][j][2], acc[tt][j][3]};
+              float qv[4];
+              quant_div_clamp(hv, sc, qv);
+              const uint32_t q = pack4_e4m3(qv[0], qv[1], qv[2], qv[3]);
               *reinterpret_cast<uint32_t*>(g.out_q + (row0 + tok) * g.n + n0 + 32 * wn + 16 * j + 4 * kq) = q;
             }
             if (wn == 0 && kq == 0)

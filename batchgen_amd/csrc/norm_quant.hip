@@ -118,11 +118,9 @@ __global__ __launch_bounds__(1024) void add_rmsnorm_fp8_quant_kernel(NormQuantAr
   constexpr float kInv448 = static_cast<float>(1.0 / 448.0);
   const float sc = fmaxf(amax * kInv448, 1e-12f);
   float qv[8];
+  quant_div_clamp(nv, sc, qv);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float qq = clamp448(nv[i] / sc);
-    qv[i] = fabsf(qq) < 1e30f ? qq : 0.0f;
-  }
+  for (int i = 0; i < 8; ++i) qv[i] = fabsf(qv[i]) < 1e30f ? qv[i] : 0.0f;
   *reinterpret_cast<uint2*>(a.q + base) =
       make_uint2(pack4_e4m3(qv[0], qv[1], qv[2], qv[3]), pack4_e4m3(qv[4], qv[5], qv[6], qv[7]));
   if ((t & 15) == 0) a.scale[row * a.srow + (int64_t)(t >> 4) * a.skb] = sc;

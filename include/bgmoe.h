@@ -407,6 +407,16 @@ int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight* gate,
 int bgmoe_selfcheck_sigmoid(uint32_t first_bits, uint64_t count, uint64_t* mismatches, uint64_t* fallbacks,
                             bgmoe_stream_t stream);
 
+/* The quantisers divide by the block scale exactly as IEEE fp32 division does (the reference's forms A-D
+ * all use a true division or `x * (1/s)`; see bgmoe_act_quant_rows) but compute the quotient as
+ * q0 = x*r, e = fma(-q0, s, x), q = fma(e, r, q0) with r = 1/s once per block.  This call draws `count`
+ * pseudo-random (s, x) pairs from the quantisers' domain (s in (1e-30, 1e30), |x| <= 448.5 s, x fp32 or
+ * bf16, signed zeros) and adds to *byte_mismatches the pairs whose e4m3 byte differs between the two
+ * divisions and to *bit_mismatches those whose normal-range quotients differ in any bit (device memory,
+ * caller-zeroed; both must stay 0).  No counterpart in the reference. */
+int bgmoe_selfcheck_scale_division(uint64_t seed, uint64_t count, uint64_t* byte_mismatches,
+                                   uint64_t* bit_mismatches, bgmoe_stream_t stream);
+
 /* ------------------------------------------------- Kimi-K3 latent-MoE seam */
 
 /* out[r, c] = bf16( beta*tanh(g/beta)*sigmoid(g) * u' ),  g = x[r, c], u = x[r, d + c] (bf16 -> fp32),

@@ -1,5 +1,7 @@
-"""The routers' short sigmoid evaluation against the library evaluation, over EVERY float bit pattern: the two
-must agree in all bits (NaN with NaN), and the short path must decide almost always."""
+"""Device self-checks of two exact short cuts.  The routers' short sigmoid evaluation against the library
+evaluation, over EVERY float bit pattern: the two must agree in all bits (NaN with NaN), and the short path
+must decide almost always.  The quantisers' division by the block scale against the IEEE division, on 2^34
+pseudo-random pairs from the quantisers' domain: identical e4m3 bytes and identical quotient bits."""
 import numpy as np
 import pytest
 import torch
@@ -42,3 +44,16 @@ def test_router_scores_still_match_the_oracle_on_awkward_logits(dev):
     gate_sigmoid_topk_cuda(logits.to(dev), bias.to(dev), 8, 1.0, ids, w)
     rid, rw = orr.gate_sigmoid_topk(logits.numpy(), bias.numpy(), 8, 1.0)
     assert np.array_equal(ids.cpu().numpy(), rid) and np.array_equal(w.cpu().numpy(), rw)
+
+
+def test_scale_division_equals_ieee_division(dev):
+    from batchgen_amd._lib import check, lib, ptr
+    counters = torch.zeros(2, dtype=torch.int64, device=dev)
+    for part in range(4):
+        say("scale-division self-check, part", part)
+        check(lib().bgmoe_selfcheck_scale_division(20261125 + part * (1 << 40), 1 << 32, ptr(counters[0:1]),
+                                                   ptr(counters[1:2]), None))
+        torch.cuda.synchronize()
+    bad_bytes, bad_bits = counters.cpu().tolist()
+    say("   e4m3 byte mismatches", bad_bytes, "quotient bit mismatches", bad_bits)
+    assert bad_bytes == 0 and bad_bits == 0

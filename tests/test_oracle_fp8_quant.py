@@ -111,3 +111,21 @@ def test_bf16_round_matches_torch():
     g = torch.Generator().manual_seed(4)
     x = torch.randn(100000, generator=g) * 3
     assert np.array_equal(oq.bf16_round(x.numpy()), x.to(torch.bfloat16).float().numpy())
+
+
+def test_short_scale_division_model_equals_ieee_division():
+    """The device quantisers compute x / s as q0 = x*r, e = fma(-q0, s, x), q = fma(e, r, q0) with r = 1/s.
+    Modelled here with a correctly rounded float32 fma, the step gives the IEEE quotient for scales and
+    values from the quantisers' domain (the device repeats the comparison on 2^34 pairs)."""
+    from oracle.norm_quant import fma_f32
+    rng = np.random.default_rng(77)
+    n = 1_000_000
+    s = (np.exp2(rng.uniform(-99, 99, n)) * rng.uniform(1, 2, n)).astype(np.float32)
+    x = (rng.uniform(-448.5, 448.5, n) * s.astype(np.float64)).astype(np.float32)
+    half = n // 2
+    x[:half] = (x[:half].view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)      # bf16 values
+    r = (np.float32(1.0) / s).astype(np.float32)
+    q0 = (x * r).astype(np.float32)
+    e = fma_f32(-q0, s, x)
+    q = np.where(e == 0, q0, fma_f32(e, r, q0))
+    assert np.array_equal(q.view(np.uint32), (x / s).astype(np.float32).view(np.uint32))
