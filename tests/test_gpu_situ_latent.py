@@ -226,3 +226,45 @@ def test_latent_situ_layer_full_size_sample(dev):
     err = og.rel_frobenius(out[sub].float().cpu().numpy(), ref["out"])
     say("   rel frobenius of the sample vs oracle:", err)
     assert err < 1e-2
+
+
+def test_new_entry_points_reject_bad_arguments(dev):
+    from batchgen_amd._lib import Mxfp4Weight, lib, ptr
+    import ctypes as C
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device=dev)
+    w = torch.ones(64, dtype=torch.bfloat16, device=dev)
+    y = torch.zeros_like(x)
+    L = lib()
+    assert L.bgmoe_rmsnorm(ptr(x), ptr(w), 4, 12, 1e-5, ptr(y), None) != 0                  # h not a multiple of 8
+    assert b"multiple of 8" in L.bgmoe_last_error()
+    assert L.bgmoe_rmsnorm(ptr(x), ptr(w), 4, 16384, 1e-5, ptr(y), None) != 0               # h too large
+    assert L.bgmoe_rmsnorm(x.data_ptr() + 2, ptr(w), 4, 56, 1e-5, ptr(y), None) != 0        # misaligned rows
+    assert L.bgmoe_rmsnorm(None, ptr(w), 4, 64, 1e-5, ptr(y), None) != 0
+    assert L.bgmoe_rmsnorm(None, None, 0, 64, 1e-5, None, None) == 0                        # nothing to do
+    assert L.bgmoe_selfcheck_sigmoid(0, 16, None, None, None) != 0
+    assert L.bgmoe_selfcheck_scale_division(1, 16, None, None, None) != 0
+    # an unknown activation code is refused before any launch
+    cnt = torch.tensor([4], dtype=torch.int32, device=dev)
+    cu = torch.tensor([0, 4], dtype=torch.int32, device=dev)
+    xk = torch.zeros(4, 128, dtype=torch.bfloat16, device=dev)
+    wp = torch.zeros(1, 128, 64, dtype=torch.uint8, device=dev)
+    ws = torch.full((1, 128, 4), 127, dtype=torch.uint8, device=dev)
+    out = torch.zeros(4, 128, dtype=torch.bfloat16, device=dev)
+    desc = Mxfp4Weight(ptr(wp), 128 * 64, None, ptr(ws), 128 * 4, None, 0, 0)
+    rc = L.bgmoe_mxfp4_fused_s1(ptr(xk), C.byref(desc), C.byref(desc), ptr(cnt), ptr(cu), 1, 4, 128, 128, ptr(out), None,
+                                2, 0, None)
+    assert rc != 0 and b"activation" in L.bgmoe_last_error()
+    with pytest.raises(RuntimeError):
+        _mg().mxfp4_fused_s1(xk, wp, ws, wp, ws, cnt, cu, activation="gelu")
+    from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
+    cfg = wl.scaled(wl.K3_LATENT, n_tokens=16, hidden=256, latent=128, inter=128, shared_inter=0, n_experts=32, e_local=4,
+                    max_tokens=16)
+    wts, _ = wl.make_mxfp4_weights(cfg, dev)
+    bias = torch.zeros(cfg.n_experts, device=dev)
+    with pytest.raises(ValueError):
+        Mxfp4MoELayer(cfg, wts, None, bias)                                                 # latent weights missing
+    lat = wl.make_latent_weights(cfg, dev)
+    with pytest.raises(ValueError):
+        Mxfp4MoELayer(cfg, wts, None, bias, latent=dict(lat, norm_weight=None))             # norm weight missing
+    with pytest.raises(ValueError):
+        Mxfp4MoELayer(wl.scaled(cfg, activation="gelu"), wts, None, bias, latent=lat)
