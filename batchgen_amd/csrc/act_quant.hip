@@ -403,6 +403,104 @@ extern "C" int bgmoe_scatter_fp8_rows(const uint8_t* xq, const float* xs, int64_
 }
 
 namespace {
+struct GroupQuantArgs {
+  const uint16_t* gate;
+  const uint16_t* up;
+  int64_t ise, iss;
+  const int32_t* counts;
+  const int32_t* starts;
+  int groups;
+  int64_t max_rows;
+  int n, form;
+  uint8_t* out;
+  int64_t ose, oss;
+  float* scale;
+  int64_t sse, sss, ssg;
+  uint16_t* prod;
+};
+
+// One wave per (group, row): 8 columns per lane and pass, 16 lanes per 128-column quantisation group.
+__global__ __launch_bounds__(256) void silu_mul_group_quant_kernel(GroupQuantArgs a) {
+  const int lane = lane_id();
+  const int64_t jobs = (int64_t)a.groups * a.max_rows;
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  for (int64_t job = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); job < jobs; job += stride) {
+    const int e = (int)(job / a.max_rows);
+    const int64_t r = job - (int64_t)e * a.max_rows;
+    if (a.counts && r >= a.counts[e]) continue;
+    const int64_t row = (a.starts ? (int64_t)a.starts[e] : 0) + r;
+    const uint16_t* gp = a.gate + e * a.ise + row * a.iss;
+    const uint16_t* upp = a.up + e * a.ise + row * a.iss;
+    uint8_t* op = a.out + e * a.ose + row * a.oss;
+    float* sp = a.scale + e * a.sse + row * a.sss;
+    for (int c0 = lane * 8; c0 < a.n; c0 += 512) {
+      const uint4 gv = *reinterpret_cast<const uint4*>(gp + c0);
+      const uint4 uv = *reinterpret_cast<const uint4*>(upp + c0);
+      const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+      float p[8];
+      uint32_t pw[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t sw = pack2_bf16(silu_exact_f32(__uint_as_float(gw[j] << 16)),
+                                       silu_exact_f32(__uint_as_float(gw[j] & 0xffff0000u)));
+        pw[j] = pack2_bf16(__uint_as_float(sw << 16) * __uint_as_float(uw[j] << 16),
+                           __uint_as_float(sw & 0xffff0000u) * __uint_as_float(uw[j] & 0xffff0000u));
+        p[2 * j] = __uint_as_float(pw[j] << 16);
+        p[2 * j + 1] = __uint_as_float(pw[j] & 0xffff0000u);
+      }
+      if (a.prod)
+        *reinterpret_cast<uint4*>(a.prod + e * a.ose + row * a.oss + c0) = make_uint4(pw[0], pw[1], pw[2], pw[3]);
+      float amax = fabsf(p[0]);
+#pragma unroll
+      for (int i = 1; i < 8; ++i) amax = fmaxf(amax, fabsf(p[i]));
+      amax = wave_max_xor<16>(amax);
+      float sc, q[8];
+      if (a.form == 1) {
+        sc = fmaxf(amax, 1e-10f) / 448.0f;
+        quant_div_clamp(p, sc, q);
+      } else {
+        constexpr float kInv448 = static_cast<float>(1.0 / 448.0);
+        sc = fmaxf(fmaxf(amax, 1.52587890625e-05f) * kInv448, 1e-12f);
+        quant_div_clamp(p, sc, q);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = fabsf(q[i]) < 1e30f ? q[i] : 0.0f;
+      }
+      *reinterpret_cast<uint2*>(op + c0) = make_uint2(pack4_e4m3(q[0], q[1], q[2], q[3]), pack4_e4m3(q[4], q[5], q[6], q[7]));
+      if ((lane & 15) == 0) sp[(int64_t)(c0 >> 7) * a.ssg] = sc;
+    }
+  }
+}
+}  // namespace
+
+extern "C" int bgmoe_silu_mul_group_quant(const uint16_t* gate, const uint16_t* up, int64_t in_stride_e,
+                                          int64_t in_stride_s, const int32_t* counts, const int32_t* starts,
+                                          int groups, int64_t max_rows, int n, int form, uint8_t* out,
+                                          int64_t out_stride_e, int64_t out_stride_s, float* scale,
+                                          int64_t scale_stride_e, int64_t scale_stride_s, int64_t scale_stride_g,
+                                          uint16_t* prod_out, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(groups >= 0 && max_rows >= 0, "silu_mul_group_quant: negative size");
+  BGMOE_REQUIRE(n > 0 && n % 128 == 0, "silu_mul_group_quant: width %d must be a positive multiple of the quant group 128", n);
+  BGMOE_REQUIRE(form == 0 || form == 1, "silu_mul_group_quant: form must be 0 (1-D quantiser) or 1 (amax / 448)");
+  if (groups == 0 || max_rows == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(gate && up && out && scale, "silu_mul_group_quant: null pointer");
+  BGMOE_REQUIRE(((uintptr_t)gate | (uintptr_t)up | (uintptr_t)prod_out) % 16 == 0 && (uintptr_t)out % 8 == 0 &&
+                    in_stride_e % 8 == 0 && in_stride_s % 8 == 0 && out_stride_e % 8 == 0 && out_stride_s % 8 == 0,
+                "silu_mul_group_quant: rows must be 16-byte aligned (strides multiples of 8 elements)");
+  BGMOE_REQUIRE(in_stride_s >= n && out_stride_s >= n, "silu_mul_group_quant: row strides smaller than the rows");
+  GroupQuantArgs a{};
+  a.gate = gate; a.up = up; a.ise = in_stride_e; a.iss = in_stride_s; a.counts = counts; a.starts = starts;
+  a.groups = groups; a.max_rows = max_rows; a.n = n; a.form = form; a.out = out; a.ose = out_stride_e;
+  a.oss = out_stride_s; a.scale = scale; a.sse = scale_stride_e; a.sss = scale_stride_s; a.ssg = scale_stride_g;
+  a.prod = prod_out;
+  int64_t blocks = ((int64_t)groups * max_rows + 3) / 4;
+  if (blocks > 16384) blocks = 16384;
+  hipStream_t st = bgmoe_stream(stream);
+  BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
+  hipLaunchKernelGGL(silu_mul_group_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a);
+  return bgmoe_check_launch("silu_mul_group_quant");
+}
+
+namespace {
 __device__ __forceinline__ uint32_t mix32(uint64_t v) {
   v ^= v >> 33; v *= 0xff51afd7ed558ccdULL; v ^= v >> 33; v *= 0xc4ceb9fe1a85ec53ULL; v ^= v >> 33;
   return (uint32_t)v;

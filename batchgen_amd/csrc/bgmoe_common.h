@@ -161,6 +161,34 @@ __device__ __forceinline__ float silu_f32(float g) { return g / (1.0f + __expf(-
 // evaluate it 64 times per lane, where the accumulation order already moves the last bits
 __device__ __forceinline__ float silu_rcp_f32(float g) { return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)); }
 
+// exp(t) for |t| <= 100, correctly rounded to fp32 but for about one input in 2^23: 2^k * P(r) in fp64 with the
+// degree-11 Taylor polynomial on |r| <= ln2/2 (truncation 2^-47), rounded once.
+__device__ __forceinline__ float exp_cr_f32(float t32) {
+  const double t = (double)t32;
+  const double k = __builtin_rint(t * 1.4426950408889634074);
+  double r = __builtin_fma(-k, 6.93147180369123816490e-01, t);
+  r = __builtin_fma(-k, 1.90821492927058770002e-10, r);
+  double p = 1.0 / 39916800.0;
+  p = __builtin_fma(p, r, 1.0 / 3628800.0);
+  p = __builtin_fma(p, r, 1.0 / 362880.0);
+  p = __builtin_fma(p, r, 1.0 / 40320.0);
+  p = __builtin_fma(p, r, 1.0 / 5040.0);
+  p = __builtin_fma(p, r, 1.0 / 720.0);
+  p = __builtin_fma(p, r, 1.0 / 120.0);
+  p = __builtin_fma(p, r, 1.0 / 24.0);
+  p = __builtin_fma(p, r, 1.0 / 6.0);
+  p = __builtin_fma(p, r, 0.5);
+  p = __builtin_fma(p, r, 1.0);
+  p = __builtin_fma(p, r, 1.0);
+  return (float)__builtin_ldexp(p, (int)k);
+}
+// PyTorch's fp32 SiLU: x / (1 + exp(-x)) as three fp32 operations (exp, add, IEEE division).  Beyond |x| = 100
+// exp(-x) is 0 or overflows to +inf in fp32 either way.
+__device__ __forceinline__ float silu_exact_f32(float g) {
+  const float e = g > 100.0f ? 0.0f : (g < -100.0f ? __builtin_huge_valf() : exp_cr_f32(-g));
+  return g / (1.0f + e);
+}
+
 // SiTU-and-multiply (Kimi-K3): beta * tanh(g / beta) * sigmoid(g), times u or, with a linear beta,
 // lbeta * tanh(u / lbeta).  fp32 throughout, the library tanhf / expf and an IEEE division; the divisions by
 // beta are multiplications by the rounded reciprocal, as in the reference kernels

@@ -191,6 +191,31 @@ int bgmoe_fused_silu_quant_3d(const uint16_t* gate, const uint16_t* up,
                               const int32_t* tokens_per_expert, int e, int mtp, int k, uint8_t* y,
                               float* scale, bgmoe_stream_t stream);
 
+/* bf16(silu(gate)) * up in bf16, then the per-row, per-128-column FP8 cast, in one pass: the activation
+ * between the two grouped GEMMs of the DeepGEMM chains and of the dense shared expert.  Replaces
+ *   form 1 (D): `silu_mul_masked_group_quant` / `silu_mul_ragged_group_quant`
+ *               (batchgen_kernels/triton/moe_masked_act_quant.py:43-376; oracle `act_reference`,
+ *               tests/test_glm52_deepgemm_masked_parity_gpu.py:128-149):
+ *               amax = max(max|p|, 1e-10), scale = amax / 448, q = clamp(p / scale, +-448);
+ *   form 0 (A): `silu_mul_per_token_blocked_quantize_bf16_to_fp8_1d`
+ *               (batchgen_kernels/triton/fp8_quantize.py:394-526): the 1-D quantiser of
+ *               bgmoe_act_quant_rows (amax floor 2^-16, scale = max(amax * (1/448), 1e-12), non-finite -> 0).
+ * In both, p = bf16( bf16(s) * up ) with s = g / (1 + exp(-g)) evaluated as the fp32 sequence
+ * exp (correctly rounded), add, IEEE division (PyTorch's SiLU, fp8_quantize.py:414-424).
+ * Row r of group e lives at element offset e*stride_e + (start_e + r)*stride_s, start_e = starts[e] or 0 when
+ * starts is NULL; rows r >= counts[e] (all max_rows rows when counts is NULL) are neither read nor written.
+ * masked [E,S,I]: stride_e = S*stride_s, starts NULL, counts = masked_m, max_rows = S;
+ * ragged [m,I]:   stride_e = 0, starts = cu_seqlens, counts = live rows, max_rows = bound on any count;
+ * 1-D [M,2I]:     groups 1, counts NULL, gate = x, up = x + I, in_stride_s = 2I, max_rows = M.
+ * Scale of (e, r, group g) at scale[e*scale_stride_e + (start_e + r)*scale_stride_s + g*scale_stride_g].
+ * prod_out (bf16, addressed like out) optionally receives p.  n a multiple of 128; 16-byte aligned rows. */
+int bgmoe_silu_mul_group_quant(const uint16_t* gate, const uint16_t* up, int64_t in_stride_e,
+                               int64_t in_stride_s, const int32_t* counts, const int32_t* starts, int groups,
+                               int64_t max_rows, int n, int form, uint8_t* out, int64_t out_stride_e,
+                               int64_t out_stride_s, float* scale, int64_t scale_stride_e,
+                               int64_t scale_stride_s, int64_t scale_stride_g, uint16_t* prod_out,
+                               bgmoe_stream_t stream);
+
 /* ------------------------------------------------------ permute / unpermute */
 
 /* Bytes of device workspace the dispatch calls need for n*k pairs. */

@@ -191,3 +191,31 @@ def swiglu_bf16(gate_f32: np.ndarray, up_f32: np.ndarray) -> np.ndarray:
     """Rounding variant (i): fp32 gate, fp32 up, fp32 silu, ONE bf16 round
     (batchgen_kernels/triton/w8a8_grouped_gemm_stage_1.py:1023-1026)."""
     return bf16_round(silu_f32(gate_f32) * up_f32.astype(F32))
+
+
+def silu_torch_f32(g) -> np.ndarray:
+    """PyTorch's fp32 SiLU, ``x / (1 + exp(-x))`` as three float32 operations -- the formula and precision the
+    reference's fused activation quantisers restate (batchgen_kernels/triton/fp8_quantize.py:414-424: libdevice
+    ``exp``, round-to-nearest division).  ``exp`` is taken correctly rounded (float64, rounded once)."""
+    g = as_f32(g)
+    with np.errstate(over="ignore"):
+        e = np.exp(-g.astype(np.float64)).astype(F32)
+        d = (F32(1.0) + e).astype(F32)
+        return (g / d).astype(F32)
+
+
+def silu_mul_bf16(gate, up) -> np.ndarray:
+    """bf16( bf16(silu(gate)) * up ): SiLU cast back to the input dtype before the multiply, bf16 product
+    (moe_masked_act_quant.py:96-99; fp8_quantize.py:425-426)."""
+    s = bf16_round(silu_torch_f32(gate))
+    return bf16_round((s * as_f32(up)).astype(F32))
+
+
+def silu_mul_group_quant(gate, up, form: str):
+    """[M, I] gate, up -> (bytes, scales, product): form "D" = ``silu_mul_{masked,ragged}_group_quant``
+    (oracle ``act_reference``, tests/test_glm52_deepgemm_masked_parity_gpu.py:128-149), form "A" =
+    ``silu_mul_per_token_blocked_quantize_bf16_to_fp8_1d``."""
+    p = silu_mul_bf16(gate, up)
+    y, s = act_quant(p, form=form)
+    return y, s, p
+

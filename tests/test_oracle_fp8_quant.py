@@ -129,3 +129,38 @@ def test_short_scale_division_model_equals_ieee_division():
     e = fma_f32(-q0, s, x)
     q = np.where(e == 0, q0, fma_f32(e, r, q0))
     assert np.array_equal(q.view(np.uint32), (x / s).astype(np.float32).view(np.uint32))
+
+
+def test_silu_in_the_reference_precision_and_the_group_quantiser_of_the_deepgemm_chain():
+    """``silu_torch_f32`` against the library's own fp32 SiLU and closed forms; ``silu_mul_group_quant`` form D
+    against the reference test's ``act_reference`` written with torch CPU operations
+    (tests/test_glm52_deepgemm_masked_parity_gpu.py:128-149)."""
+    import torch.nn.functional as F
+    gen = torch.Generator().manual_seed(11)
+    g = (torch.randn(300_000, generator=gen) * 5).to(torch.bfloat16).float()
+    mine = oq.silu_torch_f32(g.numpy())
+    lib = F.silu(g).numpy()
+    assert np.max(np.abs(mine.view(np.int32).astype(np.int64) - lib.view(np.int32).astype(np.int64))) <= 2
+    assert np.mean(oq.bf16_round(mine) != oq.bf16_round(lib)) < 1e-4
+    x64 = g.double()
+    np.testing.assert_allclose(mine, (x64 * torch.sigmoid(x64)).numpy(), rtol=3e-7, atol=1e-37)
+    special = oq.silu_torch_f32(np.array([0.0, 200.0, -200.0, 90.0, -90.0, 1e-30], dtype=np.float32))
+    assert special[0] == 0 and special[1] == 200.0 and special[2] == 0 and np.signbit(special[2])
+    assert special[3] == 90.0 and abs(special[4]) < 1e-36 and special[5] == np.float32(5e-31)
+
+    gate = (torch.randn(37, 384, generator=gen) * 3).to(torch.bfloat16)
+    up = (torch.randn(37, 384, generator=gen) * 3).to(torch.bfloat16)
+    up[3, :128] = 0                                                   # a whole zero group: floor 1e-10
+    gf = gate.float()
+    sg = (gf / (1 + torch.exp(-gf))).to(torch.bfloat16)
+    prod = (up * sg).reshape(37, 3, 128)
+    amax = prod.abs().amax(-1).float().clamp_min(1e-10)
+    s_ref = amax / 448.0
+    q_ref = (prod.float() / s_ref.unsqueeze(-1)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).reshape(37, 384)
+    y, s, p = oq.silu_mul_group_quant(gate, up, "D")
+    assert np.mean(p != prod.reshape(37, 384).float().numpy()) < 1e-3  # torch's exp vs the correctly rounded one
+    same = (p == prod.reshape(37, 384).float().numpy()).reshape(37, 3, 128).all(-1)
+    assert np.array_equal(s[same], s_ref.numpy()[same])
+    yb = q_ref.view(torch.uint8).numpy().reshape(37, 3, 128)
+    assert np.array_equal(y.reshape(37, 3, 128)[same], yb[same])
+    assert s[3, 0] == np.float32(1e-10) / np.float32(448.0) and not (y[3, :128] & 0x7F).any()    # signed zeros
