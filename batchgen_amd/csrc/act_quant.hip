@@ -439,10 +439,19 @@ __global__ __launch_bounds__(256) void silu_mul_group_quant_kernel(GroupQuantArg
       const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
       float p[8];
       uint32_t pw[4];
+      float sv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float gi = (i & 1) ? __uint_as_float(gw[i >> 1] & 0xffff0000u) : __uint_as_float(gw[i >> 1] << 16);
+        bool decided;
+        sv[i] = silu_short_f32(gi, &decided);
+        if (__any(!decided)) {                 // rare: one exact evaluation for the lanes that need it
+          if (!decided) sv[i] = silu_exact_f32(gi);
+        }
+      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t sw = pack2_bf16(silu_exact_f32(__uint_as_float(gw[j] << 16)),
-                                       silu_exact_f32(__uint_as_float(gw[j] & 0xffff0000u)));
+        const uint32_t sw = pack2_bf16(sv[2 * j], sv[2 * j + 1]);
         pw[j] = pack2_bf16(__uint_as_float(sw << 16) * __uint_as_float(uw[j] << 16),
                            __uint_as_float(sw & 0xffff0000u) * __uint_as_float(uw[j] & 0xffff0000u));
         p[2 * j] = __uint_as_float(pw[j] << 16);

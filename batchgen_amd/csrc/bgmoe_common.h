@@ -189,6 +189,22 @@ __device__ __forceinline__ float silu_exact_f32(float g) {
   return g / (1.0f + e);
 }
 
+// bf16(silu_exact_f32(g)) at a third of the cost on almost every input.  The short evaluation (hardware exp2
+// with the argument's rounding error carried separately, hardware reciprocal) stays within 4 fp32 ulps of the
+// true SiLU and silu_exact_f32 within 2; if the short result lies more than 16 ulps from the nearest bf16
+// rounding boundary both round to the same bf16.  `decided` = false asks the caller for the exact
+// evaluation (about 1 input in 2000, and every |g| > 80 or non-finite g).  Returns the fp32 value to round.
+__device__ __forceinline__ float silu_short_f32(float g, bool* decided) {
+  const float x = -g;
+  const float t_hi = x * 1.44269502162933349609375f;                         // log2(e) rounded to fp32
+  const float t_lo = __builtin_fmaf(x, 1.44269502162933349609375f, -t_hi) + x * 1.925963033500011e-08f;
+  const float e = __builtin_amdgcn_exp2f(t_hi) * __builtin_fmaf(t_lo, 0.693147182464599609375f, 1.0f);
+  const float s = g * __builtin_amdgcn_rcpf(1.0f + e);
+  const uint32_t low = __float_as_uint(s) & 0xffffu;
+  *decided = fabsf(g) <= 80.0f && (low < 0x8000u - 16u || low > 0x8000u + 16u);
+  return s;
+}
+
 // SiTU-and-multiply (Kimi-K3): beta * tanh(g / beta) * sigmoid(g), times u or, with a linear beta,
 // lbeta * tanh(u / lbeta).  fp32 throughout, the library tanhf / expf and an IEEE division; the divisions by
 // beta are multiplications by the rounded reciprocal, as in the reference kernels

@@ -119,3 +119,24 @@ def test_group_quant_argument_policy(dev):
                 torch.zeros(0, 256, dtype=torch.bfloat16, device=dev), torch.zeros(2, 4, 256, dtype=torch.bfloat16, device=dev)):
         with pytest.raises(ValueError):
             fused(bad)
+
+
+def test_silu_of_every_bf16_value_equals_the_oracle(dev):
+    """All 65536 bf16 gates against the oracle, bit for bit: with up = 1 the bf16 product the kernel can hand
+    out IS bf16(silu(gate)).  Covers the short evaluation, its hand-over to the exact one, +-0, +-inf, NaN and
+    the denormals."""
+    from batchgen_amd._lib import check, lib, ptr
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    x = torch.cat([bits.view(512, 128), torch.ones(512, 128, dtype=torch.bfloat16)], dim=1).contiguous().to(dev)
+    out = torch.empty(512, 128, dtype=torch.uint8, device=dev)
+    sc = torch.empty(512, 1, dtype=torch.float32, device=dev)
+    prod = torch.empty(512, 128, dtype=torch.bfloat16, device=dev)
+    check(lib().bgmoe_silu_mul_group_quant(ptr(x), x.data_ptr() + 256, 0, 256, None, None, 1, 512, 128, 0, ptr(out), 0,
+                                           128, ptr(sc), 0, 1, 1, ptr(prod), None))
+    got = prod.view(torch.int16).cpu().numpy().reshape(-1).view(np.uint16)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oq.bf16_round(oq.silu_torch_f32(bits.float().numpy()))
+    wb = (want.view(np.uint32) >> 16).astype(np.uint16)
+    nan = np.isnan(want)
+    assert np.array_equal(got[~nan], wb[~nan])
+    assert np.all((got[nan] & 0x7F80) == 0x7F80) and np.all((got[nan] & 0x7F) != 0)      # NaN stays NaN
