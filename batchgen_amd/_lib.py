@@ -34,7 +34,8 @@ class Mxfp4Weight(C.Structure):
 
 class Fp8Act(C.Structure):
     """bgmoe_fp8_act"""
-    _fields_ = [("x", vp), ("scale", vp), ("scale_row_stride", i64), ("scale_kb_stride", i64)]
+    _fields_ = [("x", vp), ("scale", vp), ("scale_row_stride", i64), ("scale_kb_stride", i64),
+                ("scale_group_stride", i64)]
 
 
 _SIGS = {

@@ -152,7 +152,9 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
     tok_off[i] = (uint32_t)row * (uint32_t)K + (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
     tok_on[i] = (h >> 1) < tiles;
   }
-  const float* xs_base = uniform_ptr(g.a.scale + (row0 + t0) * g.a.scale_row_stride);
+  const float* xs_base = uniform_ptr(g.a.scale_group_stride
+                                        ? g.a.scale + grp * g.a.scale_group_stride + (int64_t)t0 * g.a.scale_row_stride
+                                        : g.a.scale + (row0 + t0) * g.a.scale_row_stride);
   const uint32_t xs_off = (uint32_t)min(lane, live - 1) * (uint32_t)g.a.scale_row_stride * 4u;
 
   auto issue_tokens = [&](int kb, int slot) {

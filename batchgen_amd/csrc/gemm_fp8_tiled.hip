@@ -200,7 +200,9 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
       // row-major: row nrow; tile-major: tile nrow / 16 (16 x K bytes per row of tiles)
       w_base[i] = uniform_ptr(base + (int64_t)(LAYOUT == BGMOE_W_ROW_MAJOR ? nrow : (nrow & ~15)) * K);
     }
-    xs_base = uniform_ptr(g.a.scale + (row0 + m0) * g.a.scale_row_stride);
+    xs_base = uniform_ptr(g.a.scale_group_stride
+                              ? g.a.scale + grp * g.a.scale_group_stride + (int64_t)m0 * g.a.scale_row_stride
+                              : g.a.scale + (row0 + m0) * g.a.scale_row_stride);
     xs_off = (uint32_t)min(64 * wn + lane, cnt - 1 - m0) * (uint32_t)g.a.scale_row_stride * 4u;
     return true;
   };

@@ -338,6 +338,11 @@ typedef struct bgmoe_fp8_act {
   const float* scale;            /* element (r,kb) at r*row_stride+kb*kb_stride */
   int64_t scale_row_stride;
   int64_t scale_kb_stride;
+  /* 0: r is the row of x (cu_seqlens[g] + t).  Non-zero: scales are stored per group, token t of group g at
+   * g*scale_group_stride + t*row_stride + kb*kb_stride -- DeepGEMM's masked A-scale form, a contiguous
+   * [E, K/128, S] block viewed as [E, S, K/128]: group stride K/128*S, row stride 1, kb stride S
+   * (batchgen/models/glm/glm5/moe_deepgemm_masked.py:46-70). */
+  int64_t scale_group_stride;
 } bgmoe_fp8_act;
 
 /* Single grouped GEMM, bf16 output [m,n].  Replaces
