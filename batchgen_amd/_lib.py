@@ -54,6 +54,7 @@ _SIGS = {
     "bgmoe_set_router_gemm_plan": (i32, [i32, i32]),
     "bgmoe_add_rmsnorm_fp8_quant": (i32, [vp, vp, vp, i64, i32, f32, vp, vp, vp, i64, i64, vp, vp, vp, vp]),
     "bgmoe_selfcheck_sigmoid": (i32, [C.c_uint32, C.c_uint64, vp, vp, vp]),
+    "bgmoe_layout_to_segments": (i32, [vp, i64, i32, vp, vp, vp, vp]),
     "bgmoe_silu_mul_group_quant": (i32, [vp, vp, i64, i64, vp, vp, i32, i64, i32, i32, vp, i64, i64, vp, i64, i64, i64,
                                          vp, vp]),
     "bgmoe_selfcheck_scale_division": (i32, [C.c_uint64, C.c_uint64, vp, vp, vp]),

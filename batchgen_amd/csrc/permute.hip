@@ -459,3 +459,46 @@ extern "C" int bgmoe_compact_expert_data(const int32_t* expert_counts, int e, in
                      group_size, activated_group_idx, group_start_indices, num_active);
   return bgmoe_check_launch("compact_expert_data");
 }
+
+namespace {
+// Row -> group map (one contiguous run of rows per group, -1 on padding rows) -> (first row, live rows) per
+// group.  One block: the map is a few hundred KB at most and is read once; every output has a single writer.
+__global__ __launch_bounds__(1024) void layout_segments_kernel(const int32_t* __restrict__ layout, int64_t m, int groups,
+                                                               int32_t* __restrict__ seqlens, int32_t* __restrict__ starts,
+                                                               int32_t* __restrict__ status) {
+  __shared__ int32_t s_first[1024], s_end[1024], s_bad;
+  if (threadIdx.x == 0) s_bad = 0;
+  for (int g = threadIdx.x; g < groups; g += 1024) { s_first[g] = 0; s_end[g] = 0; }
+  __syncthreads();
+  for (int64_t r = threadIdx.x; r < m; r += 1024) {
+    const int32_t g = layout[r];
+    if (g < 0) continue;
+    if (g >= groups) { s_bad = 1; continue; }
+    if (r == 0 || layout[r - 1] != g) {
+      if (atomicAdd(&s_first[g], (int32_t)r + 1) != 0) s_bad = 2;       // a second run of the same group
+    }
+    if (r == m - 1 || layout[r + 1] != g) atomicAdd(&s_end[g], (int32_t)r + 1);
+  }
+  __syncthreads();
+  for (int g = threadIdx.x; g < groups; g += 1024) {
+    const bool live = s_first[g] != 0;
+    starts[g] = live ? s_first[g] - 1 : 0;
+    seqlens[g] = live && s_bad == 0 ? s_end[g] - (s_first[g] - 1) : 0;
+  }
+  if (threadIdx.x == 0) {
+    starts[groups] = (int32_t)m;
+    if (status) *status = s_bad;
+  }
+}
+}  // namespace
+
+extern "C" int bgmoe_layout_to_segments(const int32_t* grouped_layout, int64_t m, int groups, int32_t* seqlens,
+                                        int32_t* starts, int32_t* status, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(m >= 0 && m <= 0x7fffffffLL && groups >= 1 && groups <= 1024,
+                "layout_to_segments: m=%lld rows / %d groups out of range (groups in [1, 1024])", (long long)m, groups);
+  BGMOE_REQUIRE(seqlens && starts && (m == 0 || grouped_layout), "layout_to_segments: null pointer");
+  hipLaunchKernelGGL(layout_segments_kernel, dim3(1), dim3(1024), 0, bgmoe_stream(stream), grouped_layout, m, groups,
+                     seqlens, starts, status);
+  return bgmoe_check_launch("layout_to_segments");
+}
+

@@ -424,6 +424,16 @@ int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight* gate,
                          uint16_t* const* out_ptrs, int activation, int64_t row_bound,
                          bgmoe_stream_t stream);
 
+/* DeepGEMM's contiguous m-grouped API describes the rows by a map `grouped_layout` [m] (row -> group, -1 on
+ * alignment padding; batchgen/moe/grouped_fp8_deepgemm_moe.py:9-22, built by `build_grouped_layout`, :118-186).
+ * This call turns the map into what the grouped GEMMs here take: starts[g] = first row of group g (starts has
+ * groups + 1 entries, the last one m) and seqlens[g] = its live rows (0 for a group without rows).  Each group
+ * must own ONE contiguous run of rows; *status (optional, device) is set to 0, or to 1 for a group index
+ * >= groups and 2 for a group with two runs, in which case every seqlens entry is 0 and the GEMM that follows
+ * does nothing.  One small launch, no host synchronisation. */
+int bgmoe_layout_to_segments(const int32_t* grouped_layout, int64_t m, int groups, int32_t* seqlens,
+                             int32_t* starts, int32_t* status, bgmoe_stream_t stream);
+
 /* ---------------------------------------------------------------- self-check */
 
 /* The routers' sigmoid is the correctly rounded fp32 one (fp64 evaluation rounded once: the reference

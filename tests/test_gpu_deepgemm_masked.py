@@ -129,3 +129,61 @@ def test_layout_contract_is_enforced(dev, layer):
                      ("act_scales", torch.zeros(E, S, I // 128, device=dev))):
         with pytest.raises(RuntimeError):
             m.run_deepgemm_masked_moe(**{**good, key: bad})
+
+
+def test_contiguous_grouped_gemm_by_row_map(dev):
+    """`grouped_fp8_deepgemm_gemm` / `m_grouped_fp8_gemm_nt_contiguous`: rows described by a row -> group map
+    (128-aligned segment starts, -1 on padding, expert segments mapped to a permuted dense weight stack), both
+    activation-scale layouts; padding rows keep their sentinel; a malformed map writes nothing."""
+    from batchgen_amd._lib import check, lib, ptr
+    from batchgen_amd.moe import grouped_fp8_deepgemm_moe as dg
+    counts = np.array([0, 1, 127, 128, 129, 300, 0, 64], dtype=np.int32)
+    cu = np.concatenate([[0], np.cumsum((counts + 127) // 128 * 128)]).astype(np.int32)
+    g_, n, k = len(counts), 256, 512
+    m = int(cu[-1]) + 128
+    rng = np.random.default_rng(5)
+    wq, ws = oq.weight_block_quant((0.05 * rng.standard_normal((g_, n, k))).astype(np.float32))
+    ids = rng.permutation(g_).astype(np.int32)                        # expert segment e uses weight slot ids[e]
+    gen = torch.Generator().manual_seed(6)
+    x = rand_bf16(gen, m, k)
+    xq, xs = oq.act_quant(x, form="A")
+    d = lambda a: torch.from_numpy(a).to(dev)
+    arena = d(wq).view(torch.float8_e4m3fn)
+    stack = dg.dense_group_view([arena[i] for i in range(g_)])
+    assert stack.data_ptr() == arena.data_ptr()
+    layout = dg.build_grouped_layout(d(counts), d(cu), m, group_ids=d(ids))
+    wdeq = oq.weight_block_dequant(wq, ws)
+    xdeq = oq.act_dequant(xq, xs)
+    live = layout.cpu().numpy() >= 0
+    ref = np.zeros((m, n), dtype=np.float32)
+    for e, c in enumerate(counts):
+        ref[cu[e]:cu[e] + c] = xdeq[cu[e]:cu[e] + c] @ wdeq[ids[e]].T
+    for rows_major in (True, False):
+        out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+        scale = d(xs) if rows_major else d(np.ascontiguousarray(xs.T))
+        res = dg.grouped_fp8_deepgemm_gemm(d(xq).view(torch.float8_e4m3fn), scale, stack, d(ws), output=out,
+                                           grouped_layout=layout, x_scale_rows_major=rows_major)
+        assert res is out
+        o = out.float().cpu().numpy()
+        assert (o[~live] == 7.0).all()
+        assert calc_diff(o[live], ref[live]) < 1e-3 and og.rel_frobenius(o[live], ref[live]) < 4e-3
+    # the map's segments on the device, and a malformed map (group 2 in two runs)
+    seg = torch.full((2 * g_ + 2,), -5, dtype=torch.int32, device=dev)
+    status = torch.full((1,), -5, dtype=torch.int32, device=dev)
+    check(lib().bgmoe_layout_to_segments(ptr(layout), m, g_, ptr(seg), seg.data_ptr() + 4 * g_, ptr(status), None))
+    seqs, starts = seg[:g_].cpu().numpy(), seg[g_:].cpu().numpy()
+    assert int(status) == 0 and starts[g_] == m
+    for e, c in enumerate(counts):
+        assert seqs[ids[e]] == c and (c == 0 or starts[ids[e]] == cu[e])
+    bad = layout.clone()
+    bad[m - 1] = int(ids[2])
+    check(lib().bgmoe_layout_to_segments(ptr(bad), m, g_, ptr(seg), seg.data_ptr() + 4 * g_, ptr(status), None))
+    assert int(status) == 2 and int(seg[:g_].abs().sum()) == 0
+    out = torch.full((m, n), 7.0, dtype=torch.bfloat16, device=dev)
+    dg.m_grouped_fp8_gemm_nt_contiguous((d(xq).view(torch.float8_e4m3fn), d(xs)), (stack, d(ws)), out, bad)
+    assert (out.float() == 7.0).all()
+    with pytest.raises(ValueError):
+        dg.grouped_fp8_deepgemm_gemm(d(xq).view(torch.float8_e4m3fn), d(xs), stack, d(ws), output=out,
+                                     grouped_layout=layout[:-1], x_scale_rows_major=True)
+    with pytest.raises(ValueError):
+        dg.m_grouped_fp8_gemm_nt_contiguous((d(xq).view(torch.float8_e4m3fn), d(xs)), (stack[:, :, :256], d(ws)), out, layout)
