@@ -187,3 +187,46 @@ def test_contiguous_grouped_gemm_by_row_map(dev):
                                      grouped_layout=layout[:-1], x_scale_rows_major=True)
     with pytest.raises(ValueError):
         dg.m_grouped_fp8_gemm_nt_contiguous((d(xq).view(torch.float8_e4m3fn), d(xs)), (stack[:, :, :256], d(ws)), out, layout)
+
+
+def test_deepseek_v3_decode_wrappers_with_pointer_arrays(dev):
+    """`fused_fp8_moe_stage_1_tma_wrapper` and `fused_dequant_grouped_gemm_fp8_tma_wrapper`: 3-D masked operands,
+    one weight tensor per expert behind device pointer arrays, MN-major and row-major activation scales."""
+    from batchgen_amd.moe import grouped_gemm_kernel as gk
+    e, m_max, k, n = 6, 64, 512, 256
+    counts = [0, 1, 17, 64, 33, 5]
+    rng = np.random.default_rng(9)
+    gen = torch.Generator().manual_seed(10)
+    x = rand_bf16(gen, e * m_max, k)
+    xq, xs = oq.act_quant(x, form="A")
+    d = lambda a: torch.from_numpy(a).to(dev)
+    xq_d = d(xq).view(torch.float8_e4m3fn).view(e, m_max, k)
+    scales = {"row-major": d(xs).view(e, m_max, k // 128),
+              "MN-major": mn_major(e, m_max, k // 128, dev)}
+    scales["MN-major"].copy_(scales["row-major"])
+    def expert_weights(seed):
+        q, s = oq.weight_block_quant((0.05 * np.random.default_rng(seed).standard_normal((e, n, k))).astype(np.float32))
+        wl = [d(q[i]).view(torch.float8_e4m3fn) for i in range(e)]
+        sl = [d(s[i]) for i in range(e)]
+        tbl = lambda ts: torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device=dev)
+        return wl, tbl(wl), sl, tbl(sl), oq.weight_block_dequant(q, s)
+    gw, gp, gs, gsp, gd = expert_weights(1)
+    uw, up_, us, usp, ud = expert_weights(2)
+    cnt = torch.tensor(counts, dtype=torch.int32, device=dev)
+    xdeq = oq.act_dequant(xq, xs).reshape(e, m_max, k)
+    for name, sc in scales.items():
+        out = torch.full((e, m_max, n), 7.0, dtype=torch.bfloat16, device=dev)
+        res = gk.fused_fp8_moe_stage_1_tma_wrapper(xq_d, sc, gw, gp, uw, up_, gs, gsp, us, usp, cnt, e, out=out)
+        assert res is out
+        y = gk.fused_dequant_grouped_gemm_fp8_tma_wrapper(xq_d, sc, gw, gp, gs, gsp, cnt, e)
+        o, yv = out.float().cpu().numpy(), y.float().cpu().numpy()
+        for i, c in enumerate(counts):
+            assert (o[i, c:] == 7.0).all() and (yv[i, c:] == 0.0).all(), name
+            if c:
+                g32, u32 = xdeq[i, :c] @ gd[i].T, xdeq[i, :c] @ ud[i].T
+                assert og.rel_frobenius(o[i, :c], oq.swiglu_bf16(g32, u32)) < 5e-3, name
+                assert og.rel_frobenius(yv[i, :c], g32) < 4e-3, name
+    with pytest.raises(RuntimeError):
+        gk.fused_dequant_grouped_gemm_fp8_tma_wrapper(xq_d, scales["row-major"], gw, gp.int(), gs, gsp, cnt, e)
+    with pytest.raises(RuntimeError):
+        gk.fused_dequant_grouped_gemm_fp8_tma_wrapper(xq_d, scales["row-major"], gw, gp, gs, gsp, cnt, e + 1)
