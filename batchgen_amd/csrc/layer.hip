@@ -25,7 +25,8 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
   BGMOE_REQUIRE(L->cap_rows + n <= 2147483647LL, "moe_fp8_layer_forward: row space exceeds int32");
   if (n == 0) return BGMOE_OK;
   const bool pre_quant = L->x_fp8 != nullptr;
-  const bool own_logits = L->logits == nullptr;
+  const bool routed = L->routes_given != 0;
+  const bool own_logits = !routed && L->logits == nullptr;
   BGMOE_REQUIRE(L->bias && L->out, "moe_fp8_layer_forward: null input/output");
   BGMOE_REQUIRE(pre_quant ? L->x_scale != nullptr : L->x != nullptr,
                 "moe_fp8_layer_forward: needs x, or x_fp8 together with x_scale");
@@ -42,8 +43,10 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
   hipStream_t st = bgmoe_stream(stream);
   int rc;
 
-  // 1. router (from logits, or from the hidden states through the router GEMM)
-  if (own_logits) {
+  // 1. router (from logits, or from the hidden states through the router GEMM), unless the routes are given
+  if (routed) {
+    rc = BGMOE_OK;
+  } else if (own_logits) {
     const bool grouped = L->n_group > 1;
     rc = bgmoe_router_gemm_gate(L->router_hidden ? L->router_hidden : L->x, L->router_weight, L->bias, n, h,
                                 L->e_total, grouped ? L->n_group : 0, grouped ? L->topk_group : 0, k,

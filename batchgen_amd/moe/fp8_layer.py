@@ -38,6 +38,7 @@ class LayerStruct(C.Structure):
         ("workspace", vp), ("workspace_bytes", sz), ("out", vp),
         ("x_fp8", vp), ("x_scale", vp), ("x_scale_row_stride", i64), ("x_scale_kb_stride", i64),
         ("router_weight", vp), ("router_hidden", vp), ("router_workspace", vp), ("router_workspace_bytes", sz),
+        ("routes_given", i32),
     ]
 
 
@@ -225,7 +226,33 @@ class Fp8MoELayer:
             L.x_fp8 = L.x_scale = None
         L.n = n
         L.x = ptr(hidden_states)
+        L.routes_given = 0
         check(self._fn(C.byref(L), stream()))
+        return self.out[:n]
+
+    def forward_routed(self, hidden_states: torch.Tensor, topk_idx: torch.Tensor,
+                       topk_weight: torch.Tensor) -> torch.Tensor:
+        """The layer behind an external gate: ``topk_idx`` ``[N, K]`` (global expert ids; ids this rank does not
+        hold, and -1, contribute nothing) and ``topk_weight`` ``[N, K]`` fp32 are given, as in
+        ``WGMMAMoEBuffers.forward(layer_id, global_x, topk_idx, topk_weight)``
+        (batchgen/moe/fp8_wgmma_pipeline.py:294-372): dispatch, quantise, gate_up + SwiGLU + requant, down,
+        weighted combine (+ shared expert when the layer has one)."""
+        cfg = self.cfg
+        n = hidden_states.size(0)
+        if hidden_states.dtype != torch.bfloat16 or tuple(hidden_states.shape) != (n, cfg.hidden) or \
+                not hidden_states.is_contiguous() or n > self.n_max:
+            raise RuntimeError(f"hidden_states must be contiguous BF16 [N <= {self.n_max}, {cfg.hidden}]")
+        if tuple(topk_idx.shape) != (n, cfg.top_k) or tuple(topk_weight.shape) != (n, cfg.top_k):
+            raise RuntimeError(f"topk_idx and topk_weight must be [{n}, {cfg.top_k}]")
+        self.topk_ids[:n].copy_(topk_idx)                 # any integer dtype -> the layer's int32 buffer
+        self.topk_weights[:n].copy_(topk_weight)
+        L = self._L
+        L.logits = L.x_fp8 = L.x_scale = None
+        L.n, L.x, L.routes_given = n, ptr(hidden_states), 1
+        try:
+            check(self._fn(C.byref(L), stream()))
+        finally:
+            L.routes_given = 0
         return self.out[:n]
 
     __call__ = forward

@@ -538,6 +538,11 @@ typedef struct bgmoe_moe_fp8_layer {
   const uint16_t* router_hidden;
   void* router_workspace;
   size_t router_workspace_bytes;
+  /* non-zero: the routes are given -- topk_ids [n,top_k] and topk_weights [n,top_k] are INPUTS, the router is
+   * skipped and logits / router_weight are not read (the form of `WGMMAMoEBuffers.forward(layer_id, global_x,
+   * topk_idx, topk_weight)`, batchgen/moe/fp8_wgmma_pipeline.py:294-372).  Ids outside the local expert range
+   * (and -1) contribute nothing. */
+  int32_t routes_given;
 } bgmoe_moe_fp8_layer;
 
 int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* layer, bgmoe_stream_t stream);

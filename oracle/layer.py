@@ -53,7 +53,7 @@ def _permute(ids, expert_start, num_local, layout, max_tokens, row_align):
 
 def moe_layer_fp8(x, logits, bias, rcfg, w, expert_start, num_local,
                   layout="masked", max_tokens=0, row_align=64, shared=None,
-                  shared_mode="bf16_add"):
+                  shared_mode="bf16_add", routes=None):
     """x [N,H] bf16-valued; w = dict(gate_q,gate_s,up_q,up_s,down_q,down_s) for the
     LOCAL experts ([E_l,...] numpy); shared = same keys with a leading 1.
 
@@ -61,7 +61,9 @@ def moe_layer_fp8(x, logits, bias, rcfg, w, expert_start, num_local,
     """
     x = _q.as_f32(x)
     n, h = x.shape
-    ids, wt = route(logits, bias, rcfg)
+    # routes = (ids [N,K], weights [N,K]) from an external gate (fp8_wgmma_pipeline.py:294-307): the router is skipped
+    ids, wt = route(logits, bias, rcfg) if routes is None else (np.asarray(routes[0], dtype=np.int32),
+                                                                 np.asarray(routes[1], dtype=np.float32))
     k = ids.shape[1]
     counts, cu, pos, rows = _permute(ids, expert_start, num_local, layout, max_tokens, row_align)
     xq_tok, xs_tok = _q.act_quant(x)

@@ -284,3 +284,38 @@ def test_producer_chain_replays_from_a_hip_graph(dev):
             assert torch.equal(out_static, eager[i]), f"replay of input {i} (round {rnd}) differs from eager"
             j = (i + 1) % 3
             assert torch.equal(chain(res[j].clone(), hid[j]), eager[j])      # eager work between replays
+
+
+def test_layer_with_given_routes(dev):
+    """`forward_routed`: the layer behind an external gate.  Routes taken from the layer's own router reproduce
+    its output bit for bit; arbitrary routes (int64 ids, ids of other ranks, -1 padding, unnormalised weights)
+    match the oracle run on the same routes."""
+    from batchgen_amd import workloads as wl
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    from oracle import gemm as og
+    from oracle import layer as ol
+    cfg = wl.scaled(wl.CONFIGS[0], n_tokens=48, hidden=512, inter=256, shared_inter=256, n_experts=32, e_local=8,
+                    expert_start=8, n_group=4, topk_group=2, top_k=4, max_tokens=48)
+    inp = wl.make_inputs(cfg, "cpu")
+    w, sh = wl.make_fp8_weights(cfg, "cpu")
+    layer = Fp8MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
+                        inp["bias"].to(dev))
+    x = inp["x"].to(dev)
+    out = layer(x, inp["logits"].to(dev)).clone()
+    ids, wts = layer.topk_ids.clone(), layer.topk_weights.clone()
+    assert torch.equal(layer.forward_routed(x, ids, wts), out)
+    assert torch.equal(layer.forward_routed(x, ids.long(), wts), out)
+    g = torch.Generator().manual_seed(4)
+    rid = torch.stack([torch.randperm(cfg.n_experts, generator=g)[:cfg.top_k] for _ in range(cfg.n_tokens)])
+    rid[5] = -1                                                        # a padding row
+    rw = torch.rand(cfg.n_tokens, cfg.top_k, generator=g) * 2
+    got = layer.forward_routed(x, rid.to(dev), rw.to(dev)).float().cpu().numpy()
+    ref = ol.moe_layer_fp8(inp["x"], None, None, None, wl.weights_to_numpy(w), cfg.expert_start, cfg.e_local,
+                           layout=cfg.layout, max_tokens=cfg.max_tokens, shared=wl.weights_to_numpy(sh),
+                           routes=(rid.numpy(), rw.numpy()))
+    assert np.array_equal(layer.topk_pos.cpu().numpy(), ref["pos"])
+    assert np.array_equal(layer.expert_counts[:cfg.e_local].cpu().numpy(), ref["counts"])
+    assert og.rel_frobenius(got, ref["out"]) < 1e-2
+    assert torch.equal(layer(x, inp["logits"].to(dev)), out)          # the routed call leaves the layer as it was
+    with pytest.raises(RuntimeError):
+        layer.forward_routed(x, rid[:, :2].to(dev), rw[:, :2].to(dev))
