@@ -217,3 +217,48 @@ def test_compact_expert_data(dev):
     assert idx[:na].cpu().tolist() == nz.tolist()
     assert size[:na].cpu().tolist() == counts[nz].tolist()
     assert start[:na].cpu().tolist() == (torch.cumsum(counts[nz], 0) - counts[nz]).tolist()
+
+
+def test_legacy_combine_helpers(dev):
+    """`moe_weighted_sum_*` (dense [T, K, H]) and `scatter_weight_reduce_optimized` (sparse rows + inverse mapping)
+    against the fp32 sum in ascending k: bit-exact (the same arithmetic as reduce_weighted_scatter)."""
+    from batchgen_amd.moe import combine_variants as cv
+    g = torch.Generator().manual_seed(21)
+    t, k, h = 37, 8, 520
+    res3 = (torch.randn(t, k, h, generator=g)).to(torch.bfloat16)
+    w = torch.rand(t, k, generator=g)
+    acc = np.zeros((t, h), dtype=np.float32)
+    for j in range(k):
+        acc = (acc + (res3[:, j].float().numpy() * w[:, j:j + 1].numpy()).astype(np.float32)).astype(np.float32)
+    want = torch.from_numpy(acc).to(torch.bfloat16)
+    for fn in (cv.moe_weighted_sum_triton, cv.moe_weighted_sum_triton_v2, cv.moe_weighted_sum_v3):
+        got = fn(res3.to(dev), w.to(dev))
+        assert got.dtype == torch.bfloat16 and torch.equal(got.cpu(), want)
+    assert torch.equal(cv.moe_weighted_sum_v3(res3.to(dev), w.to(torch.bfloat16).to(dev)).cpu(),
+                       torch.from_numpy(sum_k(res3, w.to(torch.bfloat16).float())).to(torch.bfloat16))
+    # sparse form: only some (token, slot) pairs have a row, in a shuffled order, buffers oversized
+    keep = torch.rand(t, k, generator=g) < 0.6
+    tok, slot = torch.nonzero(keep, as_tuple=True)
+    order = torch.randperm(tok.numel(), generator=g)
+    tok, slot = tok[order], slot[order]
+    rows = res3[tok, slot]
+    pad = torch.zeros(50, dtype=torch.int64)
+    out = cv.scatter_weight_reduce_optimized(rows.to(dev), torch.cat([tok, pad]).to(dev), torch.cat([slot, pad]).to(dev),
+                                             w.to(dev), t, k)
+    acc = np.zeros((t, h), dtype=np.float32)
+    for j in range(k):
+        term = (res3[:, j].float().numpy() * w[:, j:j + 1].numpy()).astype(np.float32)
+        acc = np.where(keep[:, j:j + 1].numpy(), (acc + term).astype(np.float32), acc)
+    assert out.dtype == torch.float32 and np.array_equal(out.cpu().numpy(), acc)
+    m = cv.build_inverse_mapping(tok.to(dev), slot.to(dev), t, k).cpu()
+    assert m.dtype == torch.int64 and (m >= 0).sum() == tok.numel() and torch.equal(m[tok, slot], torch.arange(tok.numel()))
+    assert cv.scatter_weight_reduce_optimized(rows[:0].to(dev), tok.to(dev), slot.to(dev), w.to(dev), t, k).abs().sum() == 0
+    with pytest.raises(ValueError):
+        cv.moe_weighted_sum_triton(res3.to(dev), w[:, :4].to(dev))
+
+
+def sum_k(res3, w):
+    acc = np.zeros((res3.shape[0], res3.shape[2]), dtype=np.float32)
+    for j in range(res3.shape[1]):
+        acc = (acc + (res3[:, j].float().numpy() * w[:, j:j + 1].numpy()).astype(np.float32)).astype(np.float32)
+    return acc
