@@ -65,6 +65,7 @@ _SIGS = {
     "bgmoe_act_quant_ragged": (i32, [vp, vp, vp, i32, i64, i32, vp, vp, i32, vp]),
     "bgmoe_silu_mul_3d": (i32, [vp, vp, vp, i32, i32, i32, vp, vp]),
     "bgmoe_fused_silu_quant_3d": (i32, [vp, vp, vp, i32, i32, i32, vp, vp, vp]),
+    "bgmoe_deepep_ll_scale_repack": (i32, [vp, vp, vp, i32, i32, i32, i32, vp, vp]),
     "bgmoe_dispatch_workspace_bytes": (sz, [i64, i32]),
     "bgmoe_dispatch_scatter_3d": (i32, [vp, vp, i32, i32, i32, vp, i32, i32, i32, vp, vp, vp, vp, sz, vp]),
     "bgmoe_dispatch_scatter_ragged": (i32, [vp, vp, i32, i32, i32, vp, i64, i32, i32, vp, vp, vp, vp, i32, vp, sz, vp]),

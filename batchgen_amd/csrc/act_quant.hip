@@ -344,6 +344,55 @@ extern "C" int bgmoe_fused_silu_quant_3d(const uint16_t* gate, const uint16_t* u
   return launch<kMasked>(a, bgmoe_stream(stream));
 }
 
+namespace {
+// Copies, per expert, the first `span` columns (the live rows rounded up to span_align) of its [kb, s] scale
+// block into columns [e*s, e*s + span) of the [kb, e_count*s] matrix: 16-byte units, a fixed (experts x 8) grid
+// whose work shrinks with the counts.  A count outside [0, s] copies nothing and raises *status.
+constexpr int kRepackThreads = 256;
+constexpr int kRepackSlices = 8;
+__global__ __launch_bounds__(kRepackThreads) void scale_repack_kernel(const float* __restrict__ src,
+                                                                      const int32_t* __restrict__ recv_count,
+                                                                      float* __restrict__ dst, int experts, int kb,
+                                                                      int s, int span_align, int32_t* status) {
+  const int e = blockIdx.x;
+  const int rc = recv_count[e];
+  if (rc < 0 || rc > s) {
+    if (status && blockIdx.y == 0 && threadIdx.x == 0) atomicOr(status, 1);
+    return;
+  }
+  const int quads = (rc + span_align - 1) / span_align * (span_align / 4);
+  const float4* from = reinterpret_cast<const float4*>(src + (int64_t)e * kb * s);
+  float4* to = reinterpret_cast<float4*>(dst + (int64_t)e * s);
+  const int64_t to_pitch = (int64_t)experts * s / 4;
+  const int from_pitch = s / 4;
+  const int total = kb * quads;
+  for (int i = blockIdx.y * kRepackThreads + threadIdx.x; i < total; i += kRepackSlices * kRepackThreads) {
+    const int row = i / quads;
+    const int q = i - row * quads;
+    to[row * to_pitch + q] = from[(int64_t)row * from_pitch + q];
+  }
+}
+}  // namespace
+
+extern "C" int bgmoe_deepep_ll_scale_repack(const float* recv_scales, const int32_t* recv_count, float* out,
+                                            int experts, int kb, int s, int span_align, int32_t* status,
+                                            bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(experts > 0 && kb > 0 && s > 0, "deepep_ll_scale_repack: recv_scales must be non-empty (E=%d KB=%d S=%d)",
+                experts, kb, s);
+  BGMOE_REQUIRE((int64_t)experts * kb * s <= 0x7fffffffLL, "deepep_ll_scale_repack: recv_scales too large for int32 indexing");
+  BGMOE_REQUIRE(span_align > 0 && span_align % 4 == 0 && s % span_align == 0,
+                "deepep_ll_scale_repack: span_align (%d) must be a positive multiple of 4 dividing the expert stride %d",
+                span_align, s);
+  BGMOE_REQUIRE(recv_scales && recv_count && out, "deepep_ll_scale_repack: null pointer");
+  BGMOE_REQUIRE(((uintptr_t)recv_scales | (uintptr_t)out) % 16 == 0,
+                "deepep_ll_scale_repack: recv_scales and out must be 16-byte aligned");
+  const uintptr_t a = (uintptr_t)recv_scales, b = (uintptr_t)out, bytes = (uintptr_t)experts * kb * s * sizeof(float);
+  BGMOE_REQUIRE(a + bytes <= b || b + bytes <= a, "deepep_ll_scale_repack: recv_scales and out must not overlap");
+  hipLaunchKernelGGL(scale_repack_kernel, dim3((unsigned)experts, kRepackSlices), dim3(kRepackThreads), 0,
+                     bgmoe_stream(stream), recv_scales, recv_count, out, experts, kb, s, span_align, status);
+  return bgmoe_check_launch("deepep_ll_scale_repack");
+}
+
 int bgmoe_internal_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h, uint8_t* y,
                                  float* scale, int64_t srow, int64_t skb, int extra_rows, int64_t extra_start,
                                  hipStream_t st) {

@@ -110,3 +110,42 @@ def act_quant_rows(x, y=None, scale=None, scale_transposed=False):
     with torch.cuda.device(x.device):
         check(lib().bgmoe_act_quant_rows(ptr(x), m, k, ptr(y), ptr(scale), srow, skb, stream()))
     return y, scale
+
+
+_BAD_COUNT = {}
+
+
+def deepep_ll_scale_repack_status(device) -> torch.Tensor:
+    """int32 [1] on ``device``: becomes 1 when a ``deepep_ll_scale_repack`` call on that device met a receive
+    count outside [0, S] (the reference traps the device there; here that expert is skipped and the flag is
+    raised). Stays set until the caller zeroes it."""
+    key = str(torch.device(device))
+    t = _BAD_COUNT.get(key)
+    if t is None:
+        t = torch.zeros(1, dtype=torch.int32, device=device)
+        _BAD_COUNT[key] = t
+    return t
+
+
+def deepep_ll_scale_repack(recv_scales, recv_count, out, span_align):
+    """recv_scales: the exchange's [E, S, hidden/128] fp32 view (strides (KB*S, 1, S)) -> out [hidden/128, E*S],
+    each expert's live span (rounded up to span_align) only (fp8_blockwise_ops.cu:744-797). Returns out."""
+    ck.gpu(recv_scales, "recv_scales")
+    ck.cuda_tensor(recv_scales, recv_count, None, "recv_count")
+    ck.cuda_tensor(recv_scales, out, None, "out")
+    if recv_scales.dim() != 3 or recv_scales.dtype != torch.float32:
+        ck.fail("recv_scales must be float32 [E, S, hidden/128]")
+    e, s_, kb = recv_scales.shape
+    if e <= 0 or s_ <= 0 or kb <= 0:
+        ck.fail("recv_scales must be non-empty")
+    if tuple(recv_scales.stride()) != (kb * s_, 1, s_):
+        ck.fail(f"recv_scales must be the (1, 2)-transposed view of a contiguous [E, hidden/128, S] block, i.e. "
+                f"strides ({kb * s_}, 1, {s_}); got {tuple(recv_scales.stride())}")
+    if recv_count.dim() != 1 or recv_count.dtype != torch.int32 or recv_count.shape[0] != e:
+        ck.fail("recv_count must be int32 [E]")
+    if out.dim() != 2 or out.dtype != torch.float32 or tuple(out.shape) != (kb, e * s_) or not out.is_contiguous():
+        ck.fail(f"out must be float32 [hidden/128, E * S] = [{kb}, {e * s_}]")
+    with torch.cuda.device(recv_scales.device):
+        check(lib().bgmoe_deepep_ll_scale_repack(ptr(recv_scales), ptr(recv_count), ptr(out), e, kb, s_, int(span_align),
+                                                 ptr(deepep_ll_scale_repack_status(recv_scales.device)), stream()))
+    return out

@@ -191,6 +191,17 @@ int bgmoe_fused_silu_quant_3d(const uint16_t* gate, const uint16_t* up,
                               const int32_t* tokens_per_expert, int e, int mtp, int k, uint8_t* y,
                               float* scale, bgmoe_stream_t stream);
 
+/* Replaces `deepep_ll_scale_repack` (fp8_blockwise_ops.cu:685-797; wrapper batchgen/models/glm/glm5/moe_ragged.py:330-352):
+ * the low-latency exchange returns activation scales as a contiguous [E, KB, S] fp32 block (KB = hidden/128,
+ * S = rows per expert); out is the [KB, E*S] matrix with expert e at column e*S.  Per expert, columns
+ * [0, ceil(recv_count[e] / span_align) * span_align) of every row are copied bit for bit and the rest of `out`
+ * is left as it is.  span_align: positive multiple of 4 dividing S.  Both buffers 16-byte aligned and disjoint.
+ * A count outside [0, S] copies nothing for that expert and ORs 1 into *status (optional, device; never
+ * cleared here) where the reference traps the device.  The grouped GEMMs of this library also read the
+ * exchange's block in place (bgmoe_fp8_act.scale_group_stride), which needs no repack. */
+int bgmoe_deepep_ll_scale_repack(const float* recv_scales, const int32_t* recv_count, float* out, int experts,
+                                 int kb, int s, int span_align, int32_t* status, bgmoe_stream_t stream);
+
 /* bf16(silu(gate)) * up in bf16, then the per-row, per-128-column FP8 cast, in one pass: the activation
  * between the two grouped GEMMs of the DeepGEMM chains and of the dense shared expert.  Replaces
  *   form 1 (D): `silu_mul_masked_group_quant` / `silu_mul_ragged_group_quant`
