@@ -326,3 +326,86 @@ def test_tiled_kernel_edge_shapes(dev, n, k, layout):
     href = oq.silu_f32(ref) * up
     hh = h.float().cpu().numpy()
     assert og.rel_frobenius(hh[live], href[live]) < 4e-3 and np.all(hh[~live] == 5.0)
+
+
+def test_pointer_tables_slot_permutation_refresh_and_empty_step_under_a_graph(dev):
+    """Contract of the reference's tests/test_moe_grouped_fp8_ptrs.py restated: a captured quant -> stage 1 ->
+    quant -> down chain over pointer tables follows (a) new device-side counts, (b) a slot permutation written
+    into the tables between replays (slot s then holds another expert's weights) and (c) a step in which no
+    expert has rows, which must leave the output as it was; every replay equals the eager stacked-weight ops."""
+    groups, cap, n, k = 4, 32, 256, 384
+    g = torch.Generator().manual_seed(31)
+    x = rand_bf16(g, groups * cap, k)
+    x_d = x.to(dev)
+    mats = []
+    for shape in ((groups, n, k), (groups, n, k), (groups, k, n)):
+        wq, wsc = oq.weight_block_quant((0.03 * torch.randn(*shape, generator=g)).numpy())
+        kb = wsc.shape[2]
+        pad = np.zeros(wsc.shape[:2] + ((kb + 3) // 4 * 4,), dtype=np.float32)
+        pad[..., :kb] = wsc
+        mats.append((torch.from_numpy(wq).to(dev).view(torch.float8_e4m3fn), torch.from_numpy(pad).to(dev)))
+    cu = (torch.arange(groups + 1, dtype=torch.int32) * cap).to(dev)
+    counts = torch.zeros(groups, dtype=torch.int32, device=dev)
+    tables = [torch.zeros(groups, dtype=torch.int64, device=dev) for _ in range(6)]
+
+    def fill_tables(order):
+        for j, (w, s_) in enumerate(mats):
+            tables[2 * j].copy_(torch.tensor([w[i].data_ptr() for i in order], dtype=torch.int64))
+            tables[2 * j + 1].copy_(torch.tensor([s_[i].data_ptr() for i in order], dtype=torch.int64))
+
+    xq = torch.zeros(groups * cap, k, dtype=torch.uint8, device=dev)
+    xs = torch.zeros(k // 128, groups * cap, device=dev)
+    hq = torch.zeros(groups * cap, n, dtype=torch.uint8, device=dev)
+    hs = torch.zeros(n // 128, groups * cap, device=dev)
+    h = torch.zeros(groups * cap, n, dtype=torch.bfloat16, device=dev)
+    out = torch.zeros(groups * cap, k, dtype=torch.bfloat16, device=dev)
+    (gw, gs), (uw, us), (dw, ds) = mats
+
+    def chain(ptrs, order=None):
+        qops().act_quant_ragged(x_d, counts, cu, xq, xs, 16)
+        a = xq.view(torch.float8_e4m3fn)
+        if ptrs:
+            gm().fp8_blockwise_fused_s1_ptrs(a, gw[0], tables[0], uw[0], tables[2], counts, cu, xs, gs[0], tables[1],
+                                             us[0], tables[3], 16, output=h)
+        else:
+            o = list(order)
+            gm().fp8_blockwise_fused_s1(a, gw[o].contiguous(), uw[o].contiguous(), counts, cu, xs, gs[o].contiguous(),
+                                        us[o].contiguous(), 16, output=h)
+        qops().act_quant_ragged(h, counts, cu, hq, hs, 16)
+        b = hq.view(torch.float8_e4m3fn)
+        if ptrs:
+            gm().fp8_blockwise_grouped_gemm_ptrs(b, dw[0], tables[4], counts, cu, hs, ds[0], tables[5], 16, output=out)
+        else:
+            o = list(order)
+            gm().fp8_blockwise_grouped_gemm(b, dw[o].contiguous(), counts, cu, hs, ds[o].contiguous(), 16, output=out)
+
+    steps = [((5, 0, 32, 17), (0, 1, 2, 3)), ((1, 31, 2, 0), (2, 0, 3, 1)), ((0, 0, 0, 0), (2, 0, 3, 1)),
+             ((32, 32, 32, 32), (3, 2, 1, 0)), ((0, 9, 0, 0), (0, 1, 2, 3))]
+    fill_tables(steps[0][1])
+    counts.copy_(torch.tensor(steps[0][0], dtype=torch.int32))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain(True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain(True)
+    previous = None
+    for cnt, order in steps:
+        counts.copy_(torch.tensor(cnt, dtype=torch.int32))
+        fill_tables(order)
+        marker = out.clone() if previous is None else previous.clone()
+        out.copy_(marker)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        out.copy_(marker)
+        chain(False, order)
+        torch.cuda.synchronize()
+        say(f"graph step counts={cnt} order={order}")
+        assert torch.equal(got, out), (cnt, order)
+        if sum(cnt) == 0:
+            assert torch.equal(got, marker)
+        previous = got
