@@ -31,7 +31,15 @@ struct QuantArgs {
   int topk;
   int64_t pairs;         // gather: jobs [0,pairs) are (token,k) pairs, jobs [pairs, jobs) copy
   int64_t extra_start;   //         token (job - pairs) to row extra_start + (job - pairs)
+  int form_a;            // plain rows: amax floored at 2^-16, scale = max(amax * (1/448), 1e-12)
+  const int32_t* num_valid;  // plain rows, optional: rows at or past *num_valid get zero bytes and scale 1e-12
 };
+
+__device__ __forceinline__ float row_scale_from_amax(const QuantArgs& a, float amax, bool pad) {
+  if (!a.form_a) return quant_scale_from_amax(amax);
+  constexpr float kInv448 = 1.0f / 448.0f;
+  return pad ? 1e-12f : fmaxf(fmaxf(amax, 1.52587890625e-05f) * kInv448, 1e-12f);
+}
 
 // state of a destination row: 0 = leave untouched, 1 = valid, 2 = alignment pad
 __device__ __forceinline__ int ragged_row_state(const QuantArgs& a, int64_t row) {
@@ -100,7 +108,7 @@ __device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64
 #pragma unroll
       for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
       amax = wave_max_xor<16>(amax);
-      const float sc = quant_scale_from_amax(amax);
+      const float sc = row_scale_from_amax(a, amax, pad);
       if (in) {
         float q[8];
         quant_div_clamp(v, sc, q);
@@ -131,7 +139,7 @@ __device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64
       if (yr == nullptr) continue;
       float amax = fmaxf(fabsf(v[0]), fabsf(v[1]));
       amax = wave_max_xor<64>(amax);
-      const float sc = quant_scale_from_amax(amax);
+      const float sc = row_scale_from_amax(a, amax, pad);
       float q2[2];
       quant_div_clamp(v, sc, q2);
       const uint32_t p = pack4_e4m3(q2[0], q2[1], 0.0f, 0.0f);
@@ -149,7 +157,9 @@ __global__ __launch_bounds__(256) void act_quant_kernel(QuantArgs a) {
   for (int64_t job = (int64_t)blockIdx.x * 4 + wave; job < a.jobs; job += stride) {
     int64_t src = job, dst = job;
     bool pad = false;
-    if constexpr (MODE == kMasked) {
+    if constexpr (MODE == kPlain) {
+      if (a.num_valid) pad = job >= (int64_t)*a.num_valid;
+    } else if constexpr (MODE == kMasked) {
       const int e = (int)(job / a.mtp);
       const int t = (int)(job - (int64_t)e * a.mtp);
       if (t >= a.counts[e]) continue;
@@ -289,6 +299,18 @@ extern "C" int bgmoe_act_quant_rows(const uint16_t* x, int64_t rows, int k, uint
   QuantArgs a{};
   a.x = x; a.y = y; a.scale = scale; a.jobs = rows; a.k = k;
   a.srow = scale_row_stride; a.skb = scale_kb_stride;
+  return launch<kPlain>(a, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_act_quant_rows_1d(const uint16_t* x, int64_t rows, int k, uint8_t* y, float* scale,
+                                       int64_t scale_row_stride, int64_t scale_kb_stride,
+                                       const int32_t* num_valid_tokens, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(rows >= 0 && k >= 0, "act_quant_rows_1d: negative size");
+  BGMOE_REQUIRE(rows == 0 || k == 0 || (x && y && scale), "act_quant_rows_1d: null pointer");
+  QuantArgs a{};
+  a.x = x; a.y = y; a.scale = scale; a.jobs = rows; a.k = k;
+  a.srow = scale_row_stride; a.skb = scale_kb_stride;
+  a.form_a = 1; a.num_valid = num_valid_tokens;
   return launch<kPlain>(a, bgmoe_stream(stream));
 }
 

@@ -162,6 +162,15 @@ int bgmoe_add_rmsnorm_fp8_quant(uint16_t* residual, const uint16_t* hidden, cons
 int bgmoe_act_quant_rows(const uint16_t* x, int64_t rows, int k, uint8_t* y, float* scale,
                          int64_t scale_row_stride, int64_t scale_kb_stride, bgmoe_stream_t stream);
 
+/* The 1-D quantiser exactly: replaces `per_token_blocked_quantize_bf16_to_fp8_1d`
+ * (batchgen_kernels/triton/fp8_quantize.py:252-391): amax floored at 2^-16, s = fmaxf(amax * (1/448.f), 1e-12f),
+ * q = clamp(x/s, +-448) -> RNE e4m3fn; equals bgmoe_act_quant_rows wherever a block's amax is >= 2^-16.
+ * num_valid_tokens (optional, device int32 scalar): rows at or past it get zero bytes and scale 1e-12.
+ * Scale element (r,kb) at scale[r*srow + kb*skb]: (k/128, 1) contiguous, (1, align4(rows)) MN-major. */
+int bgmoe_act_quant_rows_1d(const uint16_t* x, int64_t rows, int k, uint8_t* y, float* scale,
+                            int64_t scale_row_stride, int64_t scale_kb_stride, const int32_t* num_valid_tokens,
+                            bgmoe_stream_t stream);
+
 /* Masked layout.  Replaces `act_quant_3d`
  * (batchgen_kernels/src/moe/fp8_blockwise/fp8_blockwise_ops.cu:39-111, 519-556).
  * x [e,mtp,k]; rows >= tokens_per_expert[e] are neither read nor written;
