@@ -45,7 +45,7 @@ enum BgmoeKernelId {
   BGMOE_K_S1_SKINNY16, BGMOE_K_S1_SKINNY64, BGMOE_K_S1_TILED,
   BGMOE_K_GEMM_SKINNY16, BGMOE_K_GEMM_SKINNY64, BGMOE_K_GEMM_TILED,
   BGMOE_K_MXFP4_S1, BGMOE_K_MXFP4_GEMM, BGMOE_K_BF16_GEMM, BGMOE_K_ROUTER_GEMM, BGMOE_K_ROUTER_GEMM_REDUCE,
-  BGMOE_K_NORM_QUANT, BGMOE_K_SITU,
+  BGMOE_K_NORM_QUANT, BGMOE_K_SITU, BGMOE_K_DENSE_GEMM,
   BGMOE_K_COUNT
 };
 extern bool g_bgmoe_prof_on;

@@ -51,7 +51,7 @@ hipEvent_t g_pending = nullptr;
 const char* kNames[BGMOE_K_COUNT] = {
     "router", "perm_hist", "perm_scan", "perm_rank", "gather_rows", "act_quant", "combine", "compact",
     "s1_skinny16", "s1_skinny64", "s1_tiled", "gemm_skinny16", "gemm_skinny64", "gemm_tiled",
-    "mxfp4_s1", "mxfp4_gemm", "bf16_gemm", "router_gemm", "router_gemm_reduce", "norm_quant", "situ_and_mul"};
+    "mxfp4_s1", "mxfp4_gemm", "bf16_gemm", "router_gemm", "router_gemm_reduce", "norm_quant", "situ_and_mul", "fp8_dense_gemm"};
 hipEvent_t take_event() {
   if (!g_free.empty()) { hipEvent_t e = g_free.back(); g_free.pop_back(); return e; }
   hipEvent_t e = nullptr;

@@ -23,6 +23,7 @@ from ..quantization.act_quant import act_quant
 
 FP8_DTYPE = torch.float8_e4m3fn
 BLOCK = 128
+DENSE_MAX_ROWS = 64        # up to here the K-split streaming kernel, above it the grouped GEMM with one group
 
 _ROWS = {}
 
@@ -67,9 +68,12 @@ def fp8_gemm_nt(lhs, rhs, d: torch.Tensor) -> None:
     if m == 0:
         return
     act = Fp8Act(ptr(a), ptr(sa), sa.stride(0), sa.stride(1), 0)
-    w = Fp8Weight(ptr(b), n * k, None, ptr(sb), (n // BLOCK) * kb, kb, None, 0, 0)
-    cu, seqlens = _one_group(m, a.device)
     with torch.cuda.device(a.device):
+        if m <= DENSE_MAX_ROWS:
+            check(lib().bgmoe_fp8_dense_gemm(C.byref(act), ptr(b), ptr(sb), kb, m, n, k, ptr(d), stream()))
+            return
+        w = Fp8Weight(ptr(b), n * k, None, ptr(sb), (n // BLOCK) * kb, kb, None, 0, 0)
+        cu, seqlens = _one_group(m, a.device)
         check(lib().bgmoe_fp8_grouped_gemm(C.byref(act), C.byref(w), seqlens, cu, 1, m, n, k, ptr(d), stream()))
 
 

@@ -374,6 +374,16 @@ int bgmoe_fp8_grouped_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* b,
                            const int32_t* seqlens, const int32_t* cu_seqlens, int groups,
                            int64_t m, int n, int k, uint16_t* out, bgmoe_stream_t stream);
 
+/* One weight matrix against few rows: out[m, n] = bf16(dequant(a) @ dequant(w)^T), w [n, k] e4m3fn row-major with
+ * block scales w_scale[(r/128)*scale_nb_stride + c/128].  Replaces `deep_gemm.fp8_gemm_nt` as the reference calls
+ * it for the dense MLP and the shared expert at decode (batchgen/attention/mla/fa3_backend.py:525-590,
+ * batchgen/models/glm/glm5/wrappers.py:448-461).  The K axis is split over the 8 waves of a block and added in a
+ * fixed order that depends on k alone, so the gate and up halves of a stacked [gate; up] weight equal two separate
+ * calls bit for bit.  a->scale_group_stride is ignored.  Weights are streamed once per 64 rows of `a`: meant for
+ * m up to 64 (measured cross-over); beyond that bgmoe_fp8_grouped_gemm with one group is the faster call.  k % 128 == 0, n % 128 == 0. */
+int bgmoe_fp8_dense_gemm(const bgmoe_fp8_act* a, const uint8_t* w, const float* w_scale, int64_t scale_nb_stride,
+                         int64_t m, int n, int k, uint16_t* out, bgmoe_stream_t stream);
+
 /* Tuning knob (no reference counterpart): groups with at most `rows` rows are served by the
  * weight-streaming kernel, larger ones by the LDS-tiled kernel.  0 sends everything to the tiled
  * kernel.  Default 256 (or the environment variable BGMOE_SKINNY_MAX_ROWS at first use).

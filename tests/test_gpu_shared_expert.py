@@ -159,3 +159,41 @@ def test_argument_policy(dev):
     with pytest.raises(RuntimeError, match="block scales"):
         Fp8DenseExpert(fused.gate, fused.gate_scale[:1], fused.up, fused.up_scale, fused.down, fused.down_scale,
                        gate_up=fused.gate_up)
+
+
+@pytest.mark.parametrize("m", [1, 4, 15, 16, 17, 32, 33, 63, 64])
+@pytest.mark.parametrize("n,k", [(128, 128), (256, 384), (1152, 1024), (8320, 256), (512, 7168), (16512, 128), (6272, 256)])
+def test_dense_k_split_gemm_vs_oracle_and_stacked_halves(dev, m, n, k):
+    """The K-split streaming GEMM (rows <= DENSE_MAX_ROWS) against the fp32 dequantise-then-matmul oracle at the
+    reference's single-GEMM gate (rtol 2e-2 / atol 5e-3, tests/test_moe_compact_ragged_fp8.py:370-377), with
+    row-major and MN-major activation scales; the two halves of the weight give the bytes of the whole."""
+    from batchgen_amd.moe.shared_expert import DENSE_MAX_ROWS, fp8_gemm_nt
+    assert m <= DENSE_MAX_ROWS
+    g = torch.Generator().manual_seed(m * 31 + n + k)
+    x = rand_bf16(g, m, k)
+    xq, xs = oq.act_quant(_bf16_np(x), form="A")
+    wq, ws = oq.weight_block_quant((0.05 * torch.randn(1, n, k, generator=g)).numpy())
+    want = og.grouped_gemm_fp8(xq, xs, wq, ws, np.array([m], np.int32), np.array([0, m], np.int32), to_bf16=False)
+    a = torch.from_numpy(xq).to(dev).view(torch.float8_e4m3fn)
+    b = torch.from_numpy(wq[0]).to(dev).view(torch.float8_e4m3fn)
+    sb = torch.from_numpy(ws[0]).to(dev)
+    sa_row = torch.from_numpy(xs).to(dev)
+    sa_mn = torch.empty(k // 128, (m + 3) // 4 * 4, device=dev).transpose(0, 1)[:m]
+    sa_mn.copy_(sa_row)
+    outs = []
+    for sa in (sa_row, sa_mn):
+        d = torch.full((m, n), -7.0, dtype=torch.bfloat16, device=dev)
+        fp8_gemm_nt((a, sa), (b, sb), d)
+        outs.append(d)
+    assert torch.equal(outs[0], outs[1])
+    got = outs[0].cpu().float().numpy()
+    np.testing.assert_allclose(got, want, rtol=2e-2, atol=5e-3)
+    rel = np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30)
+    assert rel < 4e-3, rel
+    if n >= 256:
+        half = n // 2 // 128 * 128
+        lo = torch.empty(m, half, dtype=torch.bfloat16, device=dev)
+        hi = torch.empty(m, n - half, dtype=torch.bfloat16, device=dev)
+        fp8_gemm_nt((a, sa_row), (b[:half], sb[:half // 128]), lo)
+        fp8_gemm_nt((a, sa_row), (b[half:], sb[half // 128:]), hi)
+        assert torch.equal(torch.cat([lo, hi], dim=1), outs[0])
