@@ -152,23 +152,59 @@ void launch_dense(const DenseArgs& g, hipStream_t st) {
 
 }  // namespace
 
+// defined in gemm_fp8_skinny.hip
+int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w, int64_t m, int n, int k,
+                                    int per, float* workspace, uint16_t* out, hipStream_t st);
+
+// K-blocks per slice of the split-K form for m rows, 0 = use the wave-split kernel above.  A function of m, k and
+// the layout only, never of n, so that a stacked [gate; up] weight and its halves are added in the same order.
+static int splitk_per(int64_t m, int k, int layout) {
+  const int deep = k >= 16384 ? 16 : 8;                 // measured: longer slices once K is long enough to fill the chip
+  if (layout != BGMOE_W_ROW_MAJOR || m > 64) return deep;
+  if (m <= 16) return 0;
+  if (k >= 16384) return 16;
+  return m > 32 && k >= 4096 ? 8 : 0;
+}
+
+extern "C" int64_t bgmoe_fp8_dense_gemm_workspace(int64_t m, int n, int k, int layout) {
+  if (m <= 0 || n <= 0 || k <= 0) return 0;
+  const int per = splitk_per(m, k, layout);
+  if (per <= 0) return 0;
+  return ((k / 128 + per - 1) / per) * m * n * (int64_t)sizeof(float);
+}
+
 extern "C" int bgmoe_fp8_dense_gemm(const bgmoe_fp8_act* a, const uint8_t* w, const float* w_scale,
-                                    int64_t scale_nb_stride, int64_t m, int n, int k, uint16_t* out,
-                                    bgmoe_stream_t stream) {
+                                    int64_t scale_nb_stride, int layout, int64_t m, int n, int k, uint16_t* out,
+                                    void* workspace, int64_t workspace_bytes, bgmoe_stream_t stream) {
   BGMOE_REQUIRE(a != nullptr, "fp8_dense_gemm: null operand descriptor");
   BGMOE_REQUIRE(m >= 0 && m <= 65535LL * 16, "fp8_dense_gemm: m=%lld out of range", (long long)m);
   BGMOE_REQUIRE(k > 0 && k % 128 == 0, "fp8_dense_gemm: K=%d must be a positive multiple of 128", k);
   BGMOE_REQUIRE(n > 0 && n % 128 == 0, "fp8_dense_gemm: N=%d must be a positive multiple of 128", n);
+  BGMOE_REQUIRE(layout == BGMOE_W_ROW_MAJOR || layout == BGMOE_W_TILE_MAJOR, "fp8_dense_gemm: unknown weight layout %d",
+                layout);
   if (m == 0) return BGMOE_OK;
   BGMOE_REQUIRE(a->x && a->scale && w && w_scale && out, "fp8_dense_gemm: null pointer");
   BGMOE_REQUIRE(scale_nb_stride >= k / 128, "fp8_dense_gemm: weight-scale row stride %lld < K/128 = %d",
                 (long long)scale_nb_stride, k / 128);
   BGMOE_REQUIRE(((uintptr_t)a->x | (uintptr_t)w) % 16 == 0 && (uintptr_t)out % 8 == 0,
                 "fp8_dense_gemm: x and w must be 16-byte aligned, out 8-byte aligned");
-  DenseArgs g{};
-  g.a = *a; g.w = w; g.ws = w_scale; g.ws_nb_stride = scale_nb_stride; g.m = m; g.n = n; g.k = k; g.out = out;
   hipStream_t st = bgmoe_stream(stream);
   BgmoeProf prof(BGMOE_K_DENSE_GEMM, st);
+  const int per = splitk_per(m, k, layout);
+  if (per > 0) {
+    const int64_t need = bgmoe_fp8_dense_gemm_workspace(m, n, k, layout);
+    BGMOE_REQUIRE(workspace != nullptr && workspace_bytes >= need && (uintptr_t)workspace % 16 == 0,
+                  "fp8_dense_gemm: m=%lld n=%d k=%d needs a 16-byte aligned workspace of %lld bytes "
+                  "(bgmoe_fp8_dense_gemm_workspace), got %lld", (long long)m, n, k, (long long)need,
+                  (long long)workspace_bytes);
+    bgmoe_fp8_act act = *a;
+    act.scale_group_stride = 0;
+    bgmoe_fp8_weight wd{};
+    wd.w = w; wd.scale = w_scale; wd.scale_nb_stride = scale_nb_stride; wd.layout = layout;
+    return bgmoe_internal_fp8_dense_splitk(&act, &wd, m, n, k, per, (float*)workspace, out, st);
+  }
+  DenseArgs g{};
+  g.a = *a; g.w = w; g.ws = w_scale; g.ws_nb_stride = scale_nb_stride; g.m = m; g.n = n; g.k = k; g.out = out;
   // weight tiles per block (measured): more of them re-use the token bytes a block fetches from L2, fewer of
   // them give more blocks; a handful of rows is all weight traffic and wants the blocks
   const int tiles = n / 16;

@@ -53,6 +53,8 @@ struct SkinnyArgs {
   BgmoeSplit split;           // this launch serves groups with count <= bgmoe_split_limit(...)
   int64_t row_bound;          // host-side upper bound on the total live rows
   int64_t group_bound;        // host-side upper bound on the rows of any one group (0 = unknown)
+  float* part;                // split-K launches: fp32 partial sums [slice][row][n] instead of `out`
+  int64_t part_slice_stride;
 };
 
 template <int NSC>
@@ -88,20 +90,21 @@ struct TokSlot {
 // One work item: up to 16*TT rows of one group x one n-tile, streamed over K.
 template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP>
 __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const BgmoeItem& it, float (*s_amax)[TT][16],
-                                                const uint8_t* ring, uint32_t ring_lds) {
+                                                const uint8_t* ring, uint32_t ring_lds, int kb_lo = 0, int kb_n = -1,
+                                                int slice = 0) {
   constexpr int NT = 4;                  // weight tiles per wave
   constexpr int NSC = FUSED ? 2 : 1;     // weight-scale streams per wave
   constexpr int kSlot = TokSlot<TT>::kBytes;
   constexpr int LT = TT / 2;             // token half-tile loads per wave and K-block
   const int grp = it.grp, cnt = it.cnt, ntile = it.ntile, chunk = it.chunk;
-  const int64_t row0 = g.cu[grp];
+  const int64_t row0 = g.cu ? g.cu[grp] : 0;
   const int wave = threadIdx.x >> 6;
   const uint32_t wave_u = __builtin_amdgcn_readfirstlane((uint32_t)wave);
   const int lane = threadIdx.x & 63;
   const int r16 = lane & 15;
   const int kq = lane >> 4;
   const int K = g.k;
-  const int KB = K >> 7;
+  const int KB = kb_n < 0 ? K >> 7 : kb_n;               // K-blocks [kb_lo, kb_lo + KB) of the row (split-K: a slice)
   const int n0 = ntile * (FUSED ? 128 : 256);
 
   const uint8_t* wb[2];
@@ -122,16 +125,17 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
     // a tile past N streams the last valid tile instead (its results are never stored): every load
     // below is unconditional, which lets the compiler keep precise vmcnt() waits
     const int nr = min(nrow, g.n - 16);
-    if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) wp[t] = wb[FUSED ? (t >> 1) : 0] + (int64_t)(nr + r16) * K + 16 * kq;
-    else wp[t] = wb[FUSED ? (t >> 1) : 0] + (int64_t)(nr >> 4) * K * 16 + lane * 16;
+    if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR)
+      wp[t] = wb[FUSED ? (t >> 1) : 0] + (int64_t)(nr + r16) * K + 16 * kq + ((int64_t)kb_lo << 7);
+    else wp[t] = wb[FUSED ? (t >> 1) : 0] + (int64_t)(nr >> 4) * K * 16 + lane * 16 + ((int64_t)kb_lo << 11);
   }
   const float* wsp[NSC];
   if constexpr (FUSED) {
-    wsp[0] = wsb[0] + (int64_t)(n0 >> 7) * g.w0.scale_nb_stride;
-    wsp[1] = wsb[1] + (int64_t)(n0 >> 7) * g.w1.scale_nb_stride;
+    wsp[0] = wsb[0] + (int64_t)(n0 >> 7) * g.w0.scale_nb_stride + kb_lo;
+    wsp[1] = wsb[1] + (int64_t)(n0 >> 7) * g.w1.scale_nb_stride + kb_lo;
   } else {
     const int nb = min(n0 + 64 * wave, g.n - 1) >> 7;
-    wsp[0] = wsb[0] + (int64_t)nb * g.w0.scale_nb_stride;
+    wsp[0] = wsb[0] + (int64_t)nb * g.w0.scale_nb_stride + kb_lo;
   }
 
   const int t0 = chunk * 16 * TT;
@@ -142,7 +146,7 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
   // A load covers rows 8j..8j+7 of a tile: lane p = (row p>>3, LDS chunk p&7) fetches the row's 16-byte
   // chunk (p&7) ^ (p>>3) -- whole 128-byte lines, XOR-swizzled so that the MFMA operand reads below are
   // conflict free.  Wave w loads half-tiles w*LT .. w*LT+LT-1; rows past the count re-read the last row.
-  const uint8_t* tok_base = uniform_ptr(g.a.x + (row0 + t0) * K);
+  const uint8_t* tok_base = uniform_ptr(g.a.x + (row0 + t0) * K + ((int64_t)kb_lo << 7));
   uint32_t tok_off[LT];
   bool tok_on[LT];
 #pragma unroll
@@ -152,9 +156,10 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
     tok_off[i] = (uint32_t)row * (uint32_t)K + (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
     tok_on[i] = (h >> 1) < tiles;
   }
-  const float* xs_base = uniform_ptr(g.a.scale_group_stride
-                                        ? g.a.scale + grp * g.a.scale_group_stride + (int64_t)t0 * g.a.scale_row_stride
-                                        : g.a.scale + (row0 + t0) * g.a.scale_row_stride);
+  const float* xs_base = uniform_ptr((g.a.scale_group_stride
+                                         ? g.a.scale + grp * g.a.scale_group_stride + (int64_t)t0 * g.a.scale_row_stride
+                                         : g.a.scale + (row0 + t0) * g.a.scale_row_stride) +
+                                     (int64_t)kb_lo * g.a.scale_kb_stride);
   const uint32_t xs_off = (uint32_t)min(lane, live - 1) * (uint32_t)g.a.scale_row_stride * 4u;
 
   auto issue_tokens = [&](int kb, int slot) {
@@ -293,6 +298,11 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
         if (!tv[t]) continue;
+        if (g.part != nullptr) {
+          *reinterpret_cast<floatx4*>(g.part + slice * g.part_slice_stride + (row0 + tok) * g.n + n0 + 64 * wave +
+                                      16 * t + 4 * kq) = acc[tt][t];
+          continue;
+        }
         uint2 o;
         o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
         o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
@@ -319,6 +329,46 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned 
     if (it.cnt > 16 * TT) fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, true>(g, it, s_amax, s_ring, ring_lds);
     else fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, false>(g, it, s_amax, s_ring, ring_lds);
     __syncthreads();                      // s_amax and the token ring are reused by the next item
+  }
+}
+
+// One weight matrix against m rows (host-known), K split over `ksplit` blocks per (n-tile, 64-row chunk): the
+// item function above on K-blocks [slice * per, ...), fp32 partial sums to g.part; splitk_reduce_kernel adds the
+// slices in ascending order.
+template <int LAYOUT>
+__global__ __launch_bounds__(256) void fp8_dense_splitk_kernel(SkinnyArgs g, int m, int ksplit, int per) {
+  constexpr int TT = 4, NSTAGE = 2;
+  __shared__ float s_amax[4][TT][16];
+  __shared__ __align__(16) uint8_t s_ring[NSTAGE * TokSlot<TT>::kBytes];
+  const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
+  const int ntiles = (g.n + 255) / 256;
+  unsigned b = blockIdx.x;
+  const int slice = (int)(b % (unsigned)ksplit);
+  b /= (unsigned)ksplit;
+  BgmoeItem it;
+  it.grp = 0;
+  it.cnt = m;
+  it.ntile = (int)(b % (unsigned)ntiles);
+  it.chunk = (int)(b / (unsigned)ntiles);
+  const int kb_lo = slice * per;
+  const int kb_n = min(per, (g.k >> 7) - kb_lo);                       // >= 1 by the host's choice of ksplit
+  if (m > 16 * TT) fp8_skinny_item<TT, NSTAGE, false, LAYOUT, true>(g, it, s_amax, s_ring, ring_lds, kb_lo, kb_n, slice);
+  else fp8_skinny_item<TT, NSTAGE, false, LAYOUT, false>(g, it, s_amax, s_ring, ring_lds, kb_lo, kb_n, slice);
+}
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int64_t slice_stride,
+                                                            int ksplit, int64_t quads, uint16_t* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < quads; i += (int64_t)gridDim.x * 256) {
+    floatx4 sum = *reinterpret_cast<const floatx4*>(part + 4 * i);
+    for (int s = 1; s < ksplit; ++s) {
+      const floatx4 p = *reinterpret_cast<const floatx4*>(part + s * slice_stride + 4 * i);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum[j] += p[j];
+    }
+    uint2 o;
+    o.x = pack2_bf16(sum[0], sum[1]);
+    o.y = pack2_bf16(sum[2], sum[3]);
+    *reinterpret_cast<uint2*>(out + 4 * i) = o;
   }
 }
 
@@ -500,4 +550,28 @@ extern "C" int bgmoe_fp8_fused_s1(const bgmoe_fp8_act* a, const bgmoe_fp8_weight
   g.n = n; g.k = k; g.out = out; g.out_q = out_q; g.out_s = out_scale;
   g.os_row = out_scale_row_stride; g.os_nb = out_scale_nb_stride;
   return launch_skinny(true, g, m, bgmoe_stream(stream));
+}
+
+// Split-K form of the weight-streaming GEMM for ONE group of m host-known rows (no device counts): `per`
+// K-blocks per slice; workspace holds ceil(K/128 / per) slices of m*n floats.
+int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w, int64_t m, int n, int k,
+                                    int per, float* workspace, uint16_t* out, hipStream_t st) {
+  const int kb = k >> 7;
+  const int ksplit = (kb + per - 1) / per;
+  SkinnyArgs g{};
+  g.a = *a; g.w0 = *w; g.groups = 1; g.n = n; g.k = k; g.out = out;
+  g.part = workspace; g.part_slice_stride = m * n;
+  const unsigned blocks = (unsigned)(((n + 255) / 256) * ((m + 63) / 64) * ksplit);
+  if (w->layout == BGMOE_W_TILE_MAJOR)
+    hipLaunchKernelGGL(fp8_dense_splitk_kernel<BGMOE_W_TILE_MAJOR>, dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+  else
+    hipLaunchKernelGGL(fp8_dense_splitk_kernel<BGMOE_W_ROW_MAJOR>, dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+  int rc = bgmoe_check_launch("fp8_dense_gemm (split-K)");
+  if (rc != BGMOE_OK) return rc;
+  const int64_t quads = m * n / 4;
+  int64_t rblocks = (quads + 255) / 256;
+  if (rblocks > 4096) rblocks = 4096;
+  hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)rblocks), dim3(256), 0, st, workspace, g.part_slice_stride,
+                     ksplit, quads, out);
+  return bgmoe_check_launch("fp8_dense_gemm (reduce)");
 }

@@ -23,7 +23,9 @@ from ..quantization.act_quant import act_quant
 
 FP8_DTYPE = torch.float8_e4m3fn
 BLOCK = 128
-DENSE_MAX_ROWS = 64        # up to here the K-split streaming kernel, above it the grouped GEMM with one group
+DENSE_MAX_ROWS = 64        # up to here the K-split dense kernel for any N (measured cross-overs against the
+DENSE_MAX_ROWS_NARROW = 512  # grouped GEMM with one group), up to here for N <= DENSE_NARROW_N
+DENSE_NARROW_N = 8192
 
 _ROWS = {}
 
@@ -42,9 +44,25 @@ def _one_group(m: int, device):
     return base, base + 4
 
 
-def fp8_gemm_nt(lhs, rhs, d: torch.Tensor) -> None:
+_SCRATCH = {}
+
+
+def _workspace(nbytes: int, device):
+    """Split-K partial sums: one buffer per device, grown on demand (a call that fits allocates nothing)."""
+    if nbytes <= 0:
+        return None
+    key = str(device)
+    t = _SCRATCH.get(key)
+    if t is None or t.numel() < nbytes:
+        t = torch.empty(max(nbytes, 1 << 24), dtype=torch.uint8, device=device)
+        _SCRATCH[key] = t
+    return t
+
+
+def fp8_gemm_nt(lhs, rhs, d: torch.Tensor, weight_layout: str = "row_major") -> None:
     """``d = dequant(a) @ dequant(b).T`` (bf16).  a [M, K] e4m3fn with scales [M, K/128] fp32, row-major or
-    MN-major (any strides); b [N, K] with block scales [N/128, K/128]."""
+    MN-major (any strides); b [N, K] with block scales [N/128, K/128].  ``weight_layout="tile_major"`` (no reference
+    counterpart) takes ``b`` in the resident layout of ``fp8_weight_repack``."""
     a, sa = lhs
     b, sb = rhs
     if a.dim() != 2 or b.dim() != 2 or d.dim() != 2:
@@ -67,12 +85,16 @@ def fp8_gemm_nt(lhs, rhs, d: torch.Tensor) -> None:
                            f"{sb.dtype}")
     if m == 0:
         return
+    layout = {"row_major": 0, "tile_major": 1}[weight_layout]
     act = Fp8Act(ptr(a), ptr(sa), sa.stride(0), sa.stride(1), 0)
     with torch.cuda.device(a.device):
-        if m <= DENSE_MAX_ROWS:
-            check(lib().bgmoe_fp8_dense_gemm(C.byref(act), ptr(b), ptr(sb), kb, m, n, k, ptr(d), stream()))
+        if m <= DENSE_MAX_ROWS or (m <= DENSE_MAX_ROWS_NARROW and n <= DENSE_NARROW_N):
+            need = lib().bgmoe_fp8_dense_gemm_workspace(m, n, k, layout)
+            ws = _workspace(need, a.device)
+            check(lib().bgmoe_fp8_dense_gemm(C.byref(act), ptr(b), ptr(sb), kb, layout, m, n, k, ptr(d), ptr(ws), need,
+                                             stream()))
             return
-        w = Fp8Weight(ptr(b), n * k, None, ptr(sb), (n // BLOCK) * kb, kb, None, 0, 0)
+        w = Fp8Weight(ptr(b), n * k, None, ptr(sb), (n // BLOCK) * kb, kb, None, layout, 0)
         cu, seqlens = _one_group(m, a.device)
         check(lib().bgmoe_fp8_grouped_gemm(C.byref(act), C.byref(w), seqlens, cu, 1, m, n, k, ptr(d), stream()))
 

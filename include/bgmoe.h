@@ -374,15 +374,23 @@ int bgmoe_fp8_grouped_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* b,
                            const int32_t* seqlens, const int32_t* cu_seqlens, int groups,
                            int64_t m, int n, int k, uint16_t* out, bgmoe_stream_t stream);
 
-/* One weight matrix against few rows: out[m, n] = bf16(dequant(a) @ dequant(w)^T), w [n, k] e4m3fn row-major with
- * block scales w_scale[(r/128)*scale_nb_stride + c/128].  Replaces `deep_gemm.fp8_gemm_nt` as the reference calls
- * it for the dense MLP and the shared expert at decode (batchgen/attention/mla/fa3_backend.py:525-590,
- * batchgen/models/glm/glm5/wrappers.py:448-461).  The K axis is split over the 8 waves of a block and added in a
- * fixed order that depends on k alone, so the gate and up halves of a stacked [gate; up] weight equal two separate
- * calls bit for bit.  a->scale_group_stride is ignored.  Weights are streamed once per 64 rows of `a`: meant for
- * m up to 64 (measured cross-over); beyond that bgmoe_fp8_grouped_gemm with one group is the faster call.  k % 128 == 0, n % 128 == 0. */
+/* One weight matrix against few rows: out[m, n] = bf16(dequant(a) @ dequant(w)^T), w [n, k] e4m3fn (row-major, or the
+ * tile-major resident layout) with block scales w_scale[(r/128)*scale_nb_stride + c/128].  Replaces
+ * `deep_gemm.fp8_gemm_nt` as the reference calls it for the dense MLP and the shared expert at decode
+ * (batchgen/attention/mla/fa3_backend.py:525-590, batchgen/models/glm/glm5/wrappers.py:448-461).  A grouped launch has
+ * too few work items for one group, so K is the parallel axis here, in one of two forms chosen from m, k and the
+ * layout (never from n).  Wave split: the 8 waves of a block own one K-slice each and add their partial sums through
+ * LDS in wave order (no workspace).  Block split: the weight-streaming kernel of the grouped GEMM on K-slices, fp32
+ * partial sums in `workspace` (bgmoe_fp8_dense_gemm_workspace(m, n, k, layout) bytes, 0 for the wave split; 16-byte
+ * aligned, caller-owned, contents irrelevant before and after), added in ascending slice order by a second launch.
+ * Every call is deterministic, and the gate and up halves of a stacked [gate; up] weight equal two separate
+ * calls bit for bit.  a->scale_group_stride is ignored.  Weights are streamed once per 64 rows: measured faster than
+ * bgmoe_fp8_grouped_gemm with one group up to 64 rows for any n, and up to 512 rows for n <= 8192.
+ * k % 128 == 0, n % 128 == 0. */
+int64_t bgmoe_fp8_dense_gemm_workspace(int64_t m, int n, int k, int layout);
 int bgmoe_fp8_dense_gemm(const bgmoe_fp8_act* a, const uint8_t* w, const float* w_scale, int64_t scale_nb_stride,
-                         int64_t m, int n, int k, uint16_t* out, bgmoe_stream_t stream);
+                         int layout, int64_t m, int n, int k, uint16_t* out, void* workspace, int64_t workspace_bytes,
+                         bgmoe_stream_t stream);
 
 /* Tuning knob (no reference counterpart): groups with at most `rows` rows are served by the
  * weight-streaming kernel, larger ones by the LDS-tiled kernel.  0 sends everything to the tiled

@@ -161,14 +161,16 @@ def test_argument_policy(dev):
                        gate_up=fused.gate_up)
 
 
-@pytest.mark.parametrize("m", [1, 4, 15, 16, 17, 32, 33, 63, 64])
+@pytest.mark.parametrize("m", [1, 4, 15, 16, 17, 32, 33, 63, 64, 65, 130, 257, 512])
 @pytest.mark.parametrize("n,k", [(128, 128), (256, 384), (1152, 1024), (8320, 256), (512, 7168), (16512, 128), (6272, 256)])
 def test_dense_k_split_gemm_vs_oracle_and_stacked_halves(dev, m, n, k):
-    """The K-split streaming GEMM (rows <= DENSE_MAX_ROWS) against the fp32 dequantise-then-matmul oracle at the
+    """The K-split dense GEMM (both of its forms: wave split, block split with a workspace) against the fp32 dequantise-then-matmul oracle at the
     reference's single-GEMM gate (rtol 2e-2 / atol 5e-3, tests/test_moe_compact_ragged_fp8.py:370-377), with
     row-major and MN-major activation scales; the two halves of the weight give the bytes of the whole."""
-    from batchgen_amd.moe.shared_expert import DENSE_MAX_ROWS, fp8_gemm_nt
-    assert m <= DENSE_MAX_ROWS
+    from batchgen_amd.moe.shared_expert import DENSE_MAX_ROWS, DENSE_MAX_ROWS_NARROW, DENSE_NARROW_N, fp8_gemm_nt
+    if m > DENSE_MAX_ROWS and n > DENSE_NARROW_N:
+        pytest.skip("served by the grouped GEMM")
+    assert m <= DENSE_MAX_ROWS_NARROW
     g = torch.Generator().manual_seed(m * 31 + n + k)
     x = rand_bf16(g, m, k)
     xq, xs = oq.act_quant(_bf16_np(x), form="A")
@@ -197,3 +199,26 @@ def test_dense_k_split_gemm_vs_oracle_and_stacked_halves(dev, m, n, k):
         fp8_gemm_nt((a, sa_row), (b[:half], sb[:half // 128]), lo)
         fp8_gemm_nt((a, sa_row), (b[half:], sb[half // 128:]), hi)
         assert torch.equal(torch.cat([lo, hi], dim=1), outs[0])
+
+
+@pytest.mark.parametrize("m", [3, 16, 40, 64, 200, 700])
+def test_dense_gemm_on_tile_major_weights(dev, m):
+    from batchgen_amd.kernels import load_extension
+    from batchgen_amd.moe.shared_expert import fp8_gemm_nt
+    n, k = 512, 1024
+    g = torch.Generator().manual_seed(m)
+    xq, xs = oq.act_quant(_bf16_np(rand_bf16(g, m, k)), form="A")
+    wq, ws = oq.weight_block_quant((0.05 * torch.randn(1, n, k, generator=g)).numpy())
+    want = og.grouped_gemm_fp8(xq, xs, wq, ws, np.array([m], np.int32), np.array([0, m], np.int32), to_bf16=False)
+    a = torch.from_numpy(xq).to(dev).view(torch.float8_e4m3fn)
+    b = torch.from_numpy(wq[0]).to(dev).view(torch.float8_e4m3fn)
+    tiled = load_extension("batchgen_kernels.moe._C_fp8_blockwise_gemm").fp8_weight_repack(b)
+    sa, sb = torch.from_numpy(xs).to(dev), torch.from_numpy(ws[0]).to(dev)
+    d_row = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    d_tile = torch.empty(m, n, dtype=torch.bfloat16, device=dev)
+    fp8_gemm_nt((a, sa), (b, sb), d_row)
+    fp8_gemm_nt((a, sa), (tiled, sb), d_tile, weight_layout="tile_major")
+    np.testing.assert_allclose(d_tile.cpu().float().numpy(), want, rtol=2e-2, atol=5e-3)
+    np.testing.assert_allclose(d_row.cpu().float().numpy(), want, rtol=2e-2, atol=5e-3)
+    if m > 64:                                        # both layouts take the block-split form with equal slices
+        assert torch.equal(d_row, d_tile)
