@@ -31,6 +31,7 @@ struct QuantArgs {
   int topk;
   int64_t pairs;         // gather: jobs [0,pairs) are (token,k) pairs, jobs [pairs, jobs) copy
   int64_t extra_start;   //         token (job - pairs) to row extra_start + (job - pairs)
+  int split_steps;       // 16-byte path: one wave per (row, 512 columns) instead of one wave per row
   int form_a;            // plain rows: amax floored at 2^-16, scale = max(amax * (1/448), 1e-12)
   const int32_t* num_valid;  // plain rows, optional: rows at or past *num_valid get zero bytes and scale 1e-12
 };
@@ -58,8 +59,9 @@ __device__ __forceinline__ int ragged_row_state(const QuantArgs& a, int64_t row)
   return rel < valid ? 1 : 2;
 }
 
+// VEC8: the wave quantises the 512-column pieces [s_lo, s_hi) of the row.
 template <bool VEC8>
-__device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64_t dst, bool pad) {
+__device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64_t dst, bool pad, int s_lo, int s_hi) {
   const int lane = lane_id();
   const int k = a.k;
   const uint16_t* xr = a.x + src * (int64_t)k;
@@ -70,8 +72,7 @@ __device__ __forceinline__ void quant_row(const QuantArgs& a, int64_t src, int64
 
   if constexpr (VEC8) {
     // 64 lanes x 8 elements = 4 blocks of 128 per step; 16 lanes share a block
-    const int steps = (k + 511) / 512;
-    for (int s = 0; s < steps; ++s) {
+    for (int s = s_lo; s < s_hi; ++s) {
       const int c0 = s * 512 + lane * 8;
       const bool in = c0 < k;
       float v[8];
@@ -154,7 +155,13 @@ template <int MODE, bool VEC8>
 __global__ __launch_bounds__(256) void act_quant_kernel(QuantArgs a) {
   const int wave = threadIdx.x >> 6;
   const int64_t stride = (int64_t)gridDim.x * 4;
-  for (int64_t job = (int64_t)blockIdx.x * 4 + wave; job < a.jobs; job += stride) {
+  // few rows (16-byte path): one wave per (row, 512 columns), so that they still spread over the chip and no wave
+  // carries a chain of dependent reductions; many rows: one wave per row, which overlaps the pieces' loads
+  const int pieces = (a.k + 511) / 512;
+  const int steps = VEC8 && a.split_steps ? pieces : 1;
+  for (int64_t wjob = (int64_t)blockIdx.x * 4 + wave; wjob < a.jobs * steps; wjob += stride) {
+    const int64_t job = wjob / steps;
+    const int step = (int)(wjob - job * steps);
     int64_t src = job, dst = job;
     bool pad = false;
     if constexpr (MODE == kPlain) {
@@ -178,7 +185,7 @@ __global__ __launch_bounds__(256) void act_quant_kernel(QuantArgs a) {
         dst = a.extra_start + src;
       }
     }
-    quant_row<VEC8>(a, src, dst, pad);
+    quant_row<VEC8>(a, src, dst, pad, steps > 1 ? step : 0, steps > 1 ? step + 1 : pieces);
   }
 }
 
@@ -273,14 +280,18 @@ __global__ __launch_bounds__(256) void scatter_fp8_kernel(const uint8_t* xq, con
   }
 }
 
+constexpr int64_t kSplitBelowRows = 2048;      // fewer rows than the chip has wave slots
+
 template <int MODE>
-int launch(const QuantArgs& a, hipStream_t st) {
+int launch(const QuantArgs& a_in, hipStream_t st) {
+  QuantArgs a = a_in;
   if (a.jobs <= 0 || a.k <= 0) return BGMOE_OK;
-  int64_t blocks = (a.jobs + 3) / 4;
-  if (blocks > 16384) blocks = 16384;
   auto aligned = [](const void* p, size_t n) { return p == nullptr || ((uintptr_t)p % n) == 0; };
   const bool vec = (a.k % 8 == 0) && aligned(a.x, 16) && aligned(a.up, 16) && aligned(a.y, 8) &&
                    aligned(a.h_out, 16);
+  a.split_steps = vec && a.jobs < kSplitBelowRows;
+  int64_t blocks = (a.jobs * (a.split_steps ? (a.k + 511) / 512 : 1) + 3) / 4;
+  if (blocks > 16384) blocks = 16384;
   BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
   if (vec)
     hipLaunchKernelGGL((act_quant_kernel<MODE, true>), dim3((unsigned)blocks), dim3(256), 0, st, a);
@@ -482,7 +493,7 @@ struct GroupQuantArgs {
   const int32_t* starts;
   int groups;
   int64_t max_rows;
-  int n, form;
+  int n, form, split_steps;
   uint8_t* out;
   int64_t ose, oss;
   float* scale;
@@ -490,12 +501,16 @@ struct GroupQuantArgs {
   uint16_t* prod;
 };
 
-// One wave per (group, row): 8 columns per lane and pass, 16 lanes per 128-column quantisation group.
+// 8 columns per lane and pass, 16 lanes per 128-column quantisation group.  Few rows: one wave per (group, row,
+// 512 columns); many rows: one wave per (group, row).
 __global__ __launch_bounds__(256) void silu_mul_group_quant_kernel(GroupQuantArgs a) {
   const int lane = lane_id();
-  const int64_t jobs = (int64_t)a.groups * a.max_rows;
+  const int steps = a.split_steps ? (a.n + 511) / 512 : 1;
+  const int64_t jobs = (int64_t)a.groups * a.max_rows * steps;
   const int64_t stride = (int64_t)gridDim.x * 4;
-  for (int64_t job = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); job < jobs; job += stride) {
+  for (int64_t wjob = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); wjob < jobs; wjob += stride) {
+    const int64_t job = wjob / steps;
+    const int step = (int)(wjob - job * steps);
     const int e = (int)(job / a.max_rows);
     const int64_t r = job - (int64_t)e * a.max_rows;
     if (a.counts && r >= a.counts[e]) continue;
@@ -504,7 +519,8 @@ __global__ __launch_bounds__(256) void silu_mul_group_quant_kernel(GroupQuantArg
     const uint16_t* upp = a.up + e * a.ise + row * a.iss;
     uint8_t* op = a.out + e * a.ose + row * a.oss;
     float* sp = a.scale + e * a.sse + row * a.sss;
-    for (int c0 = lane * 8; c0 < a.n; c0 += 512) {
+    const int c_end = a.split_steps ? min(a.n, (step + 1) * 512) : a.n;
+    for (int c0 = step * 512 + lane * 8; c0 < c_end; c0 += 512) {
       const uint4 gv = *reinterpret_cast<const uint4*>(gp + c0);
       const uint4 uv = *reinterpret_cast<const uint4*>(upp + c0);
       const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
@@ -572,7 +588,8 @@ extern "C" int bgmoe_silu_mul_group_quant(const uint16_t* gate, const uint16_t* 
   a.groups = groups; a.max_rows = max_rows; a.n = n; a.form = form; a.out = out; a.ose = out_stride_e;
   a.oss = out_stride_s; a.scale = scale; a.sse = scale_stride_e; a.sss = scale_stride_s; a.ssg = scale_stride_g;
   a.prod = prod_out;
-  int64_t blocks = ((int64_t)groups * max_rows + 3) / 4;
+  a.split_steps = (int64_t)groups * max_rows < kSplitBelowRows;
+  int64_t blocks = ((int64_t)groups * max_rows * (a.split_steps ? (n + 511) / 512 : 1) + 3) / 4;
   if (blocks > 16384) blocks = 16384;
   hipStream_t st = bgmoe_stream(stream);
   BgmoeProf prof(BGMOE_K_ACT_QUANT, st);

@@ -11,7 +11,8 @@ experts local, masked layout).  Prints ONE JSON line.
 
 `--op router_gemm` and `--op norm_quant` time the two producers that sit in front of the layer on the same
 configuration's shapes (hidden states -> logits -> routes in two launches; residual add + RMSNorm + FP8
-cast in one) and print the same kind of line for them.
+cast in one) and print the same kind of line for them.  `--op dense_expert [--rows R]` times the dense FP8 expert
+chain (the shared expert as the reference's model code runs it outside the grouped launch).
 """
 from __future__ import annotations
 
@@ -60,8 +61,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4, 5],
                     help="0-4: the benchmark set's configurations; 5: the Kimi-K3 latent MoE layer at its real shape")
-    ap.add_argument("--op", default="layer", choices=["layer", "router_gemm", "norm_quant"],
-                    help="what one step is: the MoE layer (default), or one of its two producers")
+    ap.add_argument("--op", default="layer", choices=["layer", "router_gemm", "norm_quant", "dense_expert"],
+                    help="what one step is: the MoE layer (default), one of its two producers, or the dense FP8 "
+                         "expert chain (the shared expert outside the grouped launch) on the configuration's shapes")
+    ap.add_argument("--rows", type=int, default=0, help="--op dense_expert: rows per step (default: the "
+                                                        "configuration's token count)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of one captured HIP graph of the layer instead of eager launches")
@@ -219,6 +223,8 @@ def bench_producer(a):
                                    "sample": f"{m} of {n} tokens, float64 BLAS product + NumPy router", "seconds": t}
         print(json.dumps(out))
         return
+    if a.op == "dense_expert":
+        return bench_dense_expert(a, cfg, dev, g, base)
     res = (torch.randn(n, h, generator=g, device=dev) * 0.9).to(torch.bfloat16)
     hid = (torch.randn(n, h, generator=g, device=dev) * 0.4).to(torch.bfloat16)
     gamma = (torch.randn(h, generator=g, device=dev) * 0.3 + 1.0).to(torch.bfloat16)
@@ -254,6 +260,67 @@ def bench_producer(a):
         t = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": alg_bytes * (m / n) / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
                                "sample": f"{m} of {n} rows, NumPy oracle, one thread", "seconds": t}
+    print(json.dumps(out))
+
+
+def bench_dense_expert(a, cfg, dev, g, base):
+    """One step = quantise(x) -> [gate; up] GEMM -> SiLU * up + quantise -> down GEMM of ONE dense FP8 expert
+    (hidden x shared_inter of the configuration) on `rows` rows."""
+    import numpy as np
+    import torch
+    from batchgen_amd import _lib
+    from batchgen_amd.moe.shared_expert import Fp8DenseExpert
+    rows = a.rows or cfg.n_tokens
+    h, inter = cfg.hidden, cfg.shared_inter or cfg.inter
+
+    def fp8_weight(n, k):
+        q = (torch.randn(n, k, generator=g, device=dev) * 64).to(torch.float8_e4m3fn)
+        sc = torch.rand(n // 128, k // 128, generator=g, device=dev) * 2e-4 + 1e-4
+        return q, sc
+    gate_up, gu_s = fp8_weight(2 * inter, h)
+    down, d_s = fp8_weight(h, inter)
+    expert = Fp8DenseExpert(gate_up[:inter], gu_s[:inter // 128].contiguous(), gate_up[inter:],
+                            gu_s[inter // 128:].contiguous(), down, d_s, gate_up=gate_up)
+    x = (torch.randn(rows, h, generator=g, device=dev) * 0.5).to(torch.bfloat16)
+    out_buf = torch.empty(rows, h, dtype=torch.bfloat16, device=dev)
+    step = lambda: expert(x, out=out_buf)
+    ms = _time(step, a.steps, a.warmup, torch)
+    _lib.prof_enable(True)
+    for _ in range(a.steps):
+        step()
+    prof = _lib.prof_collect()
+    _lib.prof_enable(False)
+    key = "fp8_dense_gemm" if "fp8_dense_gemm" in prof else "gemm_skinny16"
+    k_ms = prof[key][0] / prof[key][1]                       # average over the chain's two GEMMs
+    w_bytes = 3 * inter * h + (3 * inter * h // 16384) * 4
+    alg_bytes = w_bytes + rows * h * 2 * 2                   # weights once, bf16 rows in and out
+    gemm_bytes = w_bytes / 2                                 # per GEMM launch, averaged like k_ms
+    roof = dict(bound="hbm", kernel=key + " (average of the chain's gate_up and down GEMMs)",
+                achieved=gemm_bytes / (k_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None,
+                bytes_per_launch=gemm_bytes, avg_launch_us=k_ms * 1e3)
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    out = dict(base, metric="dense FP8 expert chain: HBM GB/s over its algorithmic bytes, 1xMI355X",
+               value=alg_bytes / (ms * 1e-3) / 1e9, unit="GB/s", ms_per_step=ms,
+               dtype="e4m3 x e4m3 -> fp32, bf16 in and out",
+               config={"workload": cfg.name + " / dense_expert", "rows": rows, "hidden": h, "intermediate": inter},
+               tokens_per_s=rows / (ms * 1e-3), kernel_ms_per_step={kk: v[0] / a.steps for kk, v in prof.items()},
+               roofline=roof)
+    if not a.no_cpu_baseline:
+        from oracle import gemm as og                        # the CPU port is the baseline leg only
+        from oracle import quant as oq
+        m = min(rows, 32)
+        one = np.array([m], np.int32), np.array([0, m], np.int32)
+        gq, gs = gate_up.cpu().view(torch.uint8).numpy()[None], gu_s.cpu().numpy()[None]
+        dq, ds = down.cpu().view(torch.uint8).numpy()[None], d_s.cpu().numpy()[None]
+        t0 = time.perf_counter()
+        xq, xs = oq.act_quant(x[:m].float().cpu().numpy(), form="A")
+        gu = og.grouped_gemm_fp8(xq, xs, gq, gs, *one)
+        hq, hs, _ = oq.silu_mul_group_quant(gu[:, :inter], gu[:, inter:], "A")
+        og.grouped_gemm_fp8(hq, hs, dq, ds, *one)
+        t = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": alg_bytes / t / 1e9, "unit": "GB/s", "cores": min(os.cpu_count() or 1, 16),
+                               "kind": "port", "sample": f"{m} of {rows} rows, NumPy oracle chain (weights "
+                               "dequantised once per call, as the algorithmic bytes count them)", "seconds": t}
     print(json.dumps(out))
 
 
