@@ -280,7 +280,8 @@ __global__ __launch_bounds__(256) void scatter_fp8_kernel(const uint8_t* xq, con
   }
 }
 
-constexpr int64_t kSplitBelowRows = 2048;      // fewer rows than the chip has wave slots
+constexpr int64_t kSplitBelowRows = 4097;      // up to about two rows per wave slot of the chip (measured cross-over
+                                               // between 4096 and 8192 fully live rows)
 
 template <int MODE>
 int launch(const QuantArgs& a_in, hipStream_t st) {
