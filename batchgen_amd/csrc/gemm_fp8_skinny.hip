@@ -88,11 +88,13 @@ struct TokSlot {
 };
 
 // One work item: up to 16*TT rows of one group x one n-tile, streamed over K.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP>
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP, int NTW = 4>
 __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const BgmoeItem& it, float (*s_amax)[TT][16],
                                                 const uint8_t* ring, uint32_t ring_lds, int kb_lo = 0, int kb_n = -1,
                                                 int slice = 0) {
-  constexpr int NT = 4;                  // weight tiles per wave
+  constexpr int NT = NTW;                // weight tiles per wave
+  static_assert(NT == 4 || (!FUSED && NT == 2), "stage 1 pairs two gate and two up tiles per wave");
+  constexpr int WCOLS = 16 * NT;         // plain GEMM: output columns per wave (4 waves per item)
   constexpr int NSC = FUSED ? 2 : 1;     // weight-scale streams per wave
   constexpr int kSlot = TokSlot<TT>::kBytes;
   constexpr int LT = TT / 2;             // token half-tile loads per wave and K-block
@@ -105,7 +107,7 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
   const int kq = lane >> 4;
   const int K = g.k;
   const int KB = kb_n < 0 ? K >> 7 : kb_n;               // K-blocks [kb_lo, kb_lo + KB) of the row (split-K: a slice)
-  const int n0 = ntile * (FUSED ? 128 : 256);
+  const int n0 = ntile * (FUSED ? 128 : 4 * WCOLS);
 
   const uint8_t* wb[2];
   const float* wsb[2];
@@ -120,7 +122,7 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
   bool tv[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const int nrow = FUSED ? n0 + 32 * wave + 16 * (t & 1) : n0 + 64 * wave + 16 * t;
+    const int nrow = FUSED ? n0 + 32 * wave + 16 * (t & 1) : n0 + WCOLS * wave + 16 * t;
     tv[t] = nrow < g.n;
     // a tile past N streams the last valid tile instead (its results are never stored): every load
     // below is unconditional, which lets the compiler keep precise vmcnt() waits
@@ -134,7 +136,7 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
     wsp[0] = wsb[0] + (int64_t)(n0 >> 7) * g.w0.scale_nb_stride + kb_lo;
     wsp[1] = wsb[1] + (int64_t)(n0 >> 7) * g.w1.scale_nb_stride + kb_lo;
   } else {
-    const int nb = min(n0 + 64 * wave, g.n - 1) >> 7;
+    const int nb = min(n0 + WCOLS * wave, g.n - 1) >> 7;
     wsp[0] = wsb[0] + (int64_t)nb * g.w0.scale_nb_stride + kb_lo;
   }
 
@@ -224,7 +226,7 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
   for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
-      wait_vm<8>();
+      wait_vm<2 * NT>();
       block_barrier();
       issue_tokens(min(kb0 + s + NSTAGE - 1, KB - 1), (s + NSTAGE - 1) % NSTAGE);
       load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
@@ -299,14 +301,14 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
       for (int t = 0; t < NT; ++t) {
         if (!tv[t]) continue;
         if (g.part != nullptr) {
-          *reinterpret_cast<floatx4*>(g.part + slice * g.part_slice_stride + (row0 + tok) * g.n + n0 + 64 * wave +
+          *reinterpret_cast<floatx4*>(g.part + slice * g.part_slice_stride + (row0 + tok) * g.n + n0 + WCOLS * wave +
                                       16 * t + 4 * kq) = acc[tt][t];
           continue;
         }
         uint2 o;
         o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
         o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
-        *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + 64 * wave + 16 * t + 4 * kq) = o;
+        *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + WCOLS * wave + 16 * t + 4 * kq) = o;
       }
     }
   }
@@ -341,7 +343,8 @@ __global__ __launch_bounds__(256) void fp8_dense_splitk_kernel(SkinnyArgs g, int
   __shared__ float s_amax[4][TT][16];
   __shared__ __align__(16) uint8_t s_ring[NSTAGE * TokSlot<TT>::kBytes];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
-  const int ntiles = (g.n + 255) / 256;
+  constexpr int NTW = 2;                                               // 128 output columns per item
+  const int ntiles = (g.n + 127) / 128;
   unsigned b = blockIdx.x;
   const int slice = (int)(b % (unsigned)ksplit);
   b /= (unsigned)ksplit;
@@ -352,8 +355,8 @@ __global__ __launch_bounds__(256) void fp8_dense_splitk_kernel(SkinnyArgs g, int
   it.chunk = (int)(b / (unsigned)ntiles);
   const int kb_lo = slice * per;
   const int kb_n = min(per, (g.k >> 7) - kb_lo);                       // >= 1 by the host's choice of ksplit
-  if (m > 16 * TT) fp8_skinny_item<TT, NSTAGE, false, LAYOUT, true>(g, it, s_amax, s_ring, ring_lds, kb_lo, kb_n, slice);
-  else fp8_skinny_item<TT, NSTAGE, false, LAYOUT, false>(g, it, s_amax, s_ring, ring_lds, kb_lo, kb_n, slice);
+  if (m > 16 * TT) fp8_skinny_item<TT, NSTAGE, false, LAYOUT, true, NTW>(g, it, s_amax, s_ring, ring_lds, kb_lo, kb_n, slice);
+  else fp8_skinny_item<TT, NSTAGE, false, LAYOUT, false, NTW>(g, it, s_amax, s_ring, ring_lds, kb_lo, kb_n, slice);
 }
 
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ part, int64_t slice_stride,
@@ -561,7 +564,7 @@ int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weig
   SkinnyArgs g{};
   g.a = *a; g.w0 = *w; g.groups = 1; g.n = n; g.k = k; g.out = out;
   g.part = workspace; g.part_slice_stride = m * n;
-  const unsigned blocks = (unsigned)(((n + 255) / 256) * ((m + 63) / 64) * ksplit);
+  const unsigned blocks = (unsigned)(((n + 127) / 128) * ((m + 63) / 64) * ksplit);
   if (w->layout == BGMOE_W_TILE_MAJOR)
     hipLaunchKernelGGL(fp8_dense_splitk_kernel<BGMOE_W_TILE_MAJOR>, dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
   else
