@@ -5,7 +5,8 @@
   262-330, 607-632): dense ``[T, K, H]`` expert results times ``[T, K]`` weights -> ``[T, H]`` in the input dtype;
 * ``build_inverse_mapping`` / ``scatter_weight_reduce_optimized``
   (batchgen/models/deepseek/deepseekv3/modeling_deepseek_v3.py:1474-1542): sparse ``[nnz, H]`` results with the
-  (token, slot) of every row -> fp32 ``[T, H]``.
+  (token, slot) of every row -> fp32 ``[T, H]``;
+* ``moe_fp32_accum_triton_v2`` (:1034-1065): expert-sorted rows and their sorting permutation -> ``[T, H]``.
 
 The block-size and version arguments select among the reference's Triton kernels, which all compute the same sum:
 accepted and ignored.
@@ -88,4 +89,28 @@ def scatter_weight_reduce_optimized(res: torch.Tensor, global_indices: torch.Ten
     with torch.cuda.device(res.device):
         check(lib().bgmoe_reduce_weighted_scatter_fp32(ptr(res), ptr(pos), ptr(topk_weight.contiguous()), num_tokens,
                                                        hidden, num_experts_per_tok, ptr(out), stream()))
+    return out
+
+
+def moe_fp32_accum_triton_v2(outs: torch.Tensor, idxs: torch.Tensor, topk_weights: torch.Tensor) -> torch.Tensor:
+    """The prefill combine of ``DeepseekV3MoE_Prefill.moe_infer``
+    (batchgen/models/deepseek/deepseekv3/modeling_deepseek_v3.py:1034-1065): ``outs`` [T * K, H] are the expert
+    outputs in expert-sorted order, ``idxs`` the sorting permutation (sorted row j came from flat (token, k) index
+    ``idxs[j]``); returns ``[T, H]`` in the dtype of ``outs``, fp32 accumulation over k ascending.  The product and
+    the sum are rounded separately here; whether the reference's Triton kernel contracts them into one fused
+    multiply-add is decided by its compiler (parity unpinned at the last fp32 bit, before the bf16 rounding)."""
+    t, k = topk_weights.shape
+    if outs.dim() != 2 or outs.shape[0] != t * k or idxs.numel() != t * k:
+        raise ValueError(f"outs must be [{t * k}, H] and idxs [{t * k}]; got {tuple(outs.shape)} and {tuple(idxs.shape)}")
+    if outs.dtype != torch.bfloat16 or not outs.is_cuda or not outs.is_contiguous() or not 1 <= k <= _MAX_K:
+        raise ValueError(f"outs must be a contiguous CUDA bfloat16 tensor and topk in [1, {_MAX_K}]")
+    h = outs.shape[1]
+    out = torch.empty((t, h), dtype=outs.dtype, device=outs.device)
+    if t == 0 or h == 0:
+        return out
+    pos = torch.empty(t * k, dtype=torch.int32, device=outs.device)
+    pos[idxs.reshape(-1).long()] = torch.arange(t * k, dtype=torch.int32, device=outs.device)
+    w = topk_weights.to(torch.float32).contiguous()
+    with torch.cuda.device(outs.device):
+        check(lib().bgmoe_reduce_weighted_scatter(ptr(outs), ptr(pos), ptr(w), t, h, k, ptr(out), -1, None, 0, stream()))
     return out

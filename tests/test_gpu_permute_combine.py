@@ -255,6 +255,12 @@ def test_legacy_combine_helpers(dev):
     assert cv.scatter_weight_reduce_optimized(rows[:0].to(dev), tok.to(dev), slot.to(dev), w.to(dev), t, k).abs().sum() == 0
     with pytest.raises(ValueError):
         cv.moe_weighted_sum_triton(res3.to(dev), w[:, :4].to(dev))
+    # expert-sorted rows + the sorting permutation (the prefill path's combine)
+    ids = torch.randint(0, 16, (t * k,), generator=g)
+    idxs = ids.argsort(stable=True)
+    sorted_rows = res3.view(t * k, h)[idxs]
+    got = cv.moe_fp32_accum_triton_v2(sorted_rows.to(dev), idxs.to(dev), w.to(dev))
+    assert got.dtype == torch.bfloat16 and torch.equal(got.cpu(), want)
 
 
 def sum_k(res3, w):
