@@ -45,3 +45,25 @@ def test_recv_count_histogram():
         m.accumulate_recv_count_histogram(torch.zeros(7, dtype=torch.int32), counts, 64)
     with pytest.raises(RuntimeError):
         m.accumulate_recv_count_histogram(hist, counts.view(2, 3), 64)
+
+
+def test_norm_quant_fuse_policy(monkeypatch):
+    from batchgen_amd.attention import norm_quant_fuse_policy as p
+    assert p.glm5_norm_quant_fuse_enabled() is True
+    assert all(p.glm5_norm_quant_fuse_site_enabled(s) for s in p.GLM5_NORM_QUANT_FUSE_SITES)
+    with pytest.raises(ValueError):
+        p.glm5_norm_quant_fuse_site_enabled("shared")
+    monkeypatch.setattr(p, "GLM5_NORM_QUANT_FUSE_DISABLED_SITES", ("q_a",))
+    assert not p.glm5_norm_quant_fuse_site_enabled("q_a") and p.glm5_norm_quant_fuse_site_enabled("shared_expert")
+    monkeypatch.setattr(p, "GLM5_NORM_QUANT_FUSE_DISABLED_SITES", ("q_b",))
+    with pytest.raises(ValueError):
+        p.glm5_norm_quant_fuse_site_enabled("q_a")
+    monkeypatch.setattr(p, "GLM5_NORM_QUANT_FUSE_DISABLED_SITES", "q_a")
+    with pytest.raises(TypeError):
+        p.glm5_norm_quant_fuse_site_enabled("q_a")
+    monkeypatch.setattr(p, "GLM5_NORM_QUANT_FUSE_DISABLED_SITES", ())
+    monkeypatch.setattr(p, "GLM5_NORM_QUANT_FUSE", False)
+    assert not p.glm5_norm_quant_fuse_site_enabled("shared_expert")
+    monkeypatch.setattr(p, "GLM5_NORM_QUANT_FUSE", 1)
+    with pytest.raises(TypeError):
+        p.glm5_norm_quant_fuse_enabled()
