@@ -2,8 +2,8 @@
 // weight-streaming kernel bound by HBM bandwidth.
 //
 // Work split: item = (group, up to 32 or 64 rows, 128 gate + 128 up output columns) for the fused
-// stage 1, (group, rows, 256 output columns) for a single GEMM; 4 waves, each owning four 16-row
-// weight tiles over the whole K.  A weight byte is read from HBM once per item, straight into
+// stage 1, (group, rows, 128 output columns) for a single GEMM; 4 waves, each owning four (stage 1) or
+// two 16-row weight tiles over the whole K.  A weight byte is read from HBM once per item, straight into
 // registers (no LDS: no other wave needs it), with 16-byte loads and a multi-stage register prefetch
 // so that each wave keeps 16-24 KB of loads in flight.  The item's tokens are needed by all four
 // waves: they go through a small LDS ring filled by asynchronous global -> LDS loads, one copy per
@@ -316,20 +316,21 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
 
 // Persistent grid: block b works on virtual blocks b, b + gridDim.x, ... until the item list ends, so
 // a launch sized from host-side bounds pays nothing for the (many) virtual blocks past the real work.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, int NTW = 4>
 __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned vblocks) {
   __shared__ float s_amax[4][TT][16];
   __shared__ __align__(16) uint8_t s_ring[NSTAGE * TokSlot<TT>::kBytes];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
-  const int ntiles = (g.n + (FUSED ? 127 : 255)) / (FUSED ? 128 : 256);
+  constexpr int kItemCols = FUSED ? 128 : 64 * NTW;
+  const int ntiles = (g.n + kItemCols - 1) / kItemCols;
   const int hi = bgmoe_split_limit(g.seqlens, g.groups, g.split);
   for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
     const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, 0, hi, 16 * TT, ntiles, vb);
     if (it.grp == BGMOE_ITEM_END) break;
     if (it.grp == BGMOE_ITEM_PAD) continue;
     // a group with several row chunks has its weights streamed once per chunk: keep them cacheable
-    if (it.cnt > 16 * TT) fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, true>(g, it, s_amax, s_ring, ring_lds);
-    else fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, false>(g, it, s_amax, s_ring, ring_lds);
+    if (it.cnt > 16 * TT) fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, true, NTW>(g, it, s_amax, s_ring, ring_lds);
+    else fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, false, NTW>(g, it, s_amax, s_ring, ring_lds);
     __syncthreads();                      // s_amax and the token ring are reused by the next item
   }
 }
@@ -418,17 +419,17 @@ static unsigned resident_blocks(K kernel, unsigned* cache) {
   return *cache;
 }
 
-template <int TT, int NS, bool FUSED, int LAYOUT>
+template <int TT, int NS, bool FUSED, int LAYOUT, int NTW = 4>
 static unsigned skinny_resident() {
   static unsigned resident = 0;
-  return resident_blocks(fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>, &resident);
+  return resident_blocks(fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW>, &resident);
 }
 
-template <int TT, int NS, bool FUSED, int LAYOUT>
+template <int TT, int NS, bool FUSED, int LAYOUT, int NTW = 4>
 static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
-  const unsigned cap = skinny_resident<TT, NS, FUSED, LAYOUT>();
+  const unsigned cap = skinny_resident<TT, NS, FUSED, LAYOUT, NTW>();
   const dim3 grid(vblocks < cap ? vblocks : cap), block(256);
-  hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks);
+  hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW>), grid, block, 0, st, g, vblocks);
 }
 
 // Stage 1 works on 32-row items (its epilogue keeps 16*TT x 8 fp32 results per lane alive next to the
@@ -441,9 +442,11 @@ static void launch_variant(bool fused, int layout, int n, int groups, int64_t bo
     if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 3, true, BGMOE_W_TILE_MAJOR>(vb, g, st);
     else launch_one<2, 3, true, BGMOE_W_ROW_MAJOR>(vb, g, st);
   } else {
-    const unsigned vb = bgmoe_item_grid((n + 255) / 256, groups, bound, hi, 64);
-    if (layout == BGMOE_W_TILE_MAJOR) launch_one<4, 2, false, BGMOE_W_TILE_MAJOR>(vb, g, st);
-    else launch_one<4, 2, false, BGMOE_W_ROW_MAJOR>(vb, g, st);
+    // 128-column items (two weight tiles per wave): twice as many, half as long as 256-column ones, which evens
+    // out the last round of the persistent grid (measured: -5% to -10% on the down projection)
+    const unsigned vb = bgmoe_item_grid((n + 127) / 128, groups, bound, hi, 64);
+    if (layout == BGMOE_W_TILE_MAJOR) launch_one<4, 2, false, BGMOE_W_TILE_MAJOR, 2>(vb, g, st);
+    else launch_one<4, 2, false, BGMOE_W_ROW_MAJOR, 2>(vb, g, st);
   }
 }
 
@@ -451,8 +454,8 @@ static void launch_variant(bool fused, int layout, int n, int groups, int64_t bo
 int bgmoe_internal_init_fp8_skinny() {
   skinny_resident<2, 3, true, BGMOE_W_TILE_MAJOR>();
   skinny_resident<2, 3, true, BGMOE_W_ROW_MAJOR>();
-  skinny_resident<4, 2, false, BGMOE_W_TILE_MAJOR>();
-  skinny_resident<4, 2, false, BGMOE_W_ROW_MAJOR>();
+  skinny_resident<4, 2, false, BGMOE_W_TILE_MAJOR, 2>();
+  skinny_resident<4, 2, false, BGMOE_W_ROW_MAJOR, 2>();
   return BGMOE_OK;
 }
 
