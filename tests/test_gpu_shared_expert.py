@@ -162,7 +162,8 @@ def test_argument_policy(dev):
 
 
 @pytest.mark.parametrize("m", [1, 4, 15, 16, 17, 32, 33, 63, 64, 65, 130, 257, 512])
-@pytest.mark.parametrize("n,k", [(128, 128), (256, 384), (1152, 1024), (8320, 256), (512, 7168), (16512, 128), (6272, 256)])
+@pytest.mark.parametrize("n,k", [(128, 128), (256, 384), (1152, 1024), (8320, 256), (512, 7168), (16512, 128), (6272, 256), (256, 1152),
+                                  (384, 2176), (256, 4224)])
 def test_dense_k_split_gemm_vs_oracle_and_stacked_halves(dev, m, n, k):
     """The K-split dense GEMM (both of its forms: wave split, block split with a workspace) against the fp32 dequantise-then-matmul oracle at the
     reference's single-GEMM gate (rtol 2e-2 / atol 5e-3, tests/test_moe_compact_ragged_fp8.py:370-377), with
