@@ -62,6 +62,8 @@ _SIGS = {
     "bgmoe_rmsnorm": (i32, [vp, vp, i64, i32, f32, vp, vp]),
     "bgmoe_act_quant_rows": (i32, [vp, i64, i32, vp, vp, i64, i64, vp]),
     "bgmoe_fp8_dense_gemm": (i32, [vp, vp, vp, i64, i32, i64, i32, i32, vp, vp, i64, vp]),
+    "bgmoe_fp8_dense_gemm_partials": (i32, [vp, vp, vp, i64, i32, i64, i32, i32, vp, i64, C.POINTER(i32), vp]),
+    "bgmoe_silu_mul_group_quant_partials": (i32, [vp, i32, i64, i64, i32, i32, vp, i64, vp, i64, i64, vp]),
     "bgmoe_fp8_dense_gemm_workspace": (i64, [i64, i32, i32, i32]),
     "bgmoe_act_quant_rows_1d": (i32, [vp, i64, i32, vp, vp, i64, i64, vp, vp]),
     "bgmoe_act_quant_3d": (i32, [vp, vp, i32, i32, i32, vp, vp, vp]),

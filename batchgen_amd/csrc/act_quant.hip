@@ -500,6 +500,9 @@ struct GroupQuantArgs {
   float* scale;
   int64_t sse, sss, ssg;
   uint16_t* prod;
+  const float* part;     // optional: gate | up as fp32 partial-sum planes [slices][rows][2n] instead of bf16 rows
+  int slices;
+  int64_t part_slice_stride;
 };
 
 // 8 columns per lane and pass, 16 lanes per 128-column quantisation group.  Few rows: one wave per (group, row,
@@ -522,9 +525,29 @@ __global__ __launch_bounds__(256) void silu_mul_group_quant_kernel(GroupQuantArg
     float* sp = a.scale + e * a.sse + row * a.sss;
     const int c_end = a.split_steps ? min(a.n, (step + 1) * 512) : a.n;
     for (int c0 = step * 512 + lane * 8; c0 < c_end; c0 += 512) {
-      const uint4 gv = *reinterpret_cast<const uint4*>(gp + c0);
-      const uint4 uv = *reinterpret_cast<const uint4*>(upp + c0);
-      const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w}, uw[4] = {uv.x, uv.y, uv.z, uv.w};
+      uint32_t gw[4], uw[4];
+      if (a.part != nullptr) {
+        // the GEMM's K-slices are added here, in slice order, and rounded to bf16 as the GEMM's own output would be
+        const float* pg = a.part + row * (2 * (int64_t)a.n) + c0;
+        floatx4 sg0 = *reinterpret_cast<const floatx4*>(pg), sg1 = *reinterpret_cast<const floatx4*>(pg + 4);
+        floatx4 su0 = *reinterpret_cast<const floatx4*>(pg + a.n), su1 = *reinterpret_cast<const floatx4*>(pg + a.n + 4);
+        for (int sl = 1; sl < a.slices; ++sl) {
+          const float* ps = pg + sl * a.part_slice_stride;
+          const floatx4 g0 = *reinterpret_cast<const floatx4*>(ps), g1 = *reinterpret_cast<const floatx4*>(ps + 4);
+          const floatx4 u0 = *reinterpret_cast<const floatx4*>(ps + a.n), u1 = *reinterpret_cast<const floatx4*>(ps + a.n + 4);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) { sg0[j] += g0[j]; sg1[j] += g1[j]; su0[j] += u0[j]; su1[j] += u1[j]; }
+        }
+        gw[0] = pack2_bf16(sg0[0], sg0[1]); gw[1] = pack2_bf16(sg0[2], sg0[3]);
+        gw[2] = pack2_bf16(sg1[0], sg1[1]); gw[3] = pack2_bf16(sg1[2], sg1[3]);
+        uw[0] = pack2_bf16(su0[0], su0[1]); uw[1] = pack2_bf16(su0[2], su0[3]);
+        uw[2] = pack2_bf16(su1[0], su1[1]); uw[3] = pack2_bf16(su1[2], su1[3]);
+      } else {
+        const uint4 gv = *reinterpret_cast<const uint4*>(gp + c0);
+        const uint4 uv = *reinterpret_cast<const uint4*>(upp + c0);
+        gw[0] = gv.x; gw[1] = gv.y; gw[2] = gv.z; gw[3] = gv.w;
+        uw[0] = uv.x; uw[1] = uv.y; uw[2] = uv.z; uw[3] = uv.w;
+      }
       float p[8];
       uint32_t pw[4];
       float sv[8];
@@ -596,6 +619,32 @@ extern "C" int bgmoe_silu_mul_group_quant(const uint16_t* gate, const uint16_t* 
   BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
   hipLaunchKernelGGL(silu_mul_group_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a);
   return bgmoe_check_launch("silu_mul_group_quant");
+}
+
+extern "C" int bgmoe_silu_mul_group_quant_partials(const float* partials, int slices, int64_t slice_stride,
+                                                   int64_t rows, int n, int form, uint8_t* out, int64_t out_stride_s,
+                                                   float* scale, int64_t scale_stride_s, int64_t scale_stride_g,
+                                                   bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(rows >= 0 && slices >= 1, "silu_mul_group_quant_partials: bad sizes rows=%lld slices=%d", (long long)rows,
+                slices);
+  BGMOE_REQUIRE(n > 0 && n % 128 == 0, "silu_mul_group_quant_partials: width %d must be a positive multiple of 128", n);
+  BGMOE_REQUIRE(form == 0 || form == 1, "silu_mul_group_quant_partials: form must be 0 or 1");
+  if (rows == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(partials && out && scale, "silu_mul_group_quant_partials: null pointer");
+  BGMOE_REQUIRE((uintptr_t)partials % 16 == 0 && slice_stride % 4 == 0 && (uintptr_t)out % 8 == 0 && out_stride_s % 8 == 0 &&
+                    out_stride_s >= n,
+                "silu_mul_group_quant_partials: misaligned buffers or row stride smaller than the row");
+  GroupQuantArgs a{};
+  a.groups = 1; a.max_rows = rows; a.n = n; a.form = form; a.out = out; a.oss = out_stride_s;
+  a.scale = scale; a.sss = scale_stride_s; a.ssg = scale_stride_g;
+  a.part = partials; a.slices = slices; a.part_slice_stride = slice_stride;
+  a.split_steps = rows < kSplitBelowRows;
+  int64_t blocks = (rows * (a.split_steps ? (n + 511) / 512 : 1) + 3) / 4;
+  if (blocks > 16384) blocks = 16384;
+  hipStream_t st = bgmoe_stream(stream);
+  BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
+  hipLaunchKernelGGL(silu_mul_group_quant_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a);
+  return bgmoe_check_launch("silu_mul_group_quant_partials");
 }
 
 namespace {

@@ -173,6 +173,37 @@ extern "C" int64_t bgmoe_fp8_dense_gemm_workspace(int64_t m, int n, int k, int l
   return ((k / 128 + per - 1) / per) * m * n * (int64_t)sizeof(float);
 }
 
+extern "C" int bgmoe_fp8_dense_gemm_partials(const bgmoe_fp8_act* a, const uint8_t* w, const float* w_scale,
+                                             int64_t scale_nb_stride, int layout, int64_t m, int n, int k,
+                                             void* workspace, int64_t workspace_bytes, int* slices,
+                                             bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(a != nullptr && slices != nullptr, "fp8_dense_gemm_partials: null argument");
+  BGMOE_REQUIRE(m > 0 && m <= 65535LL * 16, "fp8_dense_gemm_partials: m=%lld out of range", (long long)m);
+  BGMOE_REQUIRE(k > 0 && k % 128 == 0 && n > 0 && n % 128 == 0,
+                "fp8_dense_gemm_partials: K=%d and N=%d must be positive multiples of 128", k, n);
+  BGMOE_REQUIRE(layout == BGMOE_W_ROW_MAJOR || layout == BGMOE_W_TILE_MAJOR,
+                "fp8_dense_gemm_partials: unknown weight layout %d", layout);
+  const int per = splitk_per(m, k, layout);
+  BGMOE_REQUIRE(per > 0, "fp8_dense_gemm_partials: m=%lld k=%d is served without partial sums "
+                "(bgmoe_fp8_dense_gemm_workspace is 0): call bgmoe_fp8_dense_gemm", (long long)m, k);
+  const int64_t need = bgmoe_fp8_dense_gemm_workspace(m, n, k, layout);
+  BGMOE_REQUIRE(a->x && a->scale && w && w_scale, "fp8_dense_gemm_partials: null pointer");
+  BGMOE_REQUIRE(scale_nb_stride >= k / 128, "fp8_dense_gemm_partials: weight-scale row stride %lld < K/128 = %d",
+                (long long)scale_nb_stride, k / 128);
+  BGMOE_REQUIRE(((uintptr_t)a->x | (uintptr_t)w) % 16 == 0, "fp8_dense_gemm_partials: x and w must be 16-byte aligned");
+  BGMOE_REQUIRE(workspace != nullptr && workspace_bytes >= need && (uintptr_t)workspace % 16 == 0,
+                "fp8_dense_gemm_partials: needs a 16-byte aligned workspace of %lld bytes, got %lld", (long long)need,
+                (long long)workspace_bytes);
+  hipStream_t st = bgmoe_stream(stream);
+  BgmoeProf prof(BGMOE_K_DENSE_GEMM, st);
+  bgmoe_fp8_act act = *a;
+  act.scale_group_stride = 0;
+  bgmoe_fp8_weight wd{};
+  wd.w = w; wd.scale = w_scale; wd.scale_nb_stride = scale_nb_stride; wd.layout = layout;
+  *slices = (k / 128 + per - 1) / per;
+  return bgmoe_internal_fp8_dense_splitk(&act, &wd, m, n, k, per, (float*)workspace, nullptr, st);
+}
+
 extern "C" int bgmoe_fp8_dense_gemm(const bgmoe_fp8_act* a, const uint8_t* w, const float* w_scale,
                                     int64_t scale_nb_stride, int layout, int64_t m, int n, int k, uint16_t* out,
                                     void* workspace, int64_t workspace_bytes, bgmoe_stream_t stream) {

@@ -573,7 +573,7 @@ int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weig
   else
     hipLaunchKernelGGL(fp8_dense_splitk_kernel<BGMOE_W_ROW_MAJOR>, dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
   int rc = bgmoe_check_launch("fp8_dense_gemm (split-K)");
-  if (rc != BGMOE_OK) return rc;
+  if (rc != BGMOE_OK || out == nullptr) return rc;         // out == nullptr: the caller consumes the partial sums
   const int64_t quads = m * n / 4;
   int64_t rblocks = (quads + 255) / 256;
   if (rblocks > 4096) rblocks = 4096;

@@ -183,6 +183,32 @@ class Fp8DenseExpert:
         up = w8a16_gemm(self.up, self.up_scale, hidden_states, x_fp8=x_fp8)
         return w8a16_gemm(self.down, self.down_scale, torch.nn.functional.silu(gate) * up)
 
+    def _gate_up_activation_from_partials(self, x_fp8, x_scale, rows, hidden):
+        """When the [gate; up] GEMM runs in its block-split form, the activation kernel adds the K-slices itself
+        (same bits as GEMM -> bf16 -> activation, one launch and one round trip less); None when the GEMM takes
+        another form."""
+        two_i = self.gate_up.shape[0]
+        if not (rows <= DENSE_MAX_ROWS or (rows <= DENSE_MAX_ROWS_NARROW and two_i <= DENSE_NARROW_N)):
+            return None
+        need = lib().bgmoe_fp8_dense_gemm_workspace(rows, two_i, hidden, 0)
+        if need <= 0 or x_fp8.dtype != FP8_DTYPE or not x_fp8.is_contiguous():
+            return None
+        inter = two_i // 2
+        ws = _workspace(need, x_fp8.device)
+        act = Fp8Act(ptr(x_fp8), ptr(x_scale), x_scale.stride(0), x_scale.stride(1), 0)
+        slices = C.c_int32(0)
+        h_fp8 = torch.empty((rows, inter), device=x_fp8.device, dtype=FP8_DTYPE)
+        h_scale = torch.empty((inter // BLOCK, (rows + 3) // 4 * 4), device=x_fp8.device,
+                              dtype=torch.float32).transpose(0, 1)[:rows, :]
+        with torch.cuda.device(x_fp8.device):
+            check(lib().bgmoe_fp8_dense_gemm_partials(C.byref(act), ptr(self.gate_up), ptr(self.gate_up_scale),
+                                                      hidden // BLOCK, 0, rows, two_i, hidden, ptr(ws), need,
+                                                      C.byref(slices), stream()))
+            check(lib().bgmoe_silu_mul_group_quant_partials(ptr(ws), slices.value, rows * two_i, rows, inter, 0,
+                                                            ptr(h_fp8), inter, ptr(h_scale), h_scale.stride(0),
+                                                            h_scale.stride(1), stream()))
+        return h_fp8, h_scale
+
     def forward_fused_gate_up(self, hidden_states, out=None, x_fp8=None, x_scale=None):
         who = f"Layer {self.layer_idx}"
         if hidden_states.dtype != torch.bfloat16:
@@ -217,8 +243,11 @@ class Fp8DenseExpert:
             if x_scale.stride() != (1, aligned):
                 raise ValueError(f"{who}: x_scale must carry the scale_tma_aligned MN-major layout (stride "
                                  f"(1, {aligned})), got {x_scale.stride()}")
-        gate_up = torch.empty((rows, self.gate_up.shape[0]), dtype=torch.bfloat16, device=x.device)
-        fp8_gemm_nt((x_fp8, x_scale), (self.gate_up, self.gate_up_scale), gate_up)
-        h_fp8, h_scale = silu_mul_per_token_blocked_quantize_bf16_to_fp8_1d(gate_up, scale_tma_aligned=True)
+        h = self._gate_up_activation_from_partials(x_fp8, x_scale, rows, hidden)
+        if h is None:
+            gate_up = torch.empty((rows, self.gate_up.shape[0]), dtype=torch.bfloat16, device=x.device)
+            fp8_gemm_nt((x_fp8, x_scale), (self.gate_up, self.gate_up_scale), gate_up)
+            h = silu_mul_per_token_blocked_quantize_bf16_to_fp8_1d(gate_up, scale_tma_aligned=True)
+        h_fp8, h_scale = h
         fp8_gemm_nt((h_fp8, h_scale), (self.down, self.down_scale), out)
         return shaped(out)

@@ -236,6 +236,14 @@ int bgmoe_silu_mul_group_quant(const uint16_t* gate, const uint16_t* up, int64_t
                                int64_t scale_stride_s, int64_t scale_stride_g, uint16_t* prod_out,
                                bgmoe_stream_t stream);
 
+/* The same activation fed by bgmoe_fp8_dense_gemm_partials: gate | up arrive as `slices` fp32 planes of
+ * [rows, 2n] (plane stride slice_stride floats); the planes are added in ascending order and rounded to bf16, which
+ * is what the GEMM's own second launch would have stored, then processed as above (form 0 or 1).  out [rows, n]
+ * bytes with row stride out_stride_s, scale element (r, g) at scale[r*scale_stride_s + g*scale_stride_g]. */
+int bgmoe_silu_mul_group_quant_partials(const float* partials, int slices, int64_t slice_stride, int64_t rows, int n,
+                                        int form, uint8_t* out, int64_t out_stride_s, float* scale,
+                                        int64_t scale_stride_s, int64_t scale_stride_g, bgmoe_stream_t stream);
+
 /* ------------------------------------------------------ permute / unpermute */
 
 /* Bytes of device workspace the dispatch calls need for n*k pairs. */
@@ -391,6 +399,15 @@ int64_t bgmoe_fp8_dense_gemm_workspace(int64_t m, int n, int k, int layout);
 int bgmoe_fp8_dense_gemm(const bgmoe_fp8_act* a, const uint8_t* w, const float* w_scale, int64_t scale_nb_stride,
                          int layout, int64_t m, int n, int k, uint16_t* out, void* workspace, int64_t workspace_bytes,
                          bgmoe_stream_t stream);
+
+/* The block-split form of bgmoe_fp8_dense_gemm without its second launch, for a consumer that adds the K-slices
+ * itself: writes *slices planes of m*n floats (plane stride m*n) into `workspace` and sets *slices.  Fails when
+ * (m, k, layout) is served without partial sums (bgmoe_fp8_dense_gemm_workspace == 0).  No reference counterpart:
+ * it exists so that the shared expert's chain (glm5/wrappers.py:448-461) needs no launch between its first GEMM
+ * and the activation. */
+int bgmoe_fp8_dense_gemm_partials(const bgmoe_fp8_act* a, const uint8_t* w, const float* w_scale,
+                                  int64_t scale_nb_stride, int layout, int64_t m, int n, int k, void* workspace,
+                                  int64_t workspace_bytes, int* slices, bgmoe_stream_t stream);
 
 /* Tuning knob (no reference counterpart): groups with at most `rows` rows are served by the
  * weight-streaming kernel, larger ones by the LDS-tiled kernel.  0 sends everything to the tiled

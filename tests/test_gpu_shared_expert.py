@@ -223,3 +223,25 @@ def test_dense_gemm_on_tile_major_weights(dev, m):
     np.testing.assert_allclose(d_row.cpu().float().numpy(), want, rtol=2e-2, atol=5e-3)
     if m > 64:                                        # both layouts take the block-split form with equal slices
         assert torch.equal(d_row, d_tile)
+
+
+@pytest.mark.parametrize("rows,hidden,inter", [(48, 4224, 256), (200, 2176, 384), (300, 512, 256), (512, 1152, 128)])
+def test_activation_fed_by_partial_sums_equals_gemm_then_activation(dev, rows, hidden, inter):
+    """The fused chain's shortcut (the activation kernel adds the [gate; up] GEMM's K-slices itself) against the
+    plain sequence GEMM -> bf16 -> SiLU * up + cast: identical bytes and scales."""
+    from batchgen_amd.kernels.triton.fp8_quantize import (per_token_blocked_quantize_bf16_to_fp8_1d,
+                                                          silu_mul_per_token_blocked_quantize_bf16_to_fp8_1d)
+    from batchgen_amd.moe.shared_expert import fp8_gemm_nt
+    make, _ = _expert(dev, rows + hidden, hidden, inter)
+    fused = make(True)
+    x = rand_bf16(torch.Generator().manual_seed(rows), rows, hidden).to(dev)
+    x_fp8, x_scale = per_token_blocked_quantize_bf16_to_fp8_1d(x, scale_tma_aligned=True)
+    short = fused._gate_up_activation_from_partials(x_fp8, x_scale, rows, hidden)
+    assert short is not None, "this shape is meant to take the block-split GEMM"
+    gate_up = torch.empty(rows, 2 * inter, dtype=torch.bfloat16, device=dev)
+    fp8_gemm_nt((x_fp8, x_scale), (fused.gate_up, fused.gate_up_scale), gate_up)
+    h_fp8, h_scale = silu_mul_per_token_blocked_quantize_bf16_to_fp8_1d(gate_up, scale_tma_aligned=True)
+    assert torch.equal(short[0].view(torch.uint8), h_fp8.view(torch.uint8))
+    assert torch.equal(short[1], h_scale) and short[1].stride() == h_scale.stride()
+    small = fused._gate_up_activation_from_partials(x_fp8[:8], x_scale[:8], 8, hidden)
+    assert small is None                                   # a handful of rows: no partial sums exist
