@@ -209,6 +209,17 @@ class Fp8DenseExpert:
                                                             h_scale.stride(1), stream()))
         return h_fp8, h_scale
 
+    def deepgemm_forward(self, x, scale=None):
+        """``DeepseekV3MLP.deepgemm_forward(x, scale)`` (batchgen/models/deepseek/deepseekv3/
+        modeling_deepseek_v3.py:630-637): the per-projection chain, block scales optionally taken from a dict with
+        the checkpoint's ``{gate,up,down}_proj.weight_scale_inv`` keys."""
+        if scale is None:
+            return self.forward_unfused(x)
+        x_fp8 = w8a16_gemm_act_quant(x)
+        up = w8a16_gemm(self.up, scale["up_proj.weight_scale_inv"], x, x_fp8=x_fp8)
+        gate = w8a16_gemm(self.gate, scale["gate_proj.weight_scale_inv"], x, x_fp8=x_fp8)
+        return w8a16_gemm(self.down, scale["down_proj.weight_scale_inv"], torch.nn.functional.silu(gate) * up)
+
     def forward_fused_gate_up(self, hidden_states, out=None, x_fp8=None, x_scale=None):
         who = f"Layer {self.layer_idx}"
         if hidden_states.dtype != torch.bfloat16:

@@ -152,6 +152,10 @@ def test_argument_policy(dev):
     with pytest.raises(ValueError, match="shared-expert out"):
         fused(x, out=torch.zeros(4, 256, dtype=torch.bfloat16, device=dev))
     assert tuple(fused(x[:0]).shape) == (0, 512)
+    scales = {"gate_proj.weight_scale_inv": fused.gate_scale, "up_proj.weight_scale_inv": fused.up_scale,
+              "down_proj.weight_scale_inv": fused.down_scale}
+    assert torch.equal(unfused.deepgemm_forward(x, scales), unfused(x))
+    assert torch.equal(unfused.deepgemm_forward(x), unfused(x))
     from batchgen_amd.moe.shared_expert import Fp8DenseExpert
     with pytest.raises(RuntimeError, match="row halves"):
         Fp8DenseExpert(fused.gate.clone(), fused.gate_scale, fused.up, fused.up_scale, fused.down, fused.down_scale,
