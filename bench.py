@@ -284,7 +284,17 @@ def bench_dense_expert(a, cfg, dev, g, base):
     x = (torch.randn(rows, h, generator=g, device=dev) * 0.5).to(torch.bfloat16)
     out_buf = torch.empty(rows, h, dtype=torch.bfloat16, device=dev)
     step = lambda: expert(x, out=out_buf)
-    ms = _time(step, a.steps, a.warmup, torch)
+    if a.graph:                                  # replays of one captured chain: what a serving loop runs
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        ms = _time(graph.replay, a.steps, a.warmup, torch)
+        base = dict(base, launch="hip_graph")
+    else:
+        ms = _time(step, a.steps, a.warmup, torch)
     _lib.prof_enable(True)
     for _ in range(a.steps):
         step()
