@@ -1,8 +1,10 @@
 // Block-scaled FP8 GEMM of ONE weight matrix against few rows (decode-time dense MLP / shared expert outside
 // the grouped launch): out[m, n] = bf16( sum_kb (x[m, kb] . w[n, kb]) * xs[m, kb] * ws[n / 128, kb] ).
 //
-// A grouped launch has one work item per (group, 256 columns); with a single group that is N / 256 items, far
-// fewer than the chip has CUs.  Here the K axis is the parallel one: a block owns 16, 32 or 64 weight rows over
+// A grouped launch has one work item per (group, 128 columns); with a single group that is N / 128 items, fewer
+// than the chip has wave slots.  Here the K axis is the parallel one, in two forms.  This file holds the wave
+// split and the entry points; the block split (K-slices over blocks, fp32 partial sums in a caller workspace,
+// chosen for more rows) reuses the grouped kernel's work item and lives beside it.  Wave split: a block owns 16, 32 or 64 weight rows over
 // the whole K, its 8 waves own one K-slice each (a contiguous run of 128-byte scale blocks), and the partial
 // sums meet in LDS where they are added in wave order, so the result does not depend on timing.  N / 16 blocks
 // of 8 waves keep the whole weight matrix in flight at once; each wave issues all loads of up to four K-blocks
@@ -12,8 +14,8 @@
 // = B, lane l supplies row l % 16 and K-bytes {16q..16q+15, 64+16q..64+16q+15}, q = l / 16; D: lane l holds
 // token l % 16, features 4q..4q+3.
 //
-// The accumulation order is a function of K alone (slice length ceil(K/128 / 8)), never of N or of the row
-// count: the gate and up halves of a stacked [gate; up] weight give exactly the bytes of two separate calls.
+// The accumulation order is a function of K alone (slice length ceil(K/128 / 8)), and the choice between the two
+// forms a function of the row count, K and the weight layout, never of N: the gate and up halves of a stacked [gate; up] weight give exactly the bytes of two separate calls.
 //
 // Algorithmic bytes: n*k weight bytes once per 64-row chunk; the m*k token bytes are re-read per block from L2.
 #include "bgmoe_common.h"
