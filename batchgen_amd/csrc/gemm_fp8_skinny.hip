@@ -81,10 +81,11 @@ __device__ __forceinline__ intx8 load32_stream(const uint8_t* p) {
   return r;
 }
 
-// LDS ring slot of one K-block of tokens: TT 2-KiB tile images + 64 token scales
+// LDS ring slot of one K-block of tokens: TT 2-KiB tile images + one token scale per row (64 per loading wave)
 template <int TT>
 struct TokSlot {
-  static constexpr int kBytes = TT * 2048 + 256;
+  static constexpr int kScaleWaves = (TT + 3) / 4;
+  static constexpr int kBytes = TT * 2048 + 256 * kScaleWaves;
 };
 
 // One work item: up to 16*TT rows of one group x one n-tile, streamed over K.
@@ -162,14 +163,15 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
                                          ? g.a.scale + grp * g.a.scale_group_stride + (int64_t)t0 * g.a.scale_row_stride
                                          : g.a.scale + (row0 + t0) * g.a.scale_row_stride) +
                                      (int64_t)kb_lo * g.a.scale_kb_stride);
-  const uint32_t xs_off = (uint32_t)min(lane, live - 1) * (uint32_t)g.a.scale_row_stride * 4u;
+  const uint32_t xs_off = (uint32_t)min(64 * (int)wave_u + lane, live - 1) * (uint32_t)g.a.scale_row_stride * 4u;
 
   auto issue_tokens = [&](int kb, int slot) {
     const uint32_t sb = ring_lds + (uint32_t)slot * kSlot;
 #pragma unroll
     for (int i = 0; i < LT; ++i)
       if (tok_on[i]) async_load16(tok_base + (kb << 7), tok_off[i], sb + (wave_u * LT + i) * 1024);
-    if (wave_u == 0) async_load4(xs_base + (int64_t)kb * g.a.scale_kb_stride, xs_off, sb + TT * 2048);
+    if (wave_u < (uint32_t)TokSlot<TT>::kScaleWaves)        // wave w brings the scales of rows 64w .. 64w+63
+      async_load4(xs_base + (int64_t)kb * g.a.scale_kb_stride, xs_off, sb + TT * 2048 + wave_u * 256);
   };
 
   floatx4 acc[TT][NT];
@@ -338,9 +340,9 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned 
 // One weight matrix against m rows (host-known), K split over `ksplit` blocks per (n-tile, 64-row chunk): the
 // item function above on K-blocks [slice * per, ...), fp32 partial sums to g.part; splitk_reduce_kernel adds the
 // slices in ascending order.
-template <int LAYOUT>
+template <int LAYOUT, int TT>
 __global__ __launch_bounds__(256) void fp8_dense_splitk_kernel(SkinnyArgs g, int m, int ksplit, int per) {
-  constexpr int TT = 4, NSTAGE = 2;
+  constexpr int NSTAGE = 2;
   __shared__ float s_amax[4][TT][16];
   __shared__ __align__(16) uint8_t s_ring[NSTAGE * TokSlot<TT>::kBytes];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
@@ -567,11 +569,18 @@ int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weig
   SkinnyArgs g{};
   g.a = *a; g.w0 = *w; g.groups = 1; g.n = n; g.k = k; g.out = out;
   g.part = workspace; g.part_slice_stride = m * n;
-  const unsigned blocks = (unsigned)(((n + 127) / 128) * ((m + 63) / 64) * ksplit);
-  if (w->layout == BGMOE_W_TILE_MAJOR)
-    hipLaunchKernelGGL(fp8_dense_splitk_kernel<BGMOE_W_TILE_MAJOR>, dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
-  else
-    hipLaunchKernelGGL(fp8_dense_splitk_kernel<BGMOE_W_ROW_MAJOR>, dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+  // the weights are streamed once per row chunk: 128-row chunks once there are enough rows that the halved
+  // block count still fills the chip (measured: from 129 rows on for K >= 4096, from 257 rows on otherwise)
+  const int chunk_rows = m > 256 || (m > 128 && k >= 4096) ? 128 : 64;
+  const unsigned blocks = (unsigned)(((n + 127) / 128) * ((m + chunk_rows - 1) / chunk_rows) * ksplit);
+  const bool tile = w->layout == BGMOE_W_TILE_MAJOR;
+  if (chunk_rows == 128) {
+    if (tile) hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_TILE_MAJOR, 8>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+    else hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_ROW_MAJOR, 8>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+  } else {
+    if (tile) hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_TILE_MAJOR, 4>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+    else hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_ROW_MAJOR, 4>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+  }
   int rc = bgmoe_check_launch("fp8_dense_gemm (split-K)");
   if (rc != BGMOE_OK || out == nullptr) return rc;         // out == nullptr: the caller consumes the partial sums
   const int64_t quads = m * n / 4;
