@@ -61,6 +61,7 @@ int bgmoe_internal_init_fp8_skinny();
 int bgmoe_internal_init_fp8_tiled();
 int bgmoe_internal_init_mxfp4();
 int bgmoe_internal_init_router_gemm();
+int bgmoe_internal_init_permute();
 int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                             const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                             uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,

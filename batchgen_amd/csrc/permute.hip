@@ -447,6 +447,73 @@ extern "C" int bgmoe_dispatch_scatter_ragged(const uint16_t* x, const int32_t* t
   return run_gather(x, topk_pos, act_buffer, nk, k, h, bgmoe_stream(stream));
 }
 
+// ---- allocation-free variant: the chunk histograms live in a file-scope device array --------------------
+// One copy of the array exists per GPU, at its own address; the address is looked up once per device with
+// that device current (bgmoe_init, else the first call on the device) and only that pointer is ever handed
+// to kernels: the array's name is a host-side stand-in, not a device address.
+namespace {
+constexpr size_t kStaticHistInts = 262144;                 // 1 MiB per GPU, held until the process ends
+constexpr int kMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) int32_t scratch[kStaticHistInts];
+static int32_t* g_scratch_ptr[kMaxDevices] = {};
+
+static int static_hist_ptr(int32_t** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    bgmoe_set_error("dispatch_scatter_ragged_static: no current HIP device (or device index >= %d)", kMaxDevices);
+    return BGMOE_ERR_HIP;
+  }
+  if (g_scratch_ptr[dev] == nullptr) {
+    int32_t* p = nullptr;
+    const hipError_t err = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || p == nullptr) {
+      bgmoe_set_error("dispatch_scatter_ragged_static: hipGetSymbolAddress failed: %s", hipGetErrorString(err));
+      return BGMOE_ERR_HIP;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return BGMOE_OK;
+}
+
+int bgmoe_internal_init_permute() {
+  int32_t* p = nullptr;
+  return static_hist_ptr(&p);
+}
+
+extern "C" size_t bgmoe_dispatch_static_max_pairs(int num_local_experts) {
+  if (num_local_experts <= 0 || num_local_experts > kMaxLocal) return 0;
+  return (kStaticHistInts / (size_t)num_local_experts) * (size_t)kChunk;
+}
+
+extern "C" int bgmoe_dispatch_scatter_ragged_static(const uint16_t* x, const int32_t* topk_ids, int n, int k, int h,
+                                                    uint16_t* act_buffer, int64_t act_rows, int expert_start,
+                                                    int num_local_experts, int32_t* expert_counts,
+                                                    int32_t* expert_counters, int32_t* topk_pos,
+                                                    int32_t* cu_seqlens, int row_align, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n >= 0 && k > 0, "dispatch_scatter_ragged_static: bad sizes n=%d k=%d", n, k);
+  BGMOE_REQUIRE(num_local_experts > 0 && num_local_experts <= kMaxLocal,
+                "dispatch_scatter_ragged_static: num_local_experts=%d outside [1,%d]", num_local_experts, kMaxLocal);
+  const size_t need = bgmoe_dispatch_workspace_bytes((int64_t)n * k, num_local_experts);
+  if (need > kStaticHistInts * sizeof(int32_t)) {
+    bgmoe_set_error("dispatch_scatter_ragged_static: %lld pairs x %d local experts need %zu bytes of histograms, the "
+                    "static buffer holds %zu (at most %zu pairs at this expert count); use "
+                    "bgmoe_dispatch_scatter_ragged with a workspace",
+                    (long long)n * k, num_local_experts, need, kStaticHistInts * sizeof(int32_t),
+                    bgmoe_dispatch_static_max_pairs(num_local_experts));
+    return BGMOE_ERR_WORKSPACE;
+  }
+  int32_t* hist = nullptr;
+  const int rc = static_hist_ptr(&hist);
+  if (rc != BGMOE_OK) return rc;
+  // every histogram entry the scan and rank kernels read is written by the histogram kernel of the same call,
+  // so nothing has to start at zero
+  return bgmoe_dispatch_scatter_ragged(x, topk_ids, n, k, h, act_buffer, act_rows, expert_start, num_local_experts,
+                                       expert_counts, expert_counters, topk_pos, cu_seqlens, row_align, hist,
+                                       kStaticHistInts * sizeof(int32_t), stream);
+}
+
 extern "C" int bgmoe_compact_expert_data(const int32_t* expert_counts, int e, int32_t* group_size,
                                          int32_t* activated_group_idx, int32_t* group_start_indices,
                                          int32_t* num_active, bgmoe_stream_t stream) {

@@ -30,6 +30,7 @@ extern "C" int bgmoe_init(void) {
   if (rc == BGMOE_OK) rc = bgmoe_internal_init_fp8_tiled();
   if (rc == BGMOE_OK) rc = bgmoe_internal_init_mxfp4();
   if (rc == BGMOE_OK) rc = bgmoe_internal_init_router_gemm();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_permute();
   return rc;
 }
 

@@ -278,6 +278,23 @@ int bgmoe_dispatch_scatter_ragged(const uint16_t* x, const int32_t* topk_ids, in
                                   int32_t* cu_seqlens, int row_align, void* workspace,
                                   size_t workspace_bytes, bgmoe_stream_t stream);
 
+/* bgmoe_dispatch_scatter_ragged for callers that cannot allocate device memory or pass a workspace (code under
+ * HIP-graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments, outputs and results, bit for bit; the chunk histograms that the other entry
+ * point keeps in `workspace` live in a 1 MiB device array that is part of the library image (one copy per
+ * GPU, held until the process ends), so the call allocates nothing and frees nothing.  Limit:
+ * ceil(n*k / 2048) * num_local_experts <= 262144 (bgmoe_dispatch_static_max_pairs(num_local_experts) pairs:
+ * 2 097 152 at 256 local experts); larger problems are rejected with BGMOE_ERR_WORKSPACE before anything is
+ * launched.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
+ * two host threads) race; calls ordered on one stream, or separated by an event, are safe, and nothing has to
+ * be cleared between them. */
+size_t bgmoe_dispatch_static_max_pairs(int num_local_experts);
+int bgmoe_dispatch_scatter_ragged_static(const uint16_t* x, const int32_t* topk_ids, int n, int k, int h,
+                                         uint16_t* act_buffer, int64_t act_rows, int expert_start,
+                                         int num_local_experts, int32_t* expert_counts,
+                                         int32_t* expert_counters, int32_t* topk_pos, int32_t* cu_seqlens,
+                                         int row_align, bgmoe_stream_t stream);
+
 /* Quantise-while-scattering: for every pair with topk_pos[i] >= 0 write the
  * act-quant of x[i/k] to row topk_pos[i] of y / scale.  Bit-identical to a
  * scatter followed by bgmoe_act_quant_*.  No reference counterpart as one op:
