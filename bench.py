@@ -5,9 +5,12 @@
 
 A step is one forward pass of the layer (router -> permute+quant -> gate_up/SwiGLU/
 requant GEMM -> down GEMM -> combine + shared expert) over one batch of synthetic
-tokens, with weights and inputs already resident in HBM.  Default workload is
-configuration 1 of the benchmark set (DeepSeek-V3-shaped FP8 decode, 256 tokens, 32 of 256
-experts local, masked layout).  Prints ONE JSON line.
+tokens, with weights and inputs already resident in HBM.  The default run prints ONE JSON line for
+configuration 1 of the benchmark set (DeepSeek-V3-shaped FP8 decode, 256 tokens, 32 of 256 experts local, masked
+layout: the HBM GB/s half of the metric) whose `prefill` object holds configuration 2 (the same layer on 16384
+tokens, ragged layout: the FP8 TFLOP/s half), each with its roofline and CPU baseline.  `--config N` measures one
+configuration only.  Decode configurations are also timed with 512 MiB read through the chip before every pass
+(`cache_flushed`), so that nothing of the previous pass is left in the 256 MiB last-level cache.
 
 `--op router_gemm` and `--op norm_quant` time the two producers that sit in front of the layer on the same
 configuration's shapes (hidden states -> logits -> routes in two launches; residual add + RMSNorm + FP8
@@ -31,27 +34,38 @@ BF16_PEAK_TFLOPS = 2500.0       # MI355X published dense BF16 MFMA peak
 
 METRIC = "MoE layer TFLOP/s (FP8 prefill) & HBM GB/s (decode), % roofline, 1xMI355X"
 
-# HBM bytes per launch of each configuration's dominant kernel, measured with two `rocprofv3 --pmc` runs
-# (FETCH_SIZE, then WRITE_SIZE; each scaled by what the same counter reads for a plain 256 MiB copy kernel in
-# the same run: x2.000 and x1.000).  The summaries with the exact commands are under profiles/ (one file per
-# configuration).  A configuration that was not measured reports null.
 MIB = 1024 * 1024
-MEASURED_TRAFFIC_BYTES = {
-    1: int((636.8 + 1.4) * MIB),      # fp8_skinny_kernel<2,3,fused,tile_major>, config 1
-    2: int((3093.6 + 83.5) * MIB),    # fp8_tiled_kernel<fused,tile_major>, config 2
-    3: int((227.5 + 0.7) * MIB),      # mxfp4_skinny_kernel<4,3,fused,tile_major>, config 3
-    4: int((6065.8 + 154.8) * MIB),   # fp8_tiled_kernel<fused,tile_major>, config 4
-    5: int((186.7 + 1.9) * MIB),      # mxfp4_skinny_kernel<4,3,fused,tile_major>, Kimi-K3 latent layer
-}
+FLUSH_BYTES = 512 * MIB         # read between flushed replays: twice the 256 MiB last-level (Infinity) cache
 
 
-# the same for the two producers (`--op`), keyed by (op, config); summaries under profiles/ as well
-MEASURED_TRAFFIC_PRODUCER = {
-    ("router_gemm", 1): int((17.7 + 3.5) * MIB),      # router_gemm_kernel<4,4,4,split,1 wave>, 256 tokens
-    ("router_gemm", 2): int((252.3 + 16.1) * MIB),    # router_gemm_lds_kernel<whole K>, 16384 tokens
-    ("norm_quant", 1): int((7.2 + 8.8) * MIB),        # add_rmsnorm_fp8_quant_kernel, 256 rows
-    ("norm_quant", 2): int((448.1 + 563.5) * MIB),    # add_rmsnorm_fp8_quant_kernel, 16384 rows
-}
+def traffic_record(key):
+    """HBM bytes per launch of a dominant kernel, as measured with `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
+    (each scaled by what the counter reads for a plain copy kernel of known size in the same run).  The figures
+    live in the summaries under profiles/, each in a line `traffic-record: {json}` that names the workload
+    (`key`), the bytes, the git commit of the measurement and the SHA-256 of every kernel source file the
+    measured kernel is built from.  A record is used only while those files are unchanged: a figure measured on
+    another version of the kernel says nothing about this one, and null is reported instead."""
+    import glob
+    import hashlib
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*.md"))):
+        for line in open(path, encoding="utf-8"):
+            if "traffic-record:" not in line:
+                continue
+            try:
+                rec = json.loads(line.split("traffic-record:", 1)[1].strip().rstrip("->").strip())
+            except ValueError:
+                continue
+            if str(rec.get("key")) != str(key):
+                continue
+            for rel, want in rec.get("sources", {}).items():
+                try:
+                    got = hashlib.sha256(open(os.path.join(ROOT, rel), "rb").read()).hexdigest()
+                except OSError:
+                    got = None
+                if got != want:
+                    return None, f"{os.path.basename(path)}: {rel} changed since the measurement (commit {rec.get('commit')})"
+            return int(rec["fetch_bytes"]) + int(rec["write_bytes"]), f"{os.path.basename(path)} (commit {rec.get('commit')})"
+    return None, "no record under profiles/"
 
 
 def parse():
@@ -59,8 +73,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--config", type=int, default=1, choices=[0, 1, 2, 3, 4, 5],
-                    help="0-4: the benchmark set's configurations; 5: the Kimi-K3 latent MoE layer at its real shape")
+    ap.add_argument("--config", type=int, default=None, choices=[0, 1, 2, 3, 4, 5],
+                    help="0-4: the benchmark set's configurations; 5: the Kimi-K3 latent MoE layer at its real shape. "
+                         "Default: configuration 1 (decode) as the line, plus configuration 2 (prefill) in its "
+                         "`prefill` object -- the two halves of the metric")
     ap.add_argument("--op", default="layer", choices=["layer", "router_gemm", "norm_quant", "dense_expert"],
                     help="what one step is: the MoE layer (default), one of its two producers, or the dense FP8 "
                          "expert chain (the shared expert outside the grouped launch) on the configuration's shapes")
@@ -158,6 +174,8 @@ def bench_producer(a):
     from batchgen_amd import _lib, workloads as wl
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.config is None:
+        a.config = 1
     cfg = wl.CONFIGS[a.config]
     n, h, e, k = cfg.n_tokens, cfg.hidden, cfg.n_experts, cfg.top_k
     g = torch.Generator(device=dev).manual_seed(cfg.seed + 7)
@@ -198,7 +216,7 @@ def bench_producer(a):
                         peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=gb,
                         avg_launch_us=gemm_ms * 1e3)
         roof["frac"] = roof["achieved"] / roof["peak"]
-        roof["traffic"] = MEASURED_TRAFFIC_PRODUCER.get((a.op, a.config))
+        roof["traffic"], roof["traffic_source"] = traffic_record(f"{a.op}:{a.config}")
         out = dict(base, metric="router GEMM + top-k: TFLOP/s (prefill) or HBM GB/s (decode), 1xMI355X",
                    value=(flops / (ms * 1e-3) / 1e12) if mfma else (alg_bytes / (ms * 1e-3) / 1e9),
                    unit="TFLOP/s" if mfma else "GB/s", ms_per_step=ms, dtype="bf16 (fp32 accumulate)",
@@ -247,7 +265,7 @@ def bench_producer(a):
     roof = dict(bound="hbm", kernel="add_rmsnorm_fp8_quant_kernel", achieved=alg_bytes / (k_ms * 1e-3) / 1e9,
                 peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=alg_bytes, avg_launch_us=k_ms * 1e3)
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC_PRODUCER.get((a.op, a.config))
+    roof["traffic"], roof["traffic_source"] = traffic_record(f"{a.op}:{a.config}")
     out = dict(base, metric="add + RMSNorm + FP8 cast: HBM GB/s, 1xMI355X", value=alg_bytes / (ms * 1e-3) / 1e9,
                unit="GB/s", ms_per_step=ms, dtype="bf16 in, fp32 arithmetic, e4m3 + fp32 scales out",
                config={"workload": cfg.name + " / add_rmsnorm_fp8_quant", "rows": n, "hidden": h},
@@ -334,29 +352,51 @@ def bench_dense_expert(a, cfg, dev, g, base):
     print(json.dumps(out))
 
 
-def main():
-    a = parse()
-    if a.gpus != 1:
-        print("bench.py measures one GPU's expert-parallel share; this build has no multi-GPU path "
-              "(run with --gpus 1).", file=sys.stderr)
-        sys.exit(2)
-    if a.op != "layer":
-        import torch
-        if not torch.cuda.is_available():
-            print("bench.py needs a GPU", file=sys.stderr)
-            sys.exit(2)
-        return bench_producer(a)
+def cpu_baseline_mxfp4_torch(cfg, inp, w, sh, ids, wt):
+    """The reference's CPU-runnable PyTorch path on MXFP4 experts: weights dequantised to bf16 with the reference
+    recipe (oracle.layer.l1_dequant_mxfp4, batchgen/moe/mxfp4_oracle_vector.py:80-115), then the same per-expert
+    bf16 loop as the FP8 baseline (oracle.layer.moe_layer_l1_torch).  Latent configurations are not covered by that
+    loop and keep the NumPy pass."""
+    import numpy as np
+    import torch
+    from oracle import layer as ol
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    n = min(cfg.n_tokens, 128)
+    ids_n, wt_n = ids[:n], wt[:n]
+    used = np.unique(ids_n)
+    dummy = torch.zeros(1, 1, dtype=torch.bfloat16)
+    experts = []
+    for e in range(cfg.e_local):
+        if (e + cfg.expert_start) in used:
+            experts.append(tuple(ol.l1_dequant_mxfp4(w[k + "_p"][e].cpu().numpy(), w[k + "_s"][e].cpu().numpy())
+                                 for k in ("gate", "up", "down")))
+        else:
+            experts.append((dummy, dummy, dummy))
+    shared = tuple(sh[k].cpu() for k in ("gate", "up", "down")) if sh else None
+    x = inp["x"][:n].cpu()
+    ol.moe_layer_l1_torch(x, ids_n, wt_n, experts, cfg.expert_start, shared)
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ol.moe_layer_l1_torch(x, ids_n, wt_n, experts, cfg.expert_start, shared)
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[1], threads, n / cfg.n_tokens, \
+        f"{n} of {cfg.n_tokens} tokens of the workload, all experts they route to, weights dequantised to bf16 " \
+        "beforehand, 1 warm-up + median of 3"
+
+
+def measure_layer(a, config, with_cpu):
+    """One configuration of the layer: K timed passes back to back, K passes with the last-level cache flushed
+    before each (decode), K passes with per-launch events for the dominant kernel, and the CPU baseline."""
     import numpy as np
     import torch
     from batchgen_amd import _lib, workloads as wl
     from batchgen_amd.moe.fp8_layer import Fp8MoELayer
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    cfg = wl.K3_LATENT if a.config == 5 else wl.CONFIGS[a.config]
+    cfg = wl.K3_LATENT if config == 5 else wl.CONFIGS[config]
     inp = wl.make_inputs(cfg, dev)
     mx4 = cfg.weight_format == "mxfp4"
     lat = None
@@ -378,6 +418,7 @@ def main():
         cal = torch.zeros((1, 32768, 8192), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn)
         repack_tile_major(cal)
         torch.cuda.synchronize()
+        del cal
     step = lambda: layer(x, logits)
     if a.graph:
         graph = torch.cuda.CUDAGraph()
@@ -405,6 +446,29 @@ def main():
     gbps = alg_bytes / (ms * 1e-3) / 1e9
     tflops = flops / (ms * 1e-3) / 1e12
 
+    # the same passes with the last-level cache flushed before each one: a kernel that READS 512 MiB (twice the
+    # 256 MiB Infinity Cache; a write would leave dirty lines whose write-back competes with the pass that
+    # follows) runs on the stream right before the timed pass, so the pass starts on a busy queue as in the
+    # back-to-back loop.  Events bracket the pass only.
+    flush = None
+    if decode:
+        fbuf = torch.zeros(FLUSH_BYTES // 4, dtype=torch.int32, device=dev)
+        evs = []
+        for _ in range(a.steps):
+            fbuf.sum()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            step()
+            e1.record()
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        fms = float(np.median([e0.elapsed_time(e1) for e0, e1 in evs]))
+        del fbuf
+        flush = {"bytes_read_before_each_step": FLUSH_BYTES, "ms_per_step": fms,
+                 "layer_hbm_GBps": alg_bytes / (fms * 1e-3) / 1e9,
+                 "layer_frac_of_hbm_peak": alg_bytes / (fms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                 "note": "median of per-step event times; `value` and ms_per_step are the back-to-back loop"}
+
     # second timed pass with per-launch HIP events -> duration of the dominant kernel
     _lib.prof_enable(True)
     for _ in range(a.steps):
@@ -418,7 +482,7 @@ def main():
         eh = cfg.expert_hidden
         dom_bytes = active * (2 * eh * i // 2 + 2 * eh * i // 32) + rows * (eh + i) * 2
         dom_ms = prof[dom][0] / max(prof[dom][1], 1)
-        roof = dict(bound="hbm", kernel="mxfp4_skinny_kernel<TT=4,NS=3,fused,tile_major>",
+        roof = dict(bound="hbm", kernel="mxfp4_skinny_kernel<fused,tile_major>",
                     achieved=dom_bytes / (dom_ms * 1e-3) / 1e9, peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None,
                     bytes_per_launch=dom_bytes, avg_launch_us=dom_ms * 1e3)
     elif decode:
@@ -430,7 +494,7 @@ def main():
         dom_bytes = served * (2 * h * i + 2 * (h // 128) * (i // 128) * 4) + \
             srows * (h + h // 128 * 4 + i + i // 128 * 4)
         dom_ms = prof[dom][0] / max(prof[dom][1], 1)
-        roof = dict(bound="hbm", kernel="fp8_skinny_kernel<TT=2,NS=3,fused,tile_major>", achieved=dom_bytes / (dom_ms * 1e-3) / 1e9,
+        roof = dict(bound="hbm", kernel="fp8_skinny_kernel<fused,tile_major>", achieved=dom_bytes / (dom_ms * 1e-3) / 1e9,
                     peak=HBM_PEAK_GBPS, unit="GB/s", traffic=None, bytes_per_launch=dom_bytes,
                     avg_launch_us=dom_ms * 1e3)
     else:
@@ -445,7 +509,7 @@ def main():
                     peak=FP8_PEAK_TFLOPS, unit="TFLOP/s", traffic=None, flops_per_launch=dom_flops,
                     avg_launch_us=dom_ms * 1e3)
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(a.config)
+    roof["traffic"], roof["traffic_source"] = traffic_record(f"layer:{config}")
 
     out = {
         "metric": METRIC,
@@ -465,20 +529,59 @@ def main():
         "kernel_ms_per_step": per_kernel,
         "roofline": roof,
     }
-    if not a.no_cpu_baseline and mx4:
+    if flush is not None:
+        out["cache_flushed"] = flush
+    ids = layer.topk_ids.cpu().numpy()
+    wt = layer.topk_weights.cpu().numpy()
+    if with_cpu and mx4 and cfg.latent:
         t, frac, sample = cpu_baseline_mxfp4(cfg, inp, w, sh, lat)
         out["cpu_baseline"] = {"value": alg_bytes * frac / t / 1e9, "unit": out["unit"],
                                "cores": min(os.cpu_count() or 1, 16), "host_cores": os.cpu_count() or 1,
                                "kind": "port", "sample": sample + " (BLAS threads for the matrix products, one thread for the dequantisation)", "seconds": t,
                                "tokens_per_s": cfg.n_tokens * frac / t}
-    if not a.no_cpu_baseline and not mx4:
-        ids = layer.topk_ids.cpu().numpy()
-        wt = layer.topk_weights.cpu().numpy()
+    elif with_cpu and mx4:
+        t, threads, frac, sample = cpu_baseline_mxfp4_torch(cfg, inp, w, sh, ids, wt)
+        out["cpu_baseline"] = {"value": alg_bytes * frac / t / 1e9, "unit": out["unit"], "cores": threads,
+                               "host_cores": os.cpu_count() or 1, "kind": "port", "sample": sample, "seconds": t,
+                               "tokens_per_s": cfg.n_tokens * frac / t}
+    elif with_cpu:
         t, threads, cores, sample, frac = cpu_baseline(cfg, inp, w, sh, ids, wt, alg_bytes, flops)
         v = (alg_bytes * frac / t / 1e9) if decode else (flops * frac / t / 1e12)
         out["cpu_baseline"] = {"value": v, "unit": out["unit"], "cores": threads, "host_cores": cores,
                                "kind": "port", "sample": sample, "seconds": t,
                                "tokens_per_s": cfg.n_tokens * frac / t}
+    del layer, w, sh, inp, x, logits
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU's expert-parallel share; this build has no multi-GPU path "
+              "(run with --gpus 1).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    if a.op != "layer":
+        return bench_producer(a)
+    if a.config is not None:
+        print(json.dumps(measure_layer(a, a.config, not a.no_cpu_baseline)))
+        return
+    # Default run: the metric has two halves.  The line is configuration 1 (decode: HBM GB/s, the figure `value`
+    # reports); its "prefill" object is configuration 2 (prefill: FP8 TFLOP/s) measured the same way in the same
+    # process, with fewer steps because one prefill pass is ten times longer.
+    out = measure_layer(a, 1, not a.no_cpu_baseline)
+    import copy
+    b = copy.copy(a)
+    b.steps, b.warmup = max(5, a.steps // 4), max(2, a.warmup // 2)
+    pre = measure_layer(b, 2, not a.no_cpu_baseline)
+    keep = ("value", "unit", "steps", "warmup", "ms_per_step", "launch", "dtype", "config", "tokens_per_s", "layer_TFLOPs",
+            "layer_frac_of_fp8_peak", "flops", "active_local_experts", "routed_rows", "kernel_ms_per_step", "roofline",
+            "cpu_baseline")
+    out["prefill"] = {k: pre[k] for k in keep if k in pre}
     print(json.dumps(out))
 
 

@@ -154,6 +154,12 @@ def l1_dequant_weights(wq: np.ndarray, ws: np.ndarray) -> torch.Tensor:
     return e.to(torch.bfloat16)
 
 
+def l1_dequant_mxfp4(packed: np.ndarray, scales: np.ndarray) -> torch.Tensor:
+    """MXFP4 weight -> bf16 with the reference recipe (``mxfp4_dequantize_oracle``,
+    batchgen/moe/mxfp4_oracle_vector.py:80-115; every e2m1 value times a power of two is exact in bf16)."""
+    return torch.from_numpy(_mx.dequant(packed, scales)).to(torch.bfloat16)
+
+
 @torch.inference_mode()
 def moe_layer_l1_torch(x: torch.Tensor, ids: np.ndarray, wt: np.ndarray, experts, expert_start: int,
                        shared=None) -> torch.Tensor:
