@@ -1,9 +1,11 @@
 // Top-k weighted combine (un-permute) for gfx950, with the shared expert's
 // output optionally folded into the same pass.  Gather-bound: each thread owns
 // 8 consecutive columns of one token and reads K rows with 16-byte loads.
-// Every product and sum is a separately rounded fp32 operation, k ascending
-// (the build compiles with -ffp-contract=off), so the result is reproducible
-// bit for bit on the CPU.
+// The bf16 and fp32 forms accumulate acc = fma(value, weight, acc), k ascending: the
+// reference kernels' `acc += val * w[k]` (dispatch_scatter_3d.cu:386-392, 421-431) is one
+// fused multiply-add per term under nvcc's default contraction.  The ordered form rounds
+// every product and partial sum to bf16 separately.  Both are reproducible bit for bit
+// on the CPU.
 #include "bgmoe_common.h"
 
 namespace {
@@ -97,10 +99,7 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(
           float v[8];
           unpack8(raw[u], v);
 #pragma unroll
-          for (int i = 0; i < W; ++i) {
-            const float prod = v[i] * wj[u];
-            acc[i] = acc[i] + prod;
-          }
+          for (int i = 0; i < W; ++i) acc[i] = __builtin_fmaf(v[i], wj[u], acc[i]);
         }
       }
     }
@@ -117,9 +116,8 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(
       }
 #pragma unroll
       for (int i = 0; i < W; ++i) {
-        const float prod = v[i] * wj;
-        if constexpr (MODE == 2) acc[i] = bf16_round_f32(acc[i] + bf16_round_f32(prod));
-        else acc[i] = acc[i] + prod;
+        if constexpr (MODE == 2) acc[i] = bf16_round_f32(acc[i] + bf16_round_f32(v[i] * wj));
+        else acc[i] = __builtin_fmaf(v[i], wj, acc[i]);
       }
     }
   }

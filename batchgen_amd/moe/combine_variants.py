@@ -96,9 +96,10 @@ def moe_fp32_accum_triton_v2(outs: torch.Tensor, idxs: torch.Tensor, topk_weight
     """The prefill combine of ``DeepseekV3MoE_Prefill.moe_infer``
     (batchgen/models/deepseek/deepseekv3/modeling_deepseek_v3.py:1034-1065): ``outs`` [T * K, H] are the expert
     outputs in expert-sorted order, ``idxs`` the sorting permutation (sorted row j came from flat (token, k) index
-    ``idxs[j]``); returns ``[T, H]`` in the dtype of ``outs``, fp32 accumulation over k ascending.  The product and
-    the sum are rounded separately here; whether the reference's Triton kernel contracts them into one fused
-    multiply-add is decided by its compiler (parity unpinned at the last fp32 bit, before the bf16 rounding)."""
+    ``idxs[j]``); returns ``[T, H]`` in the dtype of ``outs``, fp32 accumulation over k ascending.  Each term is one
+    fused multiply-add here, as in the CUDA combine kernels; whether the reference's Triton kernel contracts the
+    product and the sum is decided by its compiler (parity unpinned at the last fp32 bit, before the bf16
+    rounding)."""
     t, k = topk_weights.shape
     if outs.dim() != 2 or outs.shape[0] != t * k or idxs.numel() != t * k:
         raise ValueError(f"outs must be [{t * k}, H] and idxs [{t * k}]; got {tuple(outs.shape)} and {tuple(idxs.shape)}")

@@ -313,7 +313,8 @@ int bgmoe_scatter_fp8_rows(const uint8_t* xq, const float* xs, int64_t xs_row_st
                            const int32_t* topk_pos, int n, int k, int h, uint8_t* y, float* scale,
                            int64_t scale_row_stride, int64_t scale_kb_stride, bgmoe_stream_t stream);
 
-/* out[t] = bf16(sum_k float(y[pos[t,k]])*w[t,k]), k ascending, pos<0 skipped.
+/* out[t] = bf16(sum_k float(y[pos[t,k]])*w[t,k]), k ascending, pos<0 skipped; every term is one fp32 fused
+ * multiply-add, acc = fma(value, weight, acc), as the reference kernel's `acc += val * w[k]` compiles.
  * Replaces `reduce_weighted_scatter` (dispatch_scatter_3d.cu:365-395, 527-556;
  * batchgen_kernels/src/moe/routing/reduce_weighted_scatter.cu:26-131).
  * num_valid_tokens > 0 limits the rows written.  shared (bf16 [n,h], may be

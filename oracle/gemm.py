@@ -73,16 +73,38 @@ def grouped_gemm_fp8_blockpromote(xq, xs, wq, ws, seqlens, cu_seqlens):
     return out
 
 
-def expert_mlp_fp8(xq, xs, gate_q, gate_s, up_q, up_s, down_q, down_s, seqlens, cu_seqlens):
-    """gate_up -> SwiGLU (fp32, one bf16 round) -> requant (form C) -> down.
+def expert_mlp_fp8(xq, xs, gate_q, gate_s, up_q, up_s, down_q, down_s, seqlens, cu_seqlens, variant="i"):
+    """gate_up -> SwiGLU -> requant -> down, with the intermediate rounded the way ``variant`` says:
 
-    Returns (y bf16-valued float32 [M,H], h bf16-valued [M,I], hq bytes, hs scales).
+    "i"    fp32 gate and up, fp32 SiLU, ONE bf16 round, requant form C: the reference's Triton stage 1
+           (w8a8_grouped_gemm_stage_1.py:1023-1026) and what the HIP kernels compute;
+    "ii"   the reference's CuTe fused stage 1 (``oracle.quant.swiglu_cute_bf16``) + requant form C
+           (``act_quant_ragged`` on its bf16 output, glm5/model.py:2560-2573);
+    "iii"  the reference's DeepGEMM chains: gate and up leave the first GEMM as bf16, then
+           ``silu_mul_{masked,ragged}_group_quant`` (bf16 SiLU, bf16 product, requant form D,
+           moe_masked_act_quant.py:96-104);
+    "fp32" no rounding that the semantics do not ask for: SwiGLU in fp32 fed straight to the requant
+           (form C), the down product left in fp32 -- the yardstick the variants' errors are measured against.
+
+    Returns (y [M,H] float32 -- bf16-valued except for "fp32" --, h [M,I], hq bytes, hs scales).
     """
+    from .quant import silu_f32, silu_mul_group_quant, swiglu_cute_bf16
     g = grouped_gemm_fp8(xq, xs, gate_q, gate_s, seqlens, cu_seqlens, to_bf16=False)
     u = grouped_gemm_fp8(xq, xs, up_q, up_s, seqlens, cu_seqlens, to_bf16=False)
-    h = swiglu_bf16(g, u)
-    hq, hs = act_quant(h)
-    y = grouped_gemm_fp8(hq, hs, down_q, down_s, seqlens, cu_seqlens, to_bf16=True)
+    if variant == "i":
+        h = swiglu_bf16(g, u)
+        hq, hs = act_quant(h)
+    elif variant == "ii":
+        h = swiglu_cute_bf16(g, u)
+        hq, hs = act_quant(h)
+    elif variant == "iii":
+        hq, hs, h = silu_mul_group_quant(bf16_round(g), bf16_round(u), "D")
+    elif variant == "fp32":
+        h = (silu_f32(g) * u.astype(F32)).astype(F32)
+        hq, hs = act_quant(h)
+    else:
+        raise ValueError(f"unknown SwiGLU rounding variant {variant!r}")
+    y = grouped_gemm_fp8(hq, hs, down_q, down_s, seqlens, cu_seqlens, to_bf16=variant != "fp32")
     return y, h, hq, hs
 
 

@@ -53,9 +53,14 @@ def _permute(ids, expert_start, num_local, layout, max_tokens, row_align):
 
 def moe_layer_fp8(x, logits, bias, rcfg, w, expert_start, num_local,
                   layout="masked", max_tokens=0, row_align=64, shared=None,
-                  shared_mode="bf16_add", routes=None):
+                  shared_mode="bf16_add", routes=None, variant="i"):
     """x [N,H] bf16-valued; w = dict(gate_q,gate_s,up_q,up_s,down_q,down_s) for the
     LOCAL experts ([E_l,...] numpy); shared = same keys with a leading 1.
+
+    ``variant`` picks the rounding of the intermediate (``oracle.gemm.expert_mlp_fp8``): "i" is what the HIP
+    path computes; "ii" and "iii" emulate the reference's own kernels; "fp32" is the fp32
+    dequantise-then-matmul yardstick (no bf16 rounding anywhere after the routing: fp32 expert outputs, fp32
+    combine, fp32 shared-expert add, fp32 result).
 
     Returns a dict with every intermediate the parity tests compare.
     """
@@ -70,15 +75,18 @@ def moe_layer_fp8(x, logits, bias, rcfg, w, expert_start, num_local,
     xq = _pm.gather_rows(xq_tok, pos, k, max(rows, 1))
     xs = _pm.gather_rows(xs_tok, pos, k, max(rows, 1))
     y, hmid, hq, hs = _gm.expert_mlp_fp8(xq, xs, w["gate_q"], w["gate_s"], w["up_q"], w["up_s"],
-                                         w["down_q"], w["down_s"], counts, cu)
+                                         w["down_q"], w["down_s"], counts, cu, variant=variant)
     y_sh = None
     if shared is not None:
         one = np.array([n], dtype=np.int32)
         zero = np.array([0, n], dtype=np.int32)
         y_sh, _, _, _ = _gm.expert_mlp_fp8(xq_tok, xs_tok, shared["gate_q"], shared["gate_s"],
                                            shared["up_q"], shared["up_s"], shared["down_q"],
-                                           shared["down_s"], one, zero)
-    out = _cb.reduce_weighted_scatter(y, pos, wt, n, k, shared=y_sh, shared_mode=shared_mode)
+                                           shared["down_s"], one, zero, variant=variant)
+    if variant == "fp32":
+        out = _cb.reduce_weighted_scatter(y, pos, wt, n, k, shared=y_sh, shared_mode="fp32")
+    else:
+        out = _cb.reduce_weighted_scatter(y, pos, wt, n, k, shared=y_sh, shared_mode=shared_mode)
     return dict(out=out, ids=ids, weights=wt, counts=counts, cu=cu, pos=pos, xq_tok=xq_tok,
                 xs_tok=xs_tok, xq=xq, xs=xs, h=hmid, hq=hq, hs=hs, y=y, y_shared=y_sh)
 

@@ -193,6 +193,24 @@ def swiglu_bf16(gate_f32: np.ndarray, up_f32: np.ndarray) -> np.ndarray:
     return bf16_round(silu_f32(gate_f32) * up_f32.astype(F32))
 
 
+def swiglu_cute_bf16(gate_f32: np.ndarray, up_f32: np.ndarray) -> np.ndarray:
+    """Rounding variant (ii), the reference's own fused stage-1 kernel
+    (batchgen_kernels/src/moe/fp8_blockwise/fp8_blockwise_s1_kernel.cuh:556-581): the gate accumulator is
+    rounded to bf16 when it is parked in shared memory, ``sigmoid = 1.0f / (1.0f + __expf(-gate))``,
+    ``(gate * sigmoid) * up`` with the fp32 up accumulator, one more bf16 round.
+
+    ``__expf(x)`` is CUDA's ``ex2.approx(x * log2e)``: the argument product is rounded to fp32 and the
+    hardware exp2 is accurate to about 2 ulp.  The emulation rounds the product exactly as the instruction
+    sequence does and takes exp2 and the division correctly rounded -- an emulation of the kernel's rounding
+    structure, not of the last bits of two approximate instructions."""
+    g = bf16_round(gate_f32)
+    t = (-g * F32(1.4426950408889634)).astype(F32)
+    with np.errstate(over="ignore"):
+        e = np.exp2(t.astype(np.float64)).astype(F32)
+        sig = (F32(1.0) / (F32(1.0) + e).astype(F32)).astype(F32)
+    return bf16_round(((g * sig).astype(F32) * as_f32(up_f32)).astype(F32))
+
+
 def silu_torch_f32(g) -> np.ndarray:
     """PyTorch's fp32 SiLU, ``x / (1 + exp(-x))`` as three float32 operations -- the formula and precision the
     reference's fused activation quantisers restate (batchgen_kernels/triton/fp8_quantize.py:414-424: libdevice
