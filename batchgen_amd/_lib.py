@@ -76,6 +76,7 @@ _SIGS = {
     "bgmoe_dispatch_scatter_ragged": (i32, [vp, vp, i32, i32, i32, vp, i64, i32, i32, vp, vp, vp, vp, i32, vp, sz, vp]),
     "bgmoe_dispatch_static_max_pairs": (sz, [i32]),
     "bgmoe_dispatch_scatter_ragged_static": (i32, [vp, vp, i32, i32, i32, vp, i64, i32, i32, vp, vp, vp, vp, i32, vp]),
+    "bgmoe_dispatch_row_metadata": (i32, [vp, vp, i64, i32, vp, i64, vp, vp, vp, vp]),
     "bgmoe_scatter_fp8_rows": (i32, [vp, vp, i64, i64, vp, i32, i32, i32, vp, vp, i64, i64, vp]),
     "bgmoe_scatter_quant": (i32, [vp, vp, i32, i32, i32, vp, vp, i64, i64, vp]),
     "bgmoe_reduce_weighted_scatter": (i32, [vp, vp, vp, i32, i32, i32, vp, i32, vp, i32, vp]),

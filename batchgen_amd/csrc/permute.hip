@@ -514,6 +514,46 @@ extern "C" int bgmoe_dispatch_scatter_ragged_static(const uint16_t* x, const int
                                        kStaticHistInts * sizeof(int32_t), stream);
 }
 
+namespace {
+// Per-row metadata of a tight (align 1) dispatch: row topk_pos[i] of pair i = (token i / k, slot i % k) gets the
+// pair's expert id, token and slot; rows at or past *total (the last entry of the offsets) get -1.  Every row
+// has exactly one writer.
+__global__ __launch_bounds__(256) void row_metadata_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ pos,
+                                                           int64_t nk, int k, const int32_t* __restrict__ total, int64_t rows,
+                                                           int32_t* __restrict__ eids, int32_t* __restrict__ toks,
+                                                           int32_t* __restrict__ slots) {
+  const int64_t live = *total;
+  const int64_t span = nk > rows ? nk : rows;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < span; i += (int64_t)gridDim.x * 256) {
+    if (i < nk) {
+      const int p = pos[i];
+      if (p >= 0 && p < rows) {
+        eids[p] = ids[i];
+        toks[p] = (int32_t)(i / k);
+        slots[p] = (int32_t)(i % k);
+      }
+    }
+    if (i < rows && i >= live) eids[i] = toks[i] = slots[i] = -1;
+  }
+}
+}  // namespace
+
+extern "C" int bgmoe_dispatch_row_metadata(const int32_t* topk_ids, const int32_t* topk_pos, int64_t nk, int k,
+                                           const int32_t* total_rows, int64_t rows, int32_t* out_eids,
+                                           int32_t* out_token_idx, int32_t* out_topk_pos, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(nk >= 0 && k > 0 && rows >= 0, "dispatch_row_metadata: bad sizes nk=%lld k=%d rows=%lld", (long long)nk, k,
+                (long long)rows);
+  if (rows == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(total_rows && out_eids && out_token_idx && out_topk_pos && (nk == 0 || (topk_ids && topk_pos)),
+                "dispatch_row_metadata: null pointer");
+  const int64_t span = nk > rows ? nk : rows;
+  int64_t blocks = (span + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(row_metadata_kernel, dim3((unsigned)blocks), dim3(256), 0, bgmoe_stream(stream), topk_ids, topk_pos, nk,
+                     k, total_rows, rows, out_eids, out_token_idx, out_topk_pos);
+  return bgmoe_check_launch("dispatch_row_metadata");
+}
+
 extern "C" int bgmoe_compact_expert_data(const int32_t* expert_counts, int e, int32_t* group_size,
                                          int32_t* activated_group_idx, int32_t* group_start_indices,
                                          int32_t* num_active, bgmoe_stream_t stream) {

@@ -102,8 +102,11 @@ def fused_moe_token_dispatch(global_x, topk_idx, token_idx, topk_pos, routed_exp
     k = topk_idx.size(1)
     e_l = int(routed_expert_end_idx - routed_expert_start_idx)
     dev = global_x.device
-    ids32 = topk_idx.to(torch.int32)
+    ids32 = topk_idx.to(torch.int32).contiguous()
     nk = n * k
+    if e_l <= 0:
+        ck.fail(f"routed_expert_end_idx ({routed_expert_end_idx}) must exceed routed_expert_start_idx "
+                f"({routed_expert_start_idx})")
     out_x = torch.empty((max(nk, 1), h), dtype=global_x.dtype, device=dev)
     counts = torch.empty(e_l, dtype=torch.int32, device=dev)
     counters = torch.empty(e_l, dtype=torch.int32, device=dev)
@@ -114,17 +117,13 @@ def fused_moe_token_dispatch(global_x, topk_idx, token_idx, topk_pos, routed_exp
         check(lib().bgmoe_dispatch_scatter_ragged(ptr(global_x), ptr(ids32), n, k, h, ptr(out_x), out_x.size(0),
                                                   int(routed_expert_start_idx), e_l, ptr(counts), ptr(counters),
                                                   ptr(pos), ptr(offsets), 1, ptr(ws), ws_bytes, stream()))
-    # per-row metadata (bookkeeping on device with torch ops; not on the hot path)
-    pos_l = pos[:nk].long()
-    live = pos_l >= 0
-    rows = pos_l[live]
-    flat = torch.arange(nk, device=dev)[live]
-    tok_src = token_idx.reshape(-1) if token_idx is not None and token_idx.numel() == n else torch.arange(n, device=dev)
-    out_eids = torch.full((max(nk, 1),), -1, dtype=torch.int32, device=dev)
-    out_tok = torch.full((max(nk, 1),), -1, dtype=torch.int32, device=dev)
-    out_pos = torch.full((max(nk, 1),), -1, dtype=torch.int32, device=dev)
-    out_eids[rows] = ids32.reshape(-1)[flat]
-    out_tok[rows] = tok_src[flat // k].to(torch.int32)
-    kpos = topk_pos.reshape(-1)[flat] if topk_pos is not None and topk_pos.numel() == nk else (flat % k)
-    out_pos[rows] = kpos.to(torch.int32)
+    # per-row metadata: one more launch, no device -> host read (the reference's kernel writes them while it copies
+    # the rows and ignores its token_idx / topk_pos arguments, fused_moe_token_dispatch.cu:59-88)
+    rows = out_x.size(0)
+    out_eids = torch.empty(rows, dtype=torch.int32, device=dev)
+    out_tok = torch.empty(rows, dtype=torch.int32, device=dev)
+    out_pos = torch.empty(rows, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        check(lib().bgmoe_dispatch_row_metadata(ptr(ids32), ptr(pos), nk, k, offsets[e_l:].data_ptr(), rows,
+                                                ptr(out_eids), ptr(out_tok), ptr(out_pos), stream()))
     return [out_x, out_eids, out_tok, out_pos, counts, offsets]

@@ -295,6 +295,15 @@ int bgmoe_dispatch_scatter_ragged_static(const uint16_t* x, const int32_t* topk_
                                          int32_t* expert_counters, int32_t* topk_pos, int32_t* cu_seqlens,
                                          int row_align, bgmoe_stream_t stream);
 
+/* The per-row outputs of `fused_moe_token_dispatch` (batchgen_kernels/src/moe/mgn/fused_moe_token_dispatch.cu:59-88:
+ * output_eids / output_token_idx / output_topk_pos) from the indices of a tight (row_align 1) ragged dispatch:
+ * row topk_pos[i] of pair i receives its expert id topk_ids[i], its token i / k and its slot i % k.  Rows at or
+ * past *total_rows (device int32: the last entry of the dispatch's cu_seqlens) receive -1, where the reference
+ * leaves them uninitialised.  One launch, nothing read back. */
+int bgmoe_dispatch_row_metadata(const int32_t* topk_ids, const int32_t* topk_pos, int64_t nk, int k,
+                                const int32_t* total_rows, int64_t rows, int32_t* out_eids,
+                                int32_t* out_token_idx, int32_t* out_topk_pos, bgmoe_stream_t stream);
+
 /* Quantise-while-scattering: for every pair with topk_pos[i] >= 0 write the
  * act-quant of x[i/k] to row topk_pos[i] of y / scale.  Bit-identical to a
  * scatter followed by bgmoe_act_quant_*.  No reference counterpart as one op:
