@@ -72,6 +72,9 @@ _SIGS = {
     "bgmoe_fused_silu_quant_3d": (i32, [vp, vp, vp, i32, i32, i32, vp, vp, vp]),
     "bgmoe_deepep_ll_scale_repack": (i32, [vp, vp, vp, i32, i32, i32, i32, vp, vp]),
     "bgmoe_dispatch_workspace_bytes": (sz, [i64, i32]),
+    "bgmoe_fp8_streamk_workspace_bytes": (sz, []),
+    "bgmoe_debug_streamk_trace": (i32, [vp]),
+    "bgmoe_set_streamk_xcd_weights": (i32, [vp]),
     "bgmoe_dispatch_scatter_3d": (i32, [vp, vp, i32, i32, i32, vp, i32, i32, i32, vp, vp, vp, vp, sz, vp]),
     "bgmoe_dispatch_scatter_ragged": (i32, [vp, vp, i32, i32, i32, vp, i64, i32, i32, vp, vp, vp, vp, i32, vp, sz, vp]),
     "bgmoe_dispatch_static_max_pairs": (sz, [i32]),
@@ -92,6 +95,10 @@ _SIGS = {
     "bgmoe_fp8_grouped_gemm": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), vp, vp, i32, i64, i32, i32, vp, vp]),
     "bgmoe_fp8_fused_s1": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), C.POINTER(Fp8Weight), vp, vp, i32,
                                  i64, i32, i32, vp, vp, vp, i64, i64, vp]),
+    "bgmoe_fp8_grouped_gemm_balanced": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), vp, vp, i32, i64, i32, i32, vp,
+                                              i64, vp, sz, vp]),
+    "bgmoe_fp8_fused_s1_balanced": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), C.POINTER(Fp8Weight), vp, vp, i32,
+                                          i64, i32, i32, vp, vp, vp, i64, i64, i64, vp, sz, vp]),
 }
 
 _lib = None

@@ -62,10 +62,36 @@ def _compile(src: str, force: bool) -> str:
     if not force and _newer(obj, deps):
         return obj
     cmd = [hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    if src in NO_SPILL:
+        cmd.insert(-4, "-Rpass-analysis=kernel-resource-usage")
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
+    if src in NO_SPILL:
+        _check_no_spill(src, r.stderr, obj)
     return obj
+
+
+# Kernels whose weight loads are issued from inline asm and waited for by hand: a register that such a load is
+# still writing must never be spilled or copied, so these files must compile without scratch memory.
+NO_SPILL = {"gemm_fp8_streamk.hip": "fp8_streamk_kernel"}
+
+
+def _check_no_spill(src: str, remarks: str, obj: str) -> None:
+    import re
+    name, bad, seen = None, [], 0
+    for line in remarks.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if m and name and NO_SPILL[src] in name:
+            seen += 1
+            if int(m.group(1)) != 0:
+                bad.append(f"{name}: {m.group(1)} bytes of scratch per lane")
+    if bad or seen == 0:
+        os.remove(obj)
+        raise RuntimeError(f"{src}: kernels must not spill registers ({'; '.join(bad) or 'no resource remarks found'})")
 
 
 def build(force: bool = False, jobs: int = 4, verbose: bool = True) -> str:

@@ -11,13 +11,16 @@
 // instruction offset is used: the hardware would add it to the LDS address as well as to the
 // global address.
 // The global address is a wave-uniform base plus a 32-bit byte offset per lane.
+// s_nop 4: the base may have just been written by a VALU instruction (v_readlane restoring a spilled SGPR, a
+// v_readfirstlane), and a vector-memory instruction that reads an SGPR needs five wait states after a VALU write
+// to it; the compiler does not look inside the asm to insert them.
 __device__ __forceinline__ void async_load16(const uint8_t* base, uint32_t lane_off, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+  asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :: "s"(lds_base), "v"(lane_off), "s"(base) : "memory", "m0");
 }
 // 64 lanes x 4 bytes -> LDS [lds_base, lds_base + 256)
 __device__ __forceinline__ void async_load4(const float* base, uint32_t lane_off, uint32_t lds_base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+  asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                :: "s"(lds_base), "v"(lane_off), "s"(base) : "memory", "m0");
 }
 template <typename T>

@@ -65,7 +65,14 @@ int bgmoe_internal_init_permute();
 int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                             const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                             uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
-                            int64_t row_bound, int64_t group_bound, hipStream_t st);
+                            int64_t row_bound, int64_t group_bound, void* streamk_ws, size_t streamk_ws_bytes,
+                            hipStream_t st);
+int bgmoe_internal_init_fp8_streamk();
+// balanced (stream-K) form of the weight-streaming kernel; BGMOE_ERR_WORKSPACE without a message = does not apply
+int bgmoe_internal_fp8_streamk(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
+                               const int32_t* seqlens, const int32_t* cu, int groups, int n, int k, uint16_t* out,
+                               uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb, int hi, int64_t row_bound,
+                               void* ws, size_t ws_bytes, hipStream_t st);
 
 // router-GEMM logits as [*nplanes_out][n][e] fp32 planes for a consumer that adds them in plane order
 int bgmoe_internal_router_gemm_planes(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,

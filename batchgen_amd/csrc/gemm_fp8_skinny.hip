@@ -55,6 +55,8 @@ struct SkinnyArgs {
   int64_t group_bound;        // host-side upper bound on the rows of any one group (0 = unknown)
   float* part;                // split-K launches: fp32 partial sums [slice][row][n] instead of `out`
   int64_t part_slice_stride;
+  void* streamk_ws;           // workspace of the balanced form (gemm_fp8_streamk.hip) or null
+  size_t streamk_ws_bytes;
 };
 
 template <int NSC>
@@ -501,6 +503,12 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
   if (hi > 0) {
     g.split = split;
     BgmoeProf prof(fused ? BGMOE_K_S1_SKINNY16 : BGMOE_K_GEMM_SKINNY16, st);
+    if (stream_only && g.streamk_ws != nullptr && g.part == nullptr) {
+      const int rc = bgmoe_internal_fp8_streamk(&g.a, &g.w0, fused ? &g.w1 : nullptr, g.seqlens, g.cu, g.groups, g.n,
+                                                g.k, g.out, g.out_q, g.out_s, g.os_row, g.os_nb, hi, bound,
+                                                g.streamk_ws, g.streamk_ws_bytes, st);
+      if (rc != BGMOE_ERR_WORKSPACE) return rc;
+    }
     launch_variant(fused, layout, g.n, g.groups, bound, hi, g, st);
     int rc = bgmoe_check_launch("fp8 grouped gemm (skinny)");
     if (rc != BGMOE_OK) return rc;
@@ -517,8 +525,10 @@ static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
 int bgmoe_internal_fp8_gemm(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, const bgmoe_fp8_weight* w1,
                             const int32_t* seqlens, const int32_t* cu, int groups, int64_t m, int n, int k,
                             uint16_t* out, uint8_t* out_q, float* out_s, int64_t os_row, int64_t os_nb,
-                            int64_t row_bound, int64_t group_bound, hipStream_t st) {
+                            int64_t row_bound, int64_t group_bound, void* streamk_ws, size_t streamk_ws_bytes,
+                            hipStream_t st) {
   SkinnyArgs g{};
+  g.streamk_ws = streamk_ws; g.streamk_ws_bytes = streamk_ws_bytes;
   g.a = *a; g.w0 = *w0; if (w1) g.w1 = *w1;
   g.seqlens = seqlens; g.cu = cu; g.groups = groups; g.n = n; g.k = k;
   g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.row_bound = row_bound;
@@ -557,6 +567,44 @@ extern "C" int bgmoe_fp8_fused_s1(const bgmoe_fp8_act* a, const bgmoe_fp8_weight
   g.a = *a; g.w0 = *gate; g.w1 = *up; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups;
   g.n = n; g.k = k; g.out = out; g.out_q = out_q; g.out_s = out_scale;
   g.os_row = out_scale_row_stride; g.os_nb = out_scale_nb_stride;
+  return launch_skinny(true, g, m, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_fp8_grouped_gemm_balanced(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* b, const int32_t* seqlens,
+                                               const int32_t* cu_seqlens, int groups, int64_t m, int n, int k,
+                                               uint16_t* out, int64_t max_group_rows, void* workspace,
+                                               size_t workspace_bytes, bgmoe_stream_t stream) {
+  int rc = check_common("fp8_grouped_gemm_balanced", a, b, seqlens, cu_seqlens, groups, m, n, k);
+  if (rc != BGMOE_OK) return rc;
+  if (groups == 0 || m == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(out && (uintptr_t)out % 8 == 0, "fp8_grouped_gemm_balanced: output must be non-null, 8-byte aligned");
+  BGMOE_REQUIRE(max_group_rows >= 0, "fp8_grouped_gemm_balanced: max_group_rows < 0");
+  SkinnyArgs g{};
+  g.a = *a; g.w0 = *b; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups; g.n = n; g.k = k;
+  g.out = out; g.group_bound = max_group_rows; g.streamk_ws = workspace; g.streamk_ws_bytes = workspace_bytes;
+  return launch_skinny(false, g, m, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_fp8_fused_s1_balanced(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* gate,
+                                           const bgmoe_fp8_weight* up, const int32_t* seqlens, const int32_t* cu_seqlens,
+                                           int groups, int64_t m, int n, int k, uint16_t* out, uint8_t* out_q,
+                                           float* out_scale, int64_t out_scale_row_stride, int64_t out_scale_nb_stride,
+                                           int64_t max_group_rows, void* workspace, size_t workspace_bytes,
+                                           bgmoe_stream_t stream) {
+  int rc = check_common("fp8_fused_s1_balanced", a, gate, seqlens, cu_seqlens, groups, m, n, k);
+  if (rc != BGMOE_OK) return rc;
+  rc = check_common("fp8_fused_s1_balanced", a, up, seqlens, cu_seqlens, groups, m, n, k);
+  if (rc != BGMOE_OK) return rc;
+  if (groups == 0 || m == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(out || out_q, "fp8_fused_s1_balanced: no output given");
+  BGMOE_REQUIRE(!out_q || out_scale, "fp8_fused_s1_balanced: out_q needs out_scale");
+  BGMOE_REQUIRE((uintptr_t)out % 8 == 0 && (uintptr_t)out_q % 4 == 0, "fp8_fused_s1_balanced: misaligned output");
+  BGMOE_REQUIRE(max_group_rows >= 0, "fp8_fused_s1_balanced: max_group_rows < 0");
+  SkinnyArgs g{};
+  g.a = *a; g.w0 = *gate; g.w1 = *up; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups;
+  g.n = n; g.k = k; g.out = out; g.out_q = out_q; g.out_s = out_scale;
+  g.os_row = out_scale_row_stride; g.os_nb = out_scale_nb_stride;
+  g.group_bound = max_group_rows; g.streamk_ws = workspace; g.streamk_ws_bytes = workspace_bytes;
   return launch_skinny(true, g, m, bgmoe_stream(stream));
 }
 

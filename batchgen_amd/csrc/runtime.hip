@@ -27,6 +27,7 @@ extern "C" int bgmoe_version(void) { return 1; }
 
 extern "C" int bgmoe_init(void) {
   int rc = bgmoe_internal_init_fp8_skinny();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_fp8_streamk();
   if (rc == BGMOE_OK) rc = bgmoe_internal_init_fp8_tiled();
   if (rc == BGMOE_OK) rc = bgmoe_internal_init_mxfp4();
   if (rc == BGMOE_OK) rc = bgmoe_internal_init_router_gemm();

@@ -94,16 +94,31 @@ def fp8_weight_repack(weight):
 
 def fp8_blockwise_grouped_gemm(x, weight, seqlens, cu_seqlens, x_scale, w_scale, num_seq_per_group_avg,
                                output=None, tma_desc=None, tiles=None, cu_tiles=None, update_tma=True,
-                               weight_layout="row_major"):
-    """Y[r,n] = sum_kb (Xq[r,kb] . Wq[g,n,kb]) * xs[kb,r] * ws[g,n/128,kb] -> bf16 [m, N]."""
+                               weight_layout="row_major", max_group_rows=0, workspace=None):
+    """Y[r,n] = sum_kb (Xq[r,kb] . Wq[g,n,kb]) * xs[kb,r] * ws[g,n/128,kb] -> bf16 [m, N].
+    ``max_group_rows`` / ``workspace`` (this build's additions): see ``streamk_workspace``."""
     m, n, k, m_pad, g = _check_inputs(x, weight, seqlens, cu_seqlens, x_scale, w_scale, output)
     if output is None:
         output = torch.empty((m, n), dtype=torch.bfloat16, device=x.device)
     a, b = _act(x, x_scale, m_pad), _stacked(weight, w_scale, weight_layout)
     with torch.cuda.device(x.device):
-        check(lib().bgmoe_fp8_grouped_gemm(C.byref(a), C.byref(b), ptr(seqlens), ptr(cu_seqlens), g, m, n, k,
-                                           ptr(output), stream()))
+        if workspace is not None:
+            check(lib().bgmoe_fp8_grouped_gemm_balanced(C.byref(a), C.byref(b), ptr(seqlens), ptr(cu_seqlens), g, m, n,
+                                                        k, ptr(output), int(max_group_rows), ptr(workspace),
+                                                        workspace.numel() * workspace.element_size(), stream()))
+        else:
+            check(lib().bgmoe_fp8_grouped_gemm(C.byref(a), C.byref(b), ptr(seqlens), ptr(cu_seqlens), g, m, n, k,
+                                               ptr(output), stream()))
     return output
+
+
+def streamk_workspace(device):
+    """A zeroed workspace for the balanced form of the grouped GEMMs (``workspace=`` of
+    fp8_blockwise_grouped_gemm / fp8_blockwise_fused_s1_quant together with ``max_group_rows``, the caller's
+    bound on the rows of any group).  Caller-owned; one per stream; calls leave its counters at zero."""
+    with torch.cuda.device(device):
+        check(lib().bgmoe_init())
+        return torch.zeros(int(lib().bgmoe_fp8_streamk_workspace_bytes()), dtype=torch.uint8, device=device)
 
 
 def fp8_blockwise_fused_s1(x, gate_weight, up_weight, seqlens, cu_seqlens, x_scale, gate_w_scale, up_w_scale,
@@ -126,7 +141,8 @@ def fp8_blockwise_fused_s1(x, gate_weight, up_weight, seqlens, cu_seqlens, x_sca
 
 
 def fp8_blockwise_fused_s1_quant(x, gate_weight, up_weight, seqlens, cu_seqlens, x_scale, gate_w_scale,
-                                 up_w_scale, out_q, out_scale_t, weight_layout="row_major"):
+                                 up_w_scale, out_q, out_scale_t, weight_layout="row_major", max_group_rows=0,
+                                 workspace=None):
     """Fused S1 with the requant in the epilogue: out_q [m,N] bytes + TRANSPOSED scale [N/128, m].
     Same bytes as fp8_blockwise_fused_s1 followed by act_quant_ragged on the live rows."""
     m, n, k, m_pad, g = _check_inputs(x, gate_weight, seqlens, cu_seqlens, x_scale, gate_w_scale, None,
@@ -139,8 +155,14 @@ def fp8_blockwise_fused_s1_quant(x, gate_weight, up_weight, seqlens, cu_seqlens,
     a = _act(x, x_scale, m_pad)
     wg, wu = _stacked(gate_weight, gate_w_scale, weight_layout), _stacked(up_weight, up_w_scale, weight_layout)
     with torch.cuda.device(x.device):
-        check(lib().bgmoe_fp8_fused_s1(C.byref(a), C.byref(wg), C.byref(wu), ptr(seqlens), ptr(cu_seqlens), g, m,
-                                       n, k, None, ptr(out_q), ptr(out_scale_t), 1, m, stream()))
+        if workspace is not None:
+            check(lib().bgmoe_fp8_fused_s1_balanced(C.byref(a), C.byref(wg), C.byref(wu), ptr(seqlens), ptr(cu_seqlens),
+                                                    g, m, n, k, None, ptr(out_q), ptr(out_scale_t), 1, m,
+                                                    int(max_group_rows), ptr(workspace),
+                                                    workspace.numel() * workspace.element_size(), stream()))
+        else:
+            check(lib().bgmoe_fp8_fused_s1(C.byref(a), C.byref(wg), C.byref(wu), ptr(seqlens), ptr(cu_seqlens), g, m,
+                                           n, k, None, ptr(out_q), ptr(out_scale_t), 1, m, stream()))
     return out_q, out_scale_t
 
 

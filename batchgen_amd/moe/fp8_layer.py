@@ -39,6 +39,7 @@ class LayerStruct(C.Structure):
         ("x_fp8", vp), ("x_scale", vp), ("x_scale_row_stride", i64), ("x_scale_kb_stride", i64),
         ("router_weight", vp), ("router_hidden", vp), ("router_workspace", vp), ("router_workspace_bytes", sz),
         ("routes_given", i32),
+        ("gemm_workspace", vp), ("gemm_workspace_bytes", sz),
     ]
 
 
@@ -46,6 +47,7 @@ _lib.register("bgmoe_moe_fp8_layer_forward", i32, [C.POINTER(LayerStruct), vp])
 
 
 W_ROW_MAJOR, W_TILE_MAJOR = 0, 1
+STREAMK_MAX_TOKENS = 256      # no group of such a batch exceeds the weight-streaming kernel's row limit
 
 
 def _check_stack(q: torch.Tensor, s: torch.Tensor):
@@ -90,7 +92,7 @@ class Fp8MoELayer:
 
     def __init__(self, cfg: MoEConfig, weights, shared, bias: torch.Tensor, max_tokens_in: Optional[int] = None,
                  shared_mode: str = "bf16_add", fold_shared: bool = True, weight_layout: str = "tile_major",
-                 router_weight: Optional[torch.Tensor] = None):
+                 router_weight: Optional[torch.Tensor] = None, balanced_gemm: bool = False):
         self.cfg = cfg
         dev = weights["gate_q"].device
         with torch.cuda.device(dev):
@@ -170,6 +172,12 @@ class Fp8MoELayer:
         L.xq, L.xs, L.hq, L.hs, L.y = ptr(self.xq), ptr(self.xs), ptr(self.hq), ptr(self.hs), ptr(self.y)
         L.workspace, L.workspace_bytes = ptr(self.workspace), self.workspace.numel()
         L.out = ptr(self.out)
+        self.gemm_workspace = None
+        if balanced_gemm and self.layout == W_TILE_MAJOR and n <= STREAMK_MAX_TOKENS:
+            # decode-sized batches: both grouped GEMMs in their balanced form (its counters start at zero)
+            gb = int(lib().bgmoe_fp8_streamk_workspace_bytes())
+            self.gemm_workspace = torch.zeros(gb, dtype=e8, device=dev)
+            L.gemm_workspace, L.gemm_workspace_bytes = ptr(self.gemm_workspace), gb
         self.router_weight = None
         if router_weight is not None:
             # the layer then routes from the hidden states: router GEMM + gate, no logits tensor

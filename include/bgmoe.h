@@ -436,6 +436,38 @@ int bgmoe_fp8_dense_gemm_partials(const bgmoe_fp8_act* a, const uint8_t* w, cons
                                   int64_t scale_nb_stride, int layout, int64_t m, int n, int k, void* workspace,
                                   int64_t workspace_bytes, int* slices, bgmoe_stream_t stream);
 
+/* Workspace of the balanced form of the weight-streaming grouped GEMM (no reference counterpart).  A decode launch
+ * has a few hundred work items of 0.25-1.8 MB for ~512 resident blocks, so whole items leave CUs idle; the
+ * balanced form cuts the sequence of all items' K-blocks into one equal share per block, streams each share
+ * without a gap across item boundaries, and finishes an item that was cut over several blocks in the block that
+ * arrives last (fp32 partial sums in this workspace, added in block order; no block waits for another).  A cut
+ * item's K-chain is summed in as many pieces as it was cut into, so its last bits depend on the group sizes of the
+ * launch (never on timing).  Layout: 4096 bytes of counters (zero before the first use, left zero by every launch)
+ * followed by the partial-sum slots. */
+size_t bgmoe_fp8_streamk_workspace_bytes(void);
+/* Tuning aid: with a device buffer of 4 * 1024 uint64 set, every share (block) of the following balanced launches
+ * records the constant-rate clock (100 MHz) at its start, before its first unit, at the end of its stream and at its
+ * end, at [4 * share .. 4 * share + 3].  NULL switches it off. */
+int bgmoe_debug_streamk_trace(uint64_t* device_buffer);
+/* Tuning knob: relative sizes of the shares of XCD 0..7 (8 ints, each in [1, 64]; default 23/21 alternating: on
+ * MI355X the odd XCDs were measured to stream about 9% slower than the even ones). */
+int bgmoe_set_streamk_xcd_weights(const int* weights);
+
+/* bgmoe_fp8_grouped_gemm / bgmoe_fp8_fused_s1 (same operands, outputs and checks) in the balanced form when it
+ * applies: tile-major weights, workspace of bgmoe_fp8_streamk_workspace_bytes() bytes, and max_group_rows -- the
+ * caller's bound on the rows of any one group (a decode batch: the number of tokens) -- within the streaming
+ * kernel's row limit.  Otherwise (max_group_rows 0 = unknown, row-major weights, NULL workspace) they are the plain
+ * calls.  No reference counterpart: the reference's ops take no workspace (fp8_blockwise_gemm.cu:564-900). */
+int bgmoe_fp8_grouped_gemm_balanced(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* b, const int32_t* seqlens,
+                                    const int32_t* cu_seqlens, int groups, int64_t m, int n, int k, uint16_t* out,
+                                    int64_t max_group_rows, void* workspace, size_t workspace_bytes,
+                                    bgmoe_stream_t stream);
+int bgmoe_fp8_fused_s1_balanced(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* gate, const bgmoe_fp8_weight* up,
+                                const int32_t* seqlens, const int32_t* cu_seqlens, int groups, int64_t m, int n, int k,
+                                uint16_t* out, uint8_t* out_q, float* out_scale, int64_t out_scale_row_stride,
+                                int64_t out_scale_nb_stride, int64_t max_group_rows, void* workspace,
+                                size_t workspace_bytes, bgmoe_stream_t stream);
+
 /* Tuning knob (no reference counterpart): groups with at most `rows` rows are served by the
  * weight-streaming kernel, larger ones by the LDS-tiled kernel.  0 sends everything to the tiled
  * kernel.  Default 256 (or the environment variable BGMOE_SKINNY_MAX_ROWS at first use).
@@ -625,6 +657,13 @@ typedef struct bgmoe_moe_fp8_layer {
    * topk_idx, topk_weight)`, batchgen/moe/fp8_wgmma_pipeline.py:294-372).  Ids outside the local expert range
    * (and -1) contribute nothing. */
   int32_t routes_given;
+  /* Optional: bgmoe_fp8_streamk_workspace_bytes() bytes, 16-byte aligned, its first 4096 bytes zero before the
+   * first call (every call leaves them zero).  With it, a batch in which no group can exceed the streaming
+   * kernel's row limit (n <= 256) runs both grouped GEMMs in their balanced form (see
+   * bgmoe_fp8_streamk_workspace_bytes); NULL / 0 = the item-per-block form.  One workspace per stream: calls that
+   * overlap on one workspace race. */
+  void* gemm_workspace;
+  size_t gemm_workspace_bytes;
 } bgmoe_moe_fp8_layer;
 
 int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* layer, bgmoe_stream_t stream);
