@@ -44,19 +44,10 @@ def _one_group(m: int, device):
     return base, base + 4
 
 
-_SCRATCH = {}
-
-
 def _workspace(nbytes: int, device):
-    """Split-K partial sums: one buffer per device, grown on demand (a call that fits allocates nothing)."""
-    if nbytes <= 0:
-        return None
-    key = str(device)
-    t = _SCRATCH.get(key)
-    if t is None or t.numel() < nbytes:
-        t = torch.empty(max(nbytes, 1 << 24), dtype=torch.uint8, device=device)
-        _SCRATCH[key] = t
-    return t
+    """Split-K partial sums: per device and stream, never freed once handed out (kernels/_workspace.py)."""
+    from ..kernels._workspace import dense_gemm_workspace
+    return dense_gemm_workspace(device, nbytes)
 
 
 def fp8_gemm_nt(lhs, rhs, d: torch.Tensor, weight_layout: str = "row_major") -> None:

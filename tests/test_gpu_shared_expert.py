@@ -249,3 +249,42 @@ def test_activation_fed_by_partial_sums_equals_gemm_then_activation(dev, rows, h
     assert torch.equal(short[1], h_scale) and short[1].stride() == h_scale.stride()
     small = fused._gate_up_activation_from_partials(x_fp8[:8], x_scale[:8], 8, hidden)
     assert small is None                                   # a handful of rows: no partial sums exist
+
+
+def test_scratch_pool_survives_growth_after_capture(dev):
+    """A graph captured while the pool's buffer was small keeps giving the right answer after an eager call has
+    made the pool allocate a larger one (the old buffer is retired, not freed), and two streams get two buffers."""
+    from batchgen_amd.kernels import _workspace as wsp
+    from batchgen_amd.kernels import load_extension
+    rt = load_extension("batchgen_kernels.moe._C_routing")
+    g = torch.Generator().manual_seed(11)
+    e, h = 64, 1024
+    w = (torch.randn(e, h, generator=g) * 0.05).to(torch.bfloat16).to(dev)
+    small = torch.randn(8, h, generator=g).to(torch.bfloat16).to(dev)
+    big = torch.randn(4096, h, generator=g).to(torch.bfloat16).to(dev)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        out_small = torch.empty((8, e), dtype=torch.float32, device=dev)
+        rt.glm5_router_gemm(small, w, None, out_small, 0, 1)          # warm-up on the capture stream
+        s.synchronize()
+        key = ("router_gemm", dev.index or 0, s.cuda_stream)
+        first = wsp._LIVE.get(key)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            rt.glm5_router_gemm(small, w, None, out_small, 0, 1)
+        want = out_small.clone()
+        from batchgen_amd._lib import lib
+        need_big = int(lib().bgmoe_router_gemm_workspace_bytes(4096, h, e))
+        out_big = torch.empty((4096, e), dtype=torch.float32, device=dev)
+        rt.glm5_router_gemm(big, w, None, out_big, 0, 1)               # may grow the pool on this stream
+        torch.zeros(1 << 22, device=dev).fill_(3.0)                   # churn the allocator
+        out_small.zero_()
+        graph.replay()
+        s.synchronize()
+        assert torch.equal(out_small, want)
+        if first is not None and need_big > first.numel():
+            assert wsp._LIVE[key] is not first and any(b is first for b in wsp._RETIRED)
+    other = wsp.scratch("router_gemm", dev, 1024)
+    with torch.cuda.stream(s):
+        mine = wsp.scratch("router_gemm", dev, 1024)
+    assert other.data_ptr() != mine.data_ptr()
