@@ -30,6 +30,10 @@ int bgmoe_internal_dispatch_index(const int32_t* ids, int64_t nk, int expert_sta
                                   int row_align, int32_t* counts, int32_t* counters, int32_t* cu,
                                   int32_t* pos, int extra_count, int64_t extra_start, void* ws,
                                   size_t ws_bytes, hipStream_t st);
+int bgmoe_internal_dispatch_scatter_quant(const int32_t* ids, int n, int k, int h, int expert_start, int e_local, int mtp,
+                                          int row_align, int32_t* counts, int32_t* counters, int32_t* cu, int32_t* pos,
+                                          int extra_count, int64_t extra_start, const uint16_t* x, uint8_t* y,
+                                          float* scale, int64_t srow, int64_t skb, hipStream_t st);
 int bgmoe_internal_scatter_quant(const uint16_t* x, const int32_t* topk_pos, int n, int k, int h, uint8_t* y,
                                  float* scale, int64_t srow, int64_t skb, int extra_rows, int64_t extra_start,
                                  hipStream_t st);

@@ -61,21 +61,29 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
   }
   if (rc != BGMOE_OK) return rc;
 
-  // 2. stable counting sort -> counts, cu_seqlens (+ the shared expert as one more group), topk_pos
-  rc = bgmoe_internal_dispatch_index(L->topk_ids, nk, L->expert_start, el, L->layout == 0 ? L->max_tokens : 0,
-                                     L->layout == 0 ? 1 : L->row_align, L->expert_counts, nullptr,
-                                     L->cu_seqlens, L->topk_pos, shared ? n : 0, L->cap_rows, L->workspace,
-                                     L->workspace_bytes, st);
-  if (rc != BGMOE_OK) return rc;
-
-  // 3. quantise while scattering; the shared expert's rows are the tokens themselves
+  // 2 + 3. stable counting sort -> counts, cu_seqlens (+ the shared expert as one more group), topk_pos; quantise
+  // while scattering (the shared expert's rows are the tokens themselves).  One launch for a decode-sized batch,
+  // two otherwise.
   const int hb = h / 128, ib = inter / 128;
-  if (pre_quant)
-    rc = bgmoe_internal_scatter_fp8(L->x_fp8, L->x_scale, L->x_scale_row_stride, L->x_scale_kb_stride,
-                                    L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0, L->cap_rows, st);
-  else
-    rc = bgmoe_internal_scatter_quant(L->x, L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0,
-                                      L->cap_rows, st);
+  rc = BGMOE_ERR_WORKSPACE;
+  if (!pre_quant)
+    rc = bgmoe_internal_dispatch_scatter_quant(L->topk_ids, n, k, h, L->expert_start, el,
+                                               L->layout == 0 ? L->max_tokens : 0, L->layout == 0 ? 1 : L->row_align,
+                                               L->expert_counts, nullptr, L->cu_seqlens, L->topk_pos, shared ? n : 0,
+                                               L->cap_rows, L->x, L->xq, L->xs, hb, 1, st);
+  if (rc == BGMOE_ERR_WORKSPACE) {
+    rc = bgmoe_internal_dispatch_index(L->topk_ids, nk, L->expert_start, el, L->layout == 0 ? L->max_tokens : 0,
+                                       L->layout == 0 ? 1 : L->row_align, L->expert_counts, nullptr,
+                                       L->cu_seqlens, L->topk_pos, shared ? n : 0, L->cap_rows, L->workspace,
+                                       L->workspace_bytes, st);
+    if (rc != BGMOE_OK) return rc;
+    if (pre_quant)
+      rc = bgmoe_internal_scatter_fp8(L->x_fp8, L->x_scale, L->x_scale_row_stride, L->x_scale_kb_stride,
+                                      L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0, L->cap_rows, st);
+    else
+      rc = bgmoe_internal_scatter_quant(L->x, L->topk_pos, n, k, h, L->xq, L->xs, hb, 1, shared ? n : 0,
+                                        L->cap_rows, st);
+  }
   if (rc != BGMOE_OK) return rc;
 
   // 4/5. gate_up + SwiGLU + requant, then down

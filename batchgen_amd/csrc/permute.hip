@@ -198,10 +198,10 @@ __global__ __launch_bounds__(256) void perm_rank_kernel(PermArgs a) {
 // one global load, a few LDS round trips per sub-step.
 constexpr int kSmallLocal = 256;
 constexpr int kSmallPairsMax = 64 * 16 * 8;
+// `global`: this block writes counts, offsets and positions to memory; `s_pos` (optional): the positions in LDS.
 template <int S>
-__global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
-  __shared__ int32_t whist[16][kSmallLocal];   // per-wave counts, then exclusive offsets over the waves
-  __shared__ int32_t s_cu[kSmallLocal + 1];
+__device__ __forceinline__ void perm_small_body(const PermArgs& a, int32_t (*whist)[kSmallLocal], int32_t* s_cu,
+                                                int32_t* s_pos, bool global) {
   const int wave = threadIdx.x >> 6;
   const int lane = lane_id();
   const int el = a.e_local;
@@ -240,8 +240,10 @@ __global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
       run += t;
     }
     const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
-    a.counts[e] = cnt;
-    if (a.counters) a.counters[e] = cnt;
+    if (global) {
+      a.counts[e] = cnt;
+      if (a.counters) a.counters[e] = cnt;
+    }
     s_cu[e + 1] = cnt;
   }
   __syncthreads();
@@ -263,11 +265,11 @@ __global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
       __builtin_amdgcn_wave_barrier();          // everybody has read s_cu[g + 1] before s_cu[g] is overwritten
       if (g < el) {
         s_cu[g] = (int32_t)(base + inc - span);
-        if (a.cu) a.cu[g] = (int32_t)(base + inc - span);
+        if (a.cu && global) a.cu[g] = (int32_t)(base + inc - span);
       }
       base += __shfl(inc, 63, BGMOE_WAVE);
     }
-    if (lane == 0) write_tail(a, base);
+    if (lane == 0 && global) write_tail(a, base);
   }
   __syncthreads();
 #pragma unroll
@@ -280,10 +282,88 @@ __global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
         if (a.mtp > 0) p = slot < a.mtp ? le[s] * a.mtp + slot : -1;
         else p = s_cu[le[s]] + slot;
       }
-      a.pos[i] = p;
+      if (global) a.pos[i] = p;
+      if (s_pos) s_pos[i] = p;
     }
   }
 }
+
+template <int S>
+__global__ __launch_bounds__(1024) void perm_small_kernel(PermArgs a) {
+  __shared__ int32_t whist[16][kSmallLocal];   // per-wave counts, then exclusive offsets over the waves
+  __shared__ int32_t s_cu[kSmallLocal + 1];
+  perm_small_body<S>(a, whist, s_cu, nullptr, true);
+}
+
+// Decode-sized batches (at most 2048 pairs): permutation indices, FP8 quantisation and the scatter in ONE launch.
+// Every block repeats the whole (small) index computation above and keeps the positions in LDS -- cheaper than a
+// second launch that waits for them -- block 0 also writes counts, offsets and positions to memory; then each
+// wave quantises one (token, 512 columns) piece once and writes bytes and scales to every row the token is routed
+// to and to its identity row (the shared expert), exactly as scatter_quant_kernel does.
+struct FusedQuantArgs {
+  const uint16_t* x;
+  uint8_t* y;
+  float* scale;
+  int64_t srow, skb;
+  int n, topk, h, steps, extra_rows;
+  int64_t extra_start;
+};
+
+__global__ __launch_bounds__(1024) void perm_quant_small_kernel(PermArgs a, FusedQuantArgs q) {
+  __shared__ int32_t whist[16][kSmallLocal];
+  __shared__ int32_t s_cu[kSmallLocal + 1];
+  __shared__ int32_t s_pos[kChunk];
+  perm_small_body<2>(a, whist, s_cu, s_pos, blockIdx.x == 0);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6;
+  const int lane = lane_id();
+  const int k = q.h;
+  const int64_t njobs = (int64_t)q.n * q.steps;
+  for (int64_t job = (int64_t)blockIdx.x * 16 + wave; job < njobs; job += (int64_t)gridDim.x * 16) {
+    const int64_t tok = job / q.steps;
+    const int c0 = (int)(job - tok * q.steps) * 512 + lane * 8;
+    const bool in = c0 < k;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+    if (in) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(q.x + tok * (int64_t)k + c0);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] = bf16_bits_to_f32(w[i] & 0xffffu);
+        v[2 * i + 1] = bf16_bits_to_f32(w[i] >> 16);
+      }
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    amax = wave_max_xor<16>(amax);
+    const float sc = quant_scale_from_amax(amax);
+    uint2 o;
+    {
+      float qv[8];
+      quant_div_clamp(v, sc, qv);
+      o.x = pack4_e4m3(qv[0], qv[1], qv[2], qv[3]);
+      o.y = pack4_e4m3(qv[4], qv[5], qv[6], qv[7]);
+    }
+    const bool lead = (lane & 15) == 0;
+    int mine = -1;
+    if (lane < q.topk) mine = s_pos[tok * q.topk + lane];
+    else if (lane == q.topk && tok < q.extra_rows) mine = (int)(q.extra_start + tok);
+    unsigned long long live = __ballot(mine >= 0);
+    while (live) {
+      const int j = __ffsll((long long)live) - 1;
+      live &= live - 1;
+      const int64_t dst = __builtin_amdgcn_readlane(mine, j);
+      if (in) {
+        *reinterpret_cast<uint2*>(q.y + dst * (int64_t)k + c0) = o;
+        if (lead) q.scale[dst * q.srow + (int64_t)(c0 >> 7) * q.skb] = sc;
+      }
+    }
+  }
+}
+
 
 // one wave per pair: act[pos] = x[token]
 __global__ __launch_bounds__(256) void gather_rows_kernel(const uint16_t* __restrict__ x,
@@ -382,6 +462,29 @@ int bgmoe_internal_dispatch_index(const int32_t* ids, int64_t nk, int expert_sta
   a.row_align = row_align; a.counts = counts; a.counters = counters; a.cu = cu; a.pos = pos;
   a.extra_count = extra_count; a.extra_start = extra_start;
   return run_index(a, ws, ws_bytes, st);
+}
+
+// Index + quantise + scatter in one launch for decode-sized batches.  BGMOE_ERR_WORKSPACE (no message): does not
+// apply (too many pairs or experts, odd shapes), the caller runs the two steps separately.
+int bgmoe_internal_dispatch_scatter_quant(const int32_t* ids, int n, int k, int h, int expert_start, int e_local, int mtp,
+                                          int row_align, int32_t* counts, int32_t* counters, int32_t* cu, int32_t* pos,
+                                          int extra_count, int64_t extra_start, const uint16_t* x, uint8_t* y,
+                                          float* scale, int64_t srow, int64_t skb, hipStream_t st) {
+  const int64_t nk = (int64_t)n * k;
+  if (nk <= 0 || nk > kChunk || e_local > kSmallLocal || k >= 64 || h <= 0 || h % 8 != 0 ||
+      (uintptr_t)x % 16 != 0 || (uintptr_t)y % 8 != 0 || extra_count > n)
+    return BGMOE_ERR_WORKSPACE;
+  PermArgs a{};
+  a.ids = ids; a.nk = nk; a.expert_start = expert_start; a.e_local = e_local; a.mtp = mtp;
+  a.row_align = row_align; a.counts = counts; a.counters = counters; a.cu = cu; a.pos = pos;
+  a.extra_count = extra_count; a.extra_start = extra_start; a.nchunks = 1;
+  FusedQuantArgs q{};
+  q.x = x; q.y = y; q.scale = scale; q.srow = srow; q.skb = skb; q.n = n; q.topk = k; q.h = h;
+  q.steps = (h + 511) / 512; q.extra_rows = extra_count > 0 ? extra_count : 0; q.extra_start = extra_start;
+  const int64_t blocks = ((int64_t)n * q.steps + 15) / 16;
+  BgmoeProf prof(BGMOE_K_ACT_QUANT, st);
+  hipLaunchKernelGGL(perm_quant_small_kernel, dim3((unsigned)blocks), dim3(1024), 0, st, a, q);
+  return bgmoe_check_launch("dispatch + scatter_quant");
 }
 
 extern "C" size_t bgmoe_dispatch_workspace_bytes(int64_t nk, int num_local_experts) {
