@@ -94,6 +94,53 @@ def _check_no_spill(src: str, remarks: str, obj: str) -> None:
         raise RuntimeError(f"{src}: kernels must not spill registers ({'; '.join(bad) or 'no resource remarks found'})")
 
 
+# ---- PyTorch C++ extension modules (host code over the C ABI) --------------------------------------------------
+EXT_SRC = os.path.join(HERE, "ext", "bgmoe_torch.cc")
+EXT_ROOT = os.path.join(HERE, "ext", "build")              # put on sys.path: holds the batchgen_kernels/... tree
+EXT_MODULES = (
+    "moe/_C_routing", "common/_C_mgn_ops", "moe/_C_dispatch_scatter_3d", "moe/_C_fp8_blockwise_gemm",
+    "moe/_C_fp8_blockwise_ops", "attention/_C_add_rmsnorm_fp8_quant",
+)
+
+
+def build_extensions(force: bool = False, verbose: bool = True) -> str:
+    """Compile batchgen_amd/ext/bgmoe_torch.cc once (g++: host code only) against the torch headers and libbgmoe.so,
+    and install the shared object as batchgen_kernels/<pkg>/<module>.so under batchgen_amd/ext/build: the module and
+    op names of the reference's compiled extensions (batchgen_kernels/__init__.py:24-45 imports them by these
+    names).  Returns the directory to put on sys.path."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension as ce
+    if not os.path.exists(LIB):
+        raise RuntimeError(f"{LIB} is missing: build the HIP library first")
+    os.makedirs(EXT_ROOT, exist_ok=True)
+    one = os.path.join(EXT_ROOT, "_bgmoe_torch.so")
+    deps = [EXT_SRC, os.path.join(INCLUDE, "bgmoe.h")]
+    if force or not _newer(one, deps):
+        tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+        rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+        cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-w", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+               f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"]
+        cmd += [f"-I{p}" for p in ce.include_paths()] + [f"-I{sysconfig.get_paths()['include']}", f"-I{rocm}/include"]
+        cmd += [EXT_SRC, "-o", one, f"-L{tlib}", f"-L{LIB_DIR}", "-ltorch_python", "-ltorch", "-ltorch_cpu", "-lc10",
+                "-lc10_hip", "-ltorch_hip", "-lbgmoe", f"-Wl,-rpath,{tlib}", "-Wl,-rpath,$ORIGIN/../../../lib",
+                "-Wl,-rpath,$ORIGIN/../../../../lib"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"g++ failed for {EXT_SRC}:\n{r.stdout[-3000:]}\n{r.stderr[-6000:]}")
+    suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+    for mod in EXT_MODULES:
+        pkg, name = mod.split("/")
+        d = os.path.join(EXT_ROOT, "batchgen_kernels", pkg)
+        os.makedirs(d, exist_ok=True)
+        dst = os.path.join(d, name + suffix)
+        if force or not _newer(dst, [one]):
+            shutil.copyfile(one, dst)
+    if verbose:
+        print(f"built {len(EXT_MODULES)} extension modules under {EXT_ROOT}/batchgen_kernels")
+    return EXT_ROOT
+
+
 def build(force: bool = False, jobs: int = 4, verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -113,10 +160,13 @@ def build(force: bool = False, jobs: int = 4, verbose: bool = True) -> str:
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--ext", action="store_true", help="also build the PyTorch C++ extension modules")
     ap.add_argument("-j", type=int, default=4)
     a = ap.parse_args()
     try:
         build(force=a.force, jobs=a.j)
+        if a.ext:
+            build_extensions(force=a.force)
     except RuntimeError as e:
         print(e, file=sys.stderr)
         sys.exit(1)
