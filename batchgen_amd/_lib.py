@@ -72,6 +72,8 @@ _SIGS = {
     "bgmoe_fused_silu_quant_3d": (i32, [vp, vp, vp, i32, i32, i32, vp, vp, vp]),
     "bgmoe_deepep_ll_scale_repack": (i32, [vp, vp, vp, i32, i32, i32, i32, vp, vp]),
     "bgmoe_dispatch_workspace_bytes": (sz, [i64, i32]),
+    "bgmoe_silu_and_mul": (i32, [vp, i64, i32, i64, vp, i64, vp]),
+    "bgmoe_bf16_linear": (i32, [vp, vp, i32, i32, i32, vp, vp, sz, vp]),
     "bgmoe_fp8_streamk_workspace_bytes": (sz, []),
     "bgmoe_debug_streamk_trace": (i32, [vp]),
     "bgmoe_set_streamk_xcd_weights": (i32, [vp]),

@@ -14,9 +14,16 @@ struct SituArgs {
   int d;
   float beta, inv_beta, lbeta, inv_lbeta;
   int has_linear;
+  int swiglu;              // bf16(bf16(silu(g)) * u) instead: PyTorch's F.silu(gate) * up on bf16 tensors
 };
 
 __device__ __forceinline__ float situ_one(const SituArgs& a, float g, float u) {
+  if (a.swiglu) {
+    bool decided;
+    float sv = silu_short_f32(g, &decided);
+    if (!decided) sv = silu_exact_f32(g);
+    return bf16_round_f32(sv) * u;
+  }
   const float lin = a.has_linear ? situ_linear_f32(u, a.lbeta, a.inv_lbeta) : u;
   return situ_gate_f32(g, a.beta, a.inv_beta) * lin;
 }
@@ -50,18 +57,31 @@ __global__ __launch_bounds__(256) void situ_and_mul_kernel(SituArgs a) {
 
 }  // namespace
 
+static int act_and_mul(const uint16_t* x, int64_t rows, int d, int64_t x_row_stride, float beta, float linear_beta,
+                       int swiglu, uint16_t* out, int64_t out_row_stride, bgmoe_stream_t stream);
+
 extern "C" int bgmoe_situ_and_mul(const uint16_t* x, int64_t rows, int d, int64_t x_row_stride, float beta,
                                   float linear_beta, uint16_t* out, int64_t out_row_stride,
                                   bgmoe_stream_t stream) {
-  BGMOE_REQUIRE(rows >= 0 && d >= 0, "situ_and_mul: bad sizes rows=%lld d=%d", (long long)rows, d);
   BGMOE_REQUIRE(beta > 0.0f, "situ_and_mul: beta must be positive, got %g", (double)beta);
+  return act_and_mul(x, rows, d, x_row_stride, beta, linear_beta, 0, out, out_row_stride, stream);
+}
+
+extern "C" int bgmoe_silu_and_mul(const uint16_t* x, int64_t rows, int d, int64_t x_row_stride, uint16_t* out,
+                                  int64_t out_row_stride, bgmoe_stream_t stream) {
+  return act_and_mul(x, rows, d, x_row_stride, 1.0f, 0.0f, 1, out, out_row_stride, stream);
+}
+
+static int act_and_mul(const uint16_t* x, int64_t rows, int d, int64_t x_row_stride, float beta, float linear_beta,
+                       int swiglu, uint16_t* out, int64_t out_row_stride, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(rows >= 0 && d >= 0, "situ_and_mul: bad sizes rows=%lld d=%d", (long long)rows, d);
   if (rows == 0 || d == 0) return BGMOE_OK;
   BGMOE_REQUIRE(x && out, "situ_and_mul: null pointer");
   BGMOE_REQUIRE(x_row_stride >= 2 * (int64_t)d && out_row_stride >= d, "situ_and_mul: row strides smaller than the rows");
   BGMOE_REQUIRE((const void*)x != (const void*)out, "situ_and_mul: out must not alias x");
   SituArgs a{};
   a.x = x; a.out = out; a.rows = rows; a.xs = x_row_stride; a.os = out_row_stride; a.d = d;
-  a.beta = beta; a.inv_beta = 1.0f / beta;
+  a.beta = beta; a.inv_beta = 1.0f / beta; a.swiglu = swiglu;
   a.has_linear = linear_beta > 0.0f;
   a.lbeta = a.has_linear ? linear_beta : 1.0f;
   a.inv_lbeta = 1.0f / a.lbeta;

@@ -27,6 +27,7 @@ struct RouterGemmArgs {
   const uint16_t* x;             // [n,h] bf16
   const uint16_t* w;             // [e,h] bf16
   float* out;                    // whole: logits [n,e]; split: planes [nseg][n][e]
+  uint16_t* out16;               // optional: the result rounded to bf16 [n,e] instead of `out` (a linear layer)
   const int64_t* rank_counts;    // whole only: rows past a rank's count get 0
   int bucket, world;
   int n, h, e, nseg;
@@ -38,6 +39,22 @@ struct Stage {
   intx4 a[NE][2];                // NE expert tiles x two 16-byte halves of the lane's 32 bytes
   intx4 b[TM][2];                // TM token tiles
 };
+
+// four consecutive results of one row as bf16 (`left` = columns left in the row from the first of them)
+__device__ __forceinline__ void store_bf16x4(uint16_t* dst, floatx4 v, int left, bool vec) {
+  if (vec) {
+    if (left > 0) {
+      uint2 o;
+      o.x = pack2_bf16(v[0], v[1]);
+      o.y = pack2_bf16(v[2], v[3]);
+      *reinterpret_cast<uint2*>(dst) = o;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < left) dst[i] = (uint16_t)f32_to_bf16_bits(v[i]);
+  }
+}
 
 __device__ __forceinline__ bool row_is_padding(const RouterGemmArgs& a, int row) {
   if (!a.rank_counts) return false;
@@ -212,6 +229,10 @@ __global__ __launch_bounds__(64 * WAVES) void router_gemm_kernel(RouterGemmArgs 
     for (int tn = 0; tn < NE; ++tn) {
       const int ex = e0 + tn * 16 + q * 4;
       floatx4 v = pad ? floatx4{0.f, 0.f, 0.f, 0.f} : tot[tm][tn];
+      if (!SPLIT && a.out16 != nullptr) {
+        store_bf16x4(a.out16 + (int64_t)token * a.e + ex, v, a.e - ex, vec);
+        continue;
+      }
       float* dst = plane + (int64_t)token * a.e + ex;
       if (vec) {
         if (ex < a.e) *reinterpret_cast<floatx4*>(dst) = v;
@@ -362,6 +383,10 @@ __global__ __launch_bounds__(64 * kLdsWaves) void router_gemm_lds_kernel(RouterG
     for (int tn = 0; tn < 4; ++tn) {
       const int ex = e0 + we * 64 + tn * 16 + q * 4;
       const floatx4 v = pad ? floatx4{0.f, 0.f, 0.f, 0.f} : tot[tm][tn];
+      if (!SPLIT && a.out16 != nullptr) {
+        store_bf16x4(a.out16 + (int64_t)token * a.e + ex, v, a.e - ex, vec);
+        continue;
+      }
       float* dst = a.out + (SPLIT ? (int64_t)seg * a.n * a.e : 0) + (int64_t)token * a.e + ex;
       if (vec) {
         if (ex < a.e) *reinterpret_cast<floatx4*>(dst) = v;
@@ -383,7 +408,8 @@ __global__ __launch_bounds__(256) void router_gemm_reduce_kernel(RouterGemmArgs 
   float v = 0.0f;
   if (!row_is_padding(a, row))
     for (int s = 0; s < a.nseg; ++s) v += planes[(int64_t)s * total + i];
-  a.out[i] = v;
+  if (a.out16 != nullptr) a.out16[i] = (uint16_t)f32_to_bf16_bits(v);
+  else a.out[i] = v;
 }
 
 int g_plan_tm = -1, g_plan_split = -1;
@@ -524,21 +550,41 @@ int bgmoe_internal_router_gemm_planes(const uint16_t* hidden, const uint16_t* we
   return bgmoe_check_launch("router_gemm");
 }
 
+static int router_gemm_run(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,
+                           const int64_t* rank_token_counts, int bucket_size, int world_size, float* logits,
+                           uint16_t* out16, void* workspace, size_t workspace_bytes, bgmoe_stream_t stream);
+
 extern "C" int bgmoe_router_gemm(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,
                                  const int64_t* rank_token_counts, int bucket_size, int world_size,
                                  float* logits, void* workspace, size_t workspace_bytes,
                                  bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n == 0 || logits, "router_gemm: null pointer");
+  return router_gemm_run(hidden, weight, n, h, e, rank_token_counts, bucket_size, world_size, logits, nullptr, workspace,
+                         workspace_bytes, stream);
+}
+
+extern "C" int bgmoe_bf16_linear(const uint16_t* x, const uint16_t* weight, int n, int h, int e, uint16_t* out,
+                                 void* workspace, size_t workspace_bytes, bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n == 0 || out, "bf16_linear: null output");
+  BGMOE_REQUIRE(e % 4 == 0 || (uintptr_t)out % 2 == 0, "bf16_linear: misaligned output");
+  BGMOE_REQUIRE(e % 4 != 0 || (uintptr_t)out % 8 == 0, "bf16_linear: output must be 8-byte aligned");
+  return router_gemm_run(x, weight, n, h, e, nullptr, 0, 0, nullptr, out, workspace, workspace_bytes, stream);
+}
+
+static int router_gemm_run(const uint16_t* hidden, const uint16_t* weight, int n, int h, int e,
+                           const int64_t* rank_token_counts, int bucket_size, int world_size, float* logits,
+                           uint16_t* out16, void* workspace, size_t workspace_bytes, bgmoe_stream_t stream) {
   if (int rc = check_shapes(n, h, e)) return rc;
   if (rank_token_counts) {
     BGMOE_REQUIRE(world_size > 0, "router_gemm: world_size must be positive when rank_token_counts is provided");
     BGMOE_REQUIRE(bucket_size > 0, "router_gemm: bucket_size must be positive when rank_token_counts is provided");
   }
   if (n == 0) return BGMOE_OK;
-  BGMOE_REQUIRE(hidden && weight && logits, "router_gemm: null pointer");
+  BGMOE_REQUIRE(hidden && weight && (logits || out16), "router_gemm: null pointer");
   bgmoe_internal_init_router_gemm();
   hipStream_t st = bgmoe_stream(stream);
   RouterGemmArgs a{};
-  a.x = hidden; a.w = weight; a.n = n; a.h = h; a.e = e;
+  a.x = hidden; a.w = weight; a.n = n; a.h = h; a.e = e; a.out16 = out16;
   a.rank_counts = rank_token_counts; a.bucket = bucket_size; a.world = world_size;
   a.nseg = (h + kSeg - 1) / kSeg;
   Plan p = make_plan(n, h, e);
@@ -557,6 +603,7 @@ extern "C" int bgmoe_router_gemm(const uint16_t* hidden, const uint16_t* weight,
   {
     RouterGemmArgs g = a;
     g.out = static_cast<float*>(workspace);
+    g.out16 = nullptr;
     g.rank_counts = nullptr;
     BgmoeProf prof(BGMOE_K_ROUTER_GEMM, st);
     launch_gemm<true>(g, p, st);

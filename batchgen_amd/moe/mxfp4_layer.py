@@ -21,12 +21,11 @@ import os
 import ctypes as C
 
 import torch
-import torch.nn.functional as F
 
 from .. import _lib
 from .._lib import Mxfp4Weight, check, lib, ptr, stream
 from ..kernels import load_extension
-from .latent import rmsnorm, situ_and_mul
+from .latent import bf16_linear, rmsnorm, silu_and_mul, situ_and_mul
 from ..workloads import MoEConfig
 
 
@@ -54,7 +53,14 @@ K3_SITU_BETA, K3_SITU_LINEAR_BETA = 4.0, 25.0   # the constants the fused stage-
 
 class Mxfp4MoELayer:
     def __init__(self, cfg: MoEConfig, weights, shared_bf16, bias: torch.Tensor, shared_mode: str = "bf16_add",
-                 latent=None):
+                 latent=None, dense_backend: str = "hip"):
+        """``dense_backend``: "hip" runs the bf16 shared expert and the latent projections on this library's own
+        bf16 GEMM; "vendor" runs them on the vendor library through ``torch.mm``, as ``nn.Linear`` in the reference
+        does.  Either way the results go into buffers owned by the layer: ``forward`` allocates no tensor, and what
+        it returns is one of those buffers, overwritten by the next call."""
+        if dense_backend not in ("hip", "vendor"):
+            raise ValueError(f"dense_backend must be 'hip' or 'vendor', got {dense_backend!r}")
+        self.dense_backend = dense_backend
         self.cfg = cfg
         dev = weights["gate_p"].device
         self.device = dev
@@ -117,6 +123,34 @@ class Mxfp4MoELayer:
         L.activation = ACTIVATIONS[cfg.activation]
         self._L = L
         self._fn = lib().bgmoe_moe_mxfp4_layer_forward
+        # buffers of the dense bf16 parts (shared expert, latent projections): forward() allocates none of them
+        hid = cfg.hidden
+        use_hip = dense_backend == "hip"
+
+        def ws(nn, hh, ee):
+            if not use_hip:
+                return None
+            return torch.empty(max(int(lib().bgmoe_router_gemm_workspace_bytes(nn, hh, ee)), 16), dtype=torch.uint8,
+                               device=dev)
+        d = {}
+        if shared_bf16 is not None:
+            si2 = self._shared_gate_up.size(0)
+            d["gu"] = torch.empty((n, si2), dtype=b2, device=dev)
+            d["hh"] = torch.empty((n, si2 // 2), dtype=b2, device=dev)
+            d["sh"] = torch.empty((n, hid), dtype=b2, device=dev)
+            d["ws_gu"], d["ws_dn"] = ws(n, hid, si2), ws(n, si2 // 2, hid)
+        if latent is not None:
+            d["xlat"] = torch.empty((n, cfg.latent), dtype=b2, device=dev)
+            d["ynorm"] = torch.empty((n, cfg.latent), dtype=b2, device=dev)
+            d["yup"] = torch.empty((n, hid), dtype=b2, device=dev)
+            d["ws_lat_dn"], d["ws_lat_up"] = ws(n, hid, cfg.latent), ws(n, cfg.latent, hid)
+        self._dense = d
+
+    def _linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, workspace) -> torch.Tensor:
+        """``x @ w^T`` into ``out``: this library's bf16 GEMM, or the vendor library's through ``torch.mm``."""
+        if self.dense_backend == "hip":
+            return bf16_linear(x, w, out, workspace)
+        return torch.mm(x, w.t(), out=out)
 
     def forward(self, hidden_states: torch.Tensor, router_logits: torch.Tensor) -> torch.Tensor:
         cfg = self.cfg
@@ -129,26 +163,26 @@ class Mxfp4MoELayer:
         sh = None
         cur = torch.cuda.current_stream(self.device)
         if self.shared is not None:
-            # the dense bf16 shared expert (vendor GEMMs) runs beside the routed experts on a second stream of
+            # the dense bf16 shared expert runs beside the routed experts on a second stream of
             # the same priority: its GEMMs are MFMA-bound, the routed kernels stream weights from HBM
             side = self._side if self.overlap_shared else cur
             if side is not cur:
                 self._fork.record(cur)
                 side.wait_event(self._fork)
             with torch.cuda.stream(side):
-                gu = F.linear(hidden_states, self._shared_gate_up)
-                si = gu.size(1) // 2
+                d = self._dense
+                gu = self._linear(hidden_states, self._shared_gate_up, d["gu"][:n], d["ws_gu"])
                 if cfg.activation == "situ":
-                    hh = situ_and_mul(gu, K3_SITU_BETA, K3_SITU_LINEAR_BETA)
+                    hh = situ_and_mul(gu, K3_SITU_BETA, K3_SITU_LINEAR_BETA, out=d["hh"][:n])
                 else:
-                    hh = F.silu(gu[:, :si]) * gu[:, si:]
-                sh = F.linear(hh, self.shared["down"])
+                    hh = silu_and_mul(gu, out=d["hh"][:n])
+                sh = self._linear(hh, self.shared["down"], d["sh"][:n], d["ws_dn"])
                 if side is not cur:
                     self._join.record(side)
-                    sh.record_stream(cur)
         x_exp = hidden_states
-        if self.latent is not None:
-            x_exp = F.linear(hidden_states, self.latent["down_proj"])      # hidden -> latent, once per token
+        if self.latent is not None:                                        # hidden -> latent, once per token
+            x_exp = self._linear(hidden_states, self.latent["down_proj"], self._dense["xlat"][:n],
+                                 self._dense["ws_lat_dn"])
         L = self._L
         L.n, L.x, L.logits = n, ptr(x_exp), ptr(router_logits)
         # latent: the shared expert's rows are hidden-sized and join after the latent -> hidden projection
@@ -165,13 +199,14 @@ class Mxfp4MoELayer:
         if self.latent is None:
             return self.out[:n]
         y = self.out[:n]
+        d = self._dense
         if self.latent.get("norm_weight") is not None:
-            y = rmsnorm(y, self.latent["norm_weight"], self.latent["eps"])
-        y = F.linear(y, self.latent["up_proj"])                            # latent -> hidden
+            y = rmsnorm(y, self.latent["norm_weight"], self.latent["eps"], out=d["ynorm"][:n])
+        y = self._linear(y, self.latent["up_proj"], d["yup"][:n], d["ws_lat_up"])     # latent -> hidden
         if sh is not None:
             if self.overlap_shared and not joined:
                 cur.wait_event(self._join)
-            y = y + sh
+            y = torch.add(y, sh, out=y)
         return y
 
     __call__ = forward

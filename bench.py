@@ -83,6 +83,9 @@ def parse():
     ap.add_argument("--rows", type=int, default=0, help="--op dense_expert: rows per step (default: the "
                                                         "configuration's token count)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--dense-backend", default=None, choices=["hip", "vendor"],
+                    help="MXFP4 configurations: the bf16 shared expert and latent projections on this library's "
+                         "bf16 GEMM (hip) or on the vendor library through F.linear (vendor); default: the layer's")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of one captured HIP graph of the layer instead of eager launches")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -404,7 +407,8 @@ def measure_layer(a, config, with_cpu):
         from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
         w, sh = wl.make_mxfp4_weights(cfg, dev)
         lat = wl.make_latent_weights(cfg, dev) if cfg.latent else None
-        layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat)
+        kw = {"dense_backend": a.dense_backend} if a.dense_backend else {}
+        layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat, **kw)
     else:
         w, sh = wl.make_fp8_weights(cfg, dev)
         layer = Fp8MoELayer(cfg, w, sh, inp["bias"])

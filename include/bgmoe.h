@@ -108,6 +108,13 @@ int bgmoe_router_gemm(const uint16_t* hidden, const uint16_t* router_weight, int
                       const int64_t* rank_token_counts, int bucket_size, int world_size, float* logits,
                       void* workspace, size_t workspace_bytes, bgmoe_stream_t stream);
 
+/* out[n,e] bf16 = bf16(x[n,h] bf16 x weight[e,h]^T bf16), fp32 accumulation in the router GEMM's fixed order: a
+ * bias-free linear layer on the same kernels (`nn.Linear` of the bf16 shared expert and of the latent projections,
+ * batchgen/moe/fused_moe_mxfp4_resident.py:905-944, kimi_linear/model.py:585-603, which the reference runs on the
+ * vendor GEMM).  workspace: bgmoe_router_gemm_workspace_bytes(n,h,e) (optional, as for bgmoe_router_gemm). */
+int bgmoe_bf16_linear(const uint16_t* x, const uint16_t* weight, int n, int h, int e, uint16_t* out, void* workspace,
+                      size_t workspace_bytes, bgmoe_stream_t stream);
+
 /* Router GEMM + top-k in two launches without materialising the logits: identical ids and weights to
  * bgmoe_router_gemm followed by bgmoe_fused_gate(apply_sigmoid=1) (n_group >= 1) or by
  * bgmoe_gate_sigmoid_topk (n_group == 0; rank_token_counts / rows_per_rank as there).  The reference
@@ -580,6 +587,11 @@ int bgmoe_selfcheck_scale_division(uint64_t seed, uint64_t count, uint64_t* byte
  * x is [rows, 2d] with row stride x_row_stride (elements), out [rows, d] with out_row_stride. */
 int bgmoe_situ_and_mul(const uint16_t* x, int64_t rows, int d, int64_t x_row_stride, float beta,
                        float linear_beta, uint16_t* out, int64_t out_row_stride, bgmoe_stream_t stream);
+
+/* out[r, c] = bf16( bf16(silu(g)) * u ): PyTorch's `F.silu(gate) * up` on bf16 tensors (the SwiGLU of a bf16 shared
+ * expert, batchgen/moe/fused_moe_mxfp4_resident.py:905-944), same layout and strides as above. */
+int bgmoe_silu_and_mul(const uint16_t* x, int64_t rows, int d, int64_t x_row_stride, uint16_t* out,
+                       int64_t out_row_stride, bgmoe_stream_t stream);
 
 /* out[r, :] = bf16( x[r, :] * rsqrt(mean(x[r, :]^2) + eps) * weight ): fp32 math, one rounding.
  * Replaces `triton_rmsnorm` / `cuda_rmsnorm` as used by `KimiRMSNorm.forward`
