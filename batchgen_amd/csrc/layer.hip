@@ -91,13 +91,16 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
   const int groups = el + (folded ? 1 : 0);
   bgmoe_fp8_act ax{L->xq, L->xs, hb, 1};
   const int64_t live_bound = nk + (folded ? n : 0);       // rows that can be live in one pass
+  // Rows one group can have: the router picks distinct experts per token, so at most n; routes handed in from
+  // outside may name one expert several times in a token's row, so only n*k bounds them.
+  const int64_t group_bound = routed ? nk : n;
   rc = bgmoe_internal_fp8_gemm(&ax, &L->gate, &L->up, L->expert_counts, L->cu_seqlens, groups,
-                               folded ? rows : L->cap_rows, inter, h, nullptr, L->hq, L->hs, ib, 1, live_bound, n,
+                               folded ? rows : L->cap_rows, inter, h, nullptr, L->hq, L->hs, ib, 1, live_bound, group_bound,
                                L->gemm_workspace, L->gemm_workspace_bytes, st);
   if (rc != BGMOE_OK) return rc;
   bgmoe_fp8_act ah{L->hq, L->hs, ib, 1};
   rc = bgmoe_internal_fp8_gemm(&ah, &L->down, nullptr, L->expert_counts, L->cu_seqlens, groups,
-                               folded ? rows : L->cap_rows, h, inter, L->y, nullptr, nullptr, 0, 0, live_bound, n,
+                               folded ? rows : L->cap_rows, h, inter, L->y, nullptr, nullptr, 0, 0, live_bound, group_bound,
                                L->gemm_workspace, L->gemm_workspace_bytes, st);
   if (rc != BGMOE_OK) return rc;
   if (shared && !folded) {

@@ -92,7 +92,7 @@ __global__ __launch_bounds__(1024) void perm_scan_kernel(PermArgs a) {
       const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
       tot[e] = cnt;
       a.counts[e] = cnt;
-      if (a.counters) a.counters[e] = cnt;
+      if (a.counters) a.counters[e] = run;       // before clipping: counters[e] > counts[e] = rows were dropped
     }
   }
   __syncthreads();
@@ -142,7 +142,7 @@ __global__ __launch_bounds__(256) void perm_rank_kernel(PermArgs a) {
     if constexpr (SINGLE) {
       const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
       a.counts[e] = cnt;
-      if (a.counters) a.counters[e] = cnt;
+      if (a.counters) a.counters[e] = run;       // before clipping: counters[e] > counts[e] = rows were dropped
       s_cu[e + 1] = cnt;
     }
   }
@@ -242,7 +242,7 @@ __device__ __forceinline__ void perm_small_body(const PermArgs& a, int32_t (*whi
     const int cnt = a.mtp > 0 ? min(run, a.mtp) : run;
     if (global) {
       a.counts[e] = cnt;
-      if (a.counters) a.counters[e] = cnt;
+      if (a.counters) a.counters[e] = run;       // before clipping: counters[e] > counts[e] = rows were dropped
     }
     s_cu[e + 1] = cnt;
   }

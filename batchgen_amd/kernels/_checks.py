@@ -39,4 +39,22 @@ def cuda_tensor(ref, t, dt, name):
         dtype(t, dt, name)
 
 
+def combine_args(expert_output, topk_pos, topk_weights, output, n, h, k, out_dtype):
+    """The weighted combines read ``topk_pos`` / ``topk_weights`` [n*k] and ``expert_output`` [rows, h] and write
+    ``output`` [n, h]: dtype, device, contiguity and minimum sizes, so that no wrong-typed or short tensor is
+    ever handed to the kernel as a raw pointer."""
+    if n < 0 or h <= 0:
+        fail(f"N must be >= 0 and H positive, got N={n} H={h}")
+    cuda_tensor(None, expert_output, torch.bfloat16, "expert_output")
+    cuda_tensor(expert_output, topk_pos, torch.int32, "topk_pos")
+    cuda_tensor(expert_output, topk_weights, torch.float32, "topk_weights")
+    cuda_tensor(expert_output, output, out_dtype, "output")
+    if topk_pos.numel() < n * k or topk_weights.numel() < n * k:
+        fail(f"topk_pos / topk_weights must hold N*K = {n * k} elements")
+    if output.numel() < n * h:
+        fail(f"output must hold N*H = {n * h} elements")
+    if expert_output.numel() % h != 0:
+        fail(f"expert_output must be [rows, {h}]")
+
+
 FP8_BYTES = (torch.uint8, torch.float8_e4m3fn)

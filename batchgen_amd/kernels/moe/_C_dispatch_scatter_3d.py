@@ -16,7 +16,14 @@ def dispatch_scatter_3d(x, topk_indices, act_buffer, expert_start, num_local_exp
     """Masked [E_local, max_tokens_padded, H] layout (dispatch_scatter_3d.cu:88-137).
     Returns [expert_counts, topk_pos]."""
     ck.cuda_tensor(None, x, torch.bfloat16, "x")
+    if x.dim() != 2:
+        ck.fail("x must be BF16 [N, H]")
     n, h = x.shape
+    ck.gpu(topk_indices, "topk_indices")
+    if topk_indices.dim() != 2 or topk_indices.size(0) != n:
+        ck.fail(f"topk_indices must be int32 [N = {n}, K]")
+    if num_local_experts <= 0 or max_tokens_padded <= 0:
+        ck.fail("num_local_experts and max_tokens_padded must be positive")
     k = topk_indices.size(1)
     flat = topk_indices.reshape(-1).contiguous()
     ck.cuda_tensor(x, flat, torch.int32, "topk_indices")
@@ -28,6 +35,8 @@ def dispatch_scatter_3d(x, topk_indices, act_buffer, expert_start, num_local_exp
         ck.cuda_tensor(x, t, torch.int32, name)
     if topk_pos.numel() < n * k:
         ck.fail("topk_pos must have N*K elements")
+    if expert_counts.numel() < num_local_experts or expert_counters.numel() < num_local_experts:
+        ck.fail(f"expert_counts / expert_counters must hold E_local = {num_local_experts} elements")
     ws, ws_bytes = dispatch_workspace(x.device, n * k, num_local_experts)
     with torch.cuda.device(x.device):
         check(lib().bgmoe_dispatch_scatter_3d(ptr(x), ptr(flat), n, k, h, ptr(act_buffer), int(expert_start),
@@ -84,9 +93,10 @@ def reduce_weighted_scatter(expert_output, topk_pos, topk_weights, N, H, K, outp
     """dispatch_scatter_3d.cu:527-556 (K in {2,4,8}; output allocated when empty)."""
     if K not in (2, 4, 8):
         ck.fail(f"Unsupported K={K}")
-    ck.cuda_tensor(None, expert_output, torch.bfloat16, "expert_output")
+    ck.gpu(expert_output, "expert_output")
     if output is None or output.numel() == 0:
         output = torch.zeros((N, H), dtype=torch.bfloat16, device=expert_output.device)
+    ck.combine_args(expert_output, topk_pos, topk_weights, output, int(N), int(H), int(K), torch.bfloat16)
     with torch.cuda.device(expert_output.device):
         check(lib().bgmoe_reduce_weighted_scatter(ptr(expert_output), ptr(topk_pos), ptr(topk_weights), int(N),
                                                   int(H), int(K), ptr(output), -1, None, 0, stream()))

@@ -221,12 +221,10 @@ def reduce_weighted_scatter(expert_output, topk_pos, topk_weights, N, H, K, outp
     """out[t] = bf16(sum_k y[pos]*w), K in {2,4,8} (reduce_weighted_scatter.cu:26-131)."""
     if K not in (2, 4, 8):
         ck.fail(f"Unsupported K={K}")
-    ck.cuda_tensor(None, expert_output, torch.bfloat16, "expert_output")
-    ck.cuda_tensor(expert_output, topk_pos, torch.int32, "topk_pos")
-    ck.cuda_tensor(expert_output, topk_weights, torch.float32, "topk_weights")
+    ck.gpu(expert_output, "expert_output")
     if output is None or output.numel() == 0:
         output = torch.zeros((N, H), dtype=torch.bfloat16, device=expert_output.device)
-    ck.cuda_tensor(expert_output, output, torch.bfloat16, "output")
+    ck.combine_args(expert_output, topk_pos, topk_weights, output, int(N), int(H), int(K), torch.bfloat16)
     with torch.cuda.device(expert_output.device):
         check(lib().bgmoe_reduce_weighted_scatter(ptr(expert_output), ptr(topk_pos), ptr(topk_weights), int(N),
                                                   int(H), int(K), ptr(output), int(num_valid_tokens), None, 0,

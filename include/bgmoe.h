@@ -263,8 +263,10 @@ size_t bgmoe_dispatch_workspace_bytes(int64_t nk, int num_local_experts);
  * row le*mtp + slot, slot = number of earlier pairs (smaller i) of the same
  * expert (deterministic; the reference uses arrival order).  topk_pos[i] = row
  * or -1.  Pairs with slot >= mtp are dropped (-1) and counts are clipped.
- * expert_counters is written with the counts too.  act_buffer may be NULL to
- * compute indices only. */
+ * expert_counters[e] is written with the number of pairs routed to expert e
+ * BEFORE clipping (what the reference's atomic counter holds at the end):
+ * expert_counters[e] > expert_counts[e] tells the caller that rows of expert e
+ * were dropped.  act_buffer may be NULL to compute indices only. */
 int bgmoe_dispatch_scatter_3d(const uint16_t* x, const int32_t* topk_ids, int n, int k, int h,
                               uint16_t* act_buffer, int expert_start, int num_local_experts,
                               int max_tokens_padded, int32_t* expert_counts,
