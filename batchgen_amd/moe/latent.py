@@ -41,6 +41,15 @@ def bf16_linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tenso
     return out
 
 
+def bf16_linear_workspace_bytes(n_max: int, h: int, e: int) -> int:
+    """Bytes of workspace that serve ``bf16_linear`` for every row count up to ``n_max``: the launch shape depends
+    on the row count (few rows: fp32 partial planes per 512-wide K segment, never more than 64 MiB of them; many
+    rows: no planes), so the need is not monotonic in it and a layer sizes its buffer once with this bound."""
+    nseg = (h + 511) // 512
+    one = n_max * e * 4
+    return max(16, one, min(nseg * one, 64 << 20))
+
+
 def silu_and_mul(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``bf16(bf16(silu(x[:, :d])) * x[:, d:])``: ``F.silu(gate) * up`` on a bf16 ``[rows, 2d]`` tensor."""
     rows, d2 = x.shape

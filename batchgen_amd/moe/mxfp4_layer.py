@@ -25,7 +25,7 @@ import torch
 from .. import _lib
 from .._lib import Mxfp4Weight, check, lib, ptr, stream
 from ..kernels import load_extension
-from .latent import bf16_linear, rmsnorm, silu_and_mul, situ_and_mul
+from .latent import bf16_linear, bf16_linear_workspace_bytes, rmsnorm, silu_and_mul, situ_and_mul
 from ..workloads import MoEConfig
 
 
@@ -51,15 +51,23 @@ ACTIVATIONS = {"swiglu": 0, "situ": 1}
 K3_SITU_BETA, K3_SITU_LINEAR_BETA = 4.0, 25.0   # the constants the fused stage-1 epilogue compiles in
 
 
+# dense_backend="auto": rows up to which the library's bf16 GEMM serves the shared expert and the latent projections.
+# Measured on MI355X against the vendor GEMM: 64 rows 7168 -> 4096 24.5 vs 20.3 us and 2048 -> 7168 14.2 vs 22.1 us
+# (the pair 38.7 vs 42.4 us); 512 rows 85 vs 44 us and 50 vs 22 us.
+DENSE_HIP_MAX_ROWS = 64
+
+
 class Mxfp4MoELayer:
     def __init__(self, cfg: MoEConfig, weights, shared_bf16, bias: torch.Tensor, shared_mode: str = "bf16_add",
-                 latent=None, dense_backend: str = "hip"):
+                 latent=None, dense_backend: str = "auto"):
         """``dense_backend``: "hip" runs the bf16 shared expert and the latent projections on this library's own
         bf16 GEMM; "vendor" runs them on the vendor library through ``torch.mm``, as ``nn.Linear`` in the reference
-        does.  Either way the results go into buffers owned by the layer: ``forward`` allocates no tensor, and what
-        it returns is one of those buffers, overwritten by the next call."""
-        if dense_backend not in ("hip", "vendor"):
-            raise ValueError(f"dense_backend must be 'hip' or 'vendor', got {dense_backend!r}")
+        does; "auto" (the default) takes this library's GEMM for calls of up to ``DENSE_HIP_MAX_ROWS`` tokens,
+        where it was measured to be the faster one, and the vendor's above.  Either way the results go into
+        buffers owned by the layer: ``forward`` allocates no tensor, and what it returns is one of those buffers,
+        overwritten by the next call."""
+        if dense_backend not in ("auto", "hip", "vendor"):
+            raise ValueError(f"dense_backend must be 'auto', 'hip' or 'vendor', got {dense_backend!r}")
         self.dense_backend = dense_backend
         self.cfg = cfg
         dev = weights["gate_p"].device
@@ -125,13 +133,14 @@ class Mxfp4MoELayer:
         self._fn = lib().bgmoe_moe_mxfp4_layer_forward
         # buffers of the dense bf16 parts (shared expert, latent projections): forward() allocates none of them
         hid = cfg.hidden
-        use_hip = dense_backend == "hip"
+        use_hip = dense_backend != "vendor"
+
+        rows_hip = n if dense_backend == "hip" else min(n, DENSE_HIP_MAX_ROWS)
 
         def ws(nn, hh, ee):
             if not use_hip:
                 return None
-            return torch.empty(max(int(lib().bgmoe_router_gemm_workspace_bytes(nn, hh, ee)), 16), dtype=torch.uint8,
-                               device=dev)
+            return torch.empty(bf16_linear_workspace_bytes(rows_hip, hh, ee), dtype=torch.uint8, device=dev)
         d = {}
         if shared_bf16 is not None:
             si2 = self._shared_gate_up.size(0)
@@ -148,7 +157,7 @@ class Mxfp4MoELayer:
 
     def _linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, workspace) -> torch.Tensor:
         """``x @ w^T`` into ``out``: this library's bf16 GEMM, or the vendor library's through ``torch.mm``."""
-        if self.dense_backend == "hip":
+        if self.dense_backend == "hip" or (self.dense_backend == "auto" and x.size(0) <= DENSE_HIP_MAX_ROWS):
             return bf16_linear(x, w, out, workspace)
         return torch.mm(x, w.t(), out=out)
 

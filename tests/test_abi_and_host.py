@@ -194,3 +194,14 @@ def test_config4_routing_has_the_skew_the_baseline_names():
     assert 0.2 <= empty <= 0.4, empty
     assert counts.max() > 2000
     assert counts.sum() == cfg.n_tokens * cfg.top_k
+
+
+def test_bf16_linear_workspace_bound_covers_every_row_count():
+    """The layer sizes its GEMM workspace once: the bound must cover what the library asks for at every row count
+    up to the maximum (the launch shape, and with it the need, is not monotonic in the rows)."""
+    from batchgen_amd._lib import lib
+    from batchgen_amd.moe.latent import bf16_linear_workspace_bytes
+    for n_max, h, e in [(512, 7168, 4096), (512, 2048, 7168), (96, 1024, 1024), (64, 7168, 4096), (300, 3584, 7168)]:
+        bound = bf16_linear_workspace_bytes(n_max, h, e)
+        for n in range(1, n_max + 1):
+            assert lib().bgmoe_router_gemm_workspace_bytes(n, h, e) <= bound, (n_max, h, e, n)
