@@ -92,7 +92,10 @@ class Fp8MoELayer:
 
     def __init__(self, cfg: MoEConfig, weights, shared, bias: torch.Tensor, max_tokens_in: Optional[int] = None,
                  shared_mode: str = "bf16_add", fold_shared: bool = True, weight_layout: str = "tile_major",
-                 router_weight: Optional[torch.Tensor] = None, balanced_gemm: bool = False):
+                 router_weight: Optional[torch.Tensor] = None, balanced_gemm: bool = False,
+                 weights_repacked: bool = False):
+        """``weights_repacked``: the ``*_q`` tensors already hold the tile-major bytes (``repack_tile_major``), e.g.
+        because two layers share one resident copy; the layer then takes them as they are."""
         self.cfg = cfg
         dev = weights["gate_q"].device
         with torch.cuda.device(dev):
@@ -100,7 +103,9 @@ class Fp8MoELayer:
         if weight_layout not in ("tile_major", "row_major"):
             raise ValueError(f"unknown weight_layout {weight_layout!r}")
         self.layout = W_TILE_MAJOR if weight_layout == "tile_major" else W_ROW_MAJOR
-        if self.layout == W_TILE_MAJOR:
+        if weights_repacked and self.layout != W_TILE_MAJOR:
+            raise ValueError("weights_repacked needs weight_layout='tile_major'")
+        if self.layout == W_TILE_MAJOR and not weights_repacked:
             # resident copy in the streaming layout; the caller may drop the row-major tensors
             weights = dict(weights)
             shared = dict(shared) if shared is not None else None

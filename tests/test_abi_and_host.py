@@ -205,3 +205,27 @@ def test_bf16_linear_workspace_bound_covers_every_row_count():
         bound = bf16_linear_workspace_bytes(n_max, h, e)
         for n in range(1, n_max + 1):
             assert lib().bgmoe_router_gemm_workspace_bytes(n, h, e) <= bound, (n_max, h, e, n)
+
+
+def test_moe_base_template_names_and_config_mapping():
+    """The template class carries the reference's names (batchgen/moe/moe_base.py:75-264) and maps a model
+    configuration object to this package's workload description; a world of more than one rank is refused."""
+    from types import SimpleNamespace
+    from batchgen_amd.moe import moe_base as mb
+    for name in ("gate", "expert_compute_persistent", "expert_compute_mixed", "shared_expert_forward", "forward",
+                 "_forward_decode", "_forward_prefill", "init_buffer_manager", "init_num_tokens",
+                 "set_num_tokens_per_rank"):
+        assert callable(getattr(mb.MoEBase, name)), name
+    cfg = SimpleNamespace(hidden_size=7168, moe_intermediate_size=2048, n_routed_experts=256, num_experts_per_tok=8,
+                          n_group=8, topk_group=4, routed_scaling_factor=2.5, norm_topk_prob=True, n_shared_experts=1)
+    base = mb.MoEBase(cfg)
+    assert (base.rank, base.world_size, base.experts_per_rank, base.routed_expert_end_idx) == (0, 1, 256, 256)
+    assert base.num_persistent_local_experts == 256 and base.enable_ep_offloading is False
+    with pytest.raises(NotImplementedError):
+        base.gate(None)
+    m = mb._moe_config(cfg, 256, 32, 64, True)
+    assert (m.hidden, m.inter, m.n_experts, m.e_local, m.expert_start, m.top_k, m.n_group, m.topk_group) == \
+        (7168, 2048, 256, 32, 64, 8, 8, 4)
+    assert (m.layout, m.max_tokens, m.shared_inter, m.rsf) == ("masked", 256, 2048, 2.5)
+    big = mb._moe_config(cfg, 16384, 256, 0, False)
+    assert (big.layout, big.row_align, big.shared_inter) == ("ragged", 128, 0)
