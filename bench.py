@@ -63,7 +63,9 @@ def traffic_record(key):
                 except OSError:
                     got = None
                 if got != want:
-                    return None, f"{os.path.basename(path)}: {rel} changed since the measurement (commit {rec.get('commit')})"
+                    then = (int(rec["fetch_bytes"]) + int(rec["write_bytes"])) / 1e6
+                    return None, (f"{os.path.basename(path)}: {rel} changed since the measurement (commit "
+                                  f"{rec.get('commit')}, which read {then:.1f} MB per launch)")
             return int(rec["fetch_bytes"]) + int(rec["write_bytes"]), f"{os.path.basename(path)} (commit {rec.get('commit')})"
     return None, "no record under profiles/"
 
