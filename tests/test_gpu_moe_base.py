@@ -52,7 +52,7 @@ def test_template_layer_against_fused_layer_and_oracle(dev, n_group):
     fused = layer.forward_fused(xd).clone()
     assert torch.equal(layer._fused.topk_ids[:48], ids), "the fused call routes like gate()"
     a, b = out.float().cpu(), fused.float().cpu()
-    assert float((a - b).norm() / b.norm()) < 5e-3        # the shared expert's sums take another K order
+    assert float((a - b).norm() / b.norm()) < 8e-3        # the shared expert's sums take another K order
     ref = ol.moe_layer_fp8(x, None, None, None, wl.weights_to_numpy(w), 0, 16, layout="masked", max_tokens=64,
                            shared=wl.weights_to_numpy(sh), routes=(ids.cpu().numpy(), wts.cpu().numpy()))
     assert og.rel_frobenius(a.numpy(), ref["out"]) < 1e-2
