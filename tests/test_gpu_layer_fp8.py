@@ -319,33 +319,3 @@ def test_layer_with_given_routes(dev):
     assert torch.equal(layer(x, inp["logits"].to(dev)), out)          # the routed call leaves the layer as it was
     with pytest.raises(RuntimeError):
         layer.forward_routed(x, rid[:, :2].to(dev), rw[:, :2].to(dev))
-
-
-def test_given_routes_may_repeat_an_expert(dev):
-    """Routes from outside may name one expert several times in a token's row: a group can then hold more rows
-    than there are tokens (here 4 x 96 = 384 rows of one expert, more than the streaming kernel's 256-row limit),
-    and every row must still be computed: against the oracle on the same routes."""
-    from batchgen_amd import workloads as wl
-    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
-    from oracle import gemm as og
-    from oracle import layer as ol
-    cfg = wl.scaled(wl.CONFIGS[0], n_tokens=96, hidden=512, inter=256, shared_inter=256, n_experts=32, e_local=8,
-                    expert_start=8, n_group=4, topk_group=2, top_k=4, max_tokens=0, layout="ragged", row_align=64)
-    say("given routes with repeats", cfg.name)
-    inp = wl.make_inputs(cfg, "cpu")
-    w, sh = wl.make_fp8_weights(cfg, "cpu")
-    layer = Fp8MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
-                        inp["bias"].to(dev))
-    x = inp["x"].to(dev)
-    layer(x, inp["logits"].to(dev))                                   # leaves other values in the row buffers
-    rid = torch.full((cfg.n_tokens, cfg.top_k), 9, dtype=torch.int32)
-    rid[7, 2] = 11
-    rw = torch.rand(cfg.n_tokens, cfg.top_k, generator=torch.Generator().manual_seed(9)) + 0.25
-    got = layer.forward_routed(x, rid.to(dev), rw.to(dev)).float().cpu().numpy()
-    ref = ol.moe_layer_fp8(inp["x"], None, None, None, wl.weights_to_numpy(w), cfg.expert_start, cfg.e_local,
-                           layout=cfg.layout, max_tokens=cfg.max_tokens, row_align=cfg.row_align, shared=wl.weights_to_numpy(sh),
-                           routes=(rid.numpy(), rw.numpy()))
-    assert np.array_equal(layer.expert_counts[:cfg.e_local].cpu().numpy(), ref["counts"])
-    assert int(ref["counts"].max()) == 383
-    assert np.array_equal(layer.topk_pos.cpu().numpy(), ref["pos"])
-    assert og.rel_frobenius(got, ref["out"]) < 1e-2

@@ -269,37 +269,3 @@ def sum_k(res3, w):
         x = res3[:, j].float().numpy()
         acc = fma_f32(x, np.broadcast_to(w[:, j:j + 1].numpy(), x.shape), acc)
     return acc
-
-
-@pytest.mark.parametrize("mod", ["ds3d", "routing"])
-def test_combine_and_dispatch_reject_wrong_arguments(dev, mod):
-    """Wrong dtypes and short tensors raise before anything is launched (no raw pointer of the wrong type or
-    size reaches the kernel)."""
-    from batchgen_amd.kernels import load_extension
-    m = ds3d() if mod == "ds3d" else load_extension("batchgen_kernels.moe._C_routing")
-    n, k, h = 8, 4, 256
-    y = torch.zeros((n * k, h), dtype=torch.bfloat16, device=dev)
-    pos = torch.arange(n * k, dtype=torch.int32, device=dev)
-    w = torch.ones((n, k), dtype=torch.float32, device=dev)
-    out = torch.zeros((n, h), dtype=torch.bfloat16, device=dev)
-    m.reduce_weighted_scatter(y, pos, w, n, h, k, out)                                    # the good call
-    for bad in (dict(w=w.bfloat16()), dict(pos=pos.long()), dict(pos=pos[:-1]), dict(w=w[:, :-1].contiguous()),
-                dict(out=out[:-1]), dict(out=out.float()), dict(w=w.cpu()), dict(y=y.float())):
-        a = dict(y=y, pos=pos, w=w, out=out)
-        a.update(bad)
-        with pytest.raises(RuntimeError):
-            m.reduce_weighted_scatter(a["y"], a["pos"], a["w"], n, h, k, a["out"])
-    if mod == "ds3d":
-        x = torch.zeros((n, h), dtype=torch.bfloat16, device=dev)
-        ids = torch.zeros((n, k), dtype=torch.int32, device=dev)
-        act = torch.zeros((2 * 16, h), dtype=torch.bfloat16, device=dev)
-        cnt = torch.zeros(2, dtype=torch.int32, device=dev)
-        ctr = torch.zeros(2, dtype=torch.int32, device=dev)
-        tp = torch.zeros(n * k, dtype=torch.int32, device=dev)
-        m.dispatch_scatter_3d(x, ids, act, 0, 2, 16, cnt, ctr, tp)                        # the good call
-        for bad in (dict(cnt=cnt[:1]), dict(ctr=ctr[:1]), dict(tp=tp[:-1]), dict(ids=ids[:-1]), dict(ids=ids.view(-1)),
-                    dict(act=act[:-1])):
-            a = dict(ids=ids, act=act, cnt=cnt, ctr=ctr, tp=tp)
-            a.update(bad)
-            with pytest.raises(RuntimeError):
-                m.dispatch_scatter_3d(x, a["ids"], a["act"], 0, 2, 16, a["cnt"], a["ctr"], a["tp"])
