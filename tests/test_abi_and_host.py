@@ -229,3 +229,31 @@ def test_moe_base_template_names_and_config_mapping():
     assert (m.layout, m.max_tokens, m.shared_inter, m.rsf) == ("masked", 256, 2048, 2.5)
     big = mb._moe_config(cfg, 16384, 256, 0, False)
     assert (big.layout, big.row_align, big.shared_inter) == ("ragged", 128, 0)
+
+
+def test_bench_accounting_and_traffic_records(tmp_path, monkeypatch):
+    """The figures bench.py divides by the measured times: algorithmic bytes and flops of config 1 worked out by
+    hand for a given routing draw (19 active experts, 297 routed rows), and the rule for `roofline.traffic`: a
+    record under profiles/ counts only while every kernel source it names still has the recorded SHA-256."""
+    import hashlib
+    import json
+    import bench
+    from batchgen_amd import workloads as wl
+    cfg = wl.CONFIGS[1]
+    weights = 3 * 7168 * 2048 + 3 * 56 * 16 * 4                    # gate, up, down bytes + their 128x128 block scales
+    by_hand = 19 * weights + weights + 256 * 7168 * 2 * 2 + 297 * (7168 + 2048) * 3
+    assert wl.algorithmic_bytes_fp8(cfg, 19, 297) == by_hand == 896570368
+    assert wl.flops_routed(cfg, 297) == 297 * 6 * 7168 * 2048
+    src = tmp_path / "kernel.hip"
+    src.write_text("v1")
+    (tmp_path / "profiles").mkdir()
+    rec = dict(key="layer:1", fetch_bytes=1000, write_bytes=24, commit="abc1234",
+               sources={"kernel.hip": hashlib.sha256(b"v1").hexdigest()})
+    (tmp_path / "profiles" / "p.md").write_text(f"text\n<!-- traffic-record: {json.dumps(rec)} -->\n")
+    monkeypatch.setattr(bench, "ROOT", str(tmp_path))
+    got, where = bench.traffic_record("layer:1")
+    assert got == 1024 and "abc1234" in where
+    assert bench.traffic_record("layer:2") == (None, "no record under profiles/")
+    src.write_text("v2")
+    got, where = bench.traffic_record("layer:1")
+    assert got is None and "kernel.hip changed" in where and "abc1234" in where
