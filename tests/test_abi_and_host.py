@@ -10,6 +10,7 @@ import subprocess
 import sys
 
 import pytest
+import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "bgmoe.h")
@@ -257,3 +258,53 @@ def test_bench_accounting_and_traffic_records(tmp_path, monkeypatch):
     src.write_text("v2")
     got, where = bench.traffic_record("layer:1")
     assert got is None and "kernel.hip changed" in where and "abc1234" in where
+
+
+def test_moe_base_decode_template_on_a_toy_layer():
+    """The template's own steps (pad to the announced capacity, gate, expert compute on the padded rows, live rows
+    + shared expert, shapes, the shared buffer manager, the overflow error) with a layer whose pieces are plain
+    tensor arithmetic, on the CPU."""
+    from types import SimpleNamespace
+    from batchgen_amd.moe import moe_base as mb
+    seen = {}
+
+    class Toy(mb.MoEBase):
+        def gate(self, x):
+            seen["gate_rows"] = x.shape[0]
+            seen["pad_is_zero"] = bool((x[5:] == 0).all())
+            return torch.zeros(x.shape[0], 2, dtype=torch.int32), torch.ones(x.shape[0], 2)
+
+        def expert_compute_persistent(self, global_x, topk_idx, topk_weight):
+            return global_x * topk_weight.sum(dim=1, keepdim=True).to(global_x.dtype)     # 2 x
+
+        def shared_expert_forward(self, identity):
+            return identity * 3
+
+    cfg = SimpleNamespace(hidden_size=16, num_experts_per_tok=2, n_routed_experts=4, phase="decode")
+    layer = Toy(cfg)
+    x = torch.randn(5, 16).to(torch.bfloat16)
+    with pytest.raises(RuntimeError):
+        layer(x)                                                       # capacity not announced
+    layer.init_num_tokens(8)
+    out = layer(x)
+    assert seen == {"gate_rows": 8, "pad_is_zero": True}
+    assert torch.equal(out, x * 2 + x * 3) and out.dtype == torch.bfloat16
+    assert layer(x.view(1, 5, 16)).shape == (1, 5, 16)
+    with pytest.raises(RuntimeError, match="buffer overflow"):
+        layer(torch.zeros(9, 16, dtype=torch.bfloat16))
+    Toy.init_buffer_manager(8, 1, 16, torch.device("cpu"))
+    try:
+        assert mb.MoEBase._buffer_mgr is None, "the manager belongs to the class it was set on"
+        Toy._buffer_mgr.all_tokens.fill_(7.0)                          # stale rows of an earlier call
+        assert torch.equal(layer(x), out) and seen["pad_is_zero"]
+        layer.set_num_tokens_per_rank(12)
+        assert Toy._buffer_mgr.num_tokens_per_rank == 12 and Toy._buffer_mgr.all_tokens.shape == (12, 16)
+        assert torch.equal(layer(x), out) and seen["gate_rows"] == 12
+    finally:
+        Toy._buffer_mgr = None
+    layer.enable_ep_offloading = True
+    with pytest.raises(NotImplementedError):
+        layer(x)                                                       # the toy has no mixed path
+    cfg.phase = "prefill"
+    with pytest.raises(NotImplementedError):
+        layer(x)
