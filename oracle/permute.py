@@ -45,6 +45,19 @@ def dispatch_masked(topk_ids, expert_start: int, num_local: int, max_tokens: int
     return np.minimum(counts, max_tokens).astype(np.int32), pos
 
 
+def dispatch_masked_arrivals(topk_ids, expert_start: int, num_local: int, max_tokens: int):
+    """``dispatch_masked`` plus what the scatter kernel's atomic slot counter holds when it has run
+    (dispatch_scatter_3d.cu:66: every local pair bumps ``expert_counters[e]``, also the pairs beyond
+    ``max_tokens``): the arrivals per expert before clipping.  ``arrivals[e] > counts[e]`` is the only
+    sign a caller gets that rows of expert e were dropped.
+
+    Returns (expert_counts, topk_pos, arrivals int32 [E_l]).
+    """
+    counts, pos = dispatch_masked(topk_ids, expert_start, num_local, max_tokens)
+    _, _, arrivals, _ = _stable_ranks(topk_ids, expert_start, num_local)
+    return counts, pos, arrivals.astype(np.int32)
+
+
 def dispatch_ragged(topk_ids, expert_start: int, num_local: int, row_align: int = 1):
     """``dispatch_scatter_ragged`` index part (dispatch_scatter_3d.cu:152-358)
     and, with row_align=1, the tight forms ``dispatch_count_gather`` /

@@ -70,16 +70,18 @@ def test_full_size_layer_properties(dev, idx):
     assert err < 1e-2
 
 
-def test_full_size_mxfp4_layer_properties(dev):
-    """Config 3 (MXFP4 weights, bf16 activations) at full size: determinism, and a sample of tokens against
-    the oracle.  (No token-order check: the bf16 shared expert of this layer runs on the vendor GEMM library,
-    whose row results are not promised to be independent of the row's position.)"""
+@pytest.mark.parametrize("backend", ["hip", "vendor"])
+def test_full_size_mxfp4_layer_properties(dev, backend):
+    """Config 3 (MXFP4 weights, bf16 activations) at full size: determinism, a sample of tokens against the
+    oracle and, with the bf16 shared expert on this library's own GEMM ("hip": a row's sums are a fixed chain
+    over K whatever the row's position), token-order equivariance bit for bit.  The vendor GEMM library does
+    not promise position-independent rows, so "vendor" is not held to that."""
     from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
     cfg = wl.CONFIGS[3]
-    say("full size", cfg.name)
+    say("full size", cfg.name, backend)
     inp = wl.make_inputs(cfg, dev)
     w, sh = wl.make_mxfp4_weights(cfg, dev)
-    layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"])
+    layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], dense_backend=backend)
     x, logits = inp["x"], inp["logits"]
     n = cfg.n_tokens
     out = layer(x, logits).clone()
@@ -87,6 +89,12 @@ def test_full_size_mxfp4_layer_properties(dev):
     counts = layer.expert_counts[:cfg.e_local].cpu().numpy()
     assert torch.isfinite(out.float()).all()
     assert torch.equal(out, layer(x, logits))
+    if backend == "hip":
+        perm = torch.randperm(n, generator=torch.Generator().manual_seed(1237)).to(dev)
+        outp = layer(x[perm].contiguous(), logits[perm].contiguous())
+        assert torch.equal(layer.topk_ids, ids[perm]), "router result depends on the token's position"
+        assert torch.equal(outp, out[perm]), "a token's output depends on where it sits in the batch"
+        assert np.array_equal(layer.expert_counts[:cfg.e_local].cpu().numpy(), counts)
     fullest = int(np.argmax(counts)) + cfg.expert_start
     hit = torch.nonzero((ids == fullest).any(dim=1)).flatten().cpu().numpy()
     sample = sorted(set([0, n - 1] + hit[:2].tolist()))

@@ -54,20 +54,6 @@ def test_dispatch_masked(dev, n, k, h, et, es, el):
     assert np.array_equal(act.view(torch.int16).cpu().numpy(), ref)
 
 
-def test_dispatch_masked_overflow_rows_are_dropped(dev):
-    ids = torch.zeros((10, 2), dtype=torch.int32)
-    ids[:, 1] = 1
-    x = torch.ones((10, 64), dtype=torch.bfloat16)
-    act = torch.zeros((2 * 4, 64), dtype=torch.bfloat16, device=dev)
-    counts = torch.empty(2, dtype=torch.int32, device=dev)
-    counters = torch.empty(2, dtype=torch.int32, device=dev)
-    pos = torch.empty(20, dtype=torch.int32, device=dev)
-    ds3d().dispatch_scatter_3d(x.to(dev), ids.to(dev), act, 0, 2, 4, counts, counters, pos)
-    co, po = op_.dispatch_masked(ids.numpy(), 0, 2, 4)
-    assert counts.tolist() == [4, 4] and np.array_equal(pos.cpu().numpy(), po)
-    assert counters.tolist() == [10, 10], "expert_counters holds the arrivals before clipping (the overflow signal)"
-
-
 @pytest.mark.parametrize("row_align", [1, 64, 128])
 @pytest.mark.parametrize("n,k,h,et,es,el", CASES)
 def test_dispatch_ragged(dev, n, k, h, et, es, el, row_align):

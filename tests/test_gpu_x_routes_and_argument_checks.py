@@ -44,6 +44,33 @@ def test_given_routes_may_repeat_an_expert(dev):
     assert og.rel_frobenius(got, ref["out"]) < 1e-2
 
 
+@pytest.mark.parametrize("n,k,et,es,el,mtp", [(10, 2, 2, 0, 2, 4), (300, 8, 64, 8, 16, 7), (2000, 8, 64, 0, 64, 100),
+                                              (40, 4, 600, 100, 300, 1)])
+def test_dispatch_masked_overflow_rows_are_dropped(dev, n, k, et, es, el, mtp):
+    """More arrivals than max_tokens_padded: the extra pairs get pos -1, the count is clipped and
+    expert_counters holds the arrivals before clipping (the overflow signal), all as the oracle says; the three
+    sizes take the one-block, the multi-chunk and the four-wave index kernels."""
+    from oracle import permute as op_
+    say("dispatch_3d overflow", n, k, et, es, el, mtp)
+    g = torch.Generator().manual_seed(n + mtp)
+    ids = torch.randint(0, et, (n, k), generator=g).to(torch.int32)
+    if n == 10:
+        ids[:, 0], ids[:, 1] = 0, 1
+    x = torch.randn((n, 64), generator=g).to(torch.bfloat16)
+    act = torch.zeros((el * mtp, 64), dtype=torch.bfloat16, device=dev)
+    counts = torch.full((el,), -3, dtype=torch.int32, device=dev)
+    counters = torch.full((el,), -3, dtype=torch.int32, device=dev)
+    pos = torch.full((n * k,), -9, dtype=torch.int32, device=dev)
+    ds3d().dispatch_scatter_3d(x.to(dev), ids.to(dev), act, es, el, mtp, counts, counters, pos)
+    co, po, arrivals = op_.dispatch_masked_arrivals(ids.numpy(), es, el, mtp)
+    assert int(arrivals.max()) > mtp, "the case must overflow"
+    assert np.array_equal(counts.cpu().numpy(), co)
+    assert np.array_equal(pos.cpu().numpy(), po)
+    assert np.array_equal(counters.cpu().numpy(), arrivals)
+    ref = op_.gather_rows(x.view(torch.int16).numpy(), po, k, el * mtp)
+    assert np.array_equal(act.view(torch.int16).cpu().numpy(), ref)
+
+
 @pytest.mark.parametrize("mod", ["ds3d", "routing"])
 def test_combine_and_dispatch_reject_wrong_arguments(dev, mod):
     """Wrong dtypes and short tensors raise before anything is launched (no raw pointer of the wrong type or

@@ -41,6 +41,30 @@ def test_masked_dispatch_drops_overflow():
     assert c.tolist() == [4, 0] and pos.tolist() == [0, 1, 2, 3] + [-1] * 6
 
 
+def test_masked_arrivals_equal_the_sequential_running_counter():
+    """Arrivals before clipping = the final value of the per-expert running counter of the sequential loop
+    (every local pair counts, kept or dropped); counts = the same clipped; a dropped pair has pos -1 and the
+    kept pairs of an expert are exactly its first max_tokens arrivals in (token, k) order."""
+    rng = np.random.default_rng(7)
+    for n, k, et, es, el, mtp in [(10, 2, 2, 0, 2, 4), (40, 4, 16, 4, 8, 3), (64, 8, 32, 0, 32, 1), (9, 3, 8, 2, 4, 100)]:
+        ids = rng.integers(es - 2, es + el + 2, size=(n, k)).astype(np.int32)       # repeats and non-local ids
+        counts, pos, arrivals = op_.dispatch_masked_arrivals(ids, es, el, mtp)
+        ctr = np.zeros(el, dtype=np.int64)
+        for i, eid in enumerate(ids.reshape(-1)):
+            le = int(eid) - es
+            if 0 <= le < el:
+                want = le * mtp + ctr[le] if ctr[le] < mtp else -1
+                assert pos[i] == want
+                ctr[le] += 1
+            else:
+                assert pos[i] == -1
+        assert np.array_equal(arrivals, ctr) and np.array_equal(counts, np.minimum(ctr, mtp))
+    ids = np.zeros((10, 2), dtype=np.int32)
+    ids[:, 1] = 1
+    counts, pos, arrivals = op_.dispatch_masked_arrivals(ids, 0, 2, 4)
+    assert counts.tolist() == [4, 4] and arrivals.tolist() == [10, 10]
+
+
 def test_gather_rows_places_tokens():
     rng = np.random.default_rng(1)
     ids = _ids(rng, 20, 4, 16)
