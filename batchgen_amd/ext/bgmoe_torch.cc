@@ -163,6 +163,8 @@ std::vector<Tensor> dispatch_count_gather(Tensor x, Tensor ids, int64_t expert_s
   const int64_t n = x.size(0), h = x.size(1), k = ids.size(1);
   TORCH_CHECK(counts.numel() >= el && counters.numel() >= el && offsets.numel() >= el + 1 && pos.numel() >= n * k,
               "expert_counts / expert_counters [E], expert_offsets [E+1] or topk_pos [N*K] too small");
+  TORCH_CHECK(dispatched.dim() == 2 && dispatched.size(1) == h, "dispatched_x must be BF16 [rows, H=", h, "]");
+  for (auto* t : {&ids, &counts, &offsets, &counters, &dispatched, &pos}) same_device(x, *t, "every tensor");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
   Tensor ws = dispatch_ws(x.device(), n * k, (int)el);
   check_rc(bgmoe_dispatch_scatter_ragged(ptr<uint16_t>(x), ptr<int32_t>(ids), (int)n, (int)k, (int)h, ptr<uint16_t>(dispatched),
@@ -179,7 +181,11 @@ Tensor combine(Tensor y, Tensor pos, Tensor w, int64_t N, int64_t H, int64_t K, 
   want(w, "topk_weights", at::kFloat);
   if (!out.defined() || out.numel() == 0) out = torch::zeros({N, H}, y.options());
   want(out, "output", at::kBFloat16);
+  TORCH_CHECK(N >= 0 && H > 0, "N must be non-negative and H positive");
+  // [rows, H] or the masked buffer [E_local, max_tokens, H]: topk_pos indexes rows of H elements either way
+  TORCH_CHECK(y.dim() >= 2 && y.size(-1) == H, "expert_output must have rows of H=", H, " elements");
   TORCH_CHECK(pos.numel() >= N * K && w.numel() >= N * K && out.numel() >= N * H, "topk_pos / topk_weights / output too small");
+  for (auto* t : {&pos, &w, &out}) same_device(y, *t, "topk_pos / topk_weights / output");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(y.device());
   check_rc(bgmoe_reduce_weighted_scatter(ptr<uint16_t>(y), ptr<int32_t>(pos), ptr<float>(w), (int)N, (int)H, (int)K,
                                          ptr<uint16_t>(out), (int)num_valid, nullptr, 0, cur_stream()));
@@ -243,6 +249,8 @@ std::vector<Tensor> fused_moe_token_dispatch(Tensor x, Tensor ids, Tensor token_
   TORCH_CHECK(ids.is_contiguous(), "topk_idx must be contiguous");
   TORCH_CHECK(x.scalar_type() == at::kBFloat16, "global_x must be BF16");
   TORCH_CHECK(end > start, "routed_expert_end_idx must exceed routed_expert_start_idx");
+  TORCH_CHECK(x.dim() == 2 && ids.dim() == 2 && ids.size(0) == x.size(0), "global_x [N, H] and topk_idx [N, K] must agree in N");
+  same_device(x, ids, "topk_idx");
   const int64_t n = x.size(0), h = x.size(1), k = ids.size(1), el = end - start, nk = n * k;
   Tensor ids32 = ids.to(at::kInt).contiguous();
   auto iopt = ids32.options();
@@ -266,6 +274,7 @@ std::vector<Tensor> dispatch_scatter_3d(Tensor x, Tensor ids, Tensor act, int64_
                                         Tensor counts, Tensor counters, Tensor pos) {
   want(x, "x", at::kBFloat16);
   TORCH_CHECK(x.dim() == 2 && ids.dim() == 2, "x must be [N, H] and topk_indices [N, K]");
+  TORCH_CHECK(ids.size(0) == x.size(0), "topk_indices has ", ids.size(0), " rows, x has ", x.size(0));
   const int64_t n = x.size(0), h = x.size(1), k = ids.size(1);
   Tensor flat = ids.reshape({-1}).contiguous();
   want(flat, "topk_indices", at::kInt);
@@ -274,6 +283,7 @@ std::vector<Tensor> dispatch_scatter_3d(Tensor x, Tensor ids, Tensor act, int64_
   for (auto* t : {&counts, &counters, &pos}) want(*t, "index tensor", at::kInt);
   TORCH_CHECK(counts.numel() >= el && counters.numel() >= el, "expert_counts / expert_counters must have E_local elements");
   TORCH_CHECK(pos.numel() >= n * k, "topk_pos must have N*K elements");
+  for (auto* t : {&flat, &act, &counts, &counters, &pos}) same_device(x, *t, "every tensor");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
   Tensor ws = dispatch_ws(x.device(), n * k, (int)el);
   check_rc(bgmoe_dispatch_scatter_3d(ptr<uint16_t>(x), ptr<int32_t>(flat), (int)n, (int)k, (int)h, ptr<uint16_t>(act),
@@ -302,6 +312,7 @@ std::vector<Tensor> dispatch_scatter_ragged(Tensor x, Tensor ids, Tensor act, in
   TORCH_CHECK(counters.dim() == 1 && counters.size(0) == el, "expert_counters must be int32 [E_local]");
   TORCH_CHECK(cu.dim() == 1 && cu.size(0) == el + 1, "cu_seqlens must be int32 [E_local + 1]");
   TORCH_CHECK(pos.dim() == 1 && pos.size(0) == nk, "topk_pos must be int32 [N * K]");
+  for (auto* t : {&ids, &act, &counts, &counters, &pos, &cu}) same_device(x, *t, "every tensor");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
   Tensor ws = dispatch_ws(x.device(), nk, (int)el);
   check_rc(bgmoe_dispatch_scatter_ragged(ptr<uint16_t>(x), ptr<int32_t>(ids), (int)n, (int)k, (int)h, ptr<uint16_t>(act),
@@ -321,6 +332,7 @@ Tensor combine_fp32(Tensor y, Tensor pos, Tensor w, int64_t N, int64_t H, int64_
   TORCH_CHECK(pos.numel() >= N * K && w.numel() >= N * K, "topk_pos / topk_weights is smaller than N*K");
   TORCH_CHECK(out.dim() == 2 && out.size(0) >= N && out.size(1) == H, "output must have shape [N, H]");
   TORCH_CHECK(y.dim() == 2 && y.size(1) == H, "expert_output must have shape [rows, H]");
+  for (auto* t : {&pos, &w, &out}) same_device(y, *t, "topk_pos / topk_weights / output");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(y.device());
   check_rc(bgmoe_reduce_weighted_scatter_fp32(ptr<uint16_t>(y), ptr<int32_t>(pos), ptr<float>(w), (int)N, (int)H, (int)K,
                                               ptr<float>(out), cur_stream()));
@@ -339,6 +351,8 @@ Tensor combine_ordered(Tensor y, Tensor pos, Tensor ids, Tensor w, int64_t N, in
   TORCH_CHECK(pos.numel() == N * K && ids.numel() == N * K && w.numel() == N * K, "topk_pos / topk_indices / topk_weights must "
               "contain N*K elements");
   TORCH_CHECK(out.numel() >= N * H, "output must have shape [N, H]");
+  TORCH_CHECK(y.dim() == 2 && y.size(1) == H, "expert_output must have shape [rows, H]");
+  for (auto* t : {&pos, &ids, &w, &out}) same_device(y, *t, "topk_pos / topk_indices / topk_weights / output");
   c10::hip::HIPGuardMasqueradingAsCUDA guard(y.device());
   check_rc(bgmoe_reduce_weighted_scatter_bf16_ordered(ptr<uint16_t>(y), ptr<int32_t>(pos), ptr<int32_t>(ids), ptr<float>(w), (int)N,
                                                       (int)H, (int)K, ptr<uint16_t>(out), cur_stream()));

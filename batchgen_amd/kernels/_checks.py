@@ -53,8 +53,8 @@ def combine_args(expert_output, topk_pos, topk_weights, output, n, h, k, out_dty
         fail(f"topk_pos / topk_weights must hold N*K = {n * k} elements")
     if output.numel() < n * h:
         fail(f"output must hold N*H = {n * h} elements")
-    if expert_output.numel() % h != 0:
-        fail(f"expert_output must be [rows, {h}]")
+    if expert_output.dim() < 2 or expert_output.size(-1) != h:      # [rows, H] or the masked [E_local, max_tokens, H]
+        fail(f"expert_output must have rows of H={h} elements")
 
 
 FP8_BYTES = (torch.uint8, torch.float8_e4m3fn)

@@ -71,12 +71,17 @@ def test_dispatch_masked_overflow_rows_are_dropped(dev, n, k, et, es, el, mtp):
     assert np.array_equal(act.view(torch.int16).cpu().numpy(), ref)
 
 
-@pytest.mark.parametrize("mod", ["ds3d", "routing"])
+@pytest.mark.parametrize("mod", ["ds3d", "routing", "ds3d_compiled", "routing_compiled"])
 def test_combine_and_dispatch_reject_wrong_arguments(dev, mod):
     """Wrong dtypes and short tensors raise before anything is launched (no raw pointer of the wrong type or
-    size reaches the kernel)."""
+    size reaches the kernel): the ctypes modules and the compiled extension modules, same table."""
     from batchgen_amd.kernels import load_extension
-    m = ds3d() if mod == "ds3d" else load_extension("batchgen_kernels.moe._C_routing")
+    name = "batchgen_kernels.moe._C_dispatch_scatter_3d" if mod.startswith("ds3d") else "batchgen_kernels.moe._C_routing"
+    if mod.endswith("_compiled"):
+        from tests.test_torch_extension_modules import load
+        m = load(name)
+    else:
+        m = load_extension(name)
     n, k, h = 8, 4, 256
     y = torch.zeros((n * k, h), dtype=torch.bfloat16, device=dev)
     pos = torch.arange(n * k, dtype=torch.int32, device=dev)
@@ -84,12 +89,13 @@ def test_combine_and_dispatch_reject_wrong_arguments(dev, mod):
     out = torch.zeros((n, h), dtype=torch.bfloat16, device=dev)
     m.reduce_weighted_scatter(y, pos, w, n, h, k, out)                                    # the good call
     for bad in (dict(w=w.bfloat16()), dict(pos=pos.long()), dict(pos=pos[:-1]), dict(w=w[:, :-1].contiguous()),
-                dict(out=out[:-1]), dict(out=out.float()), dict(w=w.cpu()), dict(y=y.float())):
+                dict(out=out[:-1]), dict(out=out.float()), dict(w=w.cpu()), dict(y=y.float()),
+                dict(y=y.view(n * k * 2, h // 2))):
         a = dict(y=y, pos=pos, w=w, out=out)
         a.update(bad)
         with pytest.raises(RuntimeError):
             m.reduce_weighted_scatter(a["y"], a["pos"], a["w"], n, h, k, a["out"])
-    if mod == "ds3d":
+    if mod.startswith("ds3d"):
         x = torch.zeros((n, h), dtype=torch.bfloat16, device=dev)
         ids = torch.zeros((n, k), dtype=torch.int32, device=dev)
         act = torch.zeros((2 * 16, h), dtype=torch.bfloat16, device=dev)
