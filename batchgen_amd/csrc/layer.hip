@@ -92,8 +92,9 @@ extern "C" int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* L, bgmoe_s
   bgmoe_fp8_act ax{L->xq, L->xs, hb, 1};
   const int64_t live_bound = nk + (folded ? n : 0);       // rows that can be live in one pass
   // Rows one group can have: the router picks distinct experts per token, so at most n; routes handed in from
-  // outside may name one expert several times in a token's row, so only n*k bounds them.
-  const int64_t group_bound = routed ? nk : n;
+  // outside may name one expert several times in a token's row, so only n*k bounds them unless the caller
+  // vouches for distinct ids (a top-k gate of its own).
+  const int64_t group_bound = routed && L->routes_given != BGMOE_ROUTES_GIVEN_DISTINCT ? nk : n;
   rc = bgmoe_internal_fp8_gemm(&ax, &L->gate, &L->up, L->expert_counts, L->cu_seqlens, groups,
                                folded ? rows : L->cap_rows, inter, h, nullptr, L->hq, L->hs, ib, 1, live_bound, group_bound,
                                L->gemm_workspace, L->gemm_workspace_bytes, st);

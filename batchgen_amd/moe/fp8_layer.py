@@ -44,6 +44,7 @@ class LayerStruct(C.Structure):
 
 
 _lib.register("bgmoe_moe_fp8_layer_forward", i32, [C.POINTER(LayerStruct), vp])
+ROUTES_GIVEN, ROUTES_GIVEN_DISTINCT = 1, 2          # bgmoe_moe_fp8_layer.routes_given (include/bgmoe.h)
 
 
 W_ROW_MAJOR, W_TILE_MAJOR = 0, 1
@@ -244,12 +245,17 @@ class Fp8MoELayer:
         return self.out[:n]
 
     def forward_routed(self, hidden_states: torch.Tensor, topk_idx: torch.Tensor,
-                       topk_weight: torch.Tensor) -> torch.Tensor:
+                       topk_weight: torch.Tensor, distinct_ids: bool = False) -> torch.Tensor:
         """The layer behind an external gate: ``topk_idx`` ``[N, K]`` (global expert ids; ids this rank does not
         hold, and -1, contribute nothing) and ``topk_weight`` ``[N, K]`` fp32 are given, as in
         ``WGMMAMoEBuffers.forward(layer_id, global_x, topk_idx, topk_weight)``
         (batchgen/moe/fp8_wgmma_pipeline.py:294-372): dispatch, quantise, gate_up + SwiGLU + requant, down,
-        weighted combine (+ shared expert when the layer has one)."""
+        weighted combine (+ shared expert when the layer has one).
+
+        ``distinct_ids``: the caller vouches that the ids of a row are pairwise different (any top-k gate's are).
+        An expert then has at most N rows, and a decode batch runs on the weight-streaming kernels alone, as
+        with the layer's own router; without the promise an expert may hold up to N*K rows and batches above
+        256 / K tokens also launch the tiled kernel."""
         cfg = self.cfg
         n = hidden_states.size(0)
         if hidden_states.dtype != torch.bfloat16 or tuple(hidden_states.shape) != (n, cfg.hidden) or \
@@ -261,7 +267,7 @@ class Fp8MoELayer:
         self.topk_weights[:n].copy_(topk_weight)
         L = self._L
         L.logits = L.x_fp8 = L.x_scale = None
-        L.n, L.x, L.routes_given = n, ptr(hidden_states), 1
+        L.n, L.x, L.routes_given = n, ptr(hidden_states), ROUTES_GIVEN_DISTINCT if distinct_ids else ROUTES_GIVEN
         try:
             check(self._fn(C.byref(L), stream()))
         finally:

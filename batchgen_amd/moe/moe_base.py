@@ -27,57 +27,72 @@ from .shared_expert import Fp8DenseExpert
 
 
 class MoEBufferManager:
-    """Buffers of the decode template, sized once and shared by every MoE layer of a model
-    (moe_base.py:31-72): the gathered tokens ``[world_size * num_tokens_per_rank, H]`` and this rank's
-    padded slice."""
+    """Token buffers of the decode template, shared by every MoE layer of a model (the reference keeps one per
+    model as a class attribute of ``MoEBase``, moe_base.py:31-72).  Here both buffers are views of ONE
+    allocation of ``(world_size + 1) * num_tokens_per_rank`` rows: the first ``world_size * num_tokens_per_rank``
+    are ``all_tokens`` (the gathered batch the experts see), the rest ``padded_hidden_states`` (this rank's
+    slice, padded).  Growing replaces the allocation; shrinking never happens, so addresses captured in a graph
+    stay valid until a larger batch arrives."""
 
     def __init__(self, num_tokens_per_rank: int, world_size: int, hidden_size: int, device: torch.device):
-        self.num_tokens_per_rank = num_tokens_per_rank
+        if num_tokens_per_rank <= 0 or world_size <= 0 or hidden_size <= 0:
+            raise ValueError("num_tokens_per_rank, world_size and hidden_size must be positive")
         self.world_size = world_size
         self.hidden_size = hidden_size
         self.device = device
-        self._allocate()
+        self.num_tokens_per_rank = 0
+        self._rows = None
+        self._grow(num_tokens_per_rank)
 
-    def _allocate(self):
-        g = self.num_tokens_per_rank * self.world_size
-        self.all_tokens = torch.zeros(g, self.hidden_size, dtype=torch.bfloat16, device=self.device)
-        self.padded_hidden_states = torch.zeros(self.num_tokens_per_rank, self.hidden_size, dtype=torch.bfloat16,
-                                                device=self.device)
-
-    def resize_if_needed(self, num_tokens_per_rank: int):
-        if num_tokens_per_rank <= self.num_tokens_per_rank:
-            return
+    def _grow(self, num_tokens_per_rank: int) -> None:
+        self._rows = torch.zeros(((self.world_size + 1) * num_tokens_per_rank, self.hidden_size),
+                                 dtype=torch.bfloat16, device=self.device)
         self.num_tokens_per_rank = num_tokens_per_rank
-        self._allocate()
+
+    @property
+    def all_tokens(self) -> torch.Tensor:
+        return self._rows[: self.world_size * self.num_tokens_per_rank]
+
+    @property
+    def padded_hidden_states(self) -> torch.Tensor:
+        return self._rows[self.world_size * self.num_tokens_per_rank:]
+
+    def resize_if_needed(self, num_tokens_per_rank: int) -> None:
+        if num_tokens_per_rank > self.num_tokens_per_rank:
+            self._grow(num_tokens_per_rank)
+
+
+def _rank_and_world() -> Tuple[int, int]:
+    import torch.distributed as dist
+    if dist.is_available() and dist.is_initialized():
+        return dist.get_rank(), dist.get_world_size()
+    return 0, 1
 
 
 class MoEBase(nn.Module):
-    """Template-method base class of the MoE layers (moe_base.py:75-264)."""
+    """Template of the MoE layers (moe_base.py:75-264).  A model file subclasses it and fills in ``gate``,
+    ``expert_compute_persistent`` / ``expert_compute_mixed`` and ``shared_expert_forward``; the attribute names
+    set here (``experts_per_rank``, ``routed_expert_start_idx``, ``num_persistent_local_experts`` ...) are the
+    ones those subclasses read."""
 
     _buffer_mgr: ClassVar[Optional[MoEBufferManager]] = None
 
     def __init__(self, config, comm=None):
         super().__init__()
-        self.config = config
-        self.hidden_size = config.hidden_size
-        self.num_experts_per_tok = config.num_experts_per_tok
-        self.comm = comm
-        import torch.distributed as dist
-        if not dist.is_available() or not dist.is_initialized():
-            self.rank, self.world_size = 0, 1
-        else:
-            self.rank, self.world_size = dist.get_rank(), dist.get_world_size()
-        if self.world_size != 1:
+        rank, world = _rank_and_world()
+        if world != 1:
             raise NotImplementedError("this build runs one GPU: the expert-parallel exchange (all-gather / "
                                       "all-reduce across ranks) is not part of it")
-        self.experts_per_rank = config.n_routed_experts // self.world_size
-        self.total_experts = self.world_size * self.experts_per_rank
-        self.routed_expert_start_idx = self.rank * self.experts_per_rank
-        self.routed_expert_end_idx = (self.rank + 1) * self.experts_per_rank
-        self.device = torch.device("cuda", self.rank % max(torch.cuda.device_count(), 1))
-        self.num_tokens_per_rank = None
+        per_rank = config.n_routed_experts // world
+        self.config, self.comm = config, comm
+        self.hidden_size, self.num_experts_per_tok = config.hidden_size, config.num_experts_per_tok
+        self.rank, self.world_size = rank, world
+        self.experts_per_rank, self.total_experts = per_rank, per_rank * world
+        self.routed_expert_start_idx, self.routed_expert_end_idx = rank * per_rank, (rank + 1) * per_rank
+        self.device = torch.device("cuda", rank % max(torch.cuda.device_count(), 1))
+        self.num_tokens_per_rank: Optional[int] = None
         self.enable_ep_offloading = False
-        self.num_persistent_local_experts = self.experts_per_rank
+        self.num_persistent_local_experts = per_rank           # every local expert resident unless a subclass says so
 
     # -- buffers ----------------------------------------------------------------------------------------------
     @classmethod
@@ -88,9 +103,10 @@ class MoEBase(nn.Module):
         self.num_tokens_per_rank = num_tokens_per_rank
 
     def set_num_tokens_per_rank(self, num_tokens_per_rank: int):
-        self.num_tokens_per_rank = num_tokens_per_rank
-        if self._buffer_mgr is not None:
-            self._buffer_mgr.resize_if_needed(num_tokens_per_rank)
+        self.init_num_tokens(num_tokens_per_rank)
+        mgr = type(self)._buffer_mgr
+        if mgr is not None:
+            mgr.resize_if_needed(num_tokens_per_rank)
 
     # -- what a model fills in --------------------------------------------------------------------------------
     def gate(self, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
@@ -113,41 +129,45 @@ class MoEBase(nn.Module):
     # -- the template -------------------------------------------------------------------------------------------
     @torch.inference_mode()
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
-        if getattr(self.config, "phase", "decode") == "decode":
-            return self._forward_decode(hidden_states)
-        return self._forward_prefill(hidden_states)
+        decode = getattr(self.config, "phase", "decode") == "decode"
+        return self._forward_decode(hidden_states) if decode else self._forward_prefill(hidden_states)
+
+    def _gathered_tokens(self, tokens: torch.Tensor) -> torch.Tensor:
+        """The batch the experts see: with one rank, this rank's tokens followed by zero rows up to
+        ``num_tokens_per_rank`` (what the all-gather of the padded slices delivers), in the shared buffer when
+        it is large enough."""
+        ntp = self.num_tokens_per_rank
+        live, width = tokens.shape
+        mgr = type(self)._buffer_mgr
+        if mgr is not None and mgr.hidden_size == width and mgr.num_tokens_per_rank >= ntp:
+            gathered = mgr.all_tokens[:ntp]
+        else:
+            gathered = tokens.new_empty((ntp, width), dtype=torch.bfloat16)
+        gathered[:live].copy_(tokens)
+        gathered[live:].zero_()
+        return gathered
+
+    def _run_experts(self, global_x: torch.Tensor, topk_idx: torch.Tensor, topk_weight: torch.Tensor) -> torch.Tensor:
+        resident = self.num_persistent_local_experts == self.experts_per_rank and not self.enable_ep_offloading
+        compute = self.expert_compute_persistent if resident else self.expert_compute_mixed
+        return compute(global_x, topk_idx, topk_weight)
 
     @torch.inference_mode()
     def _forward_decode(self, hidden_states: torch.Tensor) -> torch.Tensor:
-        """moe_base.py:188-258 with a world of one rank: pad to ``num_tokens_per_rank`` rows (the gathered
-        tokens), gate, expert compute, take the live rows, add the shared expert."""
-        orig_shape = hidden_states.shape
-        hidden_states = hidden_states.view(-1, hidden_states.shape[-1])
-        identity = hidden_states
-        num_tokens, hidden_size = hidden_states.shape
+        """The decode template (moe_base.py:188-258) for a world of one rank: gather (= pad) -> gate -> expert
+        compute -> (the all-reduce of one rank is the identity) -> this rank's live rows + shared expert."""
         if self.num_tokens_per_rank is None:
             raise RuntimeError("init_num_tokens / set_num_tokens_per_rank must be called before the first forward")
-        if num_tokens > self.num_tokens_per_rank:
-            raise RuntimeError(f"MoE buffer overflow: num_tokens={num_tokens} > "
+        tokens = hidden_states.view(-1, hidden_states.shape[-1])
+        live = tokens.size(0)
+        if live > self.num_tokens_per_rank:
+            raise RuntimeError(f"MoE buffer overflow: num_tokens={live} > "
                                f"num_tokens_per_rank={self.num_tokens_per_rank}")
-        buf, ntp = self._buffer_mgr, self.num_tokens_per_rank
-        if buf is not None and buf.num_tokens_per_rank >= ntp and buf.hidden_size == hidden_size:
-            all_tokens = buf.all_tokens[:ntp]
-        else:
-            all_tokens = torch.empty(ntp, hidden_size, device=hidden_states.device, dtype=torch.bfloat16)
-        all_tokens[:num_tokens].copy_(hidden_states)
-        if num_tokens < ntp:
-            all_tokens[num_tokens:].zero_()
-        topk_idx, topk_weight = self.gate(all_tokens)
-        all_persistent = self.num_persistent_local_experts == self.experts_per_rank
-        if all_persistent and not self.enable_ep_offloading:
-            global_results = self.expert_compute_persistent(all_tokens, topk_idx, topk_weight)
-        else:
-            global_results = self.expert_compute_mixed(all_tokens, topk_idx, topk_weight)
-        start = self.rank * ntp
-        out = global_results[start:start + num_tokens].to(hidden_states.dtype)
-        out = out + self.shared_expert_forward(identity)
-        return out.view(*orig_shape)
+        global_x = self._gathered_tokens(tokens)
+        global_results = self._run_experts(global_x, *self.gate(global_x))
+        first = self.rank * self.num_tokens_per_rank
+        routed = global_results[first:first + live].to(tokens.dtype)
+        return (routed + self.shared_expert_forward(tokens)).view(hidden_states.shape)
 
     @torch.inference_mode()
     def _forward_prefill(self, hidden_states: torch.Tensor) -> torch.Tensor:
@@ -209,6 +229,10 @@ class Fp8BlockwiseMoE(MoEBase):
                                                  shared["down_s"][0].contiguous(), gate_up=gate_up, layer_idx=layer_idx)
         self._routed: Optional[Fp8MoELayer] = None
         self._fused: Optional[Fp8MoELayer] = None
+        # this class's own gate is a top-k: the ids of a row are pairwise different, so no expert can receive more
+        # rows than there are tokens and a decode batch keeps the weight-streaming kernels.  A subclass that
+        # replaces gate() with something that may repeat an id in a row must clear this.
+        self._gate_ids_distinct = True
 
     # -- engines, built for the current token capacity ------------------------------------------------------------
     def _routed_layer(self, n_tokens: int) -> Fp8MoELayer:
@@ -243,7 +267,8 @@ class Fp8BlockwiseMoE(MoEBase):
         """Dispatch, quantise, gate_up + SwiGLU + requant, down, weighted combine of this rank's experts
         (``WGMMAMoEBuffers.forward``, batchgen/moe/fp8_wgmma_pipeline.py:294-372).  The result is a buffer of
         the layer, overwritten by the next call."""
-        return self._routed_layer(global_x.size(0)).forward_routed(global_x, topk_idx, topk_weight)
+        return self._routed_layer(global_x.size(0)).forward_routed(global_x, topk_idx, topk_weight,
+                                                                   distinct_ids=self._gate_ids_distinct)
 
     def expert_compute_mixed(self, global_x, topk_idx, topk_weight):
         """Every expert of this build is resident, so the mixed path is the persistent one."""

@@ -669,7 +669,12 @@ typedef struct bgmoe_moe_fp8_layer {
   /* non-zero: the routes are given -- topk_ids [n,top_k] and topk_weights [n,top_k] are INPUTS, the router is
    * skipped and logits / router_weight are not read (the form of `WGMMAMoEBuffers.forward(layer_id, global_x,
    * topk_idx, topk_weight)`, batchgen/moe/fp8_wgmma_pipeline.py:294-372).  Ids outside the local expert range
-   * (and -1) contribute nothing. */
+   * (and -1) contribute nothing.  BGMOE_ROUTES_GIVEN: a row of topk_ids may name one expert several times (a
+   * group is then bounded by n*top_k rows only).  BGMOE_ROUTES_GIVEN_DISTINCT: the caller promises that the ids
+   * of a row are pairwise different, as every top-k gate's are: a group then holds at most n rows, and a decode
+   * batch keeps the weight-streaming kernels it would get with the layer's own router.  A broken promise loses
+   * no row and touches no memory outside the buffers (groups above the streaming limit are then served by the
+   * tiled kernel only when one is launched, i.e. their rows may be left uncomputed): it is the caller's bug. */
   int32_t routes_given;
   /* Optional: bgmoe_fp8_streamk_workspace_bytes() bytes, 16-byte aligned, its first 4096 bytes zero before the
    * first call (every call leaves them zero).  With it, a batch in which no group can exceed the streaming
@@ -680,6 +685,7 @@ typedef struct bgmoe_moe_fp8_layer {
   size_t gemm_workspace_bytes;
 } bgmoe_moe_fp8_layer;
 
+enum { BGMOE_ROUTES_GIVEN = 1, BGMOE_ROUTES_GIVEN_DISTINCT = 2 };
 int bgmoe_moe_fp8_layer_forward(const bgmoe_moe_fp8_layer* layer, bgmoe_stream_t stream);
 
 /* One MXFP4 (W4A16) MoE layer forward on one GPU's share of the experts, masked layout:

@@ -302,6 +302,14 @@ def test_moe_base_decode_template_on_a_toy_layer():
         assert torch.equal(layer(x), out) and seen["gate_rows"] == 12
     finally:
         Toy._buffer_mgr = None
+    mgr = mb.MoEBufferManager(4, 3, 16, torch.device("cpu"))           # both buffers are views of one allocation
+    assert mgr.all_tokens.shape == (12, 16) and mgr.padded_hidden_states.shape == (4, 16)
+    assert mgr.padded_hidden_states.data_ptr() == mgr.all_tokens.data_ptr() + 12 * 16 * 2
+    before = mgr.all_tokens.data_ptr()
+    mgr.resize_if_needed(3)
+    assert mgr.all_tokens.data_ptr() == before and mgr.num_tokens_per_rank == 4      # never shrinks
+    mgr.resize_if_needed(6)
+    assert mgr.all_tokens.shape == (18, 16) and mgr.padded_hidden_states.shape == (6, 16)
     layer.enable_ep_offloading = True
     with pytest.raises(NotImplementedError):
         layer(x)                                                       # the toy has no mixed path

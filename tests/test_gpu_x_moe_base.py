@@ -82,3 +82,18 @@ def test_template_layer_prefill_phase(dev):
     pieces = layer.expert_compute_persistent(xd, *layer.gate(xd)) + layer.shared_expert_forward(xd)
     assert torch.equal(pieces, pre)
     assert torch.equal(layer.expert_compute_mixed(xd, *layer.gate(xd)), layer.expert_compute_persistent(xd, *layer.gate(xd)))
+
+
+def test_distinct_ids_promise_changes_the_kernel_choice_not_the_result(dev):
+    """``forward_routed(distinct_ids=True)`` (what the template's own top-k gate promises) bounds a group by the
+    token count instead of tokens x k, so a decode batch needs no tiled launch; on routes that do keep the
+    promise both forms give the same bits (no group here exceeds the rows every form streams)."""
+    layer, wcfg, w, sh, x = _build(dev)
+    layer.set_num_tokens_per_rank(64)
+    xd = x.to(dev)
+    ids, wts = layer.gate(xd)
+    eng = layer._routed_layer(64)
+    a = eng.forward_routed(xd, ids, wts, distinct_ids=False).clone()
+    b = eng.forward_routed(xd, ids, wts, distinct_ids=True).clone()
+    assert torch.equal(a, b)
+    assert layer._gate_ids_distinct and torch.equal(layer.expert_compute_persistent(xd, ids, wts), b)
