@@ -77,6 +77,7 @@ _SIGS = {
     "bgmoe_fp8_streamk_workspace_bytes": (sz, []),
     "bgmoe_debug_streamk_trace": (i32, [vp]),
     "bgmoe_set_streamk_xcd_weights": (i32, [vp]),
+    "bgmoe_debug_streamk_status": (i32, [vp]),
     "bgmoe_dispatch_scatter_3d": (i32, [vp, vp, i32, i32, i32, vp, i32, i32, i32, vp, vp, vp, vp, sz, vp]),
     "bgmoe_dispatch_scatter_ragged": (i32, [vp, vp, i32, i32, i32, vp, i64, i32, i32, vp, vp, vp, vp, i32, vp, sz, vp]),
     "bgmoe_dispatch_static_max_pairs": (sz, [i32]),

@@ -141,6 +141,28 @@ def build_extensions(force: bool = False, verbose: bool = True) -> str:
     return EXT_ROOT
 
 
+# ---- host-compiled checks of the arithmetic shared with the kernels (g++, no GPU) -----------------------------
+HOSTCHECK_SRC = os.path.join(CSRC, "hostcheck.cc")
+HOSTCHECK_LIB = os.path.join(LIB_DIR, "libbgmoe_hostcheck.so")
+
+
+def build_hostcheck(force: bool = False, verbose: bool = True) -> str:
+    """Compile csrc/hostcheck.cc with g++ into lib/libbgmoe_hostcheck.so: the index and address arithmetic of
+    csrc/bgmoe_hostdev.h and csrc/bgmoe_tilemap.h (the very text the kernels include) behind a few C functions that
+    the CPU tests drive.  Test infrastructure; the product library does not depend on it."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    deps = [HOSTCHECK_SRC] + [os.path.join(CSRC, f) for f in ("bgmoe_hostdev.h", "bgmoe_tilemap.h")]
+    if force or not _newer(HOSTCHECK_LIB, deps):
+        cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra", "-Werror", HOSTCHECK_SRC, "-o",
+               HOSTCHECK_LIB]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"g++ failed for {HOSTCHECK_SRC}:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {HOSTCHECK_LIB}")
+    return HOSTCHECK_LIB
+
+
 def build(force: bool = False, jobs: int = 4, verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
@@ -165,6 +187,7 @@ if __name__ == "__main__":
     a = ap.parse_args()
     try:
         build(force=a.force, jobs=a.j)
+        build_hostcheck(force=a.force)
         if a.ext:
             build_extensions(force=a.force)
     except RuntimeError as e:

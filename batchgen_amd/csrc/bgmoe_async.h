@@ -6,6 +6,7 @@
 // the data visible to the other waves with block_barrier().
 #pragma once
 #include "bgmoe_common.h"
+#include "bgmoe_hostdev.h"
 
 // 64 lanes x 16 bytes -> LDS [lds_base, lds_base + 1024); lds_base must be wave-uniform.  No
 // instruction offset is used: the hardware would add it to the LDS address as well as to the
@@ -26,9 +27,10 @@ __device__ __forceinline__ void async_load4(const float* base, uint32_t lane_off
 template <typename T>
 __device__ __forceinline__ const T* uniform_ptr(const T* p) {   // tell the compiler a pointer is wave-uniform
   const uint64_t v = reinterpret_cast<uint64_t>(p);
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return reinterpret_cast<const T*>(((uint64_t)hi << 32) | lo);
+  // the builtin returns `int`: bgmoe_compose_u64 takes both halves as unsigned, so bit 31 of the low half cannot
+  // sign-extend into the high half
+  return reinterpret_cast<const T*>(bgmoe_compose_u64(__builtin_amdgcn_readfirstlane((uint32_t)v),
+                                                      __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32))));
 }
 template <int N>
 __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }

@@ -1,0 +1,160 @@
+// Index and address arithmetic that the kernels share with host-compiled checks.
+//
+// Everything here is plain C++ over fixed-width integers: hipcc compiles it for the device (and the host), g++
+// compiles the same text into the host-side check library (csrc/hostcheck.cc), whose tests walk the arithmetic
+// over random launches on the CPU.  A kernel that needs one of these computations calls the function here
+// instead of writing it out again: what the CPU tests pin is then what the GPU runs.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define BGMOE_HD __host__ __device__ __forceinline__
+#else
+#define BGMOE_HD inline
+#endif
+
+// ---- 64-bit values from 32-bit halves ----------------------------------------------------------------------
+// Both halves are taken as UNSIGNED 32-bit parameters, whatever the caller's expression type is: the wave
+// builtins (readfirstlane, readlane) return `int`, and an `int` low half widened to 64 bits sign-extends, which
+// turns every address with bit 31 set into an unmapped one.  Going through these parameters converts modulo 2^32
+// first.
+BGMOE_HD uint64_t bgmoe_compose_u64(uint32_t lo, uint32_t hi) { return ((uint64_t)hi << 32) | (uint64_t)lo; }
+
+// Lowest and highest byte a launch addresses through `base`: rows [0, rows) of `row_bytes` bytes at a pitch of
+// `pitch_bytes`.  Host-side launch checks compare this range with the allocation before anything is enqueued.
+struct BgmoeByteRange { uint64_t lo, hi; };           // [lo, hi): hi == lo for an empty range
+BGMOE_HD BgmoeByteRange bgmoe_rows_range(uint64_t base, uint64_t rows, uint64_t row_bytes, uint64_t pitch_bytes) {
+  BgmoeByteRange r{base, base};
+  if (rows != 0 && row_bytes != 0) r.hi = base + (rows - 1) * pitch_bytes + row_bytes;
+  return r;
+}
+BGMOE_HD bool bgmoe_range_inside(BgmoeByteRange r, uint64_t alloc_base, uint64_t alloc_bytes) {
+  return r.lo >= alloc_base && r.hi >= r.lo && r.hi <= alloc_base + alloc_bytes;
+}
+
+// ---- balanced (stream-K) weight-streaming GEMM: shares of the cumulative cost --------------------------------
+// The launch's work is the sequence of units (item, K-block); an item is (group, row chunk, column slab) and its
+// units follow each other in K.  Inside a group the order is row chunk by row chunk, each chunk slab by slab.
+// Every unit has a cost; share r of G owns the units whose START cost lies in [bound(r), bound(r+1)).
+struct BgmoeSkCost { int w, r, t; };   // per 2-KiB tile: weights first stream / re-stream for a later chunk / tokens
+struct BgmoeSkShape { int tt, wc; };   // token tiles (16 rows) per row chunk; weight tiles per K-block of an item
+
+// cost of ONE K-block of ALL chunks of one slab of a group with c rows
+BGMOE_HD uint32_t bgmoe_sk_group_cost_per_kb(BgmoeSkShape s, BgmoeSkCost k, int c) {
+  if (c <= 0) return 0;
+  const int chunks = (c + 16 * s.tt - 1) / (16 * s.tt);
+  const int tiles_g = (c + 15) >> 4;
+  return (uint32_t)(s.wc * (k.w + (chunks - 1) * k.r) + tiles_g * k.t);
+}
+// the most a single unit can cost (a full first chunk), and the figure the share count is sized with: that plus one
+// weight tile, so that the rounding of a share's two bounds cannot take it below a whole unit
+BGMOE_HD uint32_t bgmoe_sk_max_unit_cost(BgmoeSkShape s, BgmoeSkCost k) { return (uint32_t)(s.wc * k.w + s.tt * k.t); }
+BGMOE_HD uint32_t bgmoe_sk_share_unit(BgmoeSkShape s, BgmoeSkCost k) { return bgmoe_sk_max_unit_cost(s, k) + (uint32_t)k.w; }
+
+// Shares are numbered XCD by XCD (n8 per XCD); a share of XCD x weighs w[x].  Weight of shares 0..r-1:
+BGMOE_HD uint32_t bgmoe_sk_cum_weight(const int (&w)[8], uint32_t n8, uint32_t r) {
+  uint32_t sum = 0, left = r;
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+  for (int x = 0; x < 8; ++x) {
+    const uint32_t take = left < n8 ? left : n8;
+    sum += take * (uint32_t)w[x];
+    left -= take;
+  }
+  return sum;
+}
+// the last share r with cum_weight(r) <= t (t < the total weight)
+BGMOE_HD uint32_t bgmoe_sk_share_of_weight(const int (&w)[8], uint32_t n8, uint32_t t) {
+  uint32_t r = 0;
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
+  for (int x = 0; x < 8; ++x) {
+    const uint32_t seg = n8 * (uint32_t)w[x];
+    if (t >= seg && x < 7) {
+      t -= seg;
+      r += n8;
+    } else {
+      const uint32_t q = t / (uint32_t)w[x];
+      return r + (q < n8 - 1 ? q : n8 - 1);
+    }
+  }
+  return r;
+}
+// Number of shares for a launch of cumulative cost C on `grid` blocks: a multiple of 8 (or 1), every share at
+// least min_units times share_unit (bgmoe_sk_share_unit) ON AVERAGE.  Weighted shares are smaller than the average by up to
+// 8 * wmin / sum(w); bgmoe_sk_weights_ok() bounds that factor so that the smallest share still holds a unit.
+BGMOE_HD uint32_t bgmoe_sk_num_shares(uint32_t C, uint32_t grid, uint32_t share_unit, uint32_t min_units) {
+  uint32_t G = C / (share_unit * min_units);
+  return G < 8 ? 1u : (G > grid ? grid : G) & ~7u;
+}
+// With min_units = 8 the smallest share is >= 8 * max_unit * 8 * wmin / sum(w) minus one for the rounding of
+// its two bounds; requiring sum(w) <= 32 * wmin leaves it at two units' cost or more.
+BGMOE_HD bool bgmoe_sk_weights_ok(const int (&w)[8]) {
+  int sum = 0, wmin = w[0];
+  for (int x = 0; x < 8; ++x) {
+    if (w[x] < 1 || w[x] > 64) return false;
+    sum += w[x];
+    if (w[x] < wmin) wmin = w[x];
+  }
+  return sum <= 32 * wmin;
+}
+// cost at which share r begins (r == G: the total cost C); Wg = cum_weight(G)
+BGMOE_HD uint32_t bgmoe_sk_bound(const int (&w)[8], uint32_t n8, uint32_t Wg, uint32_t C, uint32_t r) {
+  return (uint32_t)(((uint64_t)bgmoe_sk_cum_weight(w, n8, r) * C + Wg - 1) / Wg);
+}
+// share that holds cost position x (the share an item "begins in" / "ends in")
+BGMOE_HD uint32_t bgmoe_sk_share_of_cost(const int (&w)[8], uint32_t n8, uint32_t Wg, uint32_t C, uint32_t x) {
+  return bgmoe_sk_share_of_weight(w, n8, (uint32_t)(((uint64_t)x * Wg) / C));
+}
+
+// One contiguous run of K-blocks [kb_lo, kb_hi) of one item.
+struct BgmoeSkPart {
+  int grp, ntile, chunk, cnt;
+  int kb_lo, kb_hi;
+  uint32_t start;             // cumulative cost at the item's first K-block
+  int cpk;                    // cost of one K-block of this item
+};
+// The unit search inside group g (c rows, its first unit at cost gpre): the first unit whose start cost is >= x,
+// cut at x1 (exclusive).  Returns 1 and fills p; or returns 0 with *next = the start cost of the next item when x
+// lies inside the last K-block of an item (the caller looks again from there, possibly in the next group).
+BGMOE_HD int bgmoe_sk_locate_in_group(BgmoeSkShape s, BgmoeSkCost k, int g, int c, uint32_t gpre, int ntiles, int KB,
+                                      uint32_t x, uint32_t x1, BgmoeSkPart* p, uint32_t* next) {
+  const int chunks = (c + 16 * s.tt - 1) / (16 * s.tt);
+  const int tiles_g = (c + 15) >> 4;
+  const uint32_t slabs = (uint32_t)ntiles * (uint32_t)KB;
+  const uint32_t f0 = slabs * (uint32_t)(s.wc * k.w + s.tt * k.t);             // a full first chunk, all slabs
+  const uint32_t fl = slabs * (uint32_t)(s.wc * k.r + s.tt * k.t);             // a full later chunk
+  uint32_t r = x - gpre;
+  uint32_t ch = 0;
+  if (chunks > 1 && r >= f0) {
+    r -= f0;
+    ch = r / fl;
+    if (ch > (uint32_t)(chunks - 2)) ch = (uint32_t)(chunks - 2);
+    r -= ch * fl;
+    ch += 1;
+  }
+  const int rest = tiles_g - (int)ch * s.tt;
+  const int tl = s.tt < rest ? s.tt : rest;
+  const int cpk = s.wc * (ch == 0 ? k.w : k.r) + tl * k.t;
+  const uint32_t ci = (uint32_t)KB * (uint32_t)cpk;                            // one item of this chunk
+  const uint32_t nt = r / ci;
+  r -= nt * ci;
+  const uint32_t kb = (r + (uint32_t)cpk - 1) / (uint32_t)cpk;
+  const uint32_t start = x - r;
+  if (kb >= (uint32_t)KB) {             // x lies inside the item's last K-block: the next item's first unit
+    *next = start + (uint32_t)KB * (uint32_t)cpk;
+    return 0;
+  }
+  const uint32_t hi = (x1 - start + (uint32_t)cpk - 1) / (uint32_t)cpk;
+  p->grp = g;
+  p->ntile = (int)nt;
+  p->chunk = (int)ch;
+  p->cnt = c;
+  p->kb_lo = (int)kb;
+  p->kb_hi = (int)(hi < (uint32_t)KB ? hi : (uint32_t)KB);
+  p->start = start;
+  p->cpk = cpk;
+  return 1;
+}

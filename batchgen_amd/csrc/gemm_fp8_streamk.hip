@@ -21,6 +21,7 @@
 // is the weight-streaming kernel's; see gemm_fp8_skinny.hip.
 #include "bgmoe_common.h"
 #include "bgmoe_async.h"
+#include "bgmoe_hostdev.h"
 
 namespace {
 
@@ -39,36 +40,11 @@ struct StreamKArgs {
   int32_t* counters;          // gridDim.x counters, zero before and after every launch
   uint64_t* trace;            // optional (tuning): 4 timestamps per share (start, first unit, end of stream, end)
   int xcd_w[8];               // relative size of a share on XCD 0..7 (the XCDs do not stream equally fast)
+  int32_t* error_flag;        // device word, bit 0 set by a share that found no unit (see bgmoe_debug_streamk_status)
 };
 
-// Shares are numbered XCD by XCD (n8 per XCD); share r of XCD x weighs w[x].  cum_weight(r) = weight of shares 0..r-1.
-__device__ __forceinline__ uint32_t cum_weight(const int (&w)[8], uint32_t n8, uint32_t r) {
-  uint32_t sum = 0, left = r;
-#pragma unroll
-  for (int x = 0; x < 8; ++x) {
-    const uint32_t take = left < n8 ? left : n8;
-    sum += take * (uint32_t)w[x];
-    left -= take;
-  }
-  return sum;
-}
-// the last share r with cum_weight(r) <= t (t < the total weight)
-__device__ __forceinline__ uint32_t share_of_weight(const int (&w)[8], uint32_t n8, uint32_t t) {
-  uint32_t r = 0;
-#pragma unroll
-  for (int x = 0; x < 8; ++x) {
-    const uint32_t seg = n8 * (uint32_t)w[x];
-    if (t >= seg && x < 7) {
-      t -= seg;
-      r += n8;
-    } else {
-      const uint32_t q = t / (uint32_t)w[x];
-      return r + (q < n8 - 1 ? q : n8 - 1);
-    }
-  }
-  return r;
-}
-
+// Share arithmetic (cumulative weights, share bounds, the unit search inside a group): bgmoe_hostdev.h, shared with
+// the host-compiled checks that walk it over random launches on the CPU.
 constexpr int kMaxGroups = 320;         // per-group tables live in LDS
 
 // Cost of one K-block of an item, the measure in which shares are equal: its weight tiles (2 KiB each) count kCostW
@@ -84,13 +60,11 @@ constexpr int kMaxGroups = 320;         // per-group tables live in LDS
 #define BGMOE_SK_COST_T 2
 #endif
 constexpr int kCostW = BGMOE_SK_COST_W, kCostR = BGMOE_SK_COST_R, kCostT = BGMOE_SK_COST_T;
-// cost of all K-blocks of one slab of a group with c rows (tiles of 16 rows, chunks of TT tiles), per K-block
+constexpr BgmoeSkCost kCost{kCostW, kCostR, kCostT};
+// cost of one K-block of all row chunks of one slab of a group with c rows (tiles of 16 rows, chunks of TT tiles)
 template <int TT, int WC>
 __device__ __forceinline__ uint32_t group_cost_per_kb(int c) {
-  if (c <= 0) return 0;
-  const int chunks = (c + 16 * TT - 1) / (16 * TT);
-  const int tiles_g = (c + 15) >> 4;
-  return (uint32_t)(WC * (kCostW + (chunks - 1) * kCostR) + tiles_g * kCostT);
+  return bgmoe_sk_group_cost_per_kb(BgmoeSkShape{TT, WC}, kCost, c);
 }
 
 // One prefetch stage of a wave: NT weight tiles as the two 16-byte halves a lane loads.
@@ -156,12 +130,7 @@ __device__ __forceinline__ void async_load4_ptr(const float* lane_ptr, uint32_t 
 }
 
 // One contiguous run of K-blocks [kb_lo, kb_hi) of one item; wave-uniform.
-struct Part {
-  int grp, ntile, chunk, cnt;
-  int kb_lo, kb_hi;
-  uint32_t start;             // cumulative cost at the item's first K-block
-  int cpk;                    // cost of one K-block of this item
-};
+using Part = BgmoeSkPart;
 
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ uint32_t uniu(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
@@ -182,41 +151,22 @@ __device__ __forceinline__ bool locate(const uint32_t* s_gpre, const int32_t* s_
     }
     g = uni(g);
     const int c = uni(s_cnt[g]);
-    const int chunks = (c + 16 * TT - 1) / (16 * TT);
-    const int tiles_g = (c + 15) >> 4;
     // inside a group: row chunk by row chunk, each chunk slab by slab.  Blocks that run at the same time then hold
     // the same slab of neighbouring chunks, so a group with several chunks fetches its weights from HBM once
-    const uint32_t slabs = (uint32_t)ntiles * (uint32_t)KB;
-    const uint32_t f0 = slabs * (uint32_t)(WC * kCostW + TT * kCostT);             // a full first chunk, all slabs
-    const uint32_t fl = slabs * (uint32_t)(WC * kCostR + TT * kCostT);             // a full later chunk
-    uint32_t r = x - uniu(s_gpre[g]);
-    uint32_t ch = 0;
-    if (chunks > 1 && r >= f0) {
-      r -= f0;
-      ch = r / fl;
-      if (ch > (uint32_t)(chunks - 2)) ch = (uint32_t)(chunks - 2);
-      r -= ch * fl;
-      ch += 1;
-    }
-    const int tl = min(TT, tiles_g - (int)ch * TT);
-    const int cpk = WC * (ch == 0 ? kCostW : kCostR) + tl * kCostT;
-    const uint32_t ci = (uint32_t)KB * (uint32_t)cpk;                              // one item of this chunk
-    const uint32_t nt = r / ci;
-    r -= nt * ci;
-    const uint32_t kb = (r + (uint32_t)cpk - 1) / (uint32_t)cpk;
-    const uint32_t start = x - r;
-    if (kb >= (uint32_t)KB) {             // x lies inside the item's last K-block: the next item's first unit
-      x = start + (uint32_t)KB * (uint32_t)cpk;
+    Part q;
+    uint32_t next = 0;
+    if (!bgmoe_sk_locate_in_group(BgmoeSkShape{TT, WC}, kCost, g, c, uniu(s_gpre[g]), ntiles, KB, x, x1, &q, &next)) {
+      x = next;                           // x lies inside the item's last K-block: the next item's first unit
       continue;
     }
     p.grp = g;
-    p.ntile = uni((int)nt);
-    p.chunk = uni((int)ch);
+    p.ntile = uni(q.ntile);
+    p.chunk = uni(q.chunk);
     p.cnt = c;
-    p.kb_lo = uni((int)kb);
-    p.kb_hi = uni((int)min((uint32_t)KB, (x1 - start + (uint32_t)cpk - 1) / (uint32_t)cpk));
-    p.start = uniu(start);
-    p.cpk = uni(cpk);
+    p.kb_lo = uni(q.kb_lo);
+    p.kb_hi = uni(q.kb_hi);
+    p.start = uniu(q.start);
+    p.cpk = uni(q.cpk);
     return true;
   }
   return false;
@@ -300,24 +250,26 @@ __global__ __launch_bounds__(256, 2) void fp8_streamk_kernel(StreamKArgs g) {
   // (and at least kMinUnits of them: a launch too small for that uses fewer blocks rather than cut every item into
   // single K-blocks)
   constexpr uint32_t kMinUnits = 8;
-  uint32_t G = C / ((uint32_t)((WC + 1) * kCostW + TT * kCostT) * kMinUnits);
-  G = G < 8 ? 1 : (G > grid ? grid : G) & ~7u;
+  const uint32_t G = bgmoe_sk_num_shares(C, grid, bgmoe_sk_share_unit(BgmoeSkShape{TT, WC}, kCost), kMinUnits);
   // Blocks of one XCD (blockIdx % 8) own neighbouring shares: an item's parts and the tokens of a group stay in one
   // L2.  A share's size follows its XCD's weight.
   const uint32_t n8 = G >= 8 ? G >> 3 : 1;
   if ((blockIdx.x >> 3) >= n8) return;
   const uint32_t r = (blockIdx.x & 7u) * n8 + (blockIdx.x >> 3);
   if (r >= G) return;
-  const uint32_t Wg = cum_weight(g.xcd_w, n8, G);
-  auto bound = [&](uint32_t rr) __attribute__((always_inline)) {   // cost at which share rr begins
-    return (uint32_t)(((uint64_t)cum_weight(g.xcd_w, n8, rr) * C + Wg - 1) / Wg);
-  };
-  const uint32_t x0 = bound(r);
-  const uint32_t x1 = bound(r + 1);
+  const uint32_t Wg = bgmoe_sk_cum_weight(g.xcd_w, n8, G);
+  const uint32_t x0 = bgmoe_sk_bound(g.xcd_w, n8, Wg, C, r);           // cost at which this share begins ...
+  const uint32_t x1 = bgmoe_sk_bound(g.xcd_w, n8, Wg, C, r + 1);       // ... and ends
 
   // ---- load cursor ----
   Part pl;
-  if (!locate<TT, WC>(s_gpre, s_cnt, groups, ntiles, KB, x0, x1, pl)) return;   // cannot happen for r < G
+  if (!locate<TT, WC>(s_gpre, s_cnt, groups, ntiles, KB, x0, x1, pl)) {
+    // A share without a unit: impossible while every share is at least one unit's cost (bgmoe_sk_weights_ok and
+    // the choice of G guarantee it; the host-side checks walk the same arithmetic).  Items that span this share
+    // would never complete, so say so instead of leaving stale rows silently.
+    if (tid == 0 && g.error_flag != nullptr) atomicOr(g.error_flag, 1);
+    return;
+  }
   const uint8_t* l_wp[NT];
   const float* l_ws;                          // per lane: the scale stream this lane brings
   const uint8_t* l_tok;
@@ -557,10 +509,10 @@ __global__ __launch_bounds__(256, 2) void fp8_streamk_kernel(StreamKArgs g) {
   // begins in).  The block whose increment completes an item's count adds the other parts' slots to its own sums
   // IN SHARE ORDER and runs the epilogue; it leaves the counter at zero.  Nobody waits for another block.
   auto first_block = [&](const Part& p) __attribute__((always_inline)) {
-    return uniu(share_of_weight(g.xcd_w, n8, (uint32_t)(((uint64_t)p.start * Wg) / C)));
+    return uniu(bgmoe_sk_share_of_cost(g.xcd_w, n8, Wg, C, p.start));
   };
   auto last_block = [&](const Part& p) __attribute__((always_inline)) {
-    return uniu(share_of_weight(g.xcd_w, n8, (uint32_t)(((uint64_t)(p.start + (uint32_t)(KB - 1) * (uint32_t)p.cpk) * Wg) / C)));
+    return uniu(bgmoe_sk_share_of_cost(g.xcd_w, n8, Wg, C, p.start + (uint32_t)(KB - 1) * (uint32_t)p.cpk));
   };
   Part cut_head = pc;
   bool has_head = false, has_tail = false, head_saved = false;
@@ -759,6 +711,20 @@ unsigned grid_down() { return resident(fp8_streamk_kernel<kDownTT, kDownNS, fals
 
 constexpr size_t kCounterBytes = 4096;         // 1024 counters
 uint64_t* g_trace = nullptr;
+// Sticky status word of the balanced launches on this device (one copy per GPU, at its own address there).
+__device__ int32_t g_sk_status_word;
+constexpr int kMaxDevices = 16;
+int32_t* g_sk_status_ptr[kMaxDevices] = {};
+int32_t* status_ptr() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  if (g_sk_status_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_sk_status_word)) != hipSuccess) return nullptr;
+    g_sk_status_ptr[dev] = static_cast<int32_t*>(p);
+  }
+  return g_sk_status_ptr[dev];
+}
 // measured on MI355X: the odd XCDs stream about 9% slower than the even ones
 int g_xcd_w[8] = {23, 21, 23, 21, 23, 21, 23, 21};
 
@@ -772,11 +738,39 @@ extern "C" int bgmoe_debug_streamk_trace(uint64_t* device_buffer) {
   return BGMOE_OK;
 }
 
-// Tuning knob (no reference counterpart): relative share sizes of the eight XCDs, each in [1, 64].
+// Tuning knob (no reference counterpart): relative share sizes of the eight XCDs, each in [1, 64] and their sum at
+// most 32 times the smallest: the share count is sized from the AVERAGE share, and a share far below the average
+// could fall under the cost of one unit, own nothing, and leave the items that span it unfinished.
 extern "C" int bgmoe_set_streamk_xcd_weights(const int* w) {
   BGMOE_REQUIRE(w != nullptr, "set_streamk_xcd_weights: null");
-  for (int i = 0; i < 8; ++i) BGMOE_REQUIRE(w[i] >= 1 && w[i] <= 64, "set_streamk_xcd_weights: weight %d outside [1,64]", w[i]);
+  int ww[8];
+  for (int i = 0; i < 8; ++i) {
+    BGMOE_REQUIRE(w[i] >= 1 && w[i] <= 64, "set_streamk_xcd_weights: weight %d outside [1,64]", w[i]);
+    ww[i] = w[i];
+  }
+  BGMOE_REQUIRE(bgmoe_sk_weights_ok(ww), "set_streamk_xcd_weights: the weights' sum exceeds 32 times the smallest one "
+                "(the lightest XCD's shares could fall below one unit of work)");
   for (int i = 0; i < 8; ++i) g_xcd_w[i] = w[i];
+  return BGMOE_OK;
+}
+
+// Debug aid (no reference counterpart): reads the device's sticky status word of the balanced launches into
+// *host_out and clears it; synchronises the device.  Bit 0: a share found no unit of work (its items' rows are
+// stale).  The share arithmetic makes that impossible for accepted XCD weights; the word exists so that a
+// violation would be seen rather than silently produce stale rows.
+extern "C" int bgmoe_debug_streamk_status(int32_t* host_out) {
+  BGMOE_REQUIRE(host_out != nullptr, "debug_streamk_status: null");
+  int32_t* p = status_ptr();
+  if (p == nullptr) {
+    bgmoe_set_error("debug_streamk_status: cannot locate the status word");
+    return BGMOE_ERR_HIP;
+  }
+  const int32_t zero = 0;
+  if (hipMemcpy(host_out, p, sizeof(int32_t), hipMemcpyDeviceToHost) != hipSuccess ||
+      hipMemcpy(p, &zero, sizeof(int32_t), hipMemcpyHostToDevice) != hipSuccess) {
+    bgmoe_set_error("debug_streamk_status: copy failed");
+    return BGMOE_ERR_HIP;
+  }
   return BGMOE_OK;
 }
 
@@ -813,6 +807,7 @@ int bgmoe_internal_fp8_streamk(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w
   g.seqlens = seqlens; g.cu = cu; g.groups = groups; g.n = n; g.k = k;
   g.out = out; g.out_q = out_q; g.out_s = out_s; g.os_row = os_row; g.os_nb = os_nb; g.hi = hi;
   g.trace = g_trace;
+  g.error_flag = status_ptr();
   for (int i = 0; i < 8; ++i) g.xcd_w[i] = g_xcd_w[i];
   g.counters = reinterpret_cast<int32_t*>(ws);
   g.slots = reinterpret_cast<floatx4*>(reinterpret_cast<uint8_t*>(ws) + kCounterBytes);

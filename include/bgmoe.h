@@ -458,9 +458,14 @@ size_t bgmoe_fp8_streamk_workspace_bytes(void);
  * records the constant-rate clock (100 MHz) at its start, before its first unit, at the end of its stream and at its
  * end, at [4 * share .. 4 * share + 3].  NULL switches it off. */
 int bgmoe_debug_streamk_trace(uint64_t* device_buffer);
-/* Tuning knob: relative sizes of the shares of XCD 0..7 (8 ints, each in [1, 64]; default 23/21 alternating: on
- * MI355X the odd XCDs were measured to stream about 9% slower than the even ones). */
+/* Tuning knob: relative sizes of the shares of XCD 0..7 (8 ints, each in [1, 64], their sum at most 32 times the
+ * smallest, so that the lightest share still holds a whole unit of work; default 23/21 alternating: on MI355X
+ * the odd XCDs were measured to stream about 9% slower than the even ones). */
 int bgmoe_set_streamk_xcd_weights(const int* weights);
+/* Debug aid: copies the device's sticky status word of the balanced launches to *host_out and clears it
+ * (synchronises the device; not for the hot path).  Bit 0: a share of some launch found no unit of work, which
+ * the share arithmetic rules out for accepted XCD weights; rows of the items that spanned it would be stale. */
+int bgmoe_debug_streamk_status(int32_t* host_out);
 
 /* bgmoe_fp8_grouped_gemm / bgmoe_fp8_fused_s1 (same operands, outputs and checks) in the balanced form when it
  * applies: tile-major weights, workspace of bgmoe_fp8_streamk_workspace_bytes() bytes, and max_group_rows -- the

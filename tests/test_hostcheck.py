@@ -1,0 +1,287 @@
+"""CPU checks of the arithmetic the kernels share with the host (csrc/bgmoe_hostdev.h, csrc/bgmoe_tilemap.h),
+through the g++-built lib/libbgmoe_hostcheck.so: the text the GPU runs, walked on the CPU.
+
+* pointer halves: a wave builtin's `int` low half with bit 31 set must not sign-extend into the high half;
+* launch ranges: lowest / highest byte a strided access touches against its allocation;
+* the balanced (stream-K) GEMM's share walk over random launches: no share without a unit, every unit of work
+  owned exactly once, a cut item's parts in consecutive shares with the first / last share the kernel computes;
+* the K = 64 tile images: a wave's asynchronous loads followed by its operand reads deliver, to every lane, the
+  bytes the 32x32x64 matrix instruction expects from it, without LDS bank conflicts.
+"""
+import ctypes as C
+import os
+import random
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "batchgen_amd", "lib", "libbgmoe_hostcheck.so")
+
+
+@pytest.fixture(scope="module")
+def hc():
+    if not os.path.exists(LIB):                       # nothing built yet: build it (g++, seconds)
+        from batchgen_amd import build as b
+        b.build_hostcheck(verbose=False)
+    lib = C.CDLL(LIB)
+    lib.hc_compose_from_int_halves.restype = C.c_uint64
+    lib.hc_compose_from_int_halves.argtypes = [C.c_int, C.c_int]
+    lib.hc_rows_range_inside.restype = C.c_int
+    lib.hc_rows_range_inside.argtypes = [C.c_uint64] * 6 + [C.POINTER(C.c_uint64)] * 2
+    lib.hc_sk_weights_ok.restype = C.c_int
+    lib.hc_sk_weights_ok.argtypes = [C.POINTER(C.c_int)]
+    lib.hc_sk_walk.restype = C.c_int
+    lib.hc_sk_walk.argtypes = [C.POINTER(C.c_int32), C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                               C.c_int, C.POINTER(C.c_int), C.c_uint, C.c_uint, C.POINTER(C.c_int), C.c_int,
+                               C.POINTER(C.c_uint32)]
+    lib.hc_k64_tile_roundtrip.restype = None
+    lib.hc_k64_tile_roundtrip.argtypes = [C.c_void_p, C.c_uint32, C.c_void_p]
+    lib.hc_k64_tm_tile_roundtrip.restype = None
+    lib.hc_k64_tm_tile_roundtrip.argtypes = [C.c_void_p, C.c_void_p]
+    lib.hc_k64_operand_offsets.restype = None
+    lib.hc_k64_operand_offsets.argtypes = [C.c_void_p, C.c_int]
+    lib.hc_k64_acc_coord.restype = None
+    lib.hc_k64_acc_coord.argtypes = [C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+    return lib
+
+
+def _as_int32(v):
+    return v - (1 << 32) if v >= (1 << 31) else v
+
+
+def test_pointer_halves_do_not_sign_extend(hc):
+    """The device address 0x00007f12_8000_0040 split into halves and handed over as `int` (bit 31 of the low half
+    set: a negative int) comes back whole; so do random 64-bit values."""
+    for v in [0x00007F1280000040, 0x00007FFFFFFFFFF0, 0x0000000080000000, 0xFFFFFFFFFFFFFFFF, 0x00000000FFFFFFFF]:
+        assert hc.hc_compose_from_int_halves(_as_int32(v & 0xFFFFFFFF), _as_int32(v >> 32)) == v
+    rng = random.Random(3)
+    for _ in range(2000):
+        v = rng.getrandbits(64) | (1 << 31)
+        assert hc.hc_compose_from_int_halves(_as_int32(v & 0xFFFFFFFF), _as_int32(v >> 32)) == v
+
+
+def test_launch_byte_range_against_the_allocation(hc):
+    lo, hi = C.c_uint64(), C.c_uint64()
+    base = 0x7F0000000000
+    # 256 rows of 7168 bytes at a pitch of 7168: exactly the allocation
+    assert hc.hc_rows_range_inside(base, 256, 7168, 7168, base, 256 * 7168, lo, hi) == 1
+    assert (lo.value, hi.value) == (base, base + 256 * 7168)
+    # one row too many, one byte too wide, a base in front of the allocation, an empty launch
+    assert hc.hc_rows_range_inside(base, 257, 7168, 7168, base, 256 * 7168, lo, hi) == 0
+    assert hc.hc_rows_range_inside(base, 256, 7169, 7168, base, 256 * 7168, lo, hi) == 0
+    assert hc.hc_rows_range_inside(base - 16, 1, 16, 16, base, 4096, lo, hi) == 0
+    assert hc.hc_rows_range_inside(base + 4096, 0, 64, 64, base, 4096, lo, hi) == 1 and lo.value == hi.value
+    # a pitch larger than the row: the last row ends before the pitch does
+    assert hc.hc_rows_range_inside(base, 4, 64, 1024, base, 3 * 1024 + 64, lo, hi) == 1
+    assert hc.hc_rows_range_inside(base, 4, 64, 1024, base, 3 * 1024 + 63, lo, hi) == 0
+
+
+# ---- the balanced GEMM's share walk ---------------------------------------------------------------------------
+DEFAULT_W = [23, 21, 23, 21, 23, 21, 23, 21]
+COST = (4, 2, 2)
+# local token counts of benchmark configuration 1's routing draw (32 experts) and the shared expert's 256 rows
+CONFIG1_DRAW = [14, 0, 4, 41, 0, 0, 0, 14, 0, 11, 0, 15, 0, 0, 0, 65, 0, 1, 0, 1, 13, 39, 0, 9, 3, 1, 2, 35, 0, 16, 2, 11, 256]
+
+
+def walk(hc, counts, hi, tt, wc, ntiles, kb, grid, w=DEFAULT_W, cost=COST, min_units=8):
+    arr = (C.c_int32 * len(counts))(*counts)
+    w8 = (C.c_int * 8)(*w)
+    cap = 1 << 18
+    out = (C.c_int * (10 * cap))()
+    info = (C.c_uint32 * 4)()
+    n = hc.hc_sk_walk(arr, len(counts), hi, ntiles, kb, tt, wc, cost[0], cost[1], cost[2], w8, grid, min_units, out, cap, info)
+    parts = np.ctypeslib.as_array(out)[: 10 * max(n, 0)].reshape(-1, 10).copy()
+    return n, parts, tuple(info)
+
+
+def check_walk(counts, hi, tt, ntiles, kb, n, parts, info):
+    """Every (group, chunk, slab, K-block) owned exactly once; cut items consistent with first / last share."""
+    c_total, shares, _, _ = info
+    live = [c if 0 <= c <= hi else 0 for c in counts]
+    if not any(live):
+        assert n == 0
+        return
+    assert n > 0, f"share {-n - 1} owns no unit"
+    assert set(parts[:, 0]) == set(range(shares)), "every share owns at least one part"
+    owned = {}
+    per_item = {}
+    for share, grp, ntile, chunk, cnt, kb_lo, kb_hi, first, last, cpk in parts.tolist():
+        assert cnt == live[grp] and 0 <= ntile < ntiles and 0 <= kb_lo < kb_hi <= kb and chunk * 16 * tt < cnt
+        for k in range(kb_lo, kb_hi):
+            assert (grp, chunk, ntile, k) not in owned
+            owned[(grp, chunk, ntile, k)] = share
+        per_item.setdefault((grp, chunk, ntile), []).append((share, kb_lo, kb_hi, first, last))
+    want = sum(((c + 16 * tt - 1) // (16 * tt)) * ntiles * kb for c in live if c)
+    assert len(owned) == want, "units of work missing"
+    heads = set()
+    for item, ps in per_item.items():
+        ps.sort(key=lambda p: p[1])
+        assert ps[0][1] == 0 and ps[-1][2] == kb and all(a[2] == b[1] for a, b in zip(ps, ps[1:]))
+        first, last = ps[0][3], ps[0][4]
+        assert all(p[3] == first and p[4] == last for p in ps), "every part computes the same first / last share"
+        assert [p[0] for p in ps] == list(range(first, last + 1)), "one part in each share from first to last"
+        if len(ps) > 1:                               # the counter of a cut item lives at its first share: one item each
+            assert first not in heads
+            heads.add(first)
+
+
+@pytest.mark.parametrize("shape", [(4, 16, 16, 56, 512), (4, 8, 56, 16, 768)])
+def test_share_walk_of_config_1(hc, shape):
+    """Stage 1 (2048 gate+up columns = 16 slabs, K = 7168) and the down projection (7168 columns = 56 slabs,
+    K = 2048) on configuration 1's draw."""
+    tt, wc, ntiles, kb, grid = shape
+    n, parts, info = walk(hc, CONFIG1_DRAW, 256, tt, wc, ntiles, kb, grid)
+    check_walk(CONFIG1_DRAW, 256, tt, ntiles, kb, n, parts, info)
+    assert info[1] == grid                            # enough work for every resident block
+
+
+def test_share_walk_random_launches(hc):
+    rng = random.Random(1)
+    for _ in range(300):
+        ng = rng.choice([1, 2, 5, 33, 100, 257])
+        hi = rng.choice([16, 64, 256])
+        counts = [rng.choice([0, 0, 1, 3, 16, 17, 64, 65, 200, 256, 300, -1]) for _ in range(ng)]
+        tt, wc = rng.choice([2, 4, 8]), rng.choice([8, 16])
+        ntiles, kb = rng.choice([1, 2, 16, 56]), rng.choice([1, 2, 3, 16, 56])
+        grid = rng.choice([8, 64, 512, 768, 1024])
+        n, parts, info = walk(hc, counts, hi, tt, wc, ntiles, kb, grid)
+        check_walk(counts, hi, tt, ntiles, kb, n, parts, info)
+
+
+def test_share_walk_with_every_accepted_xcd_weighting(hc):
+    """Weights the setter accepts (each in [1, 64], sum <= 32 x the smallest) never leave a share without a unit,
+    however skewed; the weighting the setter now rejects ({1, 64, 64, ...}) does, which is why it is rejected."""
+    rng = random.Random(7)
+    tried = 0
+    while tried < 150:
+        w = [rng.choice([1, 2, 3, 8, 21, 23, 40, 64]) for _ in range(8)]
+        if not hc.hc_sk_weights_ok((C.c_int * 8)(*w)):
+            continue
+        tried += 1
+        counts = [rng.choice([0, 1, 8, 16, 33, 64, 100, 256]) for _ in range(rng.choice([3, 20, 33]))]
+        tt, wc, ntiles, kb, grid = rng.choice([(4, 16, 16, 56, 512), (4, 8, 56, 16, 768), (2, 8, 4, 8, 64)])
+        n, parts, info = walk(hc, counts, 256, tt, wc, ntiles, kb, grid, w=w)
+        check_walk(counts, 256, tt, ntiles, kb, n, parts, info)
+    for w in ([1] + [64] * 7, [64] * 7 + [1], [0] + [8] * 7, [65] + [8] * 7):
+        assert not hc.hc_sk_weights_ok((C.c_int * 8)(*w))
+    assert hc.hc_sk_weights_ok((C.c_int * 8)(*DEFAULT_W))
+    bad = [1] + [64] * 7
+    starved = False
+    for counts in ([16] * 32, CONFIG1_DRAW, [1] * 8, [64] * 20):
+        for tt, wc, ntiles, kb, grid in [(4, 16, 16, 56, 512), (4, 8, 56, 16, 768)]:
+            n, _, _ = walk(hc, counts, 256, tt, wc, ntiles, kb, grid, w=bad)
+            starved = starved or n < 0
+    assert starved, "the rejected weighting was expected to starve a share on at least one of these launches"
+
+
+# ---- predicted weight traffic of the two work orders --------------------------------------------------------------
+def restream_model(hc, counts, tt, wc, ntiles, kb, grid, tile_bytes=2048, window_bytes=4 << 20):
+    """Weight bytes the balanced launch takes from HBM, under a simple L2 model: shares advance through their cost at
+    the same rate; a re-stream (chunk > 0) of a slab's K-block is an L2 hit when the same (group, slab, K-block) is
+    streamed by a share of the SAME XCD at a time (= cost offset inside the share) no further away than the time
+    the XCD needs to replace its 4 MiB L2.  Returns (first-stream bytes, re-stream bytes from HBM, from L2)."""
+    n, parts, info = walk(hc, counts, 256, tt, wc, ntiles, kb, grid)
+    assert n > 0
+    _, shares, n8, _ = info
+    # time of every unit = running cost inside its share (every share advances one cost unit per unit of time)
+    clock = {s: 0 for s in range(shares)}
+    when = {}
+    for share, grp, ntile, chunk, cnt, kb_lo, kb_hi, first, last, cpk in parts.tolist():
+        for k in range(kb_lo, kb_hi):
+            when[(grp, chunk, ntile, k)] = (share // n8 if shares >= 8 else 0, clock[share])
+            clock[share] += cpk
+    # an XCD's n8 shares move n8 cost units per unit of time; a first-stream weight tile is COST[0] cost units
+    window = window_bytes / (n8 * tile_bytes / COST[0])
+    first_b = hbm_b = l2_b = 0
+    for (grp, chunk, ntile, k), (xcd, t) in when.items():
+        nbytes = wc * tile_bytes
+        if chunk == 0:
+            first_b += nbytes
+            continue
+        hit = any((grp, c2, ntile, k) in when and when[(grp, c2, ntile, k)][0] == xcd and
+                  abs(when[(grp, c2, ntile, k)][1] - t) <= window for c2 in range(chunk))
+        if hit:
+            l2_b += nbytes
+        else:
+            hbm_b += nbytes
+    return first_b, hbm_b, l2_b
+
+
+def test_restream_model_of_the_current_cut(hc):
+    """What the chunk-by-chunk work order of the balanced launch costs in weight traffic on configuration 1's
+    draw (64-row chunks: the group of 65 rows has two, the shared expert's 256 rows four) and on 32 groups of 16
+    rows (none): with
+    single-chunk groups nothing is streamed twice; with multi-chunk groups the later chunks of a slab run a whole
+    chunk's cost later than the first, far outside one L2's reach, so every re-stream comes from HBM.  This is
+    the traffic that the item walk of the default kernel avoids by running a slab's chunks side by side."""
+    first_b, hbm_b, l2_b = restream_model(hc, [16] * 32, 4, 16, 16, 56, 512)
+    assert hbm_b == 0 and l2_b == 0 and first_b == 32 * 2 * 2048 * 7168          # every gate+up byte once
+    first_b, hbm_b, l2_b = restream_model(hc, CONFIG1_DRAW, 4, 16, 16, 56, 512)
+    active = sum(1 for c in CONFIG1_DRAW if c)
+    assert first_b == active * 2 * 2048 * 7168
+    chunks_more = sum((c + 63) // 64 - 1 for c in CONFIG1_DRAW if c)
+    assert hbm_b + l2_b == chunks_more * 2 * 2048 * 7168
+    # 4 more chunks (65 rows: 1, the shared expert's 256 rows: 3) on 21 active groups: 19% more weight bytes, and
+    # nine tenths of them come from HBM again
+    assert hbm_b / (hbm_b + l2_b) > 0.85 and hbm_b / first_b > 0.15, "the chunk-major order re-streams from HBM"
+
+
+# ---- K = 64 tile images ----------------------------------------------------------------------------------------------
+def test_k64_row_major_tile_image(hc):
+    """32 rows x 64 bytes at a pitch of 7168: after the two half-image loads, lane l's operand is row l % 32,
+    bytes 32 * (l / 32) .. + 32 of the row's 64."""
+    rng = np.random.default_rng(5)
+    pitch = 7168
+    src = rng.integers(0, 256, size=(32, pitch), dtype=np.uint8)
+    got = np.zeros((64, 32), dtype=np.uint8)
+    hc.hc_k64_tile_roundtrip(src.ctypes.data, pitch, got.ctypes.data)
+    for lane in range(64):
+        row, h = lane % 32, lane // 32
+        assert np.array_equal(got[lane], src[row, 32 * h: 32 * h + 32]), lane
+
+
+def test_k64_tile_major_tile_image(hc):
+    """Two 16-row tiles in the resident tile-major order ([K half][16-byte piece][row] per 2 KiB tile): the K half
+    that the step uses is one contiguous KiB per tile, copied linearly; lane l's operand is again row l % 32, bytes
+    32 * (l / 32) .. + 32 of the step's 64."""
+    rng = np.random.default_rng(6)
+    rows = rng.integers(0, 256, size=(32, 128), dtype=np.uint8)          # 32 weight rows x one 128-wide K-block
+    tiles = np.zeros((2, 2, 4, 16, 16), dtype=np.uint8)                   # [tile][K half][piece][row][byte]
+    for t in range(2):
+        for kh in range(2):
+            for q in range(4):
+                for r in range(16):
+                    tiles[t, kh, q, r] = rows[16 * t + r, 64 * kh + 16 * q: 64 * kh + 16 * q + 16]
+    for kh in range(2):
+        halves = np.ascontiguousarray(tiles[:, kh]).reshape(2, 1024)      # the two KiB the step loads
+        got = np.zeros((64, 32), dtype=np.uint8)
+        hc.hc_k64_tm_tile_roundtrip(halves.ctypes.data, got.ctypes.data)
+        for lane in range(64):
+            row, h = lane % 32, lane // 32
+            assert np.array_equal(got[lane], rows[row, 64 * kh + 32 * h: 64 * kh + 32 * h + 32]), (kh, lane)
+
+
+@pytest.mark.parametrize("tile_major", [0, 1])
+def test_k64_operand_reads_have_no_bank_conflicts(hc, tile_major):
+    """A 16-byte read occupies 4 of the 64 four-byte banks; any 8 consecutive lanes of one read instruction (what
+    the LDS serves per clock at 128 B/clk) must fall into 8 different 16-byte groups of the 256-byte bank row."""
+    offs = np.zeros(128, dtype=np.uint32)
+    hc.hc_k64_operand_offsets(offs.ctypes.data, tile_major)
+    for which in (offs[:64], offs[64:]):
+        assert np.all(which % 16 == 0) and which.max() < 2048
+        for g0 in range(0, 64, 8):
+            groups = (which[g0: g0 + 8] // 16) % 16
+            assert len(set(groups.tolist())) == 8, (tile_major, g0, groups)
+    assert len(set(offs.tolist())) == 128, "the 64 lanes' two pieces are 128 different pieces of the image"
+
+
+def test_accumulator_coordinates_cover_the_32x32_product(hc):
+    a, b = C.c_uint32(), C.c_uint32()
+    seen = set()
+    for lane in range(64):
+        for v in range(16):
+            hc.hc_k64_acc_coord(lane, v, a, b)
+            assert b.value == lane % 32 and a.value == 8 * (v // 4) + 4 * (lane // 32) + v % 4
+            seen.add((a.value, b.value))
+    assert len(seen) == 1024
