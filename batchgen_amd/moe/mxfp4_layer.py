@@ -5,13 +5,14 @@ Host-side counterpart of ``ResidentEPMXFP4MoELayer._expert_path`` / ``forward``
 ungrouped sigmoid top-k router -> masked dispatch of bf16 rows -> grouped MXFP4 gate_up + activation ->
 grouped MXFP4 down -> fp32 weighted combine + shared expert.  Weights are repacked once into the
 tile-major resident layout (the reference repacks to Marlin at the same point, :13-15).
-The shared expert is a plain dense bf16 MLP and runs on the library GEMM (hipBLASLt through torch).
+The shared expert is a plain dense bf16 MLP on this library's own bf16 GEMM (``bgmoe_bf16_linear``); the vendor
+library through ``torch.mm`` is an explicit option kept for comparison.
 
 With ``latent`` weights the layer is the Kimi-K3 latent MoE (:922-944, kimi_linear/model.py:585-603): the
 router sees the hidden rows, ``down_proj`` takes them to the latent width once per token, the experts and
 the combine work on latent rows, then RMSNorm (optional) and ``up_proj`` bring the result back, and the
-shared expert's output is added.  The two projections are plain bf16 GEMMs and run on the library GEMM, as
-``nn.Linear`` does in the reference.  ``activation="situ"`` selects the K3 activation for the routed experts
+shared expert's output is added.  The two projections are plain bf16 GEMMs (``nn.Linear`` in the reference) on
+the same ``bgmoe_bf16_linear``.  ``activation="situ"`` selects the K3 activation for the routed experts
 (fused into the stage-1 GEMM) and the shared expert (``situ_and_mul``).
 """
 from __future__ import annotations
@@ -51,23 +52,18 @@ ACTIVATIONS = {"swiglu": 0, "situ": 1}
 K3_SITU_BETA, K3_SITU_LINEAR_BETA = 4.0, 25.0   # the constants the fused stage-1 epilogue compiles in
 
 
-# dense_backend="auto": rows up to which the library's bf16 GEMM serves the shared expert and the latent projections.
-# Measured on MI355X against the vendor GEMM: 64 rows 7168 -> 4096 24.5 vs 20.3 us and 2048 -> 7168 14.2 vs 22.1 us
-# (the pair 38.7 vs 42.4 us); 512 rows 85 vs 44 us and 50 vs 22 us.
-DENSE_HIP_MAX_ROWS = 64
-
-
 class Mxfp4MoELayer:
     def __init__(self, cfg: MoEConfig, weights, shared_bf16, bias: torch.Tensor, shared_mode: str = "bf16_add",
-                 latent=None, dense_backend: str = "auto"):
-        """``dense_backend``: "hip" runs the bf16 shared expert and the latent projections on this library's own
-        bf16 GEMM; "vendor" runs them on the vendor library through ``torch.mm``, as ``nn.Linear`` in the reference
-        does; "auto" (the default) takes this library's GEMM for calls of up to ``DENSE_HIP_MAX_ROWS`` tokens,
-        where it was measured to be the faster one, and the vendor's above.  Either way the results go into
-        buffers owned by the layer: ``forward`` allocates no tensor, and what it returns is one of those buffers,
+                 latent=None, dense_backend: str = "hip"):
+        """``dense_backend``: "hip" (the default) runs the bf16 shared expert and the latent projections on this
+        library's own bf16 GEMM, so that the whole layer is this library's kernels and a token's result does not
+        depend on its position in the batch; "vendor" runs them on the vendor library through ``torch.mm``, as
+        ``nn.Linear`` in the reference does (faster at 512 tokens: measured 45 + 35 us against 2 x 92 us for the
+        shared expert; kept for that comparison, never chosen silently).  Either way the results go into buffers
+        owned by the layer: ``forward`` allocates no tensor, and what it returns is one of those buffers,
         overwritten by the next call."""
-        if dense_backend not in ("auto", "hip", "vendor"):
-            raise ValueError(f"dense_backend must be 'auto', 'hip' or 'vendor', got {dense_backend!r}")
+        if dense_backend not in ("hip", "vendor"):
+            raise ValueError(f"dense_backend must be 'hip' or 'vendor', got {dense_backend!r}")
         self.dense_backend = dense_backend
         self.cfg = cfg
         dev = weights["gate_p"].device
@@ -133,14 +129,12 @@ class Mxfp4MoELayer:
         self._fn = lib().bgmoe_moe_mxfp4_layer_forward
         # buffers of the dense bf16 parts (shared expert, latent projections): forward() allocates none of them
         hid = cfg.hidden
-        use_hip = dense_backend != "vendor"
-
-        rows_hip = n if dense_backend == "hip" else min(n, DENSE_HIP_MAX_ROWS)
+        use_hip = dense_backend == "hip"
 
         def ws(nn, hh, ee):
             if not use_hip:
                 return None
-            return torch.empty(bf16_linear_workspace_bytes(rows_hip, hh, ee), dtype=torch.uint8, device=dev)
+            return torch.empty(bf16_linear_workspace_bytes(nn, hh, ee), dtype=torch.uint8, device=dev)
         d = {}
         if shared_bf16 is not None:
             si2 = self._shared_gate_up.size(0)
@@ -157,7 +151,7 @@ class Mxfp4MoELayer:
 
     def _linear(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, workspace) -> torch.Tensor:
         """``x @ w^T`` into ``out``: this library's bf16 GEMM, or the vendor library's through ``torch.mm``."""
-        if self.dense_backend == "hip" or (self.dense_backend == "auto" and x.size(0) <= DENSE_HIP_MAX_ROWS):
+        if self.dense_backend == "hip":
             return bf16_linear(x, w, out, workspace)
         return torch.mm(x, w.t(), out=out)
 

@@ -85,9 +85,9 @@ def parse():
     ap.add_argument("--rows", type=int, default=0, help="--op dense_expert: rows per step (default: the "
                                                         "configuration's token count)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--dense-backend", default=None, choices=["auto", "hip", "vendor"],
+    ap.add_argument("--dense-backend", default=None, choices=["hip", "vendor"],
                     help="MXFP4 configurations: the bf16 shared expert and latent projections on this library's "
-                         "bf16 GEMM (hip) or on the vendor library through F.linear (vendor); default: the layer's")
+                         "bf16 GEMM (hip, the layer's default) or on the vendor library through torch.mm (vendor)")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of one captured HIP graph of the layer instead of eager launches")
     ap.add_argument("--copy-calibration", action="store_true",

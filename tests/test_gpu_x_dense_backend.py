@@ -1,6 +1,6 @@
 """The bf16 dense parts of the MXFP4 layer (shared expert, latent projections) on this library's own kernels:
 ``bgmoe_bf16_linear`` against fp32, ``bgmoe_silu_and_mul`` bit for bit against the oracle, and the layer with its
-dense parts on the library's GEMM, on the vendor's, and on the automatic choice between them."""
+dense parts on the library's GEMM (the default) and on the vendor's."""
 import numpy as np
 import pytest
 import torch
@@ -44,12 +44,12 @@ def test_dense_backends_agree_and_hip_allocates_nothing(dev, latent):
     assert torch.equal(y.float().cpu(), a)
     a17 = hip(x17, l17).float().cpu()
     assert float((a17 - a[:17]).norm() / a[:17].norm()) < 4e-3      # another launch shape of the routed kernels
-    # "auto": the vendor GEMM at 96 tokens, this library's at 17 (<= DENSE_HIP_MAX_ROWS)
-    auto = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat)
-    assert auto.dense_backend == "auto"
-    c = auto(inp["x"], inp["logits"]).float().cpu()
-    assert float((c - b).norm() / b.norm()) < 4e-3
-    assert torch.equal(auto(x17, l17).float().cpu(), a17)
+    # the default is this library's own GEMM: nothing of the layer runs on the vendor library unless asked for
+    default = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat)
+    assert default.dense_backend == "hip"
+    assert torch.equal(default(inp["x"], inp["logits"]).float().cpu(), a)
+    with pytest.raises(ValueError):
+        Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat, dense_backend="auto")
 
 
 @pytest.mark.parametrize("n,h,e", [(1, 512, 8), (17, 1024, 512), (96, 7168, 260), (300, 2048, 1024), (512, 1024, 4096)])
