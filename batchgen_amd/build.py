@@ -72,26 +72,51 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
-# Kernels whose weight loads are issued from inline asm and waited for by hand: a register that such a load is
-# still writing must never be spilled or copied, so these files must compile without scratch memory.
-NO_SPILL = {"gemm_fp8_streamk.hip": "fp8_streamk_kernel"}
+# Kernels whose loads are issued from inline asm and waited for by hand: a register that such a load is still
+# writing must never be spilled or copied, so these kernels must compile without scratch memory.  The LDS-tiled
+# K = 64 kernel must also keep two waves per SIMD (at most 256 registers, no AGPR copies of its accumulators) and
+# leave room for its 4 x 33 KB ring in the CU's 160 KB of LDS.  Checked on every build from the compiler's own
+# resource remarks; a kernel over budget fails the build.
+RESOURCE_GATES = {
+    "gemm_fp8_streamk.hip": dict(kernel="fp8_streamk_kernel"),
+    "gemm_fp8_tiled_k64.hip": dict(kernel="fp8_tiled_k64_kernel", max_vgprs=256, max_agprs=0,
+                                   max_static_lds=163840 - 4 * (32768 + 1024), min_occupancy=2),
+}
+NO_SPILL = RESOURCE_GATES           # (the name the compile step tests membership with)
 
 
 def _check_no_spill(src: str, remarks: str, obj: str) -> None:
     import re
+    gate = RESOURCE_GATES[src]
+    fields = {"ScratchSize [bytes/lane]": ("scratch", lambda v: v == 0, "must be 0"),
+              "VGPRs": ("max_vgprs", None, None), "AGPRs": ("max_agprs", None, None),
+              "LDS Size [bytes/block]": ("max_static_lds", None, None),
+              "Occupancy [waves/SIMD]": ("min_occupancy", None, None)}
     name, bad, seen = None, [], 0
     for line in remarks.splitlines():
         m = re.search(r"Function Name: (\S+)", line)
         if m:
             name = m.group(1)
-        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
-        if m and name and NO_SPILL[src] in name:
+            continue
+        if not name or gate["kernel"] not in name:
+            continue
+        m = re.search(r"remark:\s+([A-Za-z \[\]/]+?): (\d+)", line)
+        if not m or m.group(1) not in fields:
+            continue
+        key, _, _ = fields[m.group(1)]
+        value = int(m.group(2))
+        if key == "scratch":
             seen += 1
-            if int(m.group(1)) != 0:
-                bad.append(f"{name}: {m.group(1)} bytes of scratch per lane")
+            if value != 0:
+                bad.append(f"{name}: {value} bytes of scratch per lane")
+        elif key in gate:
+            limit = gate[key]
+            over = value < limit if key.startswith("min_") else value > limit
+            if over:
+                bad.append(f"{name}: {m.group(1)} = {value}, limit {limit}")
     if bad or seen == 0:
         os.remove(obj)
-        raise RuntimeError(f"{src}: kernels must not spill registers ({'; '.join(bad) or 'no resource remarks found'})")
+        raise RuntimeError(f"{src}: kernel resource budget violated ({'; '.join(bad) or 'no resource remarks found'})")
 
 
 # ---- PyTorch C++ extension modules (host code over the C ABI) --------------------------------------------------

@@ -31,6 +31,14 @@ BGMOE_HD uint32_t bgmoe_k64_load_src_offset(uint32_t lane, uint32_t half, uint32
   return row * pitch + (((lane & 3u) ^ bgmoe_k64_swizzle(row)) << 4);
 }
 BGMOE_HD uint32_t bgmoe_k64_load_lds_offset(uint32_t lane, uint32_t half) { return 1024u * half + 16u * lane; }
+// the same for token image `image` of a macro tile whose group has only rows 0 .. last_row of the tile left: rows
+// past the end re-read the last row (their products are never stored); the swizzle follows the image row, not the
+// row that is read
+BGMOE_HD uint32_t bgmoe_k64_token_src_offset(uint32_t lane, uint32_t half, uint32_t image, uint32_t last_row, uint32_t pitch) {
+  const uint32_t img_row = 16u * half + (lane >> 2);
+  const uint32_t tok = 32u * image + img_row;
+  return (tok < last_row ? tok : last_row) * pitch + (((lane & 3u) ^ bgmoe_k64_swizzle(img_row)) << 4);
+}
 // the two 16-byte pieces lane `lane` feeds to the matrix instruction: row lane % 32, pieces 2h and 2h + 1 of K half
 // h = lane / 32
 BGMOE_HD uint32_t bgmoe_k64_operand_lo(uint32_t lane) {
@@ -59,3 +67,25 @@ BGMOE_HD uint32_t bgmoe_k64_tm_operand_hi(uint32_t lane) {
 // from the second (tokens: the output row)
 BGMOE_HD uint32_t bgmoe_mfma32_acc_a_row(uint32_t lane, uint32_t v) { return 8u * (v >> 2) + 4u * (lane >> 5) + (v & 3u); }
 BGMOE_HD uint32_t bgmoe_mfma32_acc_b_row(uint32_t lane) { return lane & 31u; }
+
+// ---- block geometry of the K = 64 kernel -------------------------------------------------------------------------------
+// Macro tile: 256 tokens x 256 weight rows (fused stage 1: 128 gate + 128 up rows = 128 output columns), 8 waves =
+// 4 (weight rows: wn) x 2 (tokens: wm).  A ring slot holds one K-step of 64 bytes: 8 token images (image i = tokens
+// 32 i .. 32 i + 31 of the macro tile) and 8 weight images (plain: rows 32 i ..; fused: images 0..3 = gate rows
+// 32 i .., images 4..7 = up rows 32 (i - 4) ..).  Wave w loads token image w and weight image w.
+BGMOE_HD uint32_t bgmoe_k64_wave_wn(uint32_t wave) { return wave & 3u; }
+BGMOE_HD uint32_t bgmoe_k64_wave_wm(uint32_t wave) { return wave >> 2; }
+// weight image a (0, 1) and token image b (0..3) that wave (wn, wm) multiplies
+BGMOE_HD uint32_t bgmoe_k64_a_image(bool fused, uint32_t wn, uint32_t a) { return fused ? 4u * a + wn : 2u * wn + a; }
+BGMOE_HD uint32_t bgmoe_k64_b_image(uint32_t wm, uint32_t b) { return 4u * wm + b; }
+// first weight row of image i relative to the macro tile's first row n0, and the matrix it comes from (fused: 0 gate, 1 up)
+BGMOE_HD uint32_t bgmoe_k64_image_wrow(bool fused, uint32_t image) { return fused ? 32u * (image & 3u) : 32u * image; }
+BGMOE_HD uint32_t bgmoe_k64_image_matrix(bool fused, uint32_t image) { return fused ? image >> 2 : 0u; }
+// where accumulator register v of lane `lane` of product (b, a) belongs: token and output column relative to the
+// macro tile's (m0, n0).  Fused: products a = 0 (gate) and a = 1 (up) of one b hold the SAME (token, column): SwiGLU
+// pairs them in the lane.
+BGMOE_HD uint32_t bgmoe_k64_out_token(uint32_t wm, uint32_t b, uint32_t lane) { return 128u * wm + 32u * b + (lane & 31u); }
+BGMOE_HD uint32_t bgmoe_k64_out_col(bool fused, uint32_t wn, uint32_t a, uint32_t lane, uint32_t v) {
+  const uint32_t r = bgmoe_mfma32_acc_a_row(lane, v);
+  return fused ? 32u * wn + r : 64u * wn + 32u * a + r;
+}

@@ -22,11 +22,12 @@
 // work items ordered so that the blocks of one XCD (block b runs on XCD b % 8) work on a compact patch
 // of m- and n-tiles and share their operands through that XCD's L2.  Groups at or below the row limit
 // of bgmoe_split_limit() are left to the weight-streaming kernel; empty groups cost nothing.
-#include "bgmoe_common.h"
-#include "bgmoe_sched.h"
+#include "gemm_fp8_tiled.h"
 #include "bgmoe_async.h"
 
 namespace {
+
+using TiledArgs = BgmoeTiledArgs;
 
 constexpr int TM = 256;            // tokens per macro tile
 constexpr int TW = 256;            // weight rows per macro tile
@@ -37,21 +38,8 @@ constexpr int kWBytes = TW * 128;
 constexpr int kXsOff = kTokBytes + kWBytes;
 constexpr int kSlotBytes = kXsOff + TM * 4;
 constexpr int kPanel = 8;          // m-tiles per panel of the work-item order
-constexpr int kMaxGroups = 1024;
-constexpr int kMaxKB = 256;        // K <= 32768
-
-struct TiledArgs {
-  bgmoe_fp8_act a;
-  bgmoe_fp8_weight w0, w1;
-  const int32_t* seqlens;
-  const int32_t* cu;
-  int groups, n, k;
-  uint16_t* out;
-  uint8_t* out_q;
-  float* out_s;
-  int64_t os_row, os_nb;
-  BgmoeSplit split;
-};
+constexpr int kMaxGroups = kBgmoeTiledMaxGroups;
+constexpr int kMaxKB = kBgmoeTiledMaxKB;        // K <= 32768
 
 template <bool FUSED, int LAYOUT>
 __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
@@ -435,8 +423,18 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
 }
 
 int g_num_cu = 0;
+int g_variant = 0;                 // 0: this file's K = 128 kernel; 1: the K = 64 kernel where it applies
 
 }  // namespace
+
+// Which LDS-tiled kernel serves the groups above the streaming limit (no reference counterpart): 0 = the K = 128
+// kernel (16x16x128 products, two 65 KB ring slots), 1 = the K = 64 kernel (32x32x64 products accumulated in
+// place, four 33 KB slots) for K >= 256, the K = 128 kernel otherwise.  Results of the two differ in rounding only.
+extern "C" int bgmoe_set_tiled_variant(int variant) {
+  BGMOE_REQUIRE(variant == 0 || variant == 1, "set_tiled_variant: variant must be 0 (K = 128) or 1 (K = 64), got %d", variant);
+  g_variant = variant;
+  return BGMOE_OK;
+}
 
 // device query and the dynamic-LDS opt-in of every variant, once
 int bgmoe_internal_init_fp8_tiled() {
@@ -495,6 +493,10 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   if (blocks > max_items) blocks = max_items;
   if (blocks < 8) blocks = 8;
   BgmoeProf prof(w1 ? BGMOE_K_S1_TILED : BGMOE_K_GEMM_TILED, st);
+  if (g_variant == 1) {
+    const int rc = bgmoe_launch_fp8_tiled_k64(g, w1 != nullptr, m, g_num_cu, st);
+    if (rc != BGMOE_ERR_WORKSPACE) return rc;            // (without a message: the variant does not apply here)
+  }
   const dim3 grid((unsigned)blocks), block(NT);
   const bool tm = w0->layout == BGMOE_W_TILE_MAJOR;
   if (w1) {

@@ -5,6 +5,7 @@
 // way the kernels call them, and hands the result to a test that checks invariants (every unit of work owned
 // exactly once, no share without work, addresses inside their buffers, operand bytes where the matrix
 // instruction expects them).
+#include <math.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -135,6 +136,148 @@ void hc_k64_operand_offsets(uint32_t* out, int tile_major) {
 void hc_k64_acc_coord(uint32_t lane, uint32_t v, uint32_t* a_row, uint32_t* b_row) {
   *a_row = bgmoe_mfma32_acc_a_row(lane, v);
   *b_row = bgmoe_mfma32_acc_b_row(lane);
+}
+
+
+// ---- the K = 64 kernel's dataflow on one macro tile ----------------------------------------------------------------
+// Walks what fp8_tiled_k64_kernel does for ONE work item with the kernel's own maps (bgmoe_tilemap.h): per K-step
+// every wave's asynchronous loads into a ring slot (token image `wave`, weight image `wave`, clamped rows, swizzle
+// or tile-major order), every wave's operand reads, the 32x32x64 products accumulated in place with the scale
+// change at even steps, and the epilogue's (token, column) of every accumulator register.  The matrix instruction
+// itself is taken from its definition: lane l supplies row l % 32 and K half l / 32 of each operand, register v of
+// lane l receives D[8 (v / 4) + 4 (l / 32) + v % 4][l % 32].
+//
+// x: the group's tokens [cnt][K] e4m3 bytes, xs [cnt][KB] scales; w0 (and w1 when fused): [n][K] bytes, row-major or
+// tile-major; ws0 / ws1: the K-row of weight scales per 128-row block [n / 128][KB]; (m0, n0): the macro tile.
+// out [cnt][ncols_total] and written [cnt][ncols_total] (1 where the kernel stores): fused: ncols_total = n (values
+// silu(gate) * up before the bf16 rounding); plain: n.  Returns 0, or a negative number when an address left its
+// buffer.
+static float e4m3_to_float(uint8_t b) {
+  const int sign = b >> 7, e = (b >> 3) & 15, m = b & 7;
+  float v;
+  if (e == 0) v = ldexpf((float)m / 8.0f, -6);
+  else if (e == 15 && m == 7) v = NAN;
+  else v = ldexpf(1.0f + (float)m / 8.0f, e - 7);
+  return sign ? -v : v;
+}
+
+int hc_k64_emulate_item(const uint8_t* x, const float* xs, int cnt, int K, const uint8_t* w0, const uint8_t* w1,
+                        const float* ws0, const float* ws1, int n, int fused, int tile_major, int m0, int n0, float* out,
+                        uint8_t* written) {
+  const int KB = K / 128, steps = 2 * KB;
+  const bool F = fused != 0;
+  float dec[256];
+  for (int i = 0; i < 256; ++i) dec[i] = e4m3_to_float((uint8_t)i);
+  const uint64_t x_bytes = (uint64_t)cnt * K, w_bytes = (uint64_t)n * K;
+  std::vector<uint8_t> slot(2 * 8 * BGMOE_K64_TILE_BYTES);            // tokens, then weights
+  std::vector<float> acc(8 * 64 * 4 * 2 * 16, 0.0f), prev(8 * 64 * 4 * 2, 0.0f);   // [wave][lane][b][a][v]
+  auto ACC = [&](uint32_t wave, uint32_t lane, int b, int a, int v) -> float& {
+    return acc[((((size_t)wave * 64 + lane) * 4 + b) * 2 + a) * 16 + v];
+  };
+  auto PREV = [&](uint32_t wave, uint32_t lane, int b, int a) -> float& { return prev[(((size_t)wave * 64 + lane) * 4 + b) * 2 + a]; };
+  const uint32_t last = (uint32_t)(cnt - 1 - m0);
+  for (int ks = 0; ks < steps; ++ks) {
+    // ---- loads ----
+    memset(slot.data(), 0xEE, slot.size());
+    for (uint32_t wave = 0; wave < 8; ++wave) {
+      const int nrow_raw = n0 + (int)bgmoe_k64_image_wrow(F, wave);
+      const int nrow = nrow_raw < n - 32 ? nrow_raw : n - 32;
+      const uint8_t* wbase = bgmoe_k64_image_matrix(F, wave) ? w1 : w0;
+      for (uint32_t h = 0; h < 2; ++h)
+        for (uint32_t lane = 0; lane < 64; ++lane) {
+          const uint64_t src = (uint64_t)m0 * K + (uint64_t)ks * 64 + bgmoe_k64_token_src_offset(lane, h, wave, last, (uint32_t)K);
+          if (src + 16 > x_bytes) return -1;
+          memcpy(&slot[wave * BGMOE_K64_TILE_BYTES + bgmoe_k64_load_lds_offset(lane, h)], x + src, 16);
+          uint64_t wsrc;
+          if (tile_major) wsrc = (uint64_t)((nrow >> 4) + (int)h) * K * 16 + (uint64_t)ks * 1024 + lane * 16u;
+          else wsrc = (uint64_t)nrow * K + (uint64_t)ks * 64 + bgmoe_k64_load_src_offset(lane, h, (uint32_t)K);
+          if (wsrc + 16 > w_bytes) return -2;
+          memcpy(&slot[(8 + wave) * BGMOE_K64_TILE_BYTES + bgmoe_k64_load_lds_offset(lane, h)], wbase + wsrc, 16);
+        }
+    }
+    // ---- compute ----
+    const int kb = ks >> 1;
+    for (uint32_t wave = 0; wave < 8; ++wave) {
+      const uint32_t wn = bgmoe_k64_wave_wn(wave), wm = bgmoe_k64_wave_wm(wave);
+      if (!(m0 + 128 * (int)wm < cnt)) continue;                       // the kernel's wave_live
+      if ((ks & 1) == 0) {
+        const int nb0 = (n0 >> 7), nb1 = ((n0 + 128 < n ? n0 + 128 : n - 1) >> 7);
+        const float wsc0 = F ? ws0[(size_t)nb0 * KB + kb] : ws0[(size_t)nb0 * KB + kb];
+        const float wsc1 = F ? ws1[(size_t)nb0 * KB + kb] : ws0[(size_t)nb1 * KB + kb];
+        const float wa0 = F ? wsc0 : (wn >= 2u ? wsc1 : wsc0), wa1 = F ? wsc1 : wa0;
+        for (uint32_t lane = 0; lane < 64; ++lane)
+          for (int b = 0; b < 4; ++b) {
+            uint32_t t = bgmoe_k64_out_token(wm, b, lane);             // token scale the lane reads (clamped like the load)
+            const uint32_t tc = t < last ? t : last;
+            const float s = xs[(size_t)(m0 + tc) * KB + kb];
+            const float c[2] = {s * wa0, s * wa1};
+            for (int a = 0; a < 2; ++a) {
+              if (kb > 0) {
+                const float r = PREV(wave, lane, b, a) * (1.0f / c[a]);
+                for (int v = 0; v < 16; ++v) ACC(wave, lane, b, a, v) *= r;
+              }
+              PREV(wave, lane, b, a) = c[a];
+            }
+          }
+      }
+      // operands as the lanes read them
+      uint8_t A[2][64][32], B[4][64][32];
+      for (uint32_t lane = 0; lane < 64; ++lane) {
+        for (int a = 0; a < 2; ++a) {
+          const uint8_t* img = &slot[(8 + bgmoe_k64_a_image(F, wn, a)) * BGMOE_K64_TILE_BYTES];
+          memcpy(A[a][lane], img + (tile_major ? bgmoe_k64_tm_operand_lo(lane) : bgmoe_k64_operand_lo(lane)), 16);
+          memcpy(A[a][lane] + 16, img + (tile_major ? bgmoe_k64_tm_operand_hi(lane) : bgmoe_k64_operand_hi(lane)), 16);
+        }
+        for (int b = 0; b < 4; ++b) {
+          const uint8_t* img = &slot[bgmoe_k64_b_image(wm, b) * BGMOE_K64_TILE_BYTES];
+          memcpy(B[b][lane], img + bgmoe_k64_operand_lo(lane), 16);
+          memcpy(B[b][lane] + 16, img + bgmoe_k64_operand_hi(lane), 16);
+        }
+      }
+      for (int b = 0; b < 4; ++b)
+        for (int a = 0; a < 2; ++a) {
+          float D[32][32];
+          for (int i = 0; i < 32; ++i)
+            for (int j = 0; j < 32; ++j) {
+              double sum = 0.0;
+              for (int h = 0; h < 2; ++h)
+                for (int k = 0; k < 32; ++k)
+                  sum += (double)dec[A[a][i + 32 * h][k]] * (double)dec[B[b][j + 32 * h][k]];
+              D[i][j] = (float)sum;
+            }
+          for (uint32_t lane = 0; lane < 64; ++lane)
+            for (uint32_t v = 0; v < 16; ++v)
+              ACC(wave, lane, b, a, (int)v) += D[bgmoe_mfma32_acc_a_row(lane, v)][bgmoe_mfma32_acc_b_row(lane)];
+        }
+    }
+  }
+  // ---- epilogue ----
+  for (uint32_t wave = 0; wave < 8; ++wave) {
+    const uint32_t wn = bgmoe_k64_wave_wn(wave), wm = bgmoe_k64_wave_wm(wave);
+    for (uint32_t lane = 0; lane < 64; ++lane)
+      for (int b = 0; b < 4; ++b) {
+        const int tok = m0 + (int)bgmoe_k64_out_token(wm, b, lane);
+        if (tok >= cnt) continue;
+        for (int a = 0; a < (F ? 1 : 2); ++a)
+          for (uint32_t v = 0; v < 16; ++v) {
+            const int col = n0 + (int)bgmoe_k64_out_col(F, wn, (uint32_t)a, lane, v);
+            if (col >= n) continue;
+            float val;
+            if (F) {
+              const float gt = ACC(wave, lane, b, 0, (int)v) * PREV(wave, lane, b, 0);
+              const float up = ACC(wave, lane, b, 1, (int)v) * PREV(wave, lane, b, 1);
+              val = gt / (1.0f + expf(-gt)) * up;
+            } else {
+              val = ACC(wave, lane, b, a, (int)v) * PREV(wave, lane, b, a);
+            }
+            const size_t o = (size_t)tok * n + col;
+            if (written[o]) return -3;                                  // two registers claim one output element
+            written[o] = 1;
+            out[o] = val;
+          }
+      }
+  }
+  return 0;
 }
 
 }  // extern "C"

@@ -445,6 +445,15 @@ int bgmoe_fp8_dense_gemm_partials(const bgmoe_fp8_act* a, const uint8_t* w, cons
                                   int64_t scale_nb_stride, int layout, int64_t m, int n, int k, void* workspace,
                                   int64_t workspace_bytes, int* slices, bgmoe_stream_t stream);
 
+/* Which LDS-tiled kernel serves the groups above the streaming limit (tuning switch, no reference counterpart;
+ * the reference's own tile choice is `num_seq_per_group_avg` -> TileM, batchgen/moe/grouped_fp8_blockwise_moe.py:143-190):
+ * 0 (default) = K steps of 128 bytes, 16x16x128 products promoted with one fma per accumulator and scale block,
+ * two 65 KB ring slots; 1 = K steps of 64 bytes, 32x32x64 products accumulated in place in units of the current
+ * block's scale, four 33 KB ring slots (three K-steps in flight), taken for K >= 256 and the other kernel
+ * otherwise.  Results differ in rounding only.  Process-wide; not meant to be switched while launches are being
+ * enqueued from another thread. */
+int bgmoe_set_tiled_variant(int variant);
+
 /* Workspace of the balanced form of the weight-streaming grouped GEMM (no reference counterpart).  A decode launch
  * has a few hundred work items of 0.25-1.8 MB for ~512 resident blocks, so whole items leave CUs idle; the
  * balanced form cuts the sequence of all items' K-blocks into one equal share per block, streams each share

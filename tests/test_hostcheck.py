@@ -285,3 +285,76 @@ def test_accumulator_coordinates_cover_the_32x32_product(hc):
             assert b.value == lane % 32 and a.value == 8 * (v // 4) + 4 * (lane // 32) + v % 4
             seen.add((a.value, b.value))
     assert len(seen) == 1024
+
+
+# ---- the K = 64 kernel's dataflow on one macro tile, against a plain block-scaled GEMM -------------------------------
+def _e4m3_table():
+    t = np.zeros(256, dtype=np.float64)
+    for b in range(256):
+        sign, e, m = b >> 7, (b >> 3) & 15, b & 7
+        v = (m / 8.0) * 2.0 ** -6 if e == 0 else (1 + m / 8.0) * 2.0 ** (e - 7)
+        t[b] = -v if sign else v
+    return t
+
+
+def _tile_major(w):
+    """[n, K] bytes -> the resident layout: 16-row x 128-column tiles, byte half*1024 + (q*16 + r)*16 + j of tile
+    (nt, kb) = row 16 nt + r, column 128 kb + 64 half + 16 q + j."""
+    n, k = w.shape
+    t = w.reshape(n // 16, 16, k // 128, 2, 4, 16)            # [nt][r][kb][half][q][j]
+    return np.ascontiguousarray(t.transpose(0, 2, 3, 4, 1, 5)).reshape(-1)
+
+
+@pytest.mark.parametrize("fused,tile_major,cnt,m0,n,n0", [
+    (0, 0, 256, 0, 256, 0), (0, 1, 256, 0, 256, 0),            # a full tile, both weight layouts
+    (0, 0, 300, 256, 384, 256),                                 # 44 live rows (one token half dead), images past N
+    (0, 1, 130, 0, 384, 256), (1, 0, 256, 0, 256, 128), (1, 1, 300, 256, 128, 0), (1, 1, 1, 0, 256, 0),
+])
+def test_k64_kernel_dataflow_on_one_macro_tile(hc, fused, tile_major, cnt, m0, n, n0):
+    """The K = 64 kernel's loads, operand reads, in-place accumulation with the scale change per 128-K block and its
+    epilogue coordinates, walked on the CPU with the kernel's own maps: equal (up to fp32 summation order) to
+    out[t, c] = sum_kb (sum_k x[t, k] w[c, k]) xs[t, kb] ws[c / 128, kb] on exactly the elements of the macro tile
+    that lie inside the group and inside N; nothing else is written; no address leaves its buffer."""
+    rng = np.random.default_rng(fused * 100 + tile_major * 10 + cnt + n0)
+    K, KB = 512, 4
+    dec = _e4m3_table()
+    codes = np.array([b for b in range(256) if (b & 0x7F) != 0x7F and (b & 0x7F) < 0x60], dtype=np.uint8)   # |v| <= 15
+    x = codes[rng.integers(0, len(codes), size=(cnt, K))]
+    w0 = codes[rng.integers(0, len(codes), size=(n, K))]
+    w1 = codes[rng.integers(0, len(codes), size=(n, K))]
+    xs = (rng.random((cnt, KB)) * 0.02 + 0.001).astype(np.float32)
+    xs[0, 1] = np.float32(1e-12) / np.float32(448.0)            # a token block that was all zeros: the scale floor
+    x[0, 128:256] = 0
+    ws0 = (rng.random((n // 128, KB)) * 1e-3 + 1e-5).astype(np.float32)
+    ws1 = (rng.random((n // 128, KB)) * 1e-3 + 1e-5).astype(np.float32)
+    a0 = _tile_major(w0) if tile_major else np.ascontiguousarray(w0).reshape(-1)
+    a1 = _tile_major(w1) if tile_major else np.ascontiguousarray(w1).reshape(-1)
+    out = np.zeros((cnt, n), dtype=np.float32)
+    written = np.zeros((cnt, n), dtype=np.uint8)
+    hc.hc_k64_emulate_item.restype = C.c_int
+    hc.hc_k64_emulate_item.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                       C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    rc = hc.hc_k64_emulate_item(x.ctypes.data, xs.ctypes.data, cnt, K, a0.ctypes.data, a1.ctypes.data, ws0.ctypes.data,
+                                ws1.ctypes.data, n, fused, tile_major, m0, n0, out.ctypes.data, written.ctypes.data)
+    assert rc == 0, rc
+    ncols = 128 if fused else 256
+    want_mask = np.zeros((cnt, n), dtype=np.uint8)
+    want_mask[m0: min(cnt, m0 + 256), n0: min(n, n0 + ncols)] = 1
+    assert np.array_equal(written, want_mask), "the write set is the live part of the macro tile"
+    xf, rows = dec[x], slice(m0, min(cnt, m0 + 256))
+    cols = slice(n0, min(n, n0 + ncols))
+
+    def gemm(wq, ws):
+        wf = dec[wq]
+        ref = np.zeros((cnt, n))
+        for kb in range(KB):
+            part = xf[:, 128 * kb: 128 * kb + 128] @ wf[:, 128 * kb: 128 * kb + 128].T
+            ref += part * xs[:, kb: kb + 1].astype(np.float64) * np.repeat(ws[:, kb], 128)[None, :]
+        return ref
+
+    ref = gemm(w0, ws0)
+    if fused:
+        up = gemm(w1, ws1)
+        ref = ref / (1.0 + np.exp(-ref)) * up
+    got, want = out[rows, cols].astype(np.float64), ref[rows, cols]
+    assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() + 1e-30
