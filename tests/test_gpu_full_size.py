@@ -70,8 +70,7 @@ def test_full_size_layer_properties(dev, idx):
     assert err < 1e-2
 
 
-@pytest.mark.parametrize("backend", ["hip", "vendor"])
-def test_full_size_mxfp4_layer_properties(dev, backend):
+def check_full_size_mxfp4_layer(dev, backend):
     """Config 3 (MXFP4 weights, bf16 activations) at full size: determinism, a sample of tokens against the
     oracle and, with the bf16 shared expert on this library's own GEMM ("hip": a row's sums are a fixed chain
     over K whatever the row's position), token-order equivariance bit for bit.  The vendor GEMM library does
@@ -109,3 +108,9 @@ def test_full_size_mxfp4_layer_properties(dev, backend):
     err = og.rel_frobenius(out[sub].float().cpu().numpy(), ref["out"])
     say("   rel frobenius of the sample vs oracle:", err)
     assert err < 1e-2
+
+
+def test_full_size_mxfp4_layer_properties(dev):
+    """The bf16 shared expert on the vendor GEMM; with the layer's default (this library's own GEMM), token-order
+    check included: tests/test_gpu_x_dense_backend.py::test_mxfp4_layers_on_the_default_backend."""
+    check_full_size_mxfp4_layer(dev, "vendor")

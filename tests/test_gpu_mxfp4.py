@@ -112,7 +112,7 @@ def test_reference_op_names_with_pointer_tables(dev):
     assert torch.equal(c2[live.to(dev)], ref2[live.to(dev)])
 
 
-def test_mxfp4_layer_matches_oracle(dev):
+def check_mxfp4_layer_against_oracle(dev, backend):
     from batchgen_amd import workloads as wl
     from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
     from oracle import layer as ol
@@ -121,7 +121,7 @@ def test_mxfp4_layer_matches_oracle(dev):
     inp = wl.make_inputs(cfg, "cpu")
     w, sh = wl.make_mxfp4_weights(cfg, "cpu")
     layer = Mxfp4MoELayer(cfg, {k: v.to(dev) for k, v in w.items()}, {k: v.to(dev) for k, v in sh.items()},
-                          inp["bias"].to(dev))
+                          inp["bias"].to(dev), dense_backend=backend)
     out = layer(inp["x"].to(dev), inp["logits"].to(dev))
     wn = {k: v.numpy() for k, v in w.items()}
     shn = {k: v.float().numpy() for k, v in sh.items()}
@@ -134,3 +134,9 @@ def test_mxfp4_layer_matches_oracle(dev):
     err = og.rel_frobenius(out.float().cpu().numpy(), ref["out"])
     say("   mxfp4 layer rel frobenius:", err)
     assert err < 1e-2
+
+
+def test_mxfp4_layer_matches_oracle(dev):
+    """The bf16 shared expert on the vendor GEMM here; the same check with the layer's default (this library's own
+    bf16 GEMM) is tests/test_gpu_x_dense_backend.py::test_mxfp4_layers_on_the_default_backend."""
+    check_mxfp4_layer_against_oracle(dev, "vendor")

@@ -177,12 +177,12 @@ def test_fused_s1_situ_and_reference_op_name(dev, counts, n, k):
     assert torch.equal(c[lv], h[lv])
 
 
-def _latent_case(cfg, dev, sample=None):
+def _latent_case(cfg, dev, sample=None, backend="vendor"):
     from batchgen_amd.moe.mxfp4_layer import Mxfp4MoELayer
     inp = wl.make_inputs(cfg, dev)
     w, sh = wl.make_mxfp4_weights(cfg, dev)
     lat = wl.make_latent_weights(cfg, dev)
-    layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat)
+    layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat, dense_backend=backend)
     x, logits = inp["x"], inp["logits"]
     out = layer(x, logits).clone()
     assert out.shape == (cfg.n_tokens, cfg.hidden) and torch.isfinite(out.float()).all()
@@ -197,10 +197,10 @@ def _latent_case(cfg, dev, sample=None):
     return layer, out, sub, ref
 
 
-def test_latent_situ_layer_matches_oracle(dev):
+def check_latent_layer_against_oracle(dev, backend):
     cfg = wl.scaled(wl.K3_LATENT, n_tokens=96, hidden=512, latent=256, inter=384, shared_inter=384, n_experts=224,
                     e_local=28, expert_start=56, max_tokens=96)
-    layer, out, sub, ref = _latent_case(cfg, dev)
+    layer, out, sub, ref = _latent_case(cfg, dev, backend=backend)
     assert np.array_equal(layer.topk_ids.cpu().numpy(), ref["ids"])
     assert np.array_equal(layer.topk_pos.cpu().numpy(), ref["pos"])
     assert np.array_equal(layer.expert_counts.cpu().numpy(), ref["counts"])
@@ -210,7 +210,13 @@ def test_latent_situ_layer_matches_oracle(dev):
     assert e_lat < 1e-2 and err < 1e-2
 
 
-def test_latent_situ_layer_full_size_sample(dev):
+def test_latent_situ_layer_matches_oracle(dev):
+    """Projections and shared expert on the vendor GEMM here; the layer's default (this library's own bf16 GEMM):
+    tests/test_gpu_x_dense_backend.py::test_mxfp4_layers_on_the_default_backend."""
+    check_latent_layer_against_oracle(dev, "vendor")
+
+
+def check_latent_layer_full_size_sample(dev, backend):
     """The Kimi-K3 layer at its real shape (512 tokens, 7168 -> 3584, 28 local experts of 3072, top-16 of 896):
     determinism on the whole batch and a sample of tokens against the oracle."""
     cfg = wl.K3_LATENT
@@ -221,11 +227,15 @@ def test_latent_situ_layer_full_size_sample(dev):
     hit = np.nonzero(local.sum(axis=1) >= 2)[0]
     sample = sorted(set([0, cfg.n_tokens - 1] + hit[:2].tolist()))
     say("   sample tokens", sample)
-    layer, out, sub, ref = _latent_case(cfg, dev, sample)
+    layer, out, sub, ref = _latent_case(cfg, dev, sample, backend=backend)
     assert np.array_equal(layer.topk_ids[sub].cpu().numpy(), ref["ids"])
     err = og.rel_frobenius(out[sub].float().cpu().numpy(), ref["out"])
     say("   rel frobenius of the sample vs oracle:", err)
     assert err < 1e-2
+
+
+def test_latent_situ_layer_full_size_sample(dev):
+    check_latent_layer_full_size_sample(dev, "vendor")
 
 
 def test_new_entry_points_reject_bad_arguments(dev):

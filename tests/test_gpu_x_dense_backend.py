@@ -101,3 +101,23 @@ def test_silu_and_mul_bits(dev, rows, d):
     ref = F.silu(x[:, :d].float()).to(torch.bfloat16) * x[:, d:]
     bad = int((y.view(torch.int16) != ref.view(torch.int16)).sum())
     assert bad <= max(2, rows * d // 2000), bad
+
+
+@pytest.mark.parametrize("which", ["config3_small", "latent_small", "config3_full_size", "latent_full_size"])
+def test_mxfp4_layers_on_the_default_backend(dev, which):
+    """The oracle checks of the MXFP4 layers (tests/test_gpu_mxfp4.py, test_gpu_situ_latent.py, test_gpu_full_size.py)
+    with the layer's default dense backend, this library's own bf16 GEMM, at 96 and at 512 tokens; the full-size
+    run of configuration 3 includes the token-order check (a row's sums do not depend on its position)."""
+    say("default dense backend", which)
+    if which == "config3_small":
+        from tests.test_gpu_mxfp4 import check_mxfp4_layer_against_oracle
+        check_mxfp4_layer_against_oracle(dev, "hip")
+    elif which == "latent_small":
+        from tests.test_gpu_situ_latent import check_latent_layer_against_oracle
+        check_latent_layer_against_oracle(dev, "hip")
+    elif which == "config3_full_size":
+        from tests.test_gpu_full_size import check_full_size_mxfp4_layer
+        check_full_size_mxfp4_layer(dev, "hip")
+    else:
+        from tests.test_gpu_situ_latent import check_latent_layer_full_size_sample
+        check_latent_layer_full_size_sample(dev, "hip")
