@@ -777,6 +777,7 @@ extern "C" int bgmoe_debug_streamk_status(int32_t* host_out) {
 int bgmoe_internal_init_fp8_streamk() {
   grid_s1();
   grid_down();
+  (void)status_ptr();              // resolve this device's status word here, not inside a launch a caller may be capturing
   return BGMOE_OK;
 }
 
