@@ -158,3 +158,43 @@ BGMOE_HD int bgmoe_sk_locate_in_group(BgmoeSkShape s, BgmoeSkCost k, int g, int 
   p->cpk = cpk;
   return 1;
 }
+
+// ---- LDS-tiled grouped GEMM: the persistent blocks' walk over the work items ------------------------------------------
+// Work items are (group, m-tile, n-tile); `tiles` is the exclusive prefix of m-tiles per group (tiles[groups] = all),
+// ntn the n-tiles of the output.  The flat item list is cut into eight contiguous parts, one per XCD (block b runs on
+// XCD b % 8); the bstep blocks of an XCD take its items round-robin.  Inside a group items come in panels of `panel`
+// m-tiles, and inside a panel with the m-tile running fastest, so that the items an XCD works on at one time form a
+// compact (m, n) patch whose token and weight streams its L2 can share.
+struct BgmoeTiledWalk { int64_t first; int count; int bstep; };      // this block's XCD: first item, items, blocks
+BGMOE_HD BgmoeTiledWalk bgmoe_tiled_walk(int64_t total_items, unsigned grid, unsigned block) {
+  const int nx = 8;
+  const int xcd = (int)(block % nx);
+  const int per_x = (int)((total_items + nx - 1) / nx);
+  BgmoeTiledWalk w;
+  w.bstep = (int)((grid + nx - 1 - xcd) / nx);
+  w.first = (int64_t)xcd * per_x;
+  int64_t left = total_items - w.first;
+  if (left < 0) left = 0;
+  w.count = (int)(left < per_x ? left : per_x);
+  return w;
+}
+struct BgmoeTiledItem { int grp, mtile, ntile; };
+// flat item -> (group, m-tile of the group, n-tile); tiles[] may live in LDS
+BGMOE_HD BgmoeTiledItem bgmoe_tiled_decode(const int* tiles, int groups, int ntn, int panel, int64_t item) {
+  int lo = 0, hi = groups - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int64_t)tiles[mid] * ntn <= item) lo = mid; else hi = mid - 1;
+  }
+  BgmoeTiledItem it;
+  it.grp = lo;
+  const int mt_g = tiles[lo + 1] - tiles[lo];
+  const int64_t rel = item - (int64_t)tiles[lo] * ntn;
+  const int pnl = (int)(rel / ((int64_t)panel * ntn));
+  const int left = mt_g - pnl * panel;
+  const int pm = panel < left ? panel : left;
+  const int r2 = (int)(rel - (int64_t)pnl * panel * ntn);
+  it.ntile = r2 / pm;
+  it.mtile = pnl * panel + (r2 - it.ntile * pm);
+  return it;
+}

@@ -90,13 +90,11 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
   __syncthreads();
   const int total_m = s_tiles[g.groups];
   const int64_t total = (int64_t)total_m * ntn;
-  // XCD-aware walk: block b (XCD b % 8) takes items of the b%8-th eighth of the list
-  const int nx = 8;
-  const int xcd = blockIdx.x % nx;
-  const int per_x = (int)((total + nx - 1) / nx);
-  const int bstep = (gridDim.x + nx - 1 - xcd) / nx;   // blocks living on this XCD
-  const int64_t first_x = (int64_t)xcd * per_x;
-  const int cnt_x = (int)max((int64_t)0, min((int64_t)per_x, total - first_x));
+  // XCD-aware walk: block b (XCD b % 8) takes items of the b%8-th eighth of the list (bgmoe_hostdev.h)
+  const BgmoeTiledWalk walk = bgmoe_tiled_walk(total, gridDim.x, blockIdx.x);
+  const int bstep = walk.bstep;
+  const int64_t first_x = walk.first;
+  const int cnt_x = walk.count;
 
   // ---- per-item state ----
   struct Meta { int cnt, m0, n0; int64_t row0; };
@@ -117,22 +115,10 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
   // item index of this block's walk -> (group, n-tile, m-tile), its load sources and what the epilogue needs
   auto prepare = [&](int64_t itx, Meta& mt, Src& s) -> bool {
     if (itx >= cnt_x) return false;
-    const int64_t item = first_x + itx;
-    int lo_g = 0, hi_g = g.groups - 1;
-    while (lo_g < hi_g) {
-      const int mid = (lo_g + hi_g + 1) >> 1;
-      if ((int64_t)s_tiles[mid] * ntn <= item) lo_g = mid; else hi_g = mid - 1;
-    }
-    const int grp = __builtin_amdgcn_readfirstlane(lo_g);   // (LDS reads look divergent to the compiler)
-    const int mt_g = __builtin_amdgcn_readfirstlane(s_tiles[grp + 1] - s_tiles[grp]);
-    const int64_t rel = item - (int64_t)__builtin_amdgcn_readfirstlane(s_tiles[grp]) * ntn;
-    // panels of kPanel m-tiles; inside a panel n-tiles advance with m fastest, so the items an XCD works on at one
-    // time form a compact (m, n) patch: few distinct token and weight streams per L2
-    const int panel = (int)(rel / ((int64_t)kPanel * ntn));
-    const int pm = min(kPanel, mt_g - panel * kPanel);
-    const int r2 = (int)(rel - (int64_t)panel * kPanel * ntn);
-    const int nt = r2 / pm;
-    const int mtile = panel * kPanel + (r2 - nt * pm);
+    const BgmoeTiledItem it = bgmoe_tiled_decode(s_tiles, g.groups, ntn, kPanel, first_x + itx);
+    const int grp = __builtin_amdgcn_readfirstlane(it.grp);   // (LDS reads look divergent to the compiler)
+    const int nt = __builtin_amdgcn_readfirstlane(it.ntile);
+    const int mtile = __builtin_amdgcn_readfirstlane(it.mtile);
     const int cnt = g.seqlens[grp];
     const int64_t row0 = g.cu[grp];
     const int m0 = mtile * TM;
@@ -210,7 +196,7 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
   // ---- the two cursors ----
   Meta cur{}, nxt{};
   Src L{};
-  int64_t l_itx = blockIdx.x / nx;
+  int64_t l_itx = blockIdx.x / 8;
   int l_ks = 0, l_buf = 0;
   uint32_t lg = 0;                                       // global K-step the load cursor issues next (slot lg % NS)
   bool have = prepare(l_itx, cur, L);

@@ -358,3 +358,38 @@ def test_k64_kernel_dataflow_on_one_macro_tile(hc, fused, tile_major, cnt, m0, n
         ref = ref / (1.0 + np.exp(-ref)) * up
     got, want = out[rows, cols].astype(np.float64), ref[rows, cols]
     assert np.abs(got - want).max() <= 2e-5 * np.abs(want).max() + 1e-30
+
+
+# ---- the tiled kernels' walk over work items ---------------------------------------------------------------------------
+@pytest.mark.parametrize("counts,lo,ntn,grid", [
+    ([512] * 32, 64, 16, 256),                                       # benchmark configuration 2's shape, uniform
+    ([130, 0, 700, 65, 64, 3000, 1, 257, 256, 90], 64, 16, 256),     # ragged: empty, below the limit, one row over a tile
+    ([300], 0, 1, 8), ([2100, 5, 9000] + [0] * 253, 64, 28, 256), ([257] * 7, 256, 3, 24),
+])
+def test_tiled_walk_visits_every_item_once(hc, counts, lo, ntn, grid):
+    """Blocks x rounds of the persistent walk cover every (group, m-tile, n-tile) of the groups above the row limit
+    exactly once; a block only takes items of its XCD's eighth of the list; and the items one XCD holds in one
+    round form a compact patch (few distinct m-tiles and n-tiles: the streams its L2 has to hold)."""
+    hc.hc_tiled_walk.restype = C.c_int
+    hc.hc_tiled_walk.argtypes = [C.POINTER(C.c_int32), C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint, C.POINTER(C.c_int), C.c_int]
+    want = {(g, m, n) for g, c in enumerate(counts) if c > lo for m in range((c + 255) // 256) for n in range(ntn)}
+    cap = len(want) + 16
+    out = (C.c_int * (5 * cap))()
+    n = hc.hc_tiled_walk((C.c_int32 * len(counts))(*counts), len(counts), lo, ntn, 8, grid, out, cap)
+    assert n == len(want)
+    visits = np.ctypeslib.as_array(out)[: 5 * n].reshape(-1, 5)
+    seen = {tuple(v[2:]) for v in visits.tolist()}
+    assert seen == want and len(visits) == len(want)
+    per_x = -(-len(want) // 8)
+    flat = sorted(want)                                              # the list order is group-major
+    first_of_group = {}
+    for (g, m, nn) in flat:
+        first_of_group.setdefault(g, len(first_of_group))
+    by_round = {}
+    for b, rnd, g, m, nn in visits.tolist():
+        by_round.setdefault((b % 8, rnd), []).append((g, m, nn))
+    for (xcd, rnd), items in by_round.items():
+        assert len(items) <= (grid + 7 - xcd) // 8
+        if len({g for g, _, _ in items}) == 1 and len(items) >= 16:  # a round inside one group: a patch, not a line
+            ms, ns = {m for _, m, _ in items}, {nn for _, _, nn in items}
+            assert len(ms) + len(ns) <= len(items) // 2 + 9, (xcd, rnd, len(ms), len(ns), len(items))
