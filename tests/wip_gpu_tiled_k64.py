@@ -2,7 +2,11 @@
 ``bgmoe_set_tiled_variant(1)``) on the GPU, with every group forced onto the tiled kernel: against the fp32
 dequantise-then-matmul oracle at the reference's gates, write sets, the requantisation identity of the fused
 epilogue, ragged == uniform placement bit for bit, both weight layouts, and against the K = 128 kernel (the two
-differ in rounding only).  The lane maps behind it are walked on the CPU in tests/test_hostcheck.py."""
+differ in rounding only).  The lane maps behind it are walked on the CPU in tests/test_hostcheck.py.
+
+The kernel has not run on a GPU yet, so this file carries a name pytest does not collect: a test run that
+collects everything must not be the first to launch a kernel that no GPU has executed.  Run it by naming the
+file (`python -m pytest tests/wip_gpu_tiled_k64.py -m gpu`); once it is green it becomes tests/test_gpu_y_tiled_k64.py."""
 import numpy as np
 import pytest
 import torch
