@@ -26,7 +26,10 @@ own formula):
                                  (all-equal row -> ids 0..K-1, ...), sum(w)=rsf.
 * ``router.gate_sigmoid_topk``   same, plus padding rows (-1 / 0.0).
 * ``permute.*``                  sequential per-pair loop (the reference test's
-                                 ``ref_dispatch``) and the layout invariants.
+                                 ``ref_dispatch``) and the layout invariants;
+                                 ``dispatch_masked_arrivals`` (the slot counter's
+                                 final value, dispatch_scatter_3d.cu:66) against a
+                                 running counter over the pairs, kept and dropped.
 * ``combine.*``                  per-token Python loop, all-(-1) -> zeros.
 * ``mxfp4.dequant``              the frozen 16-byte vector of the reference and
                                  its unit cases.
