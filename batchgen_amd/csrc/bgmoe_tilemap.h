@@ -89,3 +89,28 @@ BGMOE_HD uint32_t bgmoe_k64_out_col(bool fused, uint32_t wn, uint32_t a, uint32_
   const uint32_t r = bgmoe_mfma32_acc_a_row(lane, v);
   return fused ? 32u * wn + r : 64u * wn + 32u * a + r;
 }
+
+// ---- epilogue regrouping through a per-wave LDS patch -------------------------------------------------------------------
+// A lane holds 4 consecutive output columns of 16 different places of one token, and the 32 lanes of a half wave hold
+// 32 different tokens: stored as they are, one store instruction touches 32 rows with 8 (bf16) or 4 (e4m3) bytes
+// each.  Each wave therefore passes its results through a private LDS patch (LDS operations of one wave execute in
+// order: no barrier) and stores whole row segments.
+constexpr uint32_t BGMOE_K64_PATCH_BYTES = 1536;
+// Plain GEMM, bf16: pass p (0..3) of token image b moves its tokens 8p .. 8p+7: 8 rows x the wave's 64 columns
+// (128 bytes) at a pitch of 144 bytes.  Writers are the 16 lanes that hold those tokens; each writes, per product a
+// and register group q, 8 bytes (registers 4q .. 4q+3 = columns 32a + 8q + 4 (lane / 32) .. + 3).  Then every lane
+// reads 16 bytes: row lane / 8, columns 8 (lane % 8) .. + 7, and a store instruction writes 8 whole 128-byte segments.
+BGMOE_HD bool bgmoe_k64_patch_writer(uint32_t lane, uint32_t p) { return ((lane & 31u) >> 3) == p; }
+BGMOE_HD uint32_t bgmoe_k64_patch_write_off(uint32_t lane, uint32_t a, uint32_t q) {
+  return (lane & 7u) * 144u + 64u * a + 16u * q + 8u * (lane >> 5);
+}
+BGMOE_HD uint32_t bgmoe_k64_patch_read_off(uint32_t lane) { return (lane >> 3) * 144u + (lane & 7u) * 16u; }
+BGMOE_HD uint32_t bgmoe_k64_patch_read_token(uint32_t p, uint32_t lane) { return 8u * p + (lane >> 3); }   // of the image's 32
+BGMOE_HD uint32_t bgmoe_k64_patch_read_col(uint32_t lane) { return (lane & 7u) * 8u; }                     // of the wave's 64
+// Fused stage 1, e4m3 bytes: all 32 tokens of token image b at once: 32 rows x the wave's 32 columns (32 bytes) at a
+// pitch of 48 bytes; a lane writes 4 bytes per register group q and reads 16 bytes: row lane / 2, columns
+// 16 (lane % 2) .. + 15; a store instruction writes 32 segments of 32 bytes.
+BGMOE_HD uint32_t bgmoe_k64_qpatch_write_off(uint32_t lane, uint32_t q) { return (lane & 31u) * 48u + 8u * q + 4u * (lane >> 5); }
+BGMOE_HD uint32_t bgmoe_k64_qpatch_read_off(uint32_t lane) { return (lane >> 1) * 48u + (lane & 1u) * 16u; }
+BGMOE_HD uint32_t bgmoe_k64_qpatch_read_token(uint32_t lane) { return lane >> 1; }                          // of the image's 32
+BGMOE_HD uint32_t bgmoe_k64_qpatch_read_col(uint32_t lane) { return (lane & 1u) * 16u; }                    // of the wave's 32

@@ -22,4 +22,5 @@ constexpr int kBgmoeTiledMaxKB = 256;          // K <= 32768: an item's weight s
 
 // K = 64 variant: BGMOE_ERR_WORKSPACE (without a message) = does not apply to these sizes, take the K = 128 kernel
 int bgmoe_internal_init_fp8_tiled_k64();
-int bgmoe_launch_fp8_tiled_k64(const BgmoeTiledArgs& g, bool fused, int64_t m, int num_cu, hipStream_t st);
+// regroup: its epilogue stores whole row segments through per-wave LDS patches where alignment allows
+int bgmoe_launch_fp8_tiled_k64(const BgmoeTiledArgs& g, bool fused, bool regroup, int64_t m, int num_cu, hipStream_t st);

@@ -423,15 +423,17 @@ __global__ __launch_bounds__(NT) void fp8_tiled_kernel(TiledArgs g) {
 }
 
 int g_num_cu = 0;
-int g_variant = 0;                 // 0: this file's K = 128 kernel; 1: the K = 64 kernel where it applies
+int g_variant = 0;                 // 0: this file's K = 128 kernel; 1, 2: the K = 64 kernel where it applies
 
 }  // namespace
 
 // Which LDS-tiled kernel serves the groups above the streaming limit (no reference counterpart): 0 = the K = 128
 // kernel (16x16x128 products, two 65 KB ring slots), 1 = the K = 64 kernel (32x32x64 products accumulated in
-// place, four 33 KB slots) for K >= 256, the K = 128 kernel otherwise.  Results of the two differ in rounding only.
+// place, four 33 KB slots) for K >= 256, the K = 128 kernel otherwise; 2 = the same with plain per-lane stores in its
+// epilogue instead of the regrouped ones (for comparison).  Results of the two kernels differ in rounding only; 1
+// and 2 give the same bits.
 extern "C" int bgmoe_set_tiled_variant(int variant) {
-  BGMOE_REQUIRE(variant == 0 || variant == 1, "set_tiled_variant: variant must be 0 (K = 128) or 1 (K = 64), got %d", variant);
+  BGMOE_REQUIRE(variant >= 0 && variant <= 2, "set_tiled_variant: variant must be 0 (K = 128), 1 or 2 (K = 64), got %d", variant);
   g_variant = variant;
   return BGMOE_OK;
 }
@@ -493,8 +495,8 @@ int bgmoe_launch_fp8_tiled(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* w0, c
   if (blocks > max_items) blocks = max_items;
   if (blocks < 8) blocks = 8;
   BgmoeProf prof(w1 ? BGMOE_K_S1_TILED : BGMOE_K_GEMM_TILED, st);
-  if (g_variant == 1) {
-    const int rc = bgmoe_launch_fp8_tiled_k64(g, w1 != nullptr, m, g_num_cu, st);
+  if (g_variant != 0) {
+    const int rc = bgmoe_launch_fp8_tiled_k64(g, w1 != nullptr, g_variant == 1, m, g_num_cu, st);
     if (rc != BGMOE_ERR_WORKSPACE) return rc;            // (without a message: the variant does not apply here)
   }
   const dim3 grid((unsigned)blocks), block(NT);

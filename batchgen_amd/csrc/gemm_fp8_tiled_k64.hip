@@ -52,9 +52,12 @@ constexpr int kMaxGroups = kBgmoeTiledMaxGroups;
 constexpr int kMaxKB = kBgmoeTiledMaxKB;
 constexpr int kLoadsPerPair = 9;   // loads a wave issues per (even, odd) pair of K-steps
 
-template <bool FUSED, int LAYOUT>
+// REGROUP: the epilogue passes the e4m3 bytes (fused) / the bf16 values (plain GEMM) through a per-wave LDS patch and
+// stores whole row segments (bgmoe_tilemap.h) instead of 4 / 8 bytes per lane and row.
+template <bool FUSED, int LAYOUT, bool REGROUP>
 __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
   extern __shared__ __align__(16) uint8_t smem[];      // NS slots
+  __shared__ __align__(16) uint8_t s_patch[REGROUP ? NT / 64 : 1][REGROUP ? BGMOE_K64_PATCH_BYTES : 16];
   __shared__ int s_tiles[kMaxGroups + 1];              // exclusive prefix of m-tiles per group
   __shared__ float s_ws[2][2][kMaxKB];                 // [buffer][row] weight scales along K of an item
   __shared__ float s_amax[2][4][4][32];                // fused epilogue: [wm][wn][b][token] amax of 32 columns
@@ -338,7 +341,25 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
                                  fmaxf(s_amax[wm][2][b][t32], s_amax[wm][3][b][t32]));
           const float sc = quant_scale_from_amax(am);
           const int tok = m0 + (int)bgmoe_k64_out_token(wm, b, lane);
-          if (tok < cnt) {
+          if constexpr (REGROUP) {
+            // every lane quantises and writes its bytes into the wave's patch (rows past the group's end included:
+            // they are simply not stored), then reads 16 bytes of one row and stores them
+            uint8_t* const patch = s_patch[wave];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float hv[4] = {acc[b][0][4 * q], acc[b][0][4 * q + 1], acc[b][0][4 * q + 2], acc[b][0][4 * q + 3]};
+              float qv[4];
+              quant_div_clamp(hv, sc, qv);
+              *reinterpret_cast<uint32_t*>(patch + bgmoe_k64_qpatch_write_off(lane, (uint32_t)q)) =
+                  pack4_e4m3(qv[0], qv[1], qv[2], qv[3]);
+            }
+            const uint4 v = *reinterpret_cast<const uint4*>(patch + bgmoe_k64_qpatch_read_off(lane));
+            const int rtok = m0 + 128 * (int)wm + 32 * b + (int)bgmoe_k64_qpatch_read_token(lane);
+            if (rtok < cnt)
+              *reinterpret_cast<uint4*>(g.out_q + (row0 + rtok) * g.n + n0 + 32 * (int)wn +
+                                        (int)bgmoe_k64_qpatch_read_col(lane)) = v;
+            if (tok < cnt && wn == 0u && lane < 32u) g.out_s[(row0 + tok) * g.os_row + (int64_t)(n0 >> 7) * g.os_nb] = sc;
+          } else if (tok < cnt) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const float hv[4] = {acc[b][0][4 * q], acc[b][0][4 * q + 1], acc[b][0][4 * q + 2], acc[b][0][4 * q + 3]};
@@ -354,21 +375,54 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
         // s_amax is written again by the next item's epilogue, at least 2 * KB >= 4 barriers from here
       }
     } else {
+      // the wave's 64 columns lie inside N or past it as a whole when N is a multiple of 64 (the launcher takes the
+      // regrouping form only then, and only for a 16-byte aligned output)
+      if constexpr (REGROUP) {
+        uint8_t* const patch = s_patch[wave];
+        const int colw = n0 + 64 * (int)wn;
+        if (colw < g.n) {                                  // wave-uniform
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int tok = m0 + (int)bgmoe_k64_out_token(wm, b, lane);
-        if (tok >= cnt) continue;
+          for (int b = 0; b < 4; ++b) {
+            if (m0 + 128 * (int)wm + 32 * b >= cnt) continue;          // no live token in this image (wave-uniform)
 #pragma unroll
-        for (int a = 0; a < 2; ++a) {
-          const int col0 = n0 + (int)bgmoe_k64_out_col(false, wn, a, lane, 0);   // this product's first column
-          if (col0 - 4 * (int)hsel >= g.n) continue;     // the whole 32-column image lies past N (wave-uniform)
-          const float s = prev[b][a];
+            for (uint32_t p = 0; p < 4; ++p) {
+              if (bgmoe_k64_patch_writer(lane, p)) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            uint2 o;
-            o.x = pack2_bf16(acc[b][a][4 * q] * s, acc[b][a][4 * q + 1] * s);
-            o.y = pack2_bf16(acc[b][a][4 * q + 2] * s, acc[b][a][4 * q + 3] * s);
-            *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + (int)bgmoe_k64_out_col(false, wn, a, lane, 4 * q)) = o;
+                for (int a = 0; a < 2; ++a) {
+                  const float s = prev[b][a];
+#pragma unroll
+                  for (int q = 0; q < 4; ++q) {
+                    uint2 o;
+                    o.x = pack2_bf16(acc[b][a][4 * q] * s, acc[b][a][4 * q + 1] * s);
+                    o.y = pack2_bf16(acc[b][a][4 * q + 2] * s, acc[b][a][4 * q + 3] * s);
+                    *reinterpret_cast<uint2*>(patch + bgmoe_k64_patch_write_off(lane, (uint32_t)a, (uint32_t)q)) = o;
+                  }
+                }
+              }
+              const uint4 v = *reinterpret_cast<const uint4*>(patch + bgmoe_k64_patch_read_off(lane));
+              const int rtok = m0 + 128 * (int)wm + 32 * b + (int)bgmoe_k64_patch_read_token(p, lane);
+              if (rtok < cnt)
+                *reinterpret_cast<uint4*>(g.out + (row0 + rtok) * g.n + colw + (int)bgmoe_k64_patch_read_col(lane)) = v;
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const int tok = m0 + (int)bgmoe_k64_out_token(wm, b, lane);
+          if (tok >= cnt) continue;
+#pragma unroll
+          for (int a = 0; a < 2; ++a) {
+            const int col0 = n0 + (int)bgmoe_k64_out_col(false, wn, a, lane, 0);   // this product's first column
+            if (col0 - 4 * (int)hsel >= g.n) continue;     // the whole 32-column image lies past N (wave-uniform)
+            const float s = prev[b][a];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              uint2 o;
+              o.x = pack2_bf16(acc[b][a][4 * q] * s, acc[b][a][4 * q + 1] * s);
+              o.y = pack2_bf16(acc[b][a][4 * q + 2] * s, acc[b][a][4 * q + 3] * s);
+              *reinterpret_cast<uint2*>(g.out + (row0 + tok) * g.n + n0 + (int)bgmoe_k64_out_col(false, wn, a, lane, 4 * q)) = o;
+            }
           }
         }
       }
@@ -388,10 +442,14 @@ bool g_ready = false;
 int bgmoe_internal_init_fp8_tiled_k64() {
   static int state = 0;                                  // 0 = not tried, 1 = ready, -1 = failed
   if (state == 0) {
-    const void* fns[4] = {reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<true, 0>),
-                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<false, 0>),
-                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<true, 1>),
-                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<false, 1>)};
+    const void* fns[8] = {reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<true, 0, false>),
+                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<false, 0, false>),
+                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<true, 1, false>),
+                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<false, 1, false>),
+                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<true, 0, true>),
+                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<false, 0, true>),
+                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<true, 1, true>),
+                          reinterpret_cast<const void*>(&fp8_tiled_k64_kernel<false, 1, true>)};
     hipError_t e1 = hipSuccess;
     for (const void* f : fns) {
       const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
@@ -404,7 +462,13 @@ int bgmoe_internal_init_fp8_tiled_k64() {
   return BGMOE_OK;
 }
 
-int bgmoe_launch_fp8_tiled_k64(const BgmoeTiledArgs& g, bool fused, int64_t m, int num_cu, hipStream_t st) {
+template <bool FUSED, int LAYOUT>
+void launch_k64(const BgmoeTiledArgs& g, bool regroup, dim3 grid, hipStream_t st) {
+  if (regroup) hipLaunchKernelGGL((fp8_tiled_k64_kernel<FUSED, LAYOUT, true>), grid, dim3(NT), kLds, st, g);
+  else hipLaunchKernelGGL((fp8_tiled_k64_kernel<FUSED, LAYOUT, false>), grid, dim3(NT), kLds, st, g);
+}
+
+int bgmoe_launch_fp8_tiled_k64(const BgmoeTiledArgs& g, bool fused, bool regroup, int64_t m, int num_cu, hipStream_t st) {
   bgmoe_internal_init_fp8_tiled_k64();
   // K >= 256: the load cursor runs three K-steps ahead and may be at most one item ahead of the compute cursor.
   // N a multiple of 32: weight images are 32 rows.  Everything else is the K = 128 kernel's contract.
@@ -416,14 +480,20 @@ int bgmoe_launch_fp8_tiled_k64(const BgmoeTiledArgs& g, bool fused, int64_t m, i
   int64_t blocks = (int64_t)(num_cu > 0 ? num_cu : 256);
   if (blocks > max_items) blocks = max_items;
   if (blocks < 8) blocks = 8;
-  const dim3 grid((unsigned)blocks), block(NT);
+  const dim3 grid((unsigned)blocks);
   const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
+  // the regrouping epilogue stores 16 bytes per lane: e4m3 rows need a 16-byte aligned base (N is a multiple of 128
+  // for stage 1), bf16 rows a 16-byte aligned base and the wave's 64 columns inside or past N as a whole
+  if (regroup) {
+    if (fused) regroup = g.out_q != nullptr && ((uintptr_t)g.out_q & 15) == 0 && g.n % 16 == 0;
+    else regroup = ((uintptr_t)g.out & 15) == 0 && g.n % 64 == 0;
+  }
   if (fused) {
-    if (tm) hipLaunchKernelGGL((fp8_tiled_k64_kernel<true, 1>), grid, block, kLds, st, g);
-    else hipLaunchKernelGGL((fp8_tiled_k64_kernel<true, 0>), grid, block, kLds, st, g);
+    if (tm) launch_k64<true, 1>(g, regroup, grid, st);
+    else launch_k64<true, 0>(g, regroup, grid, st);
   } else {
-    if (tm) hipLaunchKernelGGL((fp8_tiled_k64_kernel<false, 1>), grid, block, kLds, st, g);
-    else hipLaunchKernelGGL((fp8_tiled_k64_kernel<false, 0>), grid, block, kLds, st, g);
+    if (tm) launch_k64<false, 1>(g, regroup, grid, st);
+    else launch_k64<false, 0>(g, regroup, grid, st);
   }
   return bgmoe_check_launch("fp8 grouped gemm (tiled, K = 64)");
 }

@@ -184,8 +184,8 @@ static float e4m3_to_float(uint8_t b) {
 }
 
 int hc_k64_emulate_item(const uint8_t* x, const float* xs, int cnt, int K, const uint8_t* w0, const uint8_t* w1,
-                        const float* ws0, const float* ws1, int n, int fused, int tile_major, int m0, int n0, float* out,
-                        uint8_t* written) {
+                        const float* ws0, const float* ws1, int n, int fused, int tile_major, int regroup, int m0, int n0,
+                        float* out, uint8_t* written) {
   const int KB = K / 128, steps = 2 * KB;
   const bool F = fused != 0;
   float dec[256];
@@ -274,30 +274,84 @@ int hc_k64_emulate_item(const uint8_t* x, const float* xs, int cnt, int K, const
     }
   }
   // ---- epilogue ----
+  auto value = [&](uint32_t wave, uint32_t lane, int b, int a, uint32_t v) {
+    if (F) {
+      const float gt = ACC(wave, lane, b, 0, (int)v) * PREV(wave, lane, b, 0);
+      const float up = ACC(wave, lane, b, 1, (int)v) * PREV(wave, lane, b, 1);
+      return gt / (1.0f + expf(-gt)) * up;
+    }
+    return ACC(wave, lane, b, a, (int)v) * PREV(wave, lane, b, a);
+  };
+  auto emit = [&](int tok, int col, float val) {
+    const size_t o = (size_t)tok * n + col;
+    if (written[o]) return false;                                       // two places claim one output element
+    written[o] = 1;
+    out[o] = val;
+    return true;
+  };
   for (uint32_t wave = 0; wave < 8; ++wave) {
     const uint32_t wn = bgmoe_k64_wave_wn(wave), wm = bgmoe_k64_wave_wm(wave);
-    for (uint32_t lane = 0; lane < 64; ++lane)
-      for (int b = 0; b < 4; ++b) {
-        const int tok = m0 + (int)bgmoe_k64_out_token(wm, b, lane);
-        if (tok >= cnt) continue;
-        for (int a = 0; a < (F ? 1 : 2); ++a)
-          for (uint32_t v = 0; v < 16; ++v) {
-            const int col = n0 + (int)bgmoe_k64_out_col(F, wn, (uint32_t)a, lane, v);
-            if (col >= n) continue;
-            float val;
-            if (F) {
-              const float gt = ACC(wave, lane, b, 0, (int)v) * PREV(wave, lane, b, 0);
-              const float up = ACC(wave, lane, b, 1, (int)v) * PREV(wave, lane, b, 1);
-              val = gt / (1.0f + expf(-gt)) * up;
-            } else {
-              val = ACC(wave, lane, b, a, (int)v) * PREV(wave, lane, b, a);
+    if (!regroup) {
+      for (uint32_t lane = 0; lane < 64; ++lane)
+        for (int b = 0; b < 4; ++b) {
+          const int tok = m0 + (int)bgmoe_k64_out_token(wm, b, lane);
+          if (tok >= cnt) continue;
+          for (int a = 0; a < (F ? 1 : 2); ++a)
+            for (uint32_t v = 0; v < 16; ++v) {
+              const int col = n0 + (int)bgmoe_k64_out_col(F, wn, (uint32_t)a, lane, v);
+              if (col >= n) continue;
+              if (!emit(tok, col, value(wave, lane, b, a, v))) return -3;
             }
-            const size_t o = (size_t)tok * n + col;
-            if (written[o]) return -3;                                  // two registers claim one output element
-            written[o] = 1;
-            out[o] = val;
+        }
+      continue;
+    }
+    // through the wave's patch: one slot per output element (e4m3: one byte; bf16: two bytes), addressed with the
+    // kernel's byte offsets
+    const uint32_t esz = F ? 1u : 2u;
+    std::vector<float> patch(BGMOE_K64_PATCH_BYTES / esz, NAN);
+    if (F) {
+      for (int b = 0; b < 4; ++b) {
+        for (uint32_t lane = 0; lane < 64; ++lane)
+          for (uint32_t q = 0; q < 4; ++q) {
+            const uint32_t off = bgmoe_k64_qpatch_write_off(lane, q);
+            if (off + 4 > BGMOE_K64_PATCH_BYTES) return -4;
+            for (uint32_t i = 0; i < 4; ++i) patch[off + i] = value(wave, lane, b, 0, 4 * q + i);
           }
+        for (uint32_t lane = 0; lane < 64; ++lane) {
+          const uint32_t off = bgmoe_k64_qpatch_read_off(lane);
+          if (off % 16 != 0 || off + 16 > BGMOE_K64_PATCH_BYTES) return -5;
+          const int rtok = m0 + 128 * (int)wm + 32 * b + (int)bgmoe_k64_qpatch_read_token(lane);
+          if (rtok >= cnt) continue;
+          for (uint32_t i = 0; i < 16; ++i)
+            if (!emit(rtok, n0 + 32 * (int)wn + (int)bgmoe_k64_qpatch_read_col(lane) + (int)i, patch[off + i])) return -3;
+        }
       }
+    } else {
+      const int colw = n0 + 64 * (int)wn;
+      if (colw >= n) continue;
+      for (int b = 0; b < 4; ++b) {
+        if (m0 + 128 * (int)wm + 32 * b >= cnt) continue;
+        for (uint32_t p = 0; p < 4; ++p) {
+          for (uint32_t lane = 0; lane < 64; ++lane) {
+            if (!bgmoe_k64_patch_writer(lane, p)) continue;
+            for (uint32_t a = 0; a < 2; ++a)
+              for (uint32_t q = 0; q < 4; ++q) {
+                const uint32_t off = bgmoe_k64_patch_write_off(lane, a, q);
+                if (off % 8 != 0 || off + 8 > BGMOE_K64_PATCH_BYTES) return -4;
+                for (uint32_t i = 0; i < 4; ++i) patch[off / 2 + i] = value(wave, lane, b, (int)a, 4 * q + i);
+              }
+          }
+          for (uint32_t lane = 0; lane < 64; ++lane) {
+            const uint32_t off = bgmoe_k64_patch_read_off(lane);
+            if (off % 16 != 0 || off + 16 > BGMOE_K64_PATCH_BYTES) return -5;
+            const int rtok = m0 + 128 * (int)wm + 32 * b + (int)bgmoe_k64_patch_read_token(p, lane);
+            if (rtok >= cnt) continue;
+            for (uint32_t i = 0; i < 8; ++i)
+              if (!emit(rtok, colw + (int)bgmoe_k64_patch_read_col(lane) + (int)i, patch[off / 2 + i])) return -3;
+          }
+        }
+      }
+    }
   }
   return 0;
 }

@@ -90,9 +90,9 @@ def parse():
                          "bf16 GEMM (hip, the layer's default) or on the vendor library through torch.mm (vendor)")
     ap.add_argument("--graph", action="store_true",
                     help="time replays of one captured HIP graph of the layer instead of eager launches")
-    ap.add_argument("--tiled-variant", type=int, default=0, choices=[0, 1],
+    ap.add_argument("--tiled-variant", type=int, default=0, choices=[0, 1, 2],
                     help="which LDS-tiled kernel serves the prefill groups: 0 = K steps of 128 (default), 1 = K steps of "
-                         "64 with in-place accumulation (bgmoe_set_tiled_variant)")
+                         "64 with in-place accumulation, 2 = the same with plain per-lane stores (bgmoe_set_tiled_variant)")
     ap.add_argument("--template", action="store_true",
                     help="FP8 configurations: also time the layer as a model file runs it through the MoEBase template "
                          "(router GEMM + gate, routed experts behind the given routes, dense shared expert, add) and "
@@ -524,7 +524,7 @@ def measure_layer(a, config, with_cpu):
                     avg_launch_us=dom_ms * 1e3)
     roof["frac"] = roof["achieved"] / roof["peak"]
     roof["traffic"], roof["traffic_source"] = traffic_record(f"layer:{config}")
-    if not decode and int(getattr(a, "tiled_variant", 0)) == 1:
+    if not decode and int(getattr(a, "tiled_variant", 0)) != 0:
         roof["kernel"] = "fp8_tiled_k64_kernel<fused,tile_major>"
 
     # Decode: the figure reported as `value` is the cache-flushed one.  A decode step of a real model finds none of

@@ -450,7 +450,9 @@ int bgmoe_fp8_dense_gemm_partials(const bgmoe_fp8_act* a, const uint8_t* w, cons
  * 0 (default) = K steps of 128 bytes, 16x16x128 products promoted with one fma per accumulator and scale block,
  * two 65 KB ring slots; 1 = K steps of 64 bytes, 32x32x64 products accumulated in place in units of the current
  * block's scale, four 33 KB ring slots (three K-steps in flight), taken for K >= 256 and the other kernel
- * otherwise.  Results differ in rounding only.  Process-wide; not meant to be switched while launches are being
+ * otherwise; its epilogue stores whole row segments through per-wave LDS patches; 2 = the same kernel with plain
+ * per-lane stores (for comparison; same bits as 1).  Results of 0 and 1 differ in rounding only.  Token and
+ * weight scales must be positive for 1 and 2.  Process-wide; not meant to be switched while launches are being
  * enqueued from another thread. */
 int bgmoe_set_tiled_variant(int variant);
 

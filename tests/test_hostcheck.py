@@ -305,16 +305,18 @@ def _tile_major(w):
     return np.ascontiguousarray(t.transpose(0, 2, 3, 4, 1, 5)).reshape(-1)
 
 
+@pytest.mark.parametrize("regroup", [0, 1])
 @pytest.mark.parametrize("fused,tile_major,cnt,m0,n,n0", [
     (0, 0, 256, 0, 256, 0), (0, 1, 256, 0, 256, 0),            # a full tile, both weight layouts
     (0, 0, 300, 256, 384, 256),                                 # 44 live rows (one token half dead), images past N
     (0, 1, 130, 0, 384, 256), (1, 0, 256, 0, 256, 128), (1, 1, 300, 256, 128, 0), (1, 1, 1, 0, 256, 0),
 ])
-def test_k64_kernel_dataflow_on_one_macro_tile(hc, fused, tile_major, cnt, m0, n, n0):
+def test_k64_kernel_dataflow_on_one_macro_tile(hc, fused, tile_major, cnt, m0, n, n0, regroup):
     """The K = 64 kernel's loads, operand reads, in-place accumulation with the scale change per 128-K block and its
     epilogue coordinates, walked on the CPU with the kernel's own maps: equal (up to fp32 summation order) to
     out[t, c] = sum_kb (sum_k x[t, k] w[c, k]) xs[t, kb] ws[c / 128, kb] on exactly the elements of the macro tile
-    that lie inside the group and inside N; nothing else is written; no address leaves its buffer."""
+    that lie inside the group and inside N; nothing else is written; no address leaves its buffer.  `regroup`: the
+    epilogue through the per-wave LDS patches (whole row segments per store) instead of per-lane stores."""
     rng = np.random.default_rng(fused * 100 + tile_major * 10 + cnt + n0)
     K, KB = 512, 4
     dec = _e4m3_table()
@@ -333,9 +335,9 @@ def test_k64_kernel_dataflow_on_one_macro_tile(hc, fused, tile_major, cnt, m0, n
     written = np.zeros((cnt, n), dtype=np.uint8)
     hc.hc_k64_emulate_item.restype = C.c_int
     hc.hc_k64_emulate_item.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
-                                       C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+                                       C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
     rc = hc.hc_k64_emulate_item(x.ctypes.data, xs.ctypes.data, cnt, K, a0.ctypes.data, a1.ctypes.data, ws0.ctypes.data,
-                                ws1.ctypes.data, n, fused, tile_major, m0, n0, out.ctypes.data, written.ctypes.data)
+                                ws1.ctypes.data, n, fused, tile_major, regroup, m0, n0, out.ctypes.data, written.ctypes.data)
     assert rc == 0, rc
     ncols = 128 if fused else 256
     want_mask = np.zeros((cnt, n), dtype=np.uint8)

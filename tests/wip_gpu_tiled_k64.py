@@ -19,12 +19,13 @@ from tests.util import say
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture()
-def k64():
-    """Every group on the tiled kernel (row limit 0), K = 64 variant; both restored afterwards."""
+@pytest.fixture(params=[2, 1], ids=["plain_stores", "regrouped_stores"])
+def k64(request):
+    """Every group on the tiled kernel (row limit 0), K = 64 variant with plain per-lane stores (2) or with the
+    epilogue regrouped through per-wave LDS patches (1); both settings restored afterwards."""
     from batchgen_amd._lib import check, lib
     check(lib().bgmoe_set_skinny_max_rows(0))
-    check(lib().bgmoe_set_tiled_variant(1))
+    check(lib().bgmoe_set_tiled_variant(request.param))
     try:
         yield
     finally:
@@ -100,9 +101,10 @@ def test_k64_variant_against_the_k128_kernel_and_placement(dev):
     outs = {}
     check(lib().bgmoe_set_skinny_max_rows(0))
     try:
-        for variant in (0, 1):
+        for variant in (0, 1, 2):
             check(lib().bgmoe_set_tiled_variant(variant))
             outs[variant] = gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, cnt_d, cu_d, xs_t, ws_d, 16).float().cpu().numpy()
+        check(lib().bgmoe_set_tiled_variant(1))
         # uniform placement: group e at row 512 e
         cu2 = (np.arange(len(counts) + 1) * 512).astype(np.int32)
         m2 = int(cu2[-1])
@@ -117,6 +119,7 @@ def test_k64_variant_against_the_k128_kernel_and_placement(dev):
     finally:
         check(lib().bgmoe_set_tiled_variant(0))
         check(lib().bgmoe_set_skinny_max_rows(256))
+    assert np.array_equal(outs[1], outs[2]), "the two epilogues of the K = 64 kernel store the same bits"
     a, b = outs[0][live], outs[1][live]
     assert og.rel_frobenius(b, a) < 2e-3
     assert np.abs(a - b).max() <= 2.0 ** -6 * np.abs(a).max() + 1e-6
@@ -136,4 +139,4 @@ def test_k64_variant_declines_short_k_and_bad_arguments(dev, k64):
     assert lib().bgmoe_set_tiled_variant(0) == 0
     b = gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, cnt_d, cu_d, xs_t, ws_d, 16)
     assert torch.equal(a, b)
-    assert lib().bgmoe_set_tiled_variant(2) != 0 and lib().bgmoe_set_tiled_variant(-1) != 0
+    assert lib().bgmoe_set_tiled_variant(3) != 0 and lib().bgmoe_set_tiled_variant(-1) != 0
