@@ -35,4 +35,8 @@ __device__ __forceinline__ const T* uniform_ptr(const T* p) {   // tell the comp
 template <int N>
 __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 __device__ __forceinline__ void block_barrier() { asm volatile("s_barrier" ::: "memory"); }
+// Barrier for an exchange through LDS only: this wave's LDS writes are done (lgkmcnt(0)), then the barrier.  Unlike
+// __syncthreads() it does not wait for vector-memory operations, so asynchronous global -> LDS loads that are in
+// flight for LATER use stay in flight across it.
+__device__ __forceinline__ void lds_exchange_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 

@@ -333,7 +333,7 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
         }
       }
       if (g.out_q != nullptr) {
-        __syncthreads();
+        lds_exchange_barrier();                          // s_amax only: the next item's loads stay in flight
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
           const uint32_t t32 = lane & 31u;
