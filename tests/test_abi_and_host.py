@@ -67,6 +67,25 @@ def test_errors_are_reported_without_a_gpu():
     assert h.bgmoe_fp8_weight_repack(None, None, 1, 100, 128, None) != 0
 
 
+def test_tuning_switches_check_their_arguments():
+    """The process-wide switches are host-side state: bad values are refused with a message, good ones accepted
+    (and the defaults restored here)."""
+    from batchgen_amd import _lib
+    h = _lib.lib()
+    for bad in (-1, 3, 7):
+        assert h.bgmoe_set_tiled_variant(bad) != 0 and b"variant" in h.bgmoe_last_error()
+    for good in (1, 2, 0):
+        assert h.bgmoe_set_tiled_variant(good) == 0
+    w8 = ctypes.c_int * 8
+    for bad in ([1] + [64] * 7, [0] + [8] * 7, [65] + [8] * 7, [64] * 7 + [1]):
+        assert h.bgmoe_set_streamk_xcd_weights(w8(*bad)) != 0, bad
+    assert b"32 times the smallest" in h.bgmoe_last_error()
+    assert h.bgmoe_set_streamk_xcd_weights(None) != 0
+    for good in ([8] * 8, [2, 3] * 4, [23, 21] * 4):
+        assert h.bgmoe_set_streamk_xcd_weights(w8(*good)) == 0, good
+    assert h.bgmoe_debug_streamk_status(None) != 0
+
+
 def test_loader_and_op_names():
     from batchgen_amd.kernels import load_extension
     want = {
