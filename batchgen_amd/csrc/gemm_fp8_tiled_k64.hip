@@ -294,12 +294,18 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
 #pragma unroll
         for (int a = 0; a < 2; ++a)
           A[a] = load_image(sw + bgmoe_k64_a_image(FUSED, wn, a) * BGMOE_K64_TILE_BYTES, a_lo, a_hi);
+        // token image b + 1 is fetched from LDS while image b is multiplied
+        intx8 Bb[2];
+        Bb[0] = load_image(sl + bgmoe_k64_b_image(wm, 0) * BGMOE_K64_TILE_BYTES, b_lo, b_hi);
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
-          const intx8 B = load_image(sl + bgmoe_k64_b_image(wm, b) * BGMOE_K64_TILE_BYTES, b_lo, b_hi);
+          if (b < 3) Bb[(b + 1) & 1] = load_image(sl + bgmoe_k64_b_image(wm, b + 1) * BGMOE_K64_TILE_BYTES, b_lo, b_hi);
+          // (the scheduler would otherwise sink the prefetch below the products that do not need it)
+          __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
           for (int a = 0; a < 2; ++a)
-            acc[b][a] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[a], B, acc[b][a], 0, 0, 0, 0, 0, 0);
+            acc[b][a] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A[a], Bb[b & 1], acc[b][a], 0, 0, 0, 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
