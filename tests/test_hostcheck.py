@@ -395,3 +395,36 @@ def test_tiled_walk_visits_every_item_once(hc, counts, lo, ntn, grid):
         if len({g for g, _, _ in items}) == 1 and len(items) >= 16:  # a round inside one group: a patch, not a line
             ms, ns = {m for _, m, _ in items}, {nn for _, _, nn in items}
             assert len(ms) + len(ns) <= len(items) // 2 + 9, (xcd, rnd, len(ms), len(ns), len(items))
+
+
+def test_in_place_block_scaling_keeps_fp32_accuracy():
+    """The K = 64 kernel's arithmetic in a float32 model: accumulators kept in units of the current 128-K block's
+    scale (acc *= s[kb-1] / s[kb], then the block's products are added unscaled; out = acc * s[last]) against the
+    promotion form (acc += product * s[kb]) and the float64 sum, with a token block that was all zeros (its scale is
+    the quantiser's floor 1e-12 / 448, fourteen orders of magnitude below its neighbours): both stay within a few
+    fp32 ulps of the exact sum, also on that row, and nothing leaves the fp32 range."""
+    rng = np.random.default_rng(0)
+    kb_n, m, n = 56, 64, 64
+    f32 = np.float32
+    prod = rng.standard_normal((kb_n, m, n)) * 300.0
+    xs = (np.abs(rng.standard_normal((kb_n, m))) * 0.01 + 1e-4).astype(f32)
+    xs[3, 5] = f32(1e-12) / f32(448)
+    prod[3, 5, :] = 0.0
+    ws = (np.abs(rng.standard_normal(kb_n)) * 1e-4 + 1e-5).astype(f32)
+    exact = sum(prod[k] * xs[k][:, None].astype(np.float64) * float(ws[k]) for k in range(kb_n))
+    promoted = np.zeros((m, n), f32)
+    in_place = np.zeros((m, n), f32)
+    prev, peak = None, 0.0
+    for k in range(kb_n):
+        c = (xs[k] * ws[k]).astype(f32)
+        promoted = (prod[k].astype(f32) * c[:, None] + promoted).astype(f32)
+        if prev is not None:
+            in_place = (in_place * (prev * (f32(1) / c)).astype(f32)[:, None]).astype(f32)
+        in_place = (in_place + prod[k].astype(f32)).astype(f32)
+        peak = max(peak, float(np.abs(in_place).max()))
+        prev = c
+    out = (in_place * prev[:, None]).astype(f32)
+    err = lambda a: np.linalg.norm(a - exact) / np.linalg.norm(exact)
+    assert err(promoted) < 1e-6 and err(out) < 1e-6
+    assert np.abs(out[5] - exact[5]).max() <= 4e-6 * np.abs(exact[5]).max()
+    assert np.isfinite(out).all() and peak < 1e30
