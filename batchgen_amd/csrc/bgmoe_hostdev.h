@@ -165,7 +165,11 @@ BGMOE_HD int bgmoe_sk_locate_in_group(BgmoeSkShape s, BgmoeSkCost k, int g, int 
 // XCD b % 8); the bstep blocks of an XCD take its items round-robin.  Inside a group items come in panels of `panel`
 // m-tiles, and inside a panel with the m-tile running fastest, so that the items an XCD works on at one time form a
 // compact (m, n) patch whose token and weight streams its L2 can share.
-struct BgmoeTiledWalk { int64_t first; int count; int bstep; };      // this block's XCD: first item, items, blocks
+// Tail of the static walk: an XCD's items are dealt to its bstep blocks in rounds.  When the last round is at most
+// half full, each of its items is split into two 128-token halves taken by different blocks (a half keeps one wave
+// per SIMD busy and takes little more than half the time), so the launch ends half a round earlier.  `virt` counts
+// the XCD's virtual items (whole items, then the halves of the last round's items).
+struct BgmoeTiledWalk { int64_t first; int count; int bstep; int split_base; int virt; };
 BGMOE_HD BgmoeTiledWalk bgmoe_tiled_walk(int64_t total_items, unsigned grid, unsigned block) {
   const int nx = 8;
   const int xcd = (int)(block % nx);
@@ -176,7 +180,22 @@ BGMOE_HD BgmoeTiledWalk bgmoe_tiled_walk(int64_t total_items, unsigned grid, uns
   int64_t left = total_items - w.first;
   if (left < 0) left = 0;
   w.count = (int)(left < per_x ? left : per_x);
+  const int rounds = w.bstep > 0 ? (w.count + w.bstep - 1) / w.bstep : 0;
+  w.split_base = rounds > 0 ? (rounds - 1) * w.bstep : 0;
+  const int rem = w.count - w.split_base;
+  w.virt = (rounds > 0 && 2 * rem <= w.bstep) ? w.split_base + 2 * rem : w.count;
   return w;
+}
+// virtual item itx of the XCD's walk -> flat item and half (-1: the whole 256-token tile; 0, 1: tokens 128 * half ..)
+BGMOE_HD bool bgmoe_tiled_walk_item(const BgmoeTiledWalk& w, int64_t itx, int64_t* item, int* half) {
+  if (itx >= w.virt) return false;
+  *half = -1;
+  *item = w.first + itx;
+  if (w.virt != w.count && itx >= w.split_base) {
+    *item = w.first + w.split_base + ((itx - w.split_base) >> 1);
+    *half = (int)((itx - w.split_base) & 1);
+  }
+  return true;
 }
 struct BgmoeTiledItem { int grp, mtile, ntile; };
 // flat item -> (group, m-tile of the group, n-tile); tiles[] may live in LDS

@@ -96,8 +96,6 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
   // XCD-aware walk: block b (XCD b % 8) takes items of the b%8-th eighth of the list (bgmoe_hostdev.h)
   const BgmoeTiledWalk walk = bgmoe_tiled_walk(total, gridDim.x, blockIdx.x);
   const int bstep = walk.bstep;
-  const int64_t first_x = walk.first;
-  const int cnt_x = walk.count;
 
   // ---- per-item state ----
   struct Meta { int cnt, m0, n0; int64_t row0; };
@@ -117,14 +115,22 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
 
   // item index of this block's walk -> (group, n-tile, m-tile), its load sources and what the epilogue needs
   auto prepare = [&](int64_t itx, Meta& mt, Src& s) -> bool {
-    if (itx >= cnt_x) return false;
-    const BgmoeTiledItem it = bgmoe_tiled_decode(s_tiles, g.groups, ntn, kPanel, first_x + itx);
+    int64_t item = 0;
+    int half = -1;                                       // -1: the whole 256-token tile
+    if (!bgmoe_tiled_walk_item(walk, itx, &item, &half)) return false;
+    const BgmoeTiledItem it = bgmoe_tiled_decode(s_tiles, g.groups, ntn, kPanel, item);
     const int grp = __builtin_amdgcn_readfirstlane(it.grp);   // (LDS reads look divergent to the compiler)
     const int nt = __builtin_amdgcn_readfirstlane(it.ntile);
     const int mtile = __builtin_amdgcn_readfirstlane(it.mtile);
-    const int cnt = g.seqlens[grp];
+    int cnt = g.seqlens[grp];
     const int64_t row0 = g.cu[grp];
-    const int m0 = mtile * TM;
+    int m0 = mtile * TM;
+    if (half >= 0) {                                     // rows [m0 + 128 * half, + 128) of the tile
+      m0 += 128 * half;
+      if (m0 >= cnt) return false;                       // no live row in this half; a block has at most one split item
+                                                         // and it is its last, so it is done
+      cnt = min(cnt, m0 + 128);
+    }
     const int n0 = nt * ncols;
     mt.cnt = cnt; mt.m0 = m0; mt.n0 = n0; mt.row0 = row0;
 

@@ -96,7 +96,7 @@ int hc_sk_walk(const int32_t* seqlens, int groups, int hi_rows, int ntiles, int 
 // ---- the LDS-tiled kernels' walk over work items -----------------------------------------------------------------
 // Every block's walk as the K = 64 kernel runs it: counts -> m-tiles of 256 rows for groups above `lo` rows, the
 // XCD-wise split of the flat item list, round-robin over an XCD's blocks, item -> (group, m-tile, n-tile).
-// out: 5 ints per visited item {block, round, grp, mtile, ntile}; returns the number of visits or -1 (out too small).
+// out: 6 ints per visit {block, round, grp, mtile, ntile, half}; returns the number of visits or -1 (out too small).
 int hc_tiled_walk(const int32_t* counts, int groups, int lo, int ntn, int panel, unsigned grid, int* out, int max_items) {
   std::vector<int> tiles(groups + 1, 0);
   for (int g = 0; g < groups; ++g) tiles[g + 1] = tiles[g] + (counts[g] > lo ? (counts[g] + 255) / 256 : 0);
@@ -105,11 +105,13 @@ int hc_tiled_walk(const int32_t* counts, int groups, int lo, int ntn, int panel,
   for (unsigned b = 0; b < grid; ++b) {
     const BgmoeTiledWalk w = bgmoe_tiled_walk(total, grid, b);
     int round = 0;
-    for (int64_t itx = b / 8; itx < w.count; itx += w.bstep, ++round) {
+    int64_t item = 0;
+    int half = -1;
+    for (int64_t itx = b / 8; bgmoe_tiled_walk_item(w, itx, &item, &half); itx += w.bstep, ++round) {
       if (n >= max_items) return -1;
-      const BgmoeTiledItem it = bgmoe_tiled_decode(tiles.data(), groups, ntn, panel, w.first + itx);
-      int* o = out + 5 * n++;
-      o[0] = (int)b; o[1] = round; o[2] = it.grp; o[3] = it.mtile; o[4] = it.ntile;
+      const BgmoeTiledItem it = bgmoe_tiled_decode(tiles.data(), groups, ntn, panel, item);
+      int* o = out + 6 * n++;
+      o[0] = (int)b; o[1] = round; o[2] = it.grp; o[3] = it.mtile; o[4] = it.ntile; o[5] = half;
     }
   }
   return n;

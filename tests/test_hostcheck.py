@@ -367,21 +367,38 @@ def test_k64_kernel_dataflow_on_one_macro_tile(hc, fused, tile_major, cnt, m0, n
     ([512] * 32, 64, 16, 256),                                       # benchmark configuration 2's shape, uniform
     ([130, 0, 700, 65, 64, 3000, 1, 257, 256, 90], 64, 16, 256),     # ragged: empty, below the limit, one row over a tile
     ([300], 0, 1, 8), ([2100, 5, 9000] + [0] * 253, 64, 28, 256), ([257] * 7, 256, 3, 24),
+    ([512] * 4, 64, 16, 256),                                        # 16 items on an XCD's 32 blocks: every item split
 ])
 def test_tiled_walk_visits_every_item_once(hc, counts, lo, ntn, grid):
     """Blocks x rounds of the persistent walk cover every (group, m-tile, n-tile) of the groups above the row limit
-    exactly once; a block only takes items of its XCD's eighth of the list; and the items one XCD holds in one
-    round form a compact patch (few distinct m-tiles and n-tiles: the streams its L2 has to hold)."""
+    exactly once -- whole, or as two 128-token halves taken by two different blocks when the XCD's last round is at
+    most half full (a half is then the last thing its block does); and the items one XCD holds in one round form a
+    compact patch (few distinct m-tiles and n-tiles: the streams its L2 has to hold)."""
     hc.hc_tiled_walk.restype = C.c_int
     hc.hc_tiled_walk.argtypes = [C.POINTER(C.c_int32), C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint, C.POINTER(C.c_int), C.c_int]
     want = {(g, m, n) for g, c in enumerate(counts) if c > lo for m in range((c + 255) // 256) for n in range(ntn)}
-    cap = len(want) + 16
-    out = (C.c_int * (5 * cap))()
+    cap = 2 * len(want) + 16
+    out = (C.c_int * (6 * cap))()
     n = hc.hc_tiled_walk((C.c_int32 * len(counts))(*counts), len(counts), lo, ntn, 8, grid, out, cap)
-    assert n == len(want)
-    visits = np.ctypeslib.as_array(out)[: 5 * n].reshape(-1, 5)
-    seen = {tuple(v[2:]) for v in visits.tolist()}
-    assert seen == want and len(visits) == len(want)
+    assert n >= len(want)
+    visits = np.ctypeslib.as_array(out)[: 6 * n].reshape(-1, 6)
+    whole = [tuple(v[2:5]) for v in visits.tolist() if v[5] == -1]
+    halves = {}
+    for b, rnd, g, m, nn, half in visits.tolist():
+        if half >= 0:
+            halves.setdefault((g, m, nn), []).append((half, b))
+    assert len(whole) == len(set(whole)) and not (set(whole) & set(halves))
+    for item, hs in halves.items():                                  # both halves, taken by two different blocks
+        assert sorted(h for h, _ in hs) == [0, 1] and hs[0][1] != hs[1][1], (item, hs)
+    assert set(whole) | set(halves) == want
+    if counts == [512] * 4:
+        assert len(halves) == len(want) and not whole
+    last_round = {}
+    for b, rnd, g, m, nn, half in visits.tolist():
+        last_round[b] = max(last_round.get(b, -1), rnd)
+    for b, rnd, g, m, nn, half in visits.tolist():                   # a split item is the last thing its block does
+        assert half == -1 or rnd == last_round[b]
+    visits = visits[:, :5]
     per_x = -(-len(want) // 8)
     flat = sorted(want)                                              # the list order is group-major
     first_of_group = {}
