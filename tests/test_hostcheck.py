@@ -310,6 +310,7 @@ def _tile_major(w):
     (0, 0, 256, 0, 256, 0), (0, 1, 256, 0, 256, 0),            # a full tile, both weight layouts
     (0, 0, 300, 256, 384, 256),                                 # 44 live rows (one token half dead), images past N
     (0, 1, 130, 0, 384, 256), (1, 0, 256, 0, 256, 128), (1, 1, 300, 256, 128, 0), (1, 1, 1, 0, 256, 0),
+    (0, 1, 256, 128, 256, 0), (1, 0, 200, 128, 128, 0),        # second halves of split items (count clipped to m0 + 128)
 ])
 def test_k64_kernel_dataflow_on_one_macro_tile(hc, fused, tile_major, cnt, m0, n, n0, regroup):
     """The K = 64 kernel's loads, operand reads, in-place accumulation with the scale change per 128-K block and its
