@@ -114,3 +114,32 @@ BGMOE_HD uint32_t bgmoe_k64_qpatch_write_off(uint32_t lane, uint32_t q) { return
 BGMOE_HD uint32_t bgmoe_k64_qpatch_read_off(uint32_t lane) { return (lane >> 1) * 48u + (lane & 1u) * 16u; }
 BGMOE_HD uint32_t bgmoe_k64_qpatch_read_token(uint32_t lane) { return lane >> 1; }                          // of the image's 32
 BGMOE_HD uint32_t bgmoe_k64_qpatch_read_col(uint32_t lane) { return (lane & 1u) * 16u; }                    // of the wave's 32
+
+// ---- bf16 GEMM with 128-token x 64-output block tiles (router_gemm_lds64_kernel) ----------------------------------------
+// A K step holds 64 output ("expert") rows then 128 token rows, 128 bytes (64 bf16) each, in one LDS stage:
+// experts at byte 0, tokens at byte 64 * 128.  The block's 8 waves issue 3 loads each; issue j = 3 * wave + i covers
+// rows 8j .. 8j+7 of the list [64 expert rows; 128 token rows]; lane p of an issue moves row p / 8's 16-byte piece
+// (p % 8) ^ (row % 8) to position p % 8 of the row (XOR swizzle).  Lane (r, q) of a wave then reads logical pieces
+// 2q and 2q + 1 of row r of a 16-row tile.
+constexpr uint32_t BGMOE_RG64_EXPERTS = 64;
+BGMOE_HD bool bgmoe_rg64_issue_is_token(uint32_t wave, uint32_t i) { return 8u * (3u * wave + i) >= BGMOE_RG64_EXPERTS; }
+// first row (inside its half of the stage) of issue (wave, i)
+BGMOE_HD uint32_t bgmoe_rg64_issue_row0(uint32_t wave, uint32_t i) {
+  const uint32_t j = 3u * wave + i;
+  return bgmoe_rg64_issue_is_token(wave, i) ? 8u * j - BGMOE_RG64_EXPERTS : 8u * j;
+}
+BGMOE_HD uint32_t bgmoe_rg64_lane_row(uint32_t wave, uint32_t i, uint32_t lane) { return bgmoe_rg64_issue_row0(wave, i) + (lane >> 3); }
+BGMOE_HD uint32_t bgmoe_rg64_lane_piece(uint32_t row, uint32_t lane) { return (lane & 7u) ^ (row & 7u); }   // fetched piece
+// LDS byte offset (inside the stage) of the issue's first byte; lane p lands at + 16 p
+BGMOE_HD uint32_t bgmoe_rg64_issue_lds(uint32_t wave, uint32_t i) {
+  return (bgmoe_rg64_issue_is_token(wave, i) ? BGMOE_RG64_EXPERTS * 128u : 0u) + bgmoe_rg64_issue_row0(wave, i) * 128u;
+}
+// operand reads: output tile tn (0..3), token tile wt (0..7), lane (r = lane % 16, q = lane / 16), half jj (0, 1)
+BGMOE_HD uint32_t bgmoe_rg64_read_expert(uint32_t tn, uint32_t lane, uint32_t jj) {
+  const uint32_t r = lane & 15u, q = lane >> 4;
+  return (16u * tn + r) * 128u + (((2u * q + jj) ^ (r & 7u)) << 4);
+}
+BGMOE_HD uint32_t bgmoe_rg64_read_token(uint32_t wt, uint32_t lane, uint32_t jj) {
+  const uint32_t r = lane & 15u, q = lane >> 4;
+  return BGMOE_RG64_EXPERTS * 128u + (16u * wt + r) * 128u + (((2u * q + jj) ^ (r & 7u)) << 4);
+}

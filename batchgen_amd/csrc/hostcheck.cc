@@ -163,6 +163,35 @@ void hc_k64_acc_coord(uint32_t lane, uint32_t v, uint32_t* a_row, uint32_t* b_ro
 }
 
 
+// ---- bf16 GEMM with 128 x 64 block tiles: one K step's loads and operand reads -----------------------------------------
+// experts [64][64] and tokens [128][64] bf16 values of one K step (given as uint16); the 24 issues of the block land
+// them in a stage; got_e [4 tiles][64 lanes][2 halves][8 values] and got_t [8 token tiles][64 lanes][2][8] are what the
+// lanes read.  Returns 0, or -1 when an issue leaves the stage's 24 KB or two lanes write one place.
+int hc_rg64_step(const uint16_t* experts, const uint16_t* tokens, uint16_t* got_e, uint16_t* got_t) {
+  std::vector<uint8_t> stage(192 * 128, 0xEE), hit(192 * 8, 0);
+  for (uint32_t wave = 0; wave < 8; ++wave)
+    for (uint32_t i = 0; i < 3; ++i)
+      for (uint32_t lane = 0; lane < 64; ++lane) {
+        const bool tok = bgmoe_rg64_issue_is_token(wave, i);
+        const uint32_t row = bgmoe_rg64_lane_row(wave, i, lane);
+        const uint32_t piece = bgmoe_rg64_lane_piece(row, lane);
+        const uint32_t dst = bgmoe_rg64_issue_lds(wave, i) + 16 * lane;
+        if (dst + 16 > stage.size() || row >= (tok ? 128u : 64u)) return -1;
+        if (hit[dst / 16]++) return -1;
+        memcpy(&stage[dst], reinterpret_cast<const uint8_t*>(tok ? tokens : experts) + row * 128 + piece * 16, 16);
+      }
+  for (size_t k = 0; k < hit.size(); ++k)
+    if (hit[k] != 1) return -1;
+  for (uint32_t lane = 0; lane < 64; ++lane)
+    for (uint32_t jj = 0; jj < 2; ++jj) {
+      for (uint32_t tn = 0; tn < 4; ++tn)
+        memcpy(got_e + ((tn * 64 + lane) * 2 + jj) * 8, &stage[bgmoe_rg64_read_expert(tn, lane, jj)], 16);
+      for (uint32_t wt = 0; wt < 8; ++wt)
+        memcpy(got_t + ((wt * 64 + lane) * 2 + jj) * 8, &stage[bgmoe_rg64_read_token(wt, lane, jj)], 16);
+    }
+  return 0;
+}
+
 // ---- the K = 64 kernel's dataflow on one macro tile ----------------------------------------------------------------
 // Walks what fp8_tiled_k64_kernel does for ONE work item with the kernel's own maps (bgmoe_tilemap.h): per K-step
 // every wave's asynchronous loads into a ring slot (token image `wave`, weight image `wave`, clamped rows, swizzle

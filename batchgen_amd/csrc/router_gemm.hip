@@ -15,6 +15,7 @@
 // Experts are the MFMA's row operand, so a lane ends up with 4 consecutive experts of one token: 16-byte
 // stores.
 #include "bgmoe_async.h"
+#include "bgmoe_tilemap.h"
 #include "bgmoe_common.h"
 
 namespace {
@@ -399,6 +400,119 @@ __global__ __launch_bounds__(64 * kLdsWaves) void router_gemm_lds_kernel(RouterG
   }
 }
 
+// The same kernel with a block tile of 128 tokens x 64 experts (whole K only): for shapes whose 128 x 128 tiles
+// number fewer than the CUs (a 512-row linear layer onto 4096 columns: 128 tiles on 256 CUs), twice as many,
+// narrower tiles put every CU to work.  A K step is 64 expert rows + 128 token rows = 24 KB; 8 waves = 8 token
+// eighths, wave tile 64 experts x 16 tokens.  Every wave issues three loads per step: issue j = 3 * wave + i of the
+// block's 24 covers rows 8j .. 8j+7 of the list [64 expert rows; 128 token rows].  Lane map, swizzle, K assignment,
+// MFMA order and segment folds are the wide kernel's, hence the same bits.  Opt-in (bgmoe_set_router_gemm_plan).
+constexpr int kLds64Experts = 64;
+constexpr int kLds64Issues = (kLds64Experts + 128) / 8 / kLdsWaves;      // 3
+static_assert(kLds64Issues * kLdsWaves * 8 == kLds64Experts + 128, "24 issues of 8 rows cover the step's 192 rows");
+static_assert(kLds64Experts == (int)BGMOE_RG64_EXPERTS && kLds64Issues == 3, "the lane maps of bgmoe_tilemap.h assume this shape");
+
+__global__ __launch_bounds__(64 * kLdsWaves) void router_gemm_lds64_kernel(RouterGemmArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  constexpr int EB = kLds64Experts;
+  constexpr int kIssues = kLds64Issues;
+  const uint32_t smem_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)smem);
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int lane = lane_id();
+  const int r16 = lane & 15, q = lane >> 4;
+  const int xcd = blockIdx.x & 7, j0 = blockIdx.x >> 3;
+  const int tl = j0 / a.eblocks;
+  const int by = j0 - tl * a.eblocks;
+  const int bx = tl * 8 + xcd;
+  if (bx >= a.ttiles) return;              // whole block, before any barrier
+  const int t0 = bx * 128, e0 = by * EB;
+  const int wt = wave;                      // this wave's 16 tokens of the block tile
+
+  // loader: per issue a wave-uniform choice between the expert rows and the token rows
+  const uint8_t* src_e = uniform_ptr(reinterpret_cast<const uint8_t*>(a.w) + (int64_t)e0 * a.h * 2);
+  const uint8_t* src_t = uniform_ptr(reinterpret_cast<const uint8_t*>(a.x) + (int64_t)t0 * a.h * 2);
+  const int lim_e = a.e - e0 - 1, lim_t = a.n - t0 - 1;                 // clamp: rows past the end re-read the last
+  uint32_t loff[kIssues], ldst[kIssues];
+  bool tok[kIssues];
+#pragma unroll
+  for (int i = 0; i < kIssues; ++i) {                                   // lane maps: bgmoe_tilemap.h
+    tok[i] = bgmoe_rg64_issue_is_token((uint32_t)wave, (uint32_t)i);    // wave-uniform
+    const int row = (int)bgmoe_rg64_lane_row((uint32_t)wave, (uint32_t)i, (uint32_t)lane);
+    const uint32_t piece = bgmoe_rg64_lane_piece((uint32_t)row, (uint32_t)lane);
+    loff[i] = (uint32_t)min(row, tok[i] ? lim_t : lim_e) * (uint32_t)a.h * 2u + piece * 16u;
+    ldst[i] = smem_base + bgmoe_rg64_issue_lds((uint32_t)wave, (uint32_t)i);
+  }
+  auto issue = [&](int step) {
+    const uint32_t d = (uint32_t)(step & (kLdsStages - 1)) * kLdsStageBytes;
+    const int64_t ko = (int64_t)step * (kStep * 2);
+#pragma unroll
+    for (int i = 0; i < kIssues; ++i)
+      async_load16(uniform_ptr((tok[i] ? src_t : src_e) + ko), loff[i],
+                   __builtin_amdgcn_readfirstlane(ldst[i] + d));
+  };
+
+  floatx4 acc[4], tot[4];
+#pragma unroll
+  for (int tn = 0; tn < 4; ++tn) {
+    acc[tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+    tot[tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int nsteps = a.h / kStep;            // the host sends only h % 64 == 0 here
+
+#pragma unroll
+  for (int s = 0; s < kLdsStages - 1; ++s)
+    if (s < nsteps) issue(s);
+  for (int s = 0; s < nsteps; ++s) {
+    const int younger = min(kLdsStages - 2, nsteps - 1 - s);      // steps requested after this one
+    if (younger >= 2) wait_vm<2 * kIssues>();
+    else if (younger == 1) wait_vm<kIssues>();
+    else wait_vm<0>();
+    block_barrier();                       // everyone's loads of step s are in; everyone is done with step s-1
+    if (s + kLdsStages - 1 < nsteps) issue(s + kLdsStages - 1);   // into the slot step s-1 just freed
+    const uint8_t* sb = smem + (s & (kLdsStages - 1)) * kLdsStageBytes;
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      intx4 av[4];
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn)
+        av[tn] = *reinterpret_cast<const intx4*>(sb + bgmoe_rg64_read_expert((uint32_t)tn, (uint32_t)lane, (uint32_t)jj));
+      const intx4 bv = *reinterpret_cast<const intx4*>(sb + bgmoe_rg64_read_token((uint32_t)wt, (uint32_t)lane, (uint32_t)jj));
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn)
+        acc[tn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av[tn]),
+                                                          __builtin_bit_cast(bf16x8, bv), acc[tn], 0, 0, 0);
+    }
+    if ((s & (kStepsPerSeg - 1)) == kStepsPerSeg - 1 || s == nsteps - 1) {   // end of a segment
+#pragma unroll
+      for (int tn = 0; tn < 4; ++tn) {
+        tot[tn] += acc[tn];
+        acc[tn] = floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+  }
+
+  const bool vec = (a.e & 3) == 0;
+  const int token = t0 + wt * 16 + r16;
+  if (token >= a.n) return;
+  const bool pad = row_is_padding(a, token);
+#pragma unroll
+  for (int tn = 0; tn < 4; ++tn) {
+    const int ex = e0 + tn * 16 + q * 4;
+    const floatx4 v = pad ? floatx4{0.f, 0.f, 0.f, 0.f} : tot[tn];
+    if (a.out16 != nullptr) {
+      store_bf16x4(a.out16 + (int64_t)token * a.e + ex, v, a.e - ex, vec);
+      continue;
+    }
+    float* dst = a.out + (int64_t)token * a.e + ex;
+    if (vec) {
+      if (ex < a.e) *reinterpret_cast<floatx4*>(dst) = v;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (ex + i < a.e) dst[i] = v[i];
+    }
+  }
+}
+
 // logits = (((0 + p_0) + p_1) + ...) over the planes; rows past a rank's count get 0
 __global__ __launch_bounds__(256) void router_gemm_reduce_kernel(RouterGemmArgs a, const float* planes) {
   const int64_t total = (int64_t)a.n * a.e;
@@ -414,8 +528,9 @@ __global__ __launch_bounds__(256) void router_gemm_reduce_kernel(RouterGemmArgs 
 
 int g_plan_tm = -1, g_plan_split = -1;
 bool g_lds_ready = false;            // the LDS kernel's 128 KB opt-in succeeded on this process's device
+bool g_lds64_ready = false;          // likewise for the 64-expert-block variant (opt-in)
 
-struct Plan { int tm; int ne; int waves; bool split; bool lds; };
+struct Plan { int tm; int ne; int waves; bool split; bool lds; bool eb64; };
 
 // Launch shape from the sizes alone (results do not depend on it).
 // A CU sustains only ~35-60 GB/s of load requests whatever hits in cache, so what matters for few tokens
@@ -427,6 +542,7 @@ Plan make_plan(int n, int h, int e) {
   Plan p;
   p.ne = 4;
   p.waves = 4;
+  p.eb64 = false;
   // Measured on MI355X (h = 7168): an LDS block needs ~0.6 us per K step whatever else runs, so the whole-K LDS
   // shape costs ~67 us per round of 256 tiles; one block per segment fills the chip from ~1K tokens on at the
   // price of the planes (write + reduce); below that the one-wave register blocks win.
@@ -456,12 +572,20 @@ Plan make_plan(int n, int h, int e) {
   if (g_plan_split == 4) { p.split = true; p.waves = 4; p.lds = h % kStep == 0 && g_lds_ready; }
   if (g_plan_split == 1) { p.split = true; p.waves = 4; p.lds = false; }
   if (g_plan_split == 2) { p.split = true; p.waves = 1; p.lds = false; }
+  if (g_plan_split == 5 && h % kStep == 0 && g_lds64_ready) { p.split = false; p.waves = 4; p.lds = true; p.eb64 = true; }
   return p;
 }
 
 template <bool SPLIT>
 void launch_gemm(const RouterGemmArgs& a0, const Plan& p, hipStream_t st) {
   RouterGemmArgs a = a0;
+  if (!SPLIT && p.lds && p.eb64) {
+    a.ttiles = (a.n + 127) / 128;
+    a.eblocks = (a.e + kLds64Experts - 1) / kLds64Experts;
+    const unsigned blocks = (unsigned)(8 * ((a.ttiles + 7) / 8) * a.eblocks);
+    hipLaunchKernelGGL(router_gemm_lds64_kernel, dim3(blocks), dim3(64 * kLdsWaves), kLdsBytes, st, a);
+    return;
+  }
   if (p.lds) {
     a.ttiles = (a.n + 127) / 128;
     a.eblocks = (a.e + 127) / 128;
@@ -506,6 +630,11 @@ int bgmoe_internal_init_router_gemm() {
     state = e == hipSuccess ? 1 : -1;
     if (e != hipSuccess) (void)hipGetLastError();
     g_lds_ready = state == 1;
+    // the opt-in narrow variant on its own: a failure here leaves the kernels above as they are
+    const hipError_t e64 = hipFuncSetAttribute(reinterpret_cast<const void*>(router_gemm_lds64_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (e64 != hipSuccess) (void)hipGetLastError();
+    g_lds64_ready = e64 == hipSuccess;
   }
   return BGMOE_OK;
 }
@@ -513,7 +642,7 @@ int bgmoe_internal_init_router_gemm() {
 extern "C" int bgmoe_set_router_gemm_plan(int token_tiles, int split) {
   BGMOE_REQUIRE(token_tiles == -1 || token_tiles == 1 || token_tiles == 2 || token_tiles == 4,
                 "set_router_gemm_plan: token_tiles must be -1, 1, 2 or 4");
-  BGMOE_REQUIRE(split >= -1 && split <= 4, "set_router_gemm_plan: split must be -1 ... 4");
+  BGMOE_REQUIRE(split >= -1 && split <= 5, "set_router_gemm_plan: split must be -1 ... 5");
   g_plan_tm = token_tiles;
   g_plan_split = split;
   return BGMOE_OK;

@@ -129,8 +129,10 @@ int bgmoe_router_gemm_gate(const uint16_t* hidden, const uint16_t* router_weight
 /* Tuning/test knob (no reference counterpart): force the router GEMM's launch shape.  token_tiles in
  * {1,2,4} = 16-token tiles per wave; split 0 = one block walks all of K, 1 = one block per 512-element
  * K segment, 2 = the same with one-wave blocks (the shape for few tokens), 3 = all of K with the operands
- * shared through LDS (the shape for many tokens; h % 64 == 0), 4 = one LDS block per K segment; -1 = choose
- * from the sizes.
+ * shared through LDS (the shape for many tokens; h % 64 == 0), 4 = one LDS block per K segment, 5 = all of K
+ * through LDS with block tiles of 128 tokens x 64 outputs instead of 128 x 128 (twice as many blocks: for shapes
+ * whose wide tiles number fewer than the CUs, e.g. a 512-row linear layer; h % 64 == 0; never chosen from the
+ * sizes yet); -1 = choose from the sizes.
  * Results do not depend on it, bit for bit. */
 int bgmoe_set_router_gemm_plan(int token_tiles, int split);
 

@@ -446,3 +446,26 @@ def test_in_place_block_scaling_keeps_fp32_accuracy():
     assert err(promoted) < 1e-6 and err(out) < 1e-6
     assert np.abs(out[5] - exact[5]).max() <= 4e-6 * np.abs(exact[5]).max()
     assert np.isfinite(out).all() and peak < 1e30
+
+
+def test_narrow_bf16_gemm_tile_loads_and_reads(hc):
+    """The 128-token x 64-output block tile of the bf16 GEMM: the 24 issues of a K step fill the stage's 192 rows
+    exactly once, and lane (r, q) of a wave reads, for output tile tn and its token tile, K elements 16 q .. 16 q + 15
+    (two 16-byte pieces) of output row 16 tn + r and of token 16 wt + r -- the operand layout of the 16x16x32 bf16
+    matrix instruction as the wide kernel feeds it."""
+    rng = np.random.default_rng(11)
+    experts = rng.integers(0, 1 << 16, size=(64, 64), dtype=np.uint16)
+    tokens = rng.integers(0, 1 << 16, size=(128, 64), dtype=np.uint16)
+    got_e = np.zeros((4, 64, 2, 8), dtype=np.uint16)
+    got_t = np.zeros((8, 64, 2, 8), dtype=np.uint16)
+    hc.hc_rg64_step.restype = C.c_int
+    hc.hc_rg64_step.argtypes = [C.c_void_p] * 4
+    assert hc.hc_rg64_step(experts.ctypes.data, tokens.ctypes.data, got_e.ctypes.data, got_t.ctypes.data) == 0
+    for lane in range(64):
+        r, q = lane % 16, lane // 16
+        for jj in range(2):
+            k0 = 8 * (2 * q + jj)
+            for tn in range(4):
+                assert np.array_equal(got_e[tn, lane, jj], experts[16 * tn + r, k0: k0 + 8]), (tn, lane, jj)
+            for wt in range(8):
+                assert np.array_equal(got_t[wt, lane, jj], tokens[16 * wt + r, k0: k0 + 8]), (wt, lane, jj)
