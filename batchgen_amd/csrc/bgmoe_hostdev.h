@@ -159,6 +159,37 @@ BGMOE_HD int bgmoe_sk_locate_in_group(BgmoeSkShape s, BgmoeSkCost k, int g, int 
   return 1;
 }
 
+// ---- weight-streaming grouped GEMMs: work items ------------------------------------------------------------------------
+// A group's rows are cut into chunks of chunk_rows rows; an item is (group, chunk, n-tile) and streams the n-tile's
+// weights once.  Groups with more than tall.min_rows rows (0: no such groups) are cut into chunks of tall.rows rows
+// instead: half as many passes over their weights for twice the accumulators.
+struct BgmoeTall { int min_rows, rows; };
+BGMOE_HD int bgmoe_item_rows(int cnt, int chunk_rows, BgmoeTall tall) {
+  return tall.min_rows > 0 && cnt > tall.min_rows ? tall.rows : chunk_rows;
+}
+BGMOE_HD int bgmoe_item_chunks(int cnt, int chunk_rows, BgmoeTall tall) {
+  const int r = bgmoe_item_rows(cnt, chunk_rows, tall);
+  return (cnt + r - 1) / r;
+}
+// XCD-aware slot -> (n-tile, chunk) map inside one group.  Blocks are dispatched round-robin over the 8 XCDs (block b
+// runs on XCD b % 8), each with its own L2.  A group with several chunks streams the same weight tile once per chunk;
+// the map puts all chunks of one n-tile on the SAME XCD in neighbouring blocks: slot q of the group (q = chunk-row *
+// ntiles_pad + block % ntiles_pad, ntiles_pad = n-tiles rounded up to 8 so that every group starts on XCD 0) ->
+// n-tile 8 * (q / (8 * chunks)) + q % 8, chunk (q / 8) % chunks.  An n-tile >= the real count is padding.
+struct BgmoeItemSlot { int ntile, chunk; };
+BGMOE_HD BgmoeItemSlot bgmoe_item_slot(int crow, int chunks, int ntiles_pad, unsigned block) {
+  const int q = crow * ntiles_pad + (int)(block % (unsigned)ntiles_pad);
+  return BgmoeItemSlot{8 * (q / (8 * chunks)) + (q & 7), (q >> 3) % chunks};
+}
+// Upper bound on the virtual blocks of a launch from host-side knowledge only: `row_bound` bounds the total live
+// rows, `max_rows` the rows of any group the launch serves.  Tall items only lower the count (tall.rows >= chunk_rows).
+BGMOE_HD unsigned bgmoe_item_grid(int ntiles, int groups, int64_t row_bound, int max_rows, int chunk_rows) {
+  int64_t items = groups + row_bound / chunk_rows;                 // >= sum of ceil(count / chunk_rows)
+  const int64_t per_group = (int64_t)groups * (((int64_t)max_rows + chunk_rows - 1) / chunk_rows);
+  if (per_group < items) items = per_group;
+  return (unsigned)(((ntiles + 7) & ~7) * items);
+}
+
 // ---- LDS-tiled grouped GEMM: the persistent blocks' walk over the work items ------------------------------------------
 // Work items are (group, m-tile, n-tile); `tiles` is the exclusive prefix of m-tiles per group (tiles[groups] = all),
 // ntn the n-tiles of the output.  The flat item list is cut into eight contiguous parts, one per XCD (block b runs on

@@ -1,6 +1,7 @@
 // Device-side work scheduling shared by the weight-streaming GEMM kernels.
 #pragma once
 #include "bgmoe_common.h"
+#include "bgmoe_hostdev.h"
 
 // Which kernel serves a group.  The weight-streaming kernel re-streams a group's weights once per
 // 32-row chunk; the LDS-tiled kernel works in 256-row tiles and needs enough of them to fill the chip.
@@ -25,29 +26,31 @@ __device__ __forceinline__ int bgmoe_split_limit(const int32_t* seqlens, int gro
 
 // Row chunks of all groups with lo < count <= hi (the number of items per n-tile).  Wave-uniform; every wave
 // runs it redundantly.
-__device__ __forceinline__ int bgmoe_total_chunks(const int32_t* seqlens, int groups, int lo, int hi, int chunk_rows) {
+__device__ __forceinline__ int bgmoe_total_chunks(const int32_t* seqlens, int groups, int lo, int hi, int chunk_rows,
+                                                  BgmoeTall tall = BgmoeTall{0, 0}) {
   const int lane = threadIdx.x & 63;
   int chunks = 0;
   for (int g0 = lane; g0 < groups; g0 += 64) {
     const int c = seqlens[g0];
-    chunks += (c > lo && c <= hi) ? (c + chunk_rows - 1) / chunk_rows : 0;
+    chunks += (c > lo && c <= hi) ? bgmoe_item_chunks(c, chunk_rows, tall) : 0;
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) chunks += __shfl_xor(chunks, off, BGMOE_WAVE);
   return __builtin_amdgcn_readfirstlane(chunks);
 }
 
-// Work items of one launch: every group with lo < count <= hi contributes ceil(count / chunk_rows)
+// Work items of one launch: every group with lo < count <= hi contributes bgmoe_item_chunks(count)
 // items (ascending group, ascending chunk).  Returns the group of item `item` and its chunk index,
 // or -1 when there are fewer items.  Wave-uniform; every wave of the block runs it redundantly.
 __device__ __forceinline__ int nth_active_item(const int32_t* seqlens, int groups, int lo, int hi,
-                                               int chunk_rows, int item, int* chunk) {
+                                               int chunk_rows, int item, int* chunk,
+                                               BgmoeTall tall = BgmoeTall{0, 0}) {
   const int lane = threadIdx.x & 63;
   int base = 0;
   for (int g0 = 0; g0 < groups; g0 += 64) {
     const int gi = g0 + lane;
     const int c = gi < groups ? seqlens[gi] : 0;
-    const int mine = (c > lo && c <= hi) ? (c + chunk_rows - 1) / chunk_rows : 0;
+    const int mine = (c > lo && c <= hi) ? bgmoe_item_chunks(c, chunk_rows, tall) : 0;
     int inc = mine;                                  // inclusive prefix sum over the wave
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -68,34 +71,34 @@ __device__ __forceinline__ int nth_active_item(const int32_t* seqlens, int group
 }
 
 
-// XCD-aware block -> (n-tile, token chunk) map inside one group.  Blocks are dispatched round-robin
-// over the 8 XCDs (block b runs on XCD b % 8), each with its own L2.  A group with several token
-// chunks streams the same weight tile once per chunk; the map puts all chunks of one n-tile on the
-// SAME XCD in neighbouring blocks: block q of the group -> n-tile 8*(q / (8*chunks)) + q % 8,
-// chunk (q / 8) % chunks.  `ntiles_pad` = n-tile count rounded up to 8 so every group starts on XCD 0.
-// `block` is the virtual block index (blockIdx.x, or blockIdx.x + i * gridDim.x in a persistent kernel
-// whose grid is a multiple of 8, which keeps block % 8 == XCD).  grp == BGMOE_ITEM_END: `block` lies past
-// the last item (so do all larger ones); grp == BGMOE_ITEM_PAD: a padding n-tile, nothing to do.
-struct BgmoeItem { int grp, ntile, chunk, cnt; };
+// Virtual block -> work item.  The (n-tile, chunk) map inside a group is bgmoe_item_slot (bgmoe_hostdev.h): all
+// chunks of one n-tile on the same XCD in neighbouring blocks.  `block` is the virtual block index (blockIdx.x, or
+// blockIdx.x + i * gridDim.x in a persistent kernel whose grid is a multiple of 8, which keeps block % 8 == XCD).
+// grp == BGMOE_ITEM_END: `block` lies past the last item (so do all larger ones); grp == BGMOE_ITEM_PAD: a padding
+// n-tile, nothing to do.  rows: the item's height (chunk_rows, or tall.rows for a tall group); its rows are
+// [chunk * rows, min(cnt, (chunk + 1) * rows)).
+struct BgmoeItem { int grp, ntile, chunk, cnt, rows; };
 constexpr int BGMOE_ITEM_PAD = -1;
 constexpr int BGMOE_ITEM_END = -2;
 
 __device__ __forceinline__ BgmoeItem bgmoe_decode_item(const int32_t* seqlens, int groups, int lo, int hi,
-                                                       int chunk_rows, int ntiles, unsigned block) {
+                                                       int chunk_rows, int ntiles, unsigned block,
+                                                       BgmoeTall tall = BgmoeTall{0, 0}) {
   BgmoeItem it;
   const int ntiles_pad = (ntiles + 7) & ~7;
   int crow = 0;
-  it.grp = nth_active_item(seqlens, groups, lo, hi, chunk_rows, (int)(block / ntiles_pad), &crow);
+  it.grp = nth_active_item(seqlens, groups, lo, hi, chunk_rows, (int)(block / ntiles_pad), &crow, tall);
   it.ntile = it.chunk = it.cnt = 0;
+  it.rows = chunk_rows;
   if (__builtin_amdgcn_readfirstlane(it.grp) < 0) {
     it.grp = BGMOE_ITEM_END;
     return it;
   }
   it.cnt = seqlens[it.grp];
-  const int chunks = (it.cnt + chunk_rows - 1) / chunk_rows;
-  const int q = crow * ntiles_pad + (int)(block % ntiles_pad);
-  it.ntile = 8 * (q / (8 * chunks)) + (q & 7);
-  it.chunk = (q >> 3) % chunks;
+  const BgmoeItemSlot slot = bgmoe_item_slot(crow, bgmoe_item_chunks(it.cnt, chunk_rows, tall), ntiles_pad, block);
+  it.ntile = slot.ntile;
+  it.chunk = slot.chunk;
+  it.rows = bgmoe_item_rows(it.cnt, chunk_rows, tall);
   if (it.ntile >= ntiles) it.grp = BGMOE_ITEM_PAD;
   // the fields are wave-uniform by construction; say so, so that everything derived from them (pointers,
   // loop bounds, branches) is scalar code
@@ -103,14 +106,6 @@ __device__ __forceinline__ BgmoeItem bgmoe_decode_item(const int32_t* seqlens, i
   it.ntile = __builtin_amdgcn_readfirstlane(it.ntile);
   it.chunk = __builtin_amdgcn_readfirstlane(it.chunk);
   it.cnt = __builtin_amdgcn_readfirstlane(it.cnt);
+  it.rows = __builtin_amdgcn_readfirstlane(it.rows);
   return it;
-}
-
-// Upper bound on the virtual blocks of a launch from host-side knowledge only: `row_bound` bounds the
-// total live rows, `max_rows` the rows of any group the launch serves.
-static inline unsigned bgmoe_item_grid(int ntiles, int groups, int64_t row_bound, int max_rows, int chunk_rows) {
-  int64_t items = groups + row_bound / chunk_rows;                 // >= sum of ceil(count / chunk_rows)
-  const int64_t per_group = (int64_t)groups * (((int64_t)max_rows + chunk_rows - 1) / chunk_rows);
-  if (per_group < items) items = per_group;
-  return (unsigned)(((ntiles + 7) & ~7) * items);
 }

@@ -57,6 +57,7 @@ struct SkinnyArgs {
   int64_t part_slice_stride;
   void* streamk_ws;           // workspace of the balanced form (gemm_fp8_streamk.hip) or null
   size_t streamk_ws_bytes;
+  int tall_min;               // stage 1 with tall items: groups with more rows than this use 64-row items (0: none)
 };
 
 template <int NSC>
@@ -320,18 +321,39 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
 
 // Persistent grid: block b works on virtual blocks b, b + gridDim.x, ... until the item list ends, so
 // a launch sized from host-side bounds pays nothing for the (many) virtual blocks past the real work.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT, int NTW = 4>
+//
+// TALL > 0: groups with more than g.tall_min rows are cut into items of 16 * TALL rows (two prefetch stages instead
+// of NSTAGE: the accumulators of the extra rows take the third stage's registers), all others into items of 16 * TT
+// rows as before.  A tall item passes over its weights half as often; every output element is computed by the same
+// chain of operations whatever the item height, so the results are the same bits.
+constexpr int kTallStages = 2;
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, int NTW = 4, int TALL = 0>
 __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned vblocks) {
-  __shared__ float s_amax[4][TT][16];
-  __shared__ __align__(16) uint8_t s_ring[NSTAGE * TokSlot<TT>::kBytes];
+  constexpr int TMAX = TALL > TT ? TALL : TT;
+  constexpr int kRingShort = NSTAGE * TokSlot<TT>::kBytes;
+  constexpr int kRingTall = TALL > 0 ? kTallStages * TokSlot<TMAX>::kBytes : 0;
+  __shared__ float s_amax_raw[4 * TMAX * 16];
+  __shared__ __align__(16) uint8_t s_ring[kRingShort > kRingTall ? kRingShort : kRingTall];
+  float (*s_amax)[TT][16] = reinterpret_cast<float (*)[TT][16]>(s_amax_raw);
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
   constexpr int kItemCols = FUSED ? 128 : 64 * NTW;
   const int ntiles = (g.n + kItemCols - 1) / kItemCols;
   const int hi = bgmoe_split_limit(g.seqlens, g.groups, g.split);
+  const BgmoeTall tall{TALL > 0 ? g.tall_min : 0, 16 * TALL};
   for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
-    const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, 0, hi, 16 * TT, ntiles, vb);
+    const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, 0, hi, 16 * TT, ntiles, vb, tall);
     if (it.grp == BGMOE_ITEM_END) break;
     if (it.grp == BGMOE_ITEM_PAD) continue;
+    if constexpr (TALL > 0) {
+      if (it.rows != 16 * TT) {           // wave-uniform: a tall group's item
+        float (*s_amax_tall)[TALL][16] = reinterpret_cast<float (*)[TALL][16]>(s_amax_raw);
+        if (it.cnt > 16 * TALL)
+          fp8_skinny_item<TALL, kTallStages, FUSED, LAYOUT, true, NTW>(g, it, s_amax_tall, s_ring, ring_lds);
+        else fp8_skinny_item<TALL, kTallStages, FUSED, LAYOUT, false, NTW>(g, it, s_amax_tall, s_ring, ring_lds);
+        __syncthreads();
+        continue;
+      }
+    }
     // a group with several row chunks has its weights streamed once per chunk: keep them cacheable
     if (it.cnt > 16 * TT) fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, true, NTW>(g, it, s_amax, s_ring, ring_lds);
     else fp8_skinny_item<TT, NSTAGE, FUSED, LAYOUT, false, NTW>(g, it, s_amax, s_ring, ring_lds);
@@ -358,6 +380,7 @@ __global__ __launch_bounds__(256) void fp8_dense_splitk_kernel(SkinnyArgs g, int
   it.cnt = m;
   it.ntile = (int)(b % (unsigned)ntiles);
   it.chunk = (int)(b / (unsigned)ntiles);
+  it.rows = 16 * TT;
   const int kb_lo = slice * per;
   const int kb_n = min(per, (g.k >> 7) - kb_lo);                       // >= 1 by the host's choice of ksplit
   if (m > 16 * TT) fp8_skinny_item<TT, NSTAGE, false, LAYOUT, true, NTW>(g, it, s_amax, s_ring, ring_lds, kb_lo, kb_n, slice);
@@ -423,17 +446,17 @@ static unsigned resident_blocks(K kernel, unsigned* cache) {
   return *cache;
 }
 
-template <int TT, int NS, bool FUSED, int LAYOUT, int NTW = 4>
+template <int TT, int NS, bool FUSED, int LAYOUT, int NTW = 4, int TALL = 0>
 static unsigned skinny_resident() {
   static unsigned resident = 0;
-  return resident_blocks(fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW>, &resident);
+  return resident_blocks(fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW, TALL>, &resident);
 }
 
-template <int TT, int NS, bool FUSED, int LAYOUT, int NTW = 4>
+template <int TT, int NS, bool FUSED, int LAYOUT, int NTW = 4, int TALL = 0>
 static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
-  const unsigned cap = skinny_resident<TT, NS, FUSED, LAYOUT, NTW>();
+  const unsigned cap = skinny_resident<TT, NS, FUSED, LAYOUT, NTW, TALL>();
   const dim3 grid(vblocks < cap ? vblocks : cap), block(256);
-  hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW>), grid, block, 0, st, g, vblocks);
+  hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW, TALL>), grid, block, 0, st, g, vblocks);
 }
 
 // Stage 1 works on 32-row items (its epilogue keeps 16*TT x 8 fp32 results per lane alive next to the
@@ -442,8 +465,12 @@ static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
 static void launch_variant(bool fused, int layout, int n, int groups, int64_t bound, int hi, const SkinnyArgs& g,
                            hipStream_t st) {
   if (fused) {
+    // (tall items only lower the item count: the same bound holds)
     const unsigned vb = bgmoe_item_grid((n + 127) / 128, groups, bound, hi, 32);
-    if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 3, true, BGMOE_W_TILE_MAJOR>(vb, g, st);
+    if (g.tall_min > 0) {
+      if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 3, true, BGMOE_W_TILE_MAJOR, 4, 4>(vb, g, st);
+      else launch_one<2, 3, true, BGMOE_W_ROW_MAJOR, 4, 4>(vb, g, st);
+    } else if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 3, true, BGMOE_W_TILE_MAJOR>(vb, g, st);
     else launch_one<2, 3, true, BGMOE_W_ROW_MAJOR>(vb, g, st);
   } else {
     // 128-column items (two weight tiles per wave): twice as many, half as long as 256-column ones, which evens
@@ -460,6 +487,8 @@ int bgmoe_internal_init_fp8_skinny() {
   skinny_resident<2, 3, true, BGMOE_W_ROW_MAJOR>();
   skinny_resident<4, 2, false, BGMOE_W_TILE_MAJOR, 2>();
   skinny_resident<4, 2, false, BGMOE_W_ROW_MAJOR, 2>();
+  skinny_resident<2, 3, true, BGMOE_W_TILE_MAJOR, 4, 4>();
+  skinny_resident<2, 3, true, BGMOE_W_ROW_MAJOR, 4, 4>();
   return BGMOE_OK;
 }
 
@@ -483,7 +512,17 @@ extern "C" int bgmoe_set_skinny_max_rows(int rows) {
   return BGMOE_OK;
 }
 
+// Stage 1 with tall items (opt-in): groups with more rows than this are cut into 64-row items, 0 = all 32-row items.
+static int g_skinny_tall_min = 0;
+
+extern "C" int bgmoe_set_skinny_tall_min_rows(int rows) {
+  BGMOE_REQUIRE(rows == 0 || rows >= 32, "set_skinny_tall_min_rows: rows must be 0 (off) or at least 32");
+  g_skinny_tall_min = rows;
+  return BGMOE_OK;
+}
+
 static int launch_skinny(bool fused, SkinnyArgs& g, int64_t m, hipStream_t st) {
+  g.tall_min = fused ? g_skinny_tall_min : 0;
   const int layout = g.w0.layout;
   if (fused && g.w1.layout != layout) {
     bgmoe_set_error("fp8_fused_s1: gate and up weights must use the same layout");

@@ -163,6 +163,37 @@ void hc_k64_acc_coord(uint32_t lane, uint32_t v, uint32_t* a_row, uint32_t* b_ro
 }
 
 
+// ---- weight-streaming kernels: virtual block -> work item ----------------------------------------------------------------
+// The device finds the group of item number block / ntiles_pad with a wave-wide prefix scan of bgmoe_item_chunks over
+// the groups with lo < count <= hi; here the same search is a loop.  out: 5 ints per virtual block (grp or -1 for a
+// padding n-tile, ntile, chunk, rows, count) for blocks 0, 1, ... until the list ends; returns the number of
+// virtual blocks before the end, or -1 when it exceeds cap.
+int64_t hc_item_walk(const int32_t* counts, int groups, int lo, int hi, int chunk_rows, int tall_min, int tall_rows,
+                     int ntiles, int32_t* out, int64_t cap) {
+  const BgmoeTall tall{tall_min, tall_rows};
+  const int ntiles_pad = (ntiles + 7) & ~7;
+  for (int64_t block = 0;; ++block) {
+    const int item = (int)(block / ntiles_pad);
+    int base = 0, grp = -1, crow = 0;
+    for (int g = 0; g < groups && grp < 0; ++g) {
+      const int c = counts[g];
+      const int mine = (c > lo && c <= hi) ? bgmoe_item_chunks(c, chunk_rows, tall) : 0;
+      if (item < base + mine) { grp = g; crow = item - base; }
+      base += mine;
+    }
+    if (grp < 0) return block;
+    if (block >= cap) return -1;
+    const int c = counts[grp];
+    const BgmoeItemSlot slot = bgmoe_item_slot(crow, bgmoe_item_chunks(c, chunk_rows, tall), ntiles_pad, (unsigned)block);
+    int32_t* o = out + 5 * block;
+    o[0] = slot.ntile >= ntiles ? -1 : grp;
+    o[1] = slot.ntile; o[2] = slot.chunk; o[3] = bgmoe_item_rows(c, chunk_rows, tall); o[4] = c;
+  }
+}
+unsigned hc_item_grid(int ntiles, int groups, int64_t row_bound, int max_rows, int chunk_rows) {
+  return bgmoe_item_grid(ntiles, groups, row_bound, max_rows, chunk_rows);
+}
+
 // ---- bf16 GEMM with 128 x 64 block tiles: one K step's loads and operand reads -----------------------------------------
 // experts [64][64] and tokens [128][64] bf16 values of one K step (given as uint16); the 24 issues of the block land
 // them in a stage; got_e [4 tiles][64 lanes][2 halves][8 values] and got_t [8 token tiles][64 lanes][2][8] are what the

@@ -93,6 +93,9 @@ def parse():
     ap.add_argument("--tiled-variant", type=int, default=0, choices=[0, 1, 2],
                     help="which LDS-tiled kernel serves the prefill groups: 0 = K steps of 128 (default), 1 = K steps of "
                          "64 with in-place accumulation, 2 = the same with plain per-lane stores (bgmoe_set_tiled_variant)")
+    ap.add_argument("--tall-min-rows", type=int, default=0,
+                    help="decode: groups with more rows than this run as 64-row stage-1 items of the weight-streaming "
+                         "kernel (bgmoe_set_skinny_tall_min_rows; 0 = off, the default)")
     ap.add_argument("--template", action="store_true",
                     help="FP8 configurations: also time the layer as a model file runs it through the MoEBase template "
                          "(router GEMM + gate, routed experts behind the given routes, dense shared expert, add) and "
@@ -422,6 +425,7 @@ def measure_layer(a, config, with_cpu):
         w, sh = wl.make_fp8_weights(cfg, dev)
         layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
     _lib.check(_lib.lib().bgmoe_set_tiled_variant(int(getattr(a, "tiled_variant", 0))))
+    _lib.check(_lib.lib().bgmoe_set_skinny_tall_min_rows(int(getattr(a, "tall_min_rows", 0))))
     x, logits = inp["x"], inp["logits"]
 
     for _ in range(a.warmup):
@@ -526,6 +530,8 @@ def measure_layer(a, config, with_cpu):
     roof["traffic"], roof["traffic_source"] = traffic_record(f"layer:{config}")
     if not decode and int(getattr(a, "tiled_variant", 0)) != 0:
         roof["kernel"] = "fp8_tiled_k64_kernel<fused,tile_major>"
+    if decode and not mx4 and int(getattr(a, "tall_min_rows", 0)) != 0:
+        roof["kernel"] = "fp8_skinny_kernel<fused,tile_major,tall items>"
 
     # Decode: the figure reported as `value` is the cache-flushed one.  A decode step of a real model finds none of
     # this layer's weights in the 256 MiB last-level cache (the other layers' weights have passed through it since),

@@ -501,6 +501,14 @@ int bgmoe_fp8_fused_s1_balanced(const bgmoe_fp8_act* a, const bgmoe_fp8_weight* 
  * Results do not depend on it beyond fp32 summation order. */
 int bgmoe_set_skinny_max_rows(int rows);
 
+/* Stage 1 of the weight-streaming kernel with tall work items (process-wide, opt-in; no counterpart in the reference).
+ * Groups with more than `rows` rows are cut into 64-row items instead of 32-row items, so that their weights are
+ * passed over half as often (a 256-row shared expert folded into a decode step: 4 passes instead of 8); the other
+ * groups keep the 32-row items and their three-stage prefetch.  rows = 0 (the default) turns it off; otherwise
+ * rows >= 32.  Every output element is computed by the same chain of operations either way: the results are the
+ * same bits.  Returns BGMOE_OK or BGMOE_ERR_ARG. */
+int bgmoe_set_skinny_tall_min_rows(int rows);
+
 /* Fused stage 1: out = bf16( silu(X*Wg^T) * (X*Wu^T) ), fp32 gate and up.
  * Replaces `fp8_blockwise_fused_s1` / `_ptrs`
  * (grouped_fp8_blockwise_moe.py:423-560, fp8_blockwise_s1_kernel.cuh:425-607).

@@ -84,6 +84,10 @@ def test_tuning_switches_check_their_arguments():
     for good in ([8] * 8, [2, 3] * 4, [23, 21] * 4):
         assert h.bgmoe_set_streamk_xcd_weights(w8(*good)) == 0, good
     assert h.bgmoe_debug_streamk_status(None) != 0
+    for bad in (-1, 1, 31):
+        assert h.bgmoe_set_skinny_tall_min_rows(bad) != 0 and b"at least 32" in h.bgmoe_last_error()
+    for good in (32, 64, 200, 0):
+        assert h.bgmoe_set_skinny_tall_min_rows(good) == 0
 
 
 def test_loader_and_op_names():

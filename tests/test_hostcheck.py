@@ -469,3 +469,68 @@ def test_narrow_bf16_gemm_tile_loads_and_reads(hc):
                 assert np.array_equal(got_e[tn, lane, jj], experts[16 * tn + r, k0: k0 + 8]), (tn, lane, jj)
             for wt in range(8):
                 assert np.array_equal(got_t[wt, lane, jj], tokens[16 * wt + r, k0: k0 + 8]), (wt, lane, jj)
+
+
+def item_walk(hc, counts, lo, hi, chunk_rows, tall_min, tall_rows, ntiles):
+    arr = (C.c_int32 * len(counts))(*counts)
+    cap = 1 << 16
+    out = (C.c_int32 * (5 * cap))()
+    hc.hc_item_walk.restype = C.c_int64
+    hc.hc_item_walk.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p,
+                                C.c_int64]
+    n = hc.hc_item_walk(arr, len(counts), lo, hi, chunk_rows, tall_min, tall_rows, ntiles, out, cap)
+    assert n >= 0
+    return [tuple(out[5 * b: 5 * b + 5]) for b in range(n)]
+
+
+def check_item_walk(hc, counts, lo, hi, chunk_rows, tall_min, tall_rows, ntiles, row_bound=None):
+    """Every (group, n-tile, chunk) of the served groups is some virtual block's item exactly once; the chunks
+    partition the group's rows; all chunks of one weight tile sit on one XCD (block % 8); the host's bound on the
+    virtual blocks covers the list."""
+    items = item_walk(hc, counts, lo, hi, chunk_rows, tall_min, tall_rows, ntiles)
+    seen = {}
+    for b, (grp, ntile, chunk, rows, cnt) in enumerate(items):
+        if grp < 0:
+            assert ntile >= ntiles
+            continue
+        assert cnt == counts[grp] and lo < cnt <= hi
+        want_rows = tall_rows if tall_min > 0 and cnt > tall_min else chunk_rows
+        assert rows == want_rows
+        assert 0 <= ntile < ntiles and 0 <= chunk * rows < cnt
+        assert (grp, ntile, chunk) not in seen
+        seen[(grp, ntile, chunk)] = b
+    for g, c in enumerate(counts):
+        if not lo < c <= hi:
+            continue
+        rows = tall_rows if tall_min > 0 and c > tall_min else chunk_rows
+        chunks = -(-c // rows)
+        for t in range(ntiles):
+            blocks = [seen[(g, t, ch)] for ch in range(chunks)]          # KeyError = an item nobody works on
+            assert len({b % 8 for b in blocks}) == 1, "the chunks of one weight tile are spread over several XCDs"
+    served = [c for c in counts if lo < c <= hi]
+    assert len(seen) == sum(-(-c // (tall_rows if tall_min > 0 and c > tall_min else chunk_rows)) for c in served) * ntiles
+    hc.hc_item_grid.restype = C.c_uint
+    hc.hc_item_grid.argtypes = [C.c_int, C.c_int, C.c_int64, C.c_int, C.c_int]
+    bound = sum(counts) if row_bound is None else row_bound
+    assert hc.hc_item_grid(ntiles, len(counts), bound, hi, chunk_rows) >= len(items)
+    return len(seen)
+
+
+def test_streaming_items_with_and_without_tall_groups(hc):
+    """Work items of the weight-streaming kernels (32-row chunks for the fused stage 1), with the opt-in tall items
+    (groups above a row count in 64-row chunks): configuration 1's draw, the shapes of the kernel tests, random
+    launches.  Tall items only lower the item count, so the host's grid bound holds unchanged."""
+    n32 = check_item_walk(hc, CONFIG1_DRAW, 0, 256, 32, 0, 0, 16)
+    n_tall32 = check_item_walk(hc, CONFIG1_DRAW, 0, 256, 32, 32, 64, 16)
+    n_tall64 = check_item_walk(hc, CONFIG1_DRAW, 0, 256, 32, 64, 64, 16)
+    # passes over a weight tile, by hand: 15 groups of at most 32 rows, then 41 / 65 / 39 / 35 / 256 rows
+    assert (n32, n_tall32, n_tall64) == ((15 + 2 + 3 + 2 + 2 + 8) * 16, (15 + 1 + 2 + 1 + 1 + 4) * 16, (15 + 2 + 2 + 2 + 2 + 4) * 16)
+    rng = random.Random(5)
+    for _ in range(200):
+        groups = rng.randint(1, 70)
+        counts = [rng.choice([0, 0, 1, 5, 16, 31, 32, 33, 63, 64, 65, 100, 128, 129, 200, 256, 300]) for _ in range(groups)]
+        ntiles = rng.choice([1, 3, 8, 9, 16, 56])
+        lo, hi = rng.choice([(0, 256), (0, 64), (64, 256), (0, 1 << 30)])
+        tall_min = rng.choice([0, 32, 40, 64, 128])
+        check_item_walk(hc, counts, lo, hi, rng.choice([16, 32, 64]) if tall_min == 0 else 32, tall_min, 64, ntiles,
+                        row_bound=sum(counts))
