@@ -96,6 +96,9 @@ _SIGS = {
     "bgmoe_mxfp4_grouped_gemm": (i32, [vp, C.POINTER(Mxfp4Weight), vp, vp, i32, i64, i32, i32, vp, vp, i64, vp]),
     "bgmoe_mxfp4_fused_s1": (i32, [vp, C.POINTER(Mxfp4Weight), C.POINTER(Mxfp4Weight), vp, vp, i32, i64, i32, i32, vp,
                                    vp, i32, i64, vp]),
+    "bgmoe_mxfp4_fused_s1_gather": (i32, [vp, i64, vp, i32, C.POINTER(Mxfp4Weight), C.POINTER(Mxfp4Weight), vp, vp, i32,
+                                          i64, i32, i32, vp, vp, i32, i64, vp]),
+    "bgmoe_dispatch_index_3d": (i32, [vp, i32, i32, i32, i32, i32, vp, vp, vp, vp, vp, sz, vp]),
     "bgmoe_compact_expert_data": (i32, [vp, i32, vp, vp, vp, vp, vp]),
     "bgmoe_fp8_grouped_gemm": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), vp, vp, i32, i64, i32, i32, vp, vp]),
     "bgmoe_fp8_fused_s1": (i32, [C.POINTER(Fp8Act), C.POINTER(Fp8Weight), C.POINTER(Fp8Weight), vp, vp, i32,

@@ -28,7 +28,12 @@ namespace {
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 
 struct Mx4Args {
-  const uint16_t* x;            // [m, k] bf16
+  const uint16_t* x;            // [m, k] bf16; with row_pair: [tokens, k], row r of a group's range reads token
+                                // row_pair[r] / pair_div
+  const int32_t* row_pair;      // optional [m]: the (token, slot) pair placed in each live row (pair = token * top_k + slot)
+  int pair_div;                 // top_k
+  uint32_t last_token;          // tokens - 1: a row's token index is clamped to it (no entry of the map can make a lane
+                                // read outside the token matrix)
   bgmoe_mxfp4_weight w0, w1;
   const int32_t* seqlens;
   const int32_t* cu;
@@ -60,7 +65,7 @@ __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float scale) {
 // chunk (p&15) ^ row, so that the MFMA operand reads (16 rows, same chunk) hit 16 different bank groups.
 // KEEP: the group has more row chunks than this one, so its weights are loaded with the default cache
 // policy (the next chunk finds them in L2); otherwise as a non-temporal stream.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP, int NT>
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool KEEP, int NT, bool MAPPED = false>
 __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it, const uint8_t* ring, uint32_t ring_lds) {
   constexpr int NH = NT / 2;                      // fused: gate tiles (= up tiles) per wave
   constexpr int NW = FUSED ? 16 * NH : 16 * NT;   // output columns per wave
@@ -108,7 +113,10 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
   uint16_t* const obase = g.out_ptrs ? g.out_ptrs[grp] : g.out + row0 * g.n;
 
   // tokens: wave w loads quarter-tiles w*TT .. w*TT+TT-1 (4 rows x 256 bytes each)
-  const uint8_t* tok_base = uniform_ptr(reinterpret_cast<const uint8_t*>(g.x + (row0 + t0) * K));
+  // With a row -> pair map the rows are read where the tokens lie (no gathered copy of them exists): the base is
+  // the token matrix and a lane's offset is its row's token times the row pitch (the host checks that the whole
+  // token matrix is addressable with 32-bit offsets).  Rows past the count repeat the last live row, as without.
+  const uint8_t* tok_base = uniform_ptr(reinterpret_cast<const uint8_t*>(MAPPED ? g.x : g.x + (row0 + t0) * K));
   uint32_t tok_off[TT];
   bool tok_on[TT];
 #pragma unroll
@@ -116,7 +124,9 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
     const int qt = (int)wave_u * TT + i;                  // quarter-tile 0 .. 4*TT-1
     const int rt = 4 * (qt & 3) + (lane >> 4);            // row inside its tile
     const int row = min(16 * (qt >> 2) + rt, live - 1);
-    tok_off[i] = (uint32_t)row * (uint32_t)(2 * K) + (uint32_t)((((lane & 15) ^ rt) & 15) * 16);
+    uint32_t src = (uint32_t)row;
+    if constexpr (MAPPED) src = min((uint32_t)g.row_pair[row0 + t0 + row] / (uint32_t)g.pair_div, g.last_token);
+    tok_off[i] = src * (uint32_t)(2 * K) + (uint32_t)((((lane & 15) ^ rt) & 15) * 16);
     tok_on[i] = (qt >> 2) < tiles;
   }
   auto issue_tokens = [&](int kb, int slot) {
@@ -233,7 +243,7 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
 // Item width is chosen per launch on the device: with 4 weight tiles per wave (128 fused / 256 plain output
 // columns per item) when that already gives every resident block an item, else with 2 tiles per wave --
 // fp4 weight stages are small, so with few items twice as many narrower ones keep more loads in flight.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT>
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool MAPPED = false>
 __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned vblocks, unsigned slots) {
   __shared__ __align__(16) uint8_t s_ring[NSTAGE * TT * 4096];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
@@ -247,8 +257,8 @@ __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned v
       const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, vb);
       if (it.grp == BGMOE_ITEM_END) break;
       if (it.grp == BGMOE_ITEM_PAD) continue;
-      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 2>(g, it, s_ring, ring_lds);
-      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 2>(g, it, s_ring, ring_lds);
+      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 2, MAPPED>(g, it, s_ring, ring_lds);
+      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 2, MAPPED>(g, it, s_ring, ring_lds);
       __syncthreads();                    // the token ring is reused by the next item
     }
   } else {
@@ -256,8 +266,8 @@ __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned v
       const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles_wide, vb);
       if (it.grp == BGMOE_ITEM_END) break;
       if (it.grp == BGMOE_ITEM_PAD) continue;
-      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 4>(g, it, s_ring, ring_lds);
-      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 4>(g, it, s_ring, ring_lds);
+      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 4, MAPPED>(g, it, s_ring, ring_lds);
+      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 4, MAPPED>(g, it, s_ring, ring_lds);
       __syncthreads();
     }
   }
@@ -292,12 +302,12 @@ int check_w(const char* what, const bgmoe_mxfp4_weight* w) {
 }
 
 // blocks resident on the whole device at once, a multiple of 8 (queried once per kernel)
-template <int TT, int NS, bool FUSED, int LAYOUT>
+template <int TT, int NS, bool FUSED, int LAYOUT, bool MAPPED = false>
 unsigned mx_resident() {
   static unsigned resident = 0;
   if (resident == 0) {
     int per_cu = 0, dev = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>, 256, 0) != hipSuccess || per_cu < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT, MAPPED>, 256, 0) != hipSuccess || per_cu < 1)
       per_cu = 1;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
@@ -308,15 +318,15 @@ unsigned mx_resident() {
   return resident;
 }
 
-template <int TT, int NS, bool FUSED, int LAYOUT>
+template <int TT, int NS, bool FUSED, int LAYOUT, bool MAPPED = false>
 void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
   // Twice as many blocks as fit at once: with up to two rounds of items every block has one item and the
   // hardware hands the second round out as blocks finish, which evens out items of unequal length (a 64-row
   // item takes 1.7x a 16-row one); beyond that the blocks stride.  Measured: skewed counts 14% faster,
   // uniform ones 3% slower (the late blocks' start-up).
-  const unsigned slots = mx_resident<TT, NS, FUSED, LAYOUT>();
+  const unsigned slots = mx_resident<TT, NS, FUSED, LAYOUT, MAPPED>();
   const dim3 grid(vblocks < 2 * slots ? vblocks : 2 * slots), block(256);
-  hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT>), grid, block, 0, st, g, vblocks,
+  hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT, MAPPED>), grid, block, 0, st, g, vblocks,
                      vblocks < slots ? vblocks : slots);
 }
 
@@ -330,7 +340,10 @@ int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
   g.lo = 0; g.hi = 0x7fffffff;     // every group: more rows = more chunks (weights re-streamed)
   const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
   BgmoeProf prof(fused ? BGMOE_K_MXFP4_S1 : BGMOE_K_MXFP4_GEMM, st);
-  if (fused) {
+  if (fused && g.row_pair != nullptr) {                  // stage 1 reading its rows through the row -> pair map
+    if (tm) launch_one<TT, 3, true, 1, true>(vblocks, g, st);
+    else launch_one<TT, 3, true, 0, true>(vblocks, g, st);
+  } else if (fused) {
     if (tm) launch_one<TT, 3, true, 1>(vblocks, g, st);
     else launch_one<TT, 3, true, 0>(vblocks, g, st);
   } else {
@@ -359,6 +372,8 @@ int bgmoe_internal_init_mxfp4() {
   mx_resident<kMxTT, 3, true, 0>();
   mx_resident<kMxTT, 3, false, 1>();
   mx_resident<kMxTT, 3, false, 0>();
+  mx_resident<kMxTT, 3, true, 1, true>();
+  mx_resident<kMxTT, 3, true, 0, true>();
   return BGMOE_OK;
 }
 
@@ -393,6 +408,34 @@ extern "C" int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight*
   BGMOE_REQUIRE(gate->layout == up->layout, "mxfp4_fused_s1: gate and up weights must use the same layout");
   Mx4Args g{};
   g.x = x; g.w0 = *gate; g.w1 = *up; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups; g.n = n; g.k = k;
+  g.out = out; g.out_ptrs = out_ptrs; g.row_bound = row_bound; g.activation = activation;
+  return launch(true, g, m, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_mxfp4_fused_s1_gather(const uint16_t* x_tokens, int64_t n_tokens, const int32_t* row_pair, int top_k,
+                                           const bgmoe_mxfp4_weight* gate, const bgmoe_mxfp4_weight* up,
+                                           const int32_t* seqlens, const int32_t* cu_seqlens, int groups, int64_t m,
+                                           int n, int k, uint16_t* out, uint16_t* const* out_ptrs, int activation,
+                                           int64_t row_bound, bgmoe_stream_t stream) {
+  int rc = check_shape("mxfp4_fused_s1_gather", x_tokens, seqlens, cu_seqlens, groups, m, n, k, out, out_ptrs);
+  if (rc != BGMOE_OK) return rc;
+  BGMOE_REQUIRE(activation == BGMOE_ACT_SWIGLU || activation == BGMOE_ACT_SITU,
+                "mxfp4_fused_s1_gather: activation must be BGMOE_ACT_SWIGLU (0) or BGMOE_ACT_SITU (1)");
+  BGMOE_REQUIRE(top_k > 0 && n_tokens >= 0, "mxfp4_fused_s1_gather: bad top_k=%d or n_tokens=%lld", top_k,
+                (long long)n_tokens);
+  // a lane addresses its token row with a 32-bit byte offset from the start of the token matrix
+  BGMOE_REQUIRE(n_tokens * 2 * (int64_t)k <= 4294967296LL,
+                "mxfp4_fused_s1_gather: token matrix of %lld x %d bf16 exceeds 4 GiB", (long long)n_tokens, k);
+  if (groups == 0 || m == 0) return BGMOE_OK;
+  BGMOE_REQUIRE(row_pair != nullptr && n_tokens > 0, "mxfp4_fused_s1_gather: null row_pair or no tokens");
+  rc = check_w("mxfp4_fused_s1_gather", gate);
+  if (rc != BGMOE_OK) return rc;
+  rc = check_w("mxfp4_fused_s1_gather", up);
+  if (rc != BGMOE_OK) return rc;
+  BGMOE_REQUIRE(gate->layout == up->layout, "mxfp4_fused_s1_gather: gate and up weights must use the same layout");
+  Mx4Args g{};
+  g.x = x_tokens; g.row_pair = row_pair; g.pair_div = top_k; g.last_token = (uint32_t)(n_tokens - 1);
+  g.w0 = *gate; g.w1 = *up; g.seqlens = seqlens; g.cu = cu_seqlens; g.groups = groups; g.n = n; g.k = k;
   g.out = out; g.out_ptrs = out_ptrs; g.row_bound = row_bound; g.activation = activation;
   return launch(true, g, m, bgmoe_stream(stream));
 }

@@ -137,17 +137,27 @@ extern "C" int bgmoe_moe_mxfp4_layer_forward(const bgmoe_moe_mxfp4_layer* L, int
   int rc;
   if (stages & BGMOE_MXFP4_ROUTED) {
     BGMOE_REQUIRE(L->x && L->logits && L->bias && L->topk_ids && L->expert_counts && L->expert_counters &&
-                  L->cu_seqlens && L->act && L->hmid, "moe_mxfp4_layer_forward: null input or buffer");
+                  L->cu_seqlens && (L->act || L->row_pair) && L->hmid, "moe_mxfp4_layer_forward: null input or buffer");
     rc = bgmoe_gate_sigmoid_topk(L->logits, L->e_total, L->bias, n, L->e_total, k, L->routed_scaling_factor,
                                  L->topk_ids, 0, L->topk_weights, nullptr, nullptr, 0, nullptr, 0, 0, stream);
     if (rc != BGMOE_OK) return rc;
-    rc = bgmoe_dispatch_scatter_3d(L->x, L->topk_ids, n, k, h, L->act, L->expert_start, el, L->max_tokens,
-                                   L->expert_counts, L->expert_counters, L->topk_pos, L->workspace,
-                                   L->workspace_bytes, stream);
-    if (rc != BGMOE_OK) return rc;
     const int64_t bound = (int64_t)n * k;
-    rc = bgmoe_mxfp4_fused_s1(L->act, &L->gate, &L->up, L->expert_counts, L->cu_seqlens, el, rows, inter, h,
-                              L->hmid, nullptr, L->activation, bound, stream);
+    if (L->row_pair != nullptr) {
+      // indices only; stage 1 reads each row from its token through the row -> pair map
+      rc = bgmoe_dispatch_index_3d(L->topk_ids, n, k, L->expert_start, el, L->max_tokens, L->expert_counts,
+                                   L->expert_counters, L->topk_pos, L->row_pair, L->workspace, L->workspace_bytes,
+                                   stream);
+      if (rc != BGMOE_OK) return rc;
+      rc = bgmoe_mxfp4_fused_s1_gather(L->x, n, L->row_pair, k, &L->gate, &L->up, L->expert_counts, L->cu_seqlens,
+                                       el, rows, inter, h, L->hmid, nullptr, L->activation, bound, stream);
+    } else {
+      rc = bgmoe_dispatch_scatter_3d(L->x, L->topk_ids, n, k, h, L->act, L->expert_start, el, L->max_tokens,
+                                     L->expert_counts, L->expert_counters, L->topk_pos, L->workspace,
+                                     L->workspace_bytes, stream);
+      if (rc != BGMOE_OK) return rc;
+      rc = bgmoe_mxfp4_fused_s1(L->act, &L->gate, &L->up, L->expert_counts, L->cu_seqlens, el, rows, inter, h,
+                                L->hmid, nullptr, L->activation, bound, stream);
+    }
     if (rc != BGMOE_OK) return rc;
     rc = bgmoe_mxfp4_grouped_gemm(L->hmid, &L->down, L->expert_counts, L->cu_seqlens, el, rows, h, inter, L->y,
                                   nullptr, bound, stream);

@@ -29,6 +29,8 @@ struct PermArgs {
   int32_t* counters;       // [e_local] (may be null)
   int32_t* cu;             // [e_local+1] (ragged; may be null for masked)
   int32_t* pos;            // [nk]
+  int32_t* row_pair;       // optional inverse map: row_pair[pos[i]] = i for every placed pair (rows without a pair keep
+                           // what they held)
   int32_t* chunk_hist;     // workspace [nchunks][e_local]
   int nchunks;
   int extra_count;         // >= 0: one more group (counts[e_local] = extra_count,
@@ -188,6 +190,7 @@ __global__ __launch_bounds__(256) void perm_rank_kernel(PermArgs a) {
         else p = (SINGLE ? s_cu[le] : a.cu[le]) + slot;
       }
       a.pos[i] = p;
+      if (a.row_pair != nullptr && p >= 0) a.row_pair[p] = (int32_t)i;
     }
   }
 }
@@ -283,6 +286,7 @@ __device__ __forceinline__ void perm_small_body(const PermArgs& a, int32_t (*whi
         else p = s_cu[le[s]] + slot;
       }
       if (global) a.pos[i] = p;
+      if (global && a.row_pair != nullptr && p >= 0) a.row_pair[p] = (int32_t)i;
       if (s_pos) s_pos[i] = p;
     }
   }
@@ -516,6 +520,26 @@ extern "C" int bgmoe_dispatch_scatter_3d(const uint16_t* x, const int32_t* topk_
   if (rc != BGMOE_OK || act_buffer == nullptr) return rc;
   BGMOE_REQUIRE(n == 0 || x, "dispatch_scatter_3d: null x");
   return run_gather(x, topk_pos, act_buffer, a.nk, k, h, bgmoe_stream(stream));
+}
+
+extern "C" int bgmoe_dispatch_index_3d(const int32_t* topk_ids, int n, int k, int expert_start, int num_local_experts,
+                                       int max_tokens_padded, int32_t* expert_counts, int32_t* expert_counters,
+                                       int32_t* topk_pos, int32_t* row_pair, void* workspace, size_t workspace_bytes,
+                                       bgmoe_stream_t stream) {
+  BGMOE_REQUIRE(n >= 0 && k > 0, "dispatch_index_3d: bad sizes n=%d k=%d", n, k);
+  BGMOE_REQUIRE(num_local_experts > 0 && num_local_experts <= kMaxLocal,
+                "dispatch_index_3d: num_local_experts=%d outside [1,%d]", num_local_experts, kMaxLocal);
+  BGMOE_REQUIRE(max_tokens_padded > 0, "dispatch_index_3d: max_tokens_padded must be positive");
+  BGMOE_REQUIRE((int64_t)num_local_experts * max_tokens_padded <= 2147483647LL && (int64_t)n * k <= 2147483647LL,
+                "dispatch_index_3d: E_local*max_tokens_padded or n*k exceeds int32");
+  BGMOE_REQUIRE(expert_counts && topk_pos && row_pair, "dispatch_index_3d: null output");
+  BGMOE_REQUIRE(n == 0 || topk_ids, "dispatch_index_3d: null topk_ids");
+  PermArgs a{};
+  a.ids = topk_ids; a.nk = (int64_t)n * k; a.expert_start = expert_start;
+  a.e_local = num_local_experts; a.mtp = max_tokens_padded; a.row_align = 1;
+  a.counts = expert_counts; a.counters = expert_counters; a.cu = nullptr; a.pos = topk_pos; a.row_pair = row_pair;
+  a.extra_count = -1;
+  return run_index(a, workspace, workspace_bytes, bgmoe_stream(stream));
 }
 
 extern "C" int bgmoe_dispatch_scatter_ragged(const uint16_t* x, const int32_t* topk_ids, int n, int k,

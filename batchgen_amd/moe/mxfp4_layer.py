@@ -42,7 +42,7 @@ class Mxfp4LayerStruct(C.Structure):
         ("gate", Mxfp4Weight), ("up", Mxfp4Weight), ("down", Mxfp4Weight),
         ("topk_ids", vp), ("topk_weights", vp), ("expert_counts", vp), ("expert_counters", vp), ("cu_seqlens", vp),
         ("topk_pos", vp), ("act", vp), ("hmid", vp), ("y", vp), ("workspace", vp), ("workspace_bytes", sz),
-        ("shared_out", vp), ("out", vp), ("activation", i32),
+        ("shared_out", vp), ("out", vp), ("activation", i32), ("row_pair", vp),
     ]
 
 
@@ -54,14 +54,18 @@ K3_SITU_BETA, K3_SITU_LINEAR_BETA = 4.0, 25.0   # the constants the fused stage-
 
 class Mxfp4MoELayer:
     def __init__(self, cfg: MoEConfig, weights, shared_bf16, bias: torch.Tensor, shared_mode: str = "bf16_add",
-                 latent=None, dense_backend: str = "hip"):
+                 latent=None, dense_backend: str = "hip", fold_gather: bool = False):
         """``dense_backend``: "hip" (the default) runs the bf16 shared expert and the latent projections on this
         library's own bf16 GEMM, so that the whole layer is this library's kernels and a token's result does not
         depend on its position in the batch; "vendor" runs them on the vendor library through ``torch.mm``, as
         ``nn.Linear`` in the reference does (faster at 512 tokens: measured 45 + 35 us against 2 x 92 us for the
         shared expert; kept for that comparison, never chosen silently).  Either way the results go into buffers
         owned by the layer: ``forward`` allocates no tensor, and what it returns is one of those buffers,
-        overwritten by the next call."""
+        overwritten by the next call.
+
+        ``fold_gather`` (opt-in): the dispatch only computes indices and stage 1 reads every row from its token
+        through a row -> pair map, instead of from a gathered expert-major copy of the rows; same results, one
+        launch and one pass over the rows fewer."""
         if dense_backend not in ("hip", "vendor"):
             raise ValueError(f"dense_backend must be 'hip' or 'vendor', got {dense_backend!r}")
         self.dense_backend = dense_backend
@@ -107,7 +111,9 @@ class Mxfp4MoELayer:
         self.expert_counters = torch.zeros(el, dtype=i4, device=dev)
         self.cu = (torch.arange(el + 1, dtype=i4, device=dev) * cfg.max_tokens).contiguous()
         self.topk_pos = torch.empty(n * k, dtype=i4, device=dev)
-        self.act = torch.zeros((self.rows, h), dtype=b2, device=dev)
+        self.fold_gather = bool(fold_gather)
+        self.act = None if self.fold_gather else torch.zeros((self.rows, h), dtype=b2, device=dev)
+        self.row_pair = torch.zeros(self.rows, dtype=i4, device=dev) if self.fold_gather else None
         self.hmid = torch.zeros((self.rows, inter), dtype=b2, device=dev)
         self.y = torch.zeros((self.rows, h), dtype=b2, device=dev)
         self.out = torch.empty((n, h), dtype=b2, device=dev)
@@ -121,7 +127,9 @@ class Mxfp4MoELayer:
         L.gate, L.up, L.down = self.w["gate"][2], self.w["up"][2], self.w["down"][2]
         L.topk_ids, L.topk_weights = ptr(self.topk_ids), ptr(self.topk_weights)
         L.expert_counts, L.expert_counters, L.cu_seqlens = ptr(self.expert_counts), ptr(self.expert_counters), ptr(self.cu)
-        L.topk_pos, L.act, L.hmid, L.y = ptr(self.topk_pos), ptr(self.act), ptr(self.hmid), ptr(self.y)
+        L.topk_pos, L.hmid, L.y = ptr(self.topk_pos), ptr(self.hmid), ptr(self.y)
+        L.act = ptr(self.act) if self.act is not None else None
+        L.row_pair = ptr(self.row_pair) if self.row_pair is not None else None
         L.workspace, L.workspace_bytes = ptr(self.workspace), self.workspace.numel()
         L.out = ptr(self.out)
         L.activation = ACTIVATIONS[cfg.activation]

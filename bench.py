@@ -93,6 +93,9 @@ def parse():
     ap.add_argument("--tiled-variant", type=int, default=0, choices=[0, 1, 2],
                     help="which LDS-tiled kernel serves the prefill groups: 0 = K steps of 128 (default), 1 = K steps of "
                          "64 with in-place accumulation, 2 = the same with plain per-lane stores (bgmoe_set_tiled_variant)")
+    ap.add_argument("--fold-gather", action="store_true",
+                    help="MXFP4 configurations: stage 1 reads its rows from the tokens through the dispatch's row -> pair "
+                         "map instead of from a gathered copy (Mxfp4MoELayer(fold_gather=True))")
     ap.add_argument("--tall-min-rows", type=int, default=0,
                     help="decode: groups with more rows than this run as 64-row stage-1 items of the weight-streaming "
                          "kernel (bgmoe_set_skinny_tall_min_rows; 0 = off, the default)")
@@ -420,6 +423,8 @@ def measure_layer(a, config, with_cpu):
         w, sh = wl.make_mxfp4_weights(cfg, dev)
         lat = wl.make_latent_weights(cfg, dev) if cfg.latent else None
         kw = {"dense_backend": a.dense_backend} if a.dense_backend else {}
+        if getattr(a, "fold_gather", False):
+            kw["fold_gather"] = True
         layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], latent=lat, **kw)
     else:
         w, sh = wl.make_fp8_weights(cfg, dev)

@@ -275,6 +275,14 @@ int bgmoe_dispatch_scatter_3d(const uint16_t* x, const int32_t* topk_ids, int n,
                               int32_t* expert_counters, int32_t* topk_pos, void* workspace,
                               size_t workspace_bytes, bgmoe_stream_t stream);
 
+/* The index part of bgmoe_dispatch_scatter_3d alone, plus the inverse map (no counterpart in the reference): same
+ * expert_counts / expert_counters / topk_pos, no rows are moved, and row_pair[topk_pos[i]] = i for every placed pair
+ * i = token * k + slot (rows of the masked layout that hold no pair keep what they held).  For consumers that read
+ * a row's data from its token instead of from a gathered copy (bgmoe_mxfp4_fused_s1_gather). */
+int bgmoe_dispatch_index_3d(const int32_t* topk_ids, int n, int k, int expert_start, int num_local_experts,
+                            int max_tokens_padded, int32_t* expert_counts, int32_t* expert_counters, int32_t* topk_pos,
+                            int32_t* row_pair, void* workspace, size_t workspace_bytes, bgmoe_stream_t stream);
+
 /* Contiguous ragged layout.  Replaces `dispatch_scatter_ragged`
  * (dispatch_scatter_3d.py:112-156, dispatch_scatter_3d.cu:152-358) and, with
  * row_align = 1, `dispatch_count_gather`
@@ -573,6 +581,16 @@ int bgmoe_mxfp4_fused_s1(const uint16_t* x, const bgmoe_mxfp4_weight* gate,
                          uint16_t* const* out_ptrs, int activation, int64_t row_bound,
                          bgmoe_stream_t stream);
 
+/* The same with the rows read where the tokens lie (no counterpart in the reference, whose dispatch always copies
+ * the rows into the expert-major buffer first): x_tokens is the [n_tokens, k] token matrix, and row r of group g
+ * (r in [cu_seqlens[g], cu_seqlens[g] + seqlens[g])) is token row_pair[r] / top_k -- row_pair as written by
+ * bgmoe_dispatch_index_3d.  A token index is clamped to n_tokens - 1, so that no map entry can make the kernel read
+ * outside x_tokens; n_tokens * k * 2 must not exceed 4 GiB.  Same results as bgmoe_mxfp4_fused_s1 on the gathered rows. */
+int bgmoe_mxfp4_fused_s1_gather(const uint16_t* x_tokens, int64_t n_tokens, const int32_t* row_pair, int top_k,
+                                const bgmoe_mxfp4_weight* gate, const bgmoe_mxfp4_weight* up, const int32_t* seqlens,
+                                const int32_t* cu_seqlens, int groups, int64_t m, int n, int k, uint16_t* out,
+                                uint16_t* const* out_ptrs, int activation, int64_t row_bound, bgmoe_stream_t stream);
+
 /* DeepGEMM's contiguous m-grouped API describes the rows by a map `grouped_layout` [m] (row -> group, -1 on
  * alignment padding; batchgen/moe/grouped_fp8_deepgemm_moe.py:9-22, built by `build_grouped_layout`, :118-186).
  * This call turns the map into what the grouped GEMMs here take: starts[g] = first row of group g (starts has
@@ -745,6 +763,9 @@ typedef struct bgmoe_moe_mxfp4_layer {
   const uint16_t* shared_out;     /* [n,h] bf16 or NULL                                       */
   uint16_t* out;                  /* [n,h] bf16                                               */
   int32_t activation;             /* BGMOE_ACT_SWIGLU or BGMOE_ACT_SITU                       */
+  int32_t* row_pair;              /* NULL, or [e_local*max_tokens]: the dispatch only computes indices (this row ->
+                                   * pair map included) and stage 1 reads its rows from x through the map; `act`
+                                   * is then unused and may be NULL.  Same results.               */
 } bgmoe_moe_mxfp4_layer;
 
 int bgmoe_moe_mxfp4_layer_forward(const bgmoe_moe_mxfp4_layer* layer, int stages, bgmoe_stream_t stream);

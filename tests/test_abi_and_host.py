@@ -37,16 +37,23 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_struct_layout_matches_the_header(tmp_path):
     from batchgen_amd import _lib
     from batchgen_amd.moe.fp8_layer import LayerStruct
+    from batchgen_amd.moe.mxfp4_layer import Mxfp4LayerStruct
     prog = tmp_path / "sz.c"
     prog.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "bgmoe.h"\n'
-                    'int main(){printf("%zu %zu %zu %zu %zu %zu\\n", sizeof(bgmoe_fp8_weight), sizeof(bgmoe_fp8_act),'
+                    'int main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(bgmoe_fp8_weight),'
+                    'sizeof(bgmoe_fp8_act),'
                     'sizeof(bgmoe_moe_fp8_layer), offsetof(bgmoe_moe_fp8_layer, cap_rows),'
-                    'offsetof(bgmoe_moe_fp8_layer, gate), offsetof(bgmoe_moe_fp8_layer, out));return 0;}\n')
+                    'offsetof(bgmoe_moe_fp8_layer, gate), offsetof(bgmoe_moe_fp8_layer, out),'
+                    'sizeof(bgmoe_mxfp4_weight), sizeof(bgmoe_moe_mxfp4_layer), offsetof(bgmoe_moe_mxfp4_layer, gate),'
+                    'offsetof(bgmoe_moe_mxfp4_layer, activation), offsetof(bgmoe_moe_mxfp4_layer, row_pair));'
+                    'return 0;}\n')
     exe = tmp_path / "sz"
     subprocess.run(["gcc", f"-I{os.path.join(ROOT, 'include')}", str(prog), "-o", str(exe)], check=True)
     got = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
     want = [ctypes.sizeof(_lib.Fp8Weight), ctypes.sizeof(_lib.Fp8Act), ctypes.sizeof(LayerStruct),
-            LayerStruct.cap_rows.offset, LayerStruct.gate.offset, LayerStruct.out.offset]
+            LayerStruct.cap_rows.offset, LayerStruct.gate.offset, LayerStruct.out.offset,
+            ctypes.sizeof(_lib.Mxfp4Weight), ctypes.sizeof(Mxfp4LayerStruct), Mxfp4LayerStruct.gate.offset,
+            Mxfp4LayerStruct.activation.offset, Mxfp4LayerStruct.row_pair.offset]
     assert got == want
 
 
@@ -65,6 +72,14 @@ def test_errors_are_reported_without_a_gpu():
     assert b"act_buffer rows" in h.bgmoe_last_error()
     assert h.bgmoe_dispatch_workspace_bytes(2048, 32) == 0 and h.bgmoe_dispatch_workspace_bytes(131072, 32) == 64 * 32 * 4
     assert h.bgmoe_fp8_weight_repack(None, None, 1, 100, 128, None) != 0
+    p16 = ctypes.c_void_p(16)
+    assert h.bgmoe_dispatch_index_3d(p16, 4, 2, 0, 4, 8, p16, None, p16, None, None, 0, None) != 0
+    assert b"null output" in h.bgmoe_last_error()
+    assert h.bgmoe_dispatch_index_3d(p16, 4, 2, 0, 4, 0, p16, None, p16, p16, None, 0, None) != 0
+    assert b"max_tokens_padded" in h.bgmoe_last_error()
+    assert h.bgmoe_mxfp4_fused_s1_gather(p16, 1 << 20, p16, 8, None, None, p16, p16, 4, 64, 128, 4096, p16, None, 0, 0,
+                                         None) != 0
+    assert b"exceeds 4 GiB" in h.bgmoe_last_error()
 
 
 def test_tuning_switches_check_their_arguments():
