@@ -181,6 +181,13 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
   // K-block, loads complete in issue order, so "at most the 2*NT weight loads of the youngest stage
   // outstanding" means the stage about to be computed has landed for this wave; the barrier extends
   // that to the other waves' token loads and frees the slot refilled next.
+  // With more than three stages several younger stages are in flight at the wait: each of them has at least its
+  // 2*NT weight loads outstanding (token loads of dead tiles are skipped, so they cannot be counted on), and so has
+  // the stage about to be computed, whose weight loads follow its token loads: "at most 2*NT*(NSTAGE-1)
+  // outstanding" is then what says that this stage's tokens have landed (its weights are the compiler's own loads
+  // and waited for by the compiler).
+  constexpr int kWaitLoads = NSTAGE <= 3 ? 2 * NT : 2 * NT * (NSTAGE - 1);
+  static_assert(kWaitLoads <= 63, "s_waitcnt vmcnt holds six bits");
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s) {
     issue_tokens(min(s, KB - 1), s);
@@ -190,7 +197,7 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
   for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
-      wait_vm<2 * NT>();
+      wait_vm<kWaitLoads>();
       block_barrier();
       issue_tokens(min(kb0 + s + NSTAGE - 1, KB - 1), (s + NSTAGE - 1) % NSTAGE);
       load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
@@ -331,25 +338,37 @@ void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
 }
 
 constexpr int kMxTT = 4;           // 64-row items: every group is streamed once per 64 rows
+// The opt-in variant: 32-row items with six prefetch stages.  fp4 weight stages are small (4 KB per wave and K-block
+// against 8 KB of the FP8 kernel), so three stages keep 8 KB per wave in flight; the accumulators of the other 32 rows
+// pay for three more stages (20 KB in flight per wave) at the same two blocks per CU and the same 48 KB token ring.
+// bf16 token rows weigh four times their weights, so a 32-row item is also the better-balanced unit.
+constexpr int kMxTT2 = 2, kMxNS2 = 6;
+int g_mx_variant = 0;
+
+template <int TT, int NS>
+void launch_shape(bool fused, bool tm, unsigned vblocks, const Mx4Args& g, hipStream_t st) {
+  if (fused && g.row_pair != nullptr) {                  // stage 1 reading its rows through the row -> pair map
+    if (tm) launch_one<TT, NS, true, 1, true>(vblocks, g, st);
+    else launch_one<TT, NS, true, 0, true>(vblocks, g, st);
+  } else if (fused) {
+    if (tm) launch_one<TT, NS, true, 1>(vblocks, g, st);
+    else launch_one<TT, NS, true, 0>(vblocks, g, st);
+  } else {
+    if (tm) launch_one<TT, NS, false, 1>(vblocks, g, st);
+    else launch_one<TT, NS, false, 0>(vblocks, g, st);
+  }
+}
 
 int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
-  constexpr int TT = kMxTT;
+  const int tt = g_mx_variant == 1 ? kMxTT2 : kMxTT;
   const int ntile = fused ? 64 : 128;      // the narrow item width bounds the virtual block count of both widths
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
-  const unsigned vblocks = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 16 * TT);
+  const unsigned vblocks = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 16 * tt);
   g.lo = 0; g.hi = 0x7fffffff;     // every group: more rows = more chunks (weights re-streamed)
   const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
   BgmoeProf prof(fused ? BGMOE_K_MXFP4_S1 : BGMOE_K_MXFP4_GEMM, st);
-  if (fused && g.row_pair != nullptr) {                  // stage 1 reading its rows through the row -> pair map
-    if (tm) launch_one<TT, 3, true, 1, true>(vblocks, g, st);
-    else launch_one<TT, 3, true, 0, true>(vblocks, g, st);
-  } else if (fused) {
-    if (tm) launch_one<TT, 3, true, 1>(vblocks, g, st);
-    else launch_one<TT, 3, true, 0>(vblocks, g, st);
-  } else {
-    if (tm) launch_one<TT, 3, false, 1>(vblocks, g, st);
-    else launch_one<TT, 3, false, 0>(vblocks, g, st);
-  }
+  if (g_mx_variant == 1) launch_shape<kMxTT2, kMxNS2>(fused, tm, vblocks, g, st);
+  else launch_shape<kMxTT, 3>(fused, tm, vblocks, g, st);
   return bgmoe_check_launch("mxfp4 grouped gemm");
 }
 
@@ -374,6 +393,19 @@ int bgmoe_internal_init_mxfp4() {
   mx_resident<kMxTT, 3, false, 0>();
   mx_resident<kMxTT, 3, true, 1, true>();
   mx_resident<kMxTT, 3, true, 0, true>();
+  mx_resident<kMxTT2, kMxNS2, true, 1>();
+  mx_resident<kMxTT2, kMxNS2, true, 0>();
+  mx_resident<kMxTT2, kMxNS2, false, 1>();
+  mx_resident<kMxTT2, kMxNS2, false, 0>();
+  mx_resident<kMxTT2, kMxNS2, true, 1, true>();
+  mx_resident<kMxTT2, kMxNS2, true, 0, true>();
+  return BGMOE_OK;
+}
+
+extern "C" int bgmoe_set_mxfp4_variant(int variant) {
+  BGMOE_REQUIRE(variant == 0 || variant == 1, "set_mxfp4_variant: variant must be 0 (64-row items, three stages) or 1 "
+                                              "(32-row items, six stages), got %d", variant);
+  g_mx_variant = variant;
   return BGMOE_OK;
 }
 

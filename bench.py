@@ -93,6 +93,9 @@ def parse():
     ap.add_argument("--tiled-variant", type=int, default=0, choices=[0, 1, 2],
                     help="which LDS-tiled kernel serves the prefill groups: 0 = K steps of 128 (default), 1 = K steps of "
                          "64 with in-place accumulation, 2 = the same with plain per-lane stores (bgmoe_set_tiled_variant)")
+    ap.add_argument("--mxfp4-variant", type=int, default=0, choices=[0, 1],
+                    help="MXFP4 configurations: 0 = 64-row items with three prefetch stages (default), 1 = 32-row items "
+                         "with six (bgmoe_set_mxfp4_variant)")
     ap.add_argument("--fold-gather", action="store_true",
                     help="MXFP4 configurations: stage 1 reads its rows from the tokens through the dispatch's row -> pair "
                          "map instead of from a gathered copy (Mxfp4MoELayer(fold_gather=True))")
@@ -431,6 +434,7 @@ def measure_layer(a, config, with_cpu):
         layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
     _lib.check(_lib.lib().bgmoe_set_tiled_variant(int(getattr(a, "tiled_variant", 0))))
     _lib.check(_lib.lib().bgmoe_set_skinny_tall_min_rows(int(getattr(a, "tall_min_rows", 0))))
+    _lib.check(_lib.lib().bgmoe_set_mxfp4_variant(int(getattr(a, "mxfp4_variant", 0))))
     x, logits = inp["x"], inp["logits"]
 
     for _ in range(a.warmup):

@@ -591,6 +591,13 @@ int bgmoe_mxfp4_fused_s1_gather(const uint16_t* x_tokens, int64_t n_tokens, cons
                                 const int32_t* cu_seqlens, int groups, int64_t m, int n, int k, uint16_t* out,
                                 uint16_t* const* out_ptrs, int activation, int64_t row_bound, bgmoe_stream_t stream);
 
+/* Which shape of the MXFP4 weight-streaming kernel serves the calls above (process-wide, opt-in; no counterpart in
+ * the reference): 0 = 64-row work items with a three-stage weight prefetch (the default), 1 = 32-row items with a
+ * six-stage prefetch (2.5 times the weight bytes in flight per wave, groups above 32 rows pass over their weights
+ * once per 32 rows).  Every output element is computed by the same chain of operations: same bits.
+ * Returns BGMOE_OK or BGMOE_ERR_ARG. */
+int bgmoe_set_mxfp4_variant(int variant);
+
 /* DeepGEMM's contiguous m-grouped API describes the rows by a map `grouped_layout` [m] (row -> group, -1 on
  * alignment padding; batchgen/moe/grouped_fp8_deepgemm_moe.py:9-22, built by `build_grouped_layout`, :118-186).
  * This call turns the map into what the grouped GEMMs here take: starts[g] = first row of group g (starts has
