@@ -365,7 +365,11 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
               *reinterpret_cast<uint32_t*>(patch + bgmoe_k64_qpatch_write_off(lane, (uint32_t)q)) =
                   pack4_e4m3(qv[0], qv[1], qv[2], qv[3]);
             }
+            // (the patch goes from lane to lane inside the wave: LDS serves a wave's accesses in order, so no wait is
+            // needed; the wave barrier is no instruction, it keeps the compiler from moving accesses across it)
+            __builtin_amdgcn_wave_barrier();
             const uint4 v = *reinterpret_cast<const uint4*>(patch + bgmoe_k64_qpatch_read_off(lane));
+            __builtin_amdgcn_wave_barrier();
             const int rtok = m0 + 128 * (int)wm + 32 * b + (int)bgmoe_k64_qpatch_read_token(lane);
             if (rtok < cnt)
               *reinterpret_cast<uint4*>(g.out_q + (row0 + rtok) * g.n + n0 + 32 * (int)wn +
@@ -411,7 +415,9 @@ __global__ __launch_bounds__(NT) void fp8_tiled_k64_kernel(BgmoeTiledArgs g) {
                   }
                 }
               }
+              __builtin_amdgcn_wave_barrier();
               const uint4 v = *reinterpret_cast<const uint4*>(patch + bgmoe_k64_patch_read_off(lane));
+              __builtin_amdgcn_wave_barrier();
               const int rtok = m0 + 128 * (int)wm + 32 * b + (int)bgmoe_k64_patch_read_token(p, lane);
               if (rtok < cnt)
                 *reinterpret_cast<uint4*>(g.out + (row0 + rtok) * g.n + colw + (int)bgmoe_k64_patch_read_col(lane)) = v;

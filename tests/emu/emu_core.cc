@@ -1,0 +1,472 @@
+// TEST INFRASTRUCTURE: CPU emulator behind tests/emu/shim/hip/hip_runtime.h.  One fiber per GPU lane, blocks of a
+// launch one after the other.  Fibers run until they reach a rendezvous (a wave-wide operation or a barrier); a
+// wave-wide operation is carried out when every lane of the wave that is still running has arrived at it.  Lanes of
+// a wave are therefore NOT in lockstep between rendezvous points: code that exchanges data between lanes through LDS
+// without a barrier needs __builtin_amdgcn_wave_barrier() (a rendezvous here, no instruction on the GPU).
+// Divergence: when every running fiber of a block is waiting and a wave's lanes wait at different call sites, the
+// group at the lowest code address goes first (the taken side of a structured `if` precedes the join point).
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <sys/mman.h>
+
+#include <vector>
+
+#include "../../include/bgmoe.h"
+
+extern "C" void emu_switch(void** save_sp, void* load_sp);
+asm(R"(
+.text
+.globl emu_switch
+.type emu_switch,@function
+emu_switch:
+  pushq %rbp
+  pushq %rbx
+  pushq %r12
+  pushq %r13
+  pushq %r14
+  pushq %r15
+  movq %rsp, (%rdi)
+  movq %rsi, %rsp
+  popq %r15
+  popq %r14
+  popq %r13
+  popq %r12
+  popq %rbx
+  popq %rbp
+  ret
+.size emu_switch, .-emu_switch
+)");
+
+namespace emu {
+namespace {
+
+enum Op { OP_NONE = 0, OP_SYNC, OP_SHFL, OP_BALLOT, OP_RFL, OP_RLANE, OP_MFMA16_F8, OP_MFMA32_F8, OP_MFMA16_BF16, OP_BARRIER };
+
+struct Pending { const uint8_t* src; uint8_t* dst; unsigned bytes; };
+
+struct Fiber {
+  Lane lane;
+  void* sp = nullptr;
+  uint8_t* stack = nullptr;
+  bool done = false;
+  Op op = OP_NONE;                 // what the fiber waits at (OP_NONE: runnable)
+  const void* site = nullptr;
+  uint32_t in[40];
+  uint32_t out[16];
+  std::vector<Pending> pending;    // lazy asynchronous loads, oldest first
+  uint32_t async_seq = 0;
+};
+
+constexpr size_t kStack = 256 * 1024;
+constexpr int kMaxThreads = 1024;
+
+std::vector<Fiber> g_fibers;
+std::vector<uint8_t*> g_stacks;
+Fiber* g_cur = nullptr;
+void* g_sched_sp = nullptr;
+const std::function<void()>* g_body = nullptr;
+alignas(256) uint8_t g_dynamic_lds[160 * 1024];
+bool g_lazy = false;
+uint64_t g_stat_launches = 0, g_stat_blocks = 0, g_stat_rendezvous = 0, g_stat_async = 0;
+struct UniformTag { uint32_t seq; const void* base; uint32_t lds; bool used; };
+std::vector<UniformTag> g_uniform;   // [wave][slot]: what the first lane of a wave passed for its seq-th async load
+constexpr int kUniformSlots = 64;
+
+[[noreturn]] void die(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  fprintf(stderr, "emu: ");
+  vfprintf(stderr, fmt, ap);
+  fprintf(stderr, "\n");
+  va_end(ap);
+  fflush(stderr);
+  abort();
+}
+
+void fiber_main() {
+  (*g_body)();
+  Fiber* f = g_cur;
+  for (const Pending& p : f->pending) memcpy(p.dst, p.src, p.bytes);   // whatever was still in flight lands
+  f->pending.clear();
+  f->done = true;
+  emu_switch(&f->sp, g_sched_sp);
+  die("a finished fiber was resumed");
+}
+
+void yield_to_scheduler() {
+  Fiber* f = g_cur;
+  emu_switch(&f->sp, g_sched_sp);
+}
+
+float bf16_to_f32(uint16_t b) {
+  const uint32_t u = (uint32_t)b << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+// carries out the operation the fibers [first, first + n) of one wave wait at (all at the same site), for the
+// lanes in `who`
+void perform(Fiber* wave, const std::vector<int>& who) {
+  const Op op = wave[who[0]].op;
+  ++g_stat_rendezvous;
+  switch (op) {
+    case OP_SYNC:
+    case OP_BARRIER:
+      break;
+    case OP_SHFL:
+    case OP_RLANE:
+      for (int l : who) {
+        const int src = (int)(wave[l].in[1] & 63u);
+        bool present = false;
+        for (int m : who) present = present || m == src;
+        wave[l].out[0] = present ? wave[src].in[0] : wave[l].in[0];
+      }
+      break;
+    case OP_BALLOT: {
+      uint64_t m = 0;
+      for (int l : who) m |= (uint64_t)(wave[l].in[0] != 0) << l;
+      for (int l : who) { wave[l].out[0] = (uint32_t)m; wave[l].out[1] = (uint32_t)(m >> 32); }
+      break;
+    }
+    case OP_RFL:
+      for (int l : who) wave[l].out[0] = wave[who[0]].in[0];
+      break;
+    case OP_MFMA16_F8: {
+      // A: lane l = row l % 16, K bytes 32 (l / 16) .. + 31; B likewise with its column; D[i][j]: lane j + 16 (i / 4),
+      // register i % 4
+      if (who.size() != 64) die("matrix instruction with %zu of 64 lanes", who.size());
+      float A[16][128], B[16][128];
+      for (int l = 0; l < 64; ++l) {
+        const uint8_t* a = reinterpret_cast<const uint8_t*>(wave[l].in);
+        const uint8_t* b = reinterpret_cast<const uint8_t*>(wave[l].in + 8);
+        for (int k = 0; k < 32; ++k) {
+          A[l & 15][32 * (l >> 4) + k] = e4m3_to_f32(a[k]);
+          B[l & 15][32 * (l >> 4) + k] = e4m3_to_f32(b[k]);
+        }
+      }
+      for (int l = 0; l < 64; ++l)
+        for (int r = 0; r < 4; ++r) {
+          const int i = 4 * (l >> 4) + r, j = l & 15;
+          float c;
+          memcpy(&c, &wave[l].in[16 + r], 4);
+          float s = 0.0f;
+          for (int k = 0; k < 128; ++k) s += A[i][k] * B[j][k];
+          const float d = c + s;
+          memcpy(&wave[l].out[r], &d, 4);
+        }
+      break;
+    }
+    case OP_MFMA32_F8: {
+      // A: lane l = row l % 32, K bytes 32 (l / 32) .. + 31; B likewise; D[i][j]: lane j + 32 ((i / 4) % 2),
+      // register 4 (i / 8) + i % 4
+      if (who.size() != 64) die("matrix instruction with %zu of 64 lanes", who.size());
+      static float A[32][64], B[32][64];
+      for (int l = 0; l < 64; ++l) {
+        const uint8_t* a = reinterpret_cast<const uint8_t*>(wave[l].in);
+        const uint8_t* b = reinterpret_cast<const uint8_t*>(wave[l].in + 8);
+        for (int k = 0; k < 32; ++k) {
+          A[l & 31][32 * (l >> 5) + k] = e4m3_to_f32(a[k]);
+          B[l & 31][32 * (l >> 5) + k] = e4m3_to_f32(b[k]);
+        }
+      }
+      for (int l = 0; l < 64; ++l)
+        for (int v = 0; v < 16; ++v) {
+          const int i = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3), j = l & 31;
+          float c;
+          memcpy(&c, &wave[l].in[16 + v], 4);
+          float s = 0.0f;
+          for (int k = 0; k < 64; ++k) s += A[i][k] * B[j][k];
+          const float d = c + s;
+          memcpy(&wave[l].out[v], &d, 4);
+        }
+      break;
+    }
+    case OP_MFMA16_BF16: {
+      // A: lane l = row l % 16, K elements 8 (l / 16) .. + 7; B likewise; D as the 16x16 form above
+      if (who.size() != 64) die("matrix instruction with %zu of 64 lanes", who.size());
+      float A[16][32], B[16][32];
+      for (int l = 0; l < 64; ++l) {
+        const uint16_t* a = reinterpret_cast<const uint16_t*>(wave[l].in);
+        const uint16_t* b = reinterpret_cast<const uint16_t*>(wave[l].in + 4);
+        for (int k = 0; k < 8; ++k) {
+          A[l & 15][8 * (l >> 4) + k] = bf16_to_f32(a[k]);
+          B[l & 15][8 * (l >> 4) + k] = bf16_to_f32(b[k]);
+        }
+      }
+      for (int l = 0; l < 64; ++l)
+        for (int r = 0; r < 4; ++r) {
+          const int i = 4 * (l >> 4) + r, j = l & 15;
+          float c;
+          memcpy(&c, &wave[l].in[8 + r], 4);
+          float s = 0.0f;
+          for (int k = 0; k < 32; ++k) s += A[i][k] * B[j][k];
+          const float d = c + s;
+          memcpy(&wave[l].out[r], &d, 4);
+        }
+      break;
+    }
+    default:
+      die("unknown rendezvous %d", (int)op);
+  }
+  for (int l : who) wave[l].op = OP_NONE;
+}
+
+// the lanes of `wave` (nl of them) that still run all wait at one wave-wide operation at one site: carry it out
+bool try_wave(Fiber* wave, int nl) {
+  const void* site = nullptr;
+  Op op = OP_NONE;
+  std::vector<int> who;
+  for (int l = 0; l < nl; ++l) {
+    if (wave[l].done) continue;
+    if (wave[l].op == OP_NONE || wave[l].op == OP_BARRIER) return false;
+    if (who.empty()) { site = wave[l].site; op = wave[l].op; }
+    else if (wave[l].site != site || wave[l].op != op) return false;
+    who.push_back(l);
+  }
+  if (who.empty()) return false;
+  perform(wave, who);
+  return true;
+}
+
+// rendezvous of the calling lane: deposit is done, wait until the operation has been carried out
+void rendezvous(Op op, const void* site) {
+  Fiber* f = g_cur;
+  f->op = op;
+  f->site = site;
+  if (op != OP_BARRIER) {
+    Fiber* wave = &g_fibers[f->lane.wave * 64];
+    const int nl = (int)std::min<size_t>(64, g_fibers.size() - f->lane.wave * 64);
+    if (try_wave(wave, nl)) return;          // this lane was the last to arrive: everybody may go on
+  }
+  while (f->op != OP_NONE) yield_to_scheduler();
+}
+
+void run_block(dim3 grid, dim3 block, dim3 bid) {
+  const int nt = (int)(block.x * block.y * block.z);
+  if (nt > kMaxThreads) die("block of %d threads", nt);
+  g_fibers.assign((size_t)nt, Fiber());
+  while ((int)g_stacks.size() < nt) {
+    void* p = mmap(nullptr, kStack, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0);
+    if (p == MAP_FAILED) die("no memory for a fiber stack");
+    mprotect(p, 4096, PROT_NONE);            // guard page under the stack
+    g_stacks.push_back(static_cast<uint8_t*>(p));
+  }
+  g_uniform.assign((size_t)((nt + 63) / 64) * kUniformSlots, UniformTag{0, nullptr, 0, false});
+  for (int t = 0; t < nt; ++t) {
+    Fiber& f = g_fibers[t];
+    f.lane.tid = dim3(t % block.x, (t / block.x) % block.y, t / (block.x * block.y));
+    f.lane.bid = bid;
+    f.lane.bdim = block;
+    f.lane.gdim = grid;
+    f.lane.lane = (unsigned)t & 63u;
+    f.lane.wave = (unsigned)t >> 6;
+    f.stack = g_stacks[t];
+    uint64_t* top = reinterpret_cast<uint64_t*>(f.stack + kStack);
+    *--top = 0;                               // keeps the entry frame aligned as after a call
+    *--top = reinterpret_cast<uint64_t>(&fiber_main);
+    for (int r = 0; r < 6; ++r) *--top = 0;
+    f.sp = top;
+  }
+  int running = nt;
+  while (running > 0) {
+    bool progressed = false;
+    for (int t = 0; t < nt; ++t) {
+      Fiber& f = g_fibers[t];
+      if (f.done || f.op != OP_NONE) continue;
+      g_cur = &f;
+      emu_switch(&g_sched_sp, f.sp);
+      g_cur = nullptr;
+      progressed = true;
+      if (f.done) --running;
+    }
+    if (running == 0) break;
+    if (progressed) {
+      bool any_runnable = false;
+      for (int t = 0; t < nt; ++t) any_runnable = any_runnable || (!g_fibers[t].done && g_fibers[t].op == OP_NONE);
+      if (any_runnable) continue;
+    }
+    // every running fiber waits.  Waves whose lanes all wait at one operation were served on arrival; what is left:
+    // the block barrier (everybody at it), lanes that ended since (a wave's remaining lanes now agree), divergence.
+    bool all_barrier = true;
+    for (int t = 0; t < nt; ++t) all_barrier = all_barrier && (g_fibers[t].done || g_fibers[t].op == OP_BARRIER);
+    if (all_barrier) {
+      ++g_stat_rendezvous;
+      for (int t = 0; t < nt; ++t) g_fibers[t].op = OP_NONE;
+      continue;
+    }
+    bool served = false;
+    for (int w = 0; w * 64 < nt && !served; ++w) served = try_wave(&g_fibers[w * 64], std::min(64, nt - w * 64));
+    if (served) continue;
+    // divergence: in some wave, serve the waiting group at the lowest code address
+    for (int w = 0; w * 64 < nt && !served; ++w) {
+      Fiber* wave = &g_fibers[w * 64];
+      const int nl = std::min(64, nt - w * 64);
+      const void* lowest = nullptr;
+      for (int l = 0; l < nl; ++l)
+        if (!wave[l].done && wave[l].op != OP_NONE && wave[l].op != OP_BARRIER && (lowest == nullptr || wave[l].site < lowest))
+          lowest = wave[l].site;
+      if (lowest == nullptr) continue;
+      std::vector<int> who;
+      for (int l = 0; l < nl; ++l)
+        if (!wave[l].done && wave[l].site == lowest && wave[l].op != OP_NONE && wave[l].op != OP_BARRIER) who.push_back(l);
+      perform(wave, who);
+      served = true;
+    }
+    if (!served) die("deadlock: every fiber of block %u waits and nothing can be served", bid.x);
+  }
+}
+
+uint8_t* lds_pointer(uint32_t lds32, unsigned bytes) {
+  // kernels hold LDS addresses as 32-bit values; every LDS object of this emulation (function-local statics of the
+  // kernels, g_dynamic_lds) lies in this shared object's data, whose upper address half g_dynamic_lds shares
+  const uintptr_t hi = reinterpret_cast<uintptr_t>(g_dynamic_lds) & ~uintptr_t(0xffffffffu);
+  uint8_t* p = reinterpret_cast<uint8_t*>(hi | lds32);
+  (void)bytes;
+  return p;
+}
+
+}  // namespace
+
+Lane& lane() { return g_cur->lane; }
+uint8_t* dynamic_lds() { return g_dynamic_lds; }
+
+void launch(dim3 grid, dim3 block, size_t dynamic_lds_bytes, const std::function<void()>& body) {
+  if (g_cur != nullptr) die("nested launch");
+  if (dynamic_lds_bytes > sizeof(g_dynamic_lds)) die("%zu bytes of dynamic LDS", dynamic_lds_bytes);
+  ++g_stat_launches;
+  g_body = &body;
+  for (unsigned z = 0; z < grid.z; ++z)
+    for (unsigned y = 0; y < grid.y; ++y)
+      for (unsigned x = 0; x < grid.x; ++x) {
+        ++g_stat_blocks;
+        run_block(grid, block, dim3(x, y, z));
+      }
+  g_body = nullptr;
+}
+
+void block_barrier() { rendezvous(OP_BARRIER, __builtin_return_address(0)); }
+__attribute__((noinline)) void wave_sync() { rendezvous(OP_SYNC, __builtin_return_address(0)); }
+__attribute__((noinline)) uint32_t shfl32(uint32_t v, int src) {
+  g_cur->in[0] = v;
+  g_cur->in[1] = (uint32_t)src;
+  rendezvous(OP_SHFL, __builtin_return_address(0));
+  return g_cur->out[0];
+}
+__attribute__((noinline)) uint32_t readlane32(uint32_t v, int l) {
+  g_cur->in[0] = v;
+  g_cur->in[1] = (uint32_t)l;
+  rendezvous(OP_RLANE, __builtin_return_address(0));
+  return g_cur->out[0];
+}
+__attribute__((noinline)) uint64_t ballot(bool pred) {
+  g_cur->in[0] = pred;
+  rendezvous(OP_BALLOT, __builtin_return_address(0));
+  return (uint64_t)g_cur->out[0] | ((uint64_t)g_cur->out[1] << 32);
+}
+__attribute__((noinline)) uint32_t readfirstlane32(uint32_t v) {
+  g_cur->in[0] = v;
+  rendezvous(OP_RFL, __builtin_return_address(0));
+  return g_cur->out[0];
+}
+__attribute__((noinline)) void mfma_16x16x128_f8(const int32_t* a8, const int32_t* b8, const float* c4, float* d4) {
+  memcpy(g_cur->in, a8, 32);
+  memcpy(g_cur->in + 8, b8, 32);
+  memcpy(g_cur->in + 16, c4, 16);
+  rendezvous(OP_MFMA16_F8, __builtin_return_address(0));
+  memcpy(d4, g_cur->out, 16);
+}
+__attribute__((noinline)) void mfma_32x32x64_f8(const int32_t* a8, const int32_t* b8, const float* c16, float* d16) {
+  memcpy(g_cur->in, a8, 32);
+  memcpy(g_cur->in + 8, b8, 32);
+  memcpy(g_cur->in + 16, c16, 64);
+  rendezvous(OP_MFMA32_F8, __builtin_return_address(0));
+  memcpy(d16, g_cur->out, 64);
+}
+__attribute__((noinline)) void mfma_16x16x32_bf16(const uint16_t* a8, const uint16_t* b8, const float* c4, float* d4) {
+  memcpy(g_cur->in, a8, 16);
+  memcpy(g_cur->in + 4, b8, 16);
+  memcpy(g_cur->in + 8, c4, 16);
+  rendezvous(OP_MFMA16_BF16, __builtin_return_address(0));
+  memcpy(d4, g_cur->out, 16);
+}
+
+void async_load(const void* base, uint32_t lane_off, uint32_t lds_base, unsigned bytes) {
+  Fiber* f = g_cur;
+  ++g_stat_async;
+  // base and LDS address are scalar operands of the instruction: every lane of the wave must pass the same
+  UniformTag& tag = g_uniform[(size_t)f->lane.wave * kUniformSlots + f->async_seq % kUniformSlots];
+  if (!tag.used || tag.seq != f->async_seq) tag = UniformTag{f->async_seq, base, lds_base, true};
+  else if (tag.base != base || tag.lds != lds_base)
+    die("asynchronous load %u of wave %u: lane %u passes another base or LDS address than an earlier lane", f->async_seq,
+        f->lane.wave, f->lane.lane);
+  ++f->async_seq;
+  const uint8_t* src = static_cast<const uint8_t*>(base) + lane_off;
+  uint8_t* dst = lds_pointer(lds_base, bytes) + (size_t)bytes * f->lane.lane;
+  if (g_lazy) f->pending.push_back(Pending{src, dst, bytes});
+  else memcpy(dst, src, bytes);
+}
+
+void wait_vm(int n) {
+  Fiber* f = g_cur;
+  if (!g_lazy) return;
+  const size_t keep = (size_t)(n < 0 ? 0 : n);
+  if (f->pending.size() <= keep) return;
+  const size_t land = f->pending.size() - keep;
+  for (size_t i = 0; i < land; ++i) memcpy(f->pending[i].dst, f->pending[i].src, f->pending[i].bytes);
+  f->pending.erase(f->pending.begin(), f->pending.begin() + (long)land);
+}
+
+float e4m3_to_f32(uint8_t b) {
+  const int s = b >> 7, e = (b >> 3) & 15, m = b & 7;
+  float v;
+  if (e == 15 && m == 7) v = NAN;
+  else if (e == 0) v = ldexpf((float)m, -9);
+  else v = ldexpf((float)(8 + m), e - 10);
+  return s ? -v : v;
+}
+
+// round to nearest even, saturating at +-448 (the library clamps before it converts), NaN -> 0x7f
+uint8_t f32_to_e4m3(float f) {
+  if (f != f) return 0x7f;
+  const uint8_t sign = signbit(f) ? 0x80 : 0;
+  float a = fabsf(f);
+  if (a >= 448.0f) return sign | 0x7e;
+  if (a < ldexpf(1.0f, -10)) return sign;                        // below half of the smallest denormal (2^-9)
+  int e;
+  (void)frexpf(a, &e);                                           // a = m 2^e, m in [0.5, 1)
+  int exp = e - 1;                                               // a = 1.xxx 2^exp
+  if (exp < -6) exp = -6;                                        // denormal range: fixed exponent
+  const float q = rintf(ldexpf(a, 3 - exp));                     // mantissa in units of 2^(exp-3), ties to even
+  int mant = (int)q, be = exp + 7;
+  if (exp == -6 && mant < 8) return sign | (uint8_t)mant;        // denormal (or zero)
+  if (mant == 16) { mant = 8; ++be; }
+  if (be > 15 || (be == 15 && mant - 8 > 6)) return sign | 0x7e;
+  return sign | (uint8_t)(be << 3) | (uint8_t)(mant - 8);
+}
+
+}  // namespace emu
+
+// ---- the pieces of the library's runtime that the staged kernel sources link against ---------------------------------
+static char g_error[512];
+void bgmoe_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+int bgmoe_check_launch(const char*) { return BGMOE_OK; }
+bool g_bgmoe_prof_on = false;
+void bgmoe_prof_mark(int, hipStream_t, bool) {}
+
+extern "C" {
+const char* bgmoe_last_error(void) { return g_error; }
+void emu_set_async_mode(int lazy) { emu::g_lazy = lazy != 0; }
+void emu_stats(uint64_t* out4) {
+  out4[0] = emu::g_stat_launches; out4[1] = emu::g_stat_blocks; out4[2] = emu::g_stat_rendezvous; out4[3] = emu::g_stat_async;
+}
+float emu_e4m3_to_f32(uint8_t b) { return emu::e4m3_to_f32(b); }
+uint8_t emu_f32_to_e4m3(float f) { return emu::f32_to_e4m3(f); }
+}

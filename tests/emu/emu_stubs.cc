@@ -1,0 +1,12 @@
+// TEST INFRASTRUCTURE: entry points of translation units that are not part of the emulation build, as far as the
+// staged sources refer to them.
+#include <hip/hip_runtime.h>
+
+#include "../../include/bgmoe.h"
+
+// the balanced (stream-K) form is not emulated: "does not apply", the caller launches the plain form
+int bgmoe_internal_fp8_streamk(const bgmoe_fp8_act*, const bgmoe_fp8_weight*, const bgmoe_fp8_weight*, const int32_t*,
+                               const int32_t*, int, int, int, uint16_t*, uint8_t*, float*, int64_t, int64_t, int, int64_t,
+                               void*, size_t, hipStream_t) {
+  return BGMOE_ERR_WORKSPACE;
+}
