@@ -20,6 +20,7 @@ def load():
             if fn is not None:
                 fn.restype, fn.argtypes = res, args
         h.emu_set_async_mode.argtypes = [C.c_int]
+        h.emu_set_schedule.argtypes = [C.c_int]
         h.emu_stats.argtypes = [C.c_void_p]
         h.emu_e4m3_to_f32.restype, h.emu_e4m3_to_f32.argtypes = C.c_float, [C.c_uint8]
         h.emu_f32_to_e4m3.restype, h.emu_f32_to_e4m3.argtypes = C.c_uint8, [C.c_float]

@@ -69,6 +69,7 @@ void* g_sched_sp = nullptr;
 const std::function<void()>* g_body = nullptr;
 alignas(256) uint8_t g_dynamic_lds[160 * 1024];
 bool g_lazy = false;
+int g_schedule = 0;
 uint64_t g_stat_launches = 0, g_stat_blocks = 0, g_stat_rendezvous = 0, g_stat_async = 0;
 struct UniformTag { uint32_t seq; const void* base; uint32_t lds; bool used; };
 std::vector<UniformTag> g_uniform;   // [wave][slot]: what the first lane of a wave passed for its seq-th async load
@@ -271,16 +272,27 @@ void run_block(dim3 grid, dim3 block, dim3 bid) {
     f.sp = top;
   }
   int running = nt;
+  const int nw = (nt + 63) / 64;
   while (running > 0) {
     bool progressed = false;
-    for (int t = 0; t < nt; ++t) {
-      Fiber& f = g_fibers[t];
-      if (f.done || f.op != OP_NONE) continue;
-      g_cur = &f;
-      emu_switch(&g_sched_sp, f.sp);
-      g_cur = nullptr;
-      progressed = true;
-      if (f.done) --running;
+    // schedule 0: every wave advances by one rendezvous per sweep (the waves stay close together); 1 / 2: the
+    // lowest / highest wave runs until it can go no further (a block barrier, its end) before the next one starts,
+    // the largest skew between waves that the kernel's barriers allow
+    for (int wi = 0; wi < nw; ++wi) {
+      const int w = g_schedule == 2 ? nw - 1 - wi : wi;
+      bool ran;
+      do {
+        ran = false;
+        for (int t = w * 64; t < std::min(nt, w * 64 + 64); ++t) {
+          Fiber& f = g_fibers[t];
+          if (f.done || f.op != OP_NONE) continue;
+          g_cur = &f;
+          emu_switch(&g_sched_sp, f.sp);
+          g_cur = nullptr;
+          ran = progressed = true;
+          if (f.done) --running;
+        }
+      } while (ran && g_schedule != 0);
     }
     if (running == 0) break;
     if (progressed) {
@@ -464,6 +476,7 @@ void bgmoe_prof_mark(int, hipStream_t, bool) {}
 extern "C" {
 const char* bgmoe_last_error(void) { return g_error; }
 void emu_set_async_mode(int lazy) { emu::g_lazy = lazy != 0; }
+void emu_set_schedule(int mode) { emu::g_schedule = mode; }
 void emu_stats(uint64_t* out4) {
   out4[0] = emu::g_stat_launches; out4[1] = emu::g_stat_blocks; out4[2] = emu::g_stat_rendezvous; out4[3] = emu::g_stat_async;
 }

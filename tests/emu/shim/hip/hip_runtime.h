@@ -55,7 +55,7 @@ struct Lane {
   unsigned lane, wave;
 };
 Lane& lane();                                   // the fiber that is running
-constexpr int kCus = 8;                         // the emulated device: 8 compute units (one per XCD)
+constexpr int kCus = 16;                        // the emulated device: 16 compute units (two per XCD)
 void launch(dim3 grid, dim3 block, size_t dynamic_lds, const std::function<void()>& body);
 uint8_t* dynamic_lds();
 void block_barrier();

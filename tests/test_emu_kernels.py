@@ -179,6 +179,7 @@ def tiled_only(h):
         ok(h, h.bgmoe_set_tiled_variant(0))
         ok(h, h.bgmoe_set_skinny_max_rows(256))
         h.emu_set_async_mode(0)
+        h.emu_set_schedule(0)
 
 
 K64_CASES = [  # counts, n, k
@@ -188,17 +189,24 @@ K64_CASES = [  # counts, n, k
 ]
 
 
-@pytest.mark.parametrize("mode", ["eager", "lazy"])
+# asynchronous loads land at once / as late as the waits allow; waves advance together / the first or the last wave
+# runs ahead as far as the barriers let it
+K64_MODES = [("eager", 0), ("lazy", 0), ("eager", 1), ("eager", 2), ("lazy", 2)]
+
+
+@pytest.mark.parametrize("mode,schedule", K64_MODES, ids=[f"{m}_sched{s}" for m, s in K64_MODES])
 @pytest.mark.parametrize("variant", [2, 1], ids=["plain_stores", "regrouped_stores"])
 @pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
 @pytest.mark.parametrize("counts,n,k", K64_CASES, ids=["k256", "k384", "k512"])
-def test_k64_tiled_kernel_on_the_emulator(h, tiled_only, counts, n, k, layout, variant, mode):
+def test_k64_tiled_kernel_on_the_emulator(h, tiled_only, counts, n, k, layout, variant, mode, schedule):
     """The K = 64 LDS-tiled kernel (no GPU has run it): plain GEMM and fused stage 1 against the oracle, with the
-    asynchronous loads landing at once (a slot refilled too early would corrupt a step still being read) and as late
-    as the kernel's wait counts allow (a wait that is too lenient would leave a step stale)."""
+    asynchronous loads landing at once (a slot refilled too early would corrupt a step still being read -- most
+    visibly when one wave runs ahead of the others) and as late as the kernel's wait counts allow (a wait that is
+    too lenient would leave a step stale)."""
     counts, cu, m, xq, xs, ws, live = _problem(10 + n + k, counts, n, k, nmat=2)
     ok(h, h.bgmoe_set_tiled_variant(variant))
     h.emu_set_async_mode(1 if mode == "lazy" else 0)
+    h.emu_set_schedule(schedule)
     before = emu.stats(h)
     wq = np.ascontiguousarray(ws[0][0])
     out = run_gemm(h, counts, cu, m, xq, xs, (_tile_major(h, wq) if layout else wq, ws[0][1]), n, k, layout)
@@ -209,3 +217,26 @@ def test_k64_tiled_kernel_on_the_emulator(h, tiled_only, counts, n, k, layout, v
     got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
     check_s1_against_oracle(xq, xs, ws[0], ws[1], counts, cu, live, got)
     assert emu.stats(h)["async_loads"] > before["async_loads"]
+
+
+@pytest.mark.parametrize("mode", ["eager", "lazy"])
+def test_k64_split_tail_on_the_emulator(h, tiled_only, mode):
+    """24 work items on the emulated device's 16 blocks (two per XCD): every XCD has three items, so its last round
+    holds one, which is split into two 128-token halves taken by its two blocks -- including a half whose rows all
+    lie past the group's end (the 300-row group's second tile has 44 rows) and a half that starts mid-group."""
+    import ctypes
+    from batchgen_amd.build import build_hostcheck
+    counts0 = (512, 300, 256, 700, 1000)
+    n, k = 256, 256
+    hc = ctypes.CDLL(build_hostcheck())
+    hc.hc_tiled_walk.restype = C.c_int
+    hc.hc_tiled_walk.argtypes = [C.POINTER(C.c_int32), C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint, C.POINTER(C.c_int), C.c_int]
+    out = (C.c_int * (6 * 128))()
+    nv = hc.hc_tiled_walk((C.c_int32 * 5)(*counts0), 5, 0, 2, 8, 16, out, 128)
+    visits = np.ctypeslib.as_array(out)[: 6 * nv].reshape(-1, 6)
+    assert (visits[:, 5] >= 0).sum() == 16, "the shape is meant to split one item per XCD"
+    counts, cu, m, xq, xs, ws, live = _problem(99, counts0, n, k, nmat=2)
+    ok(h, h.bgmoe_set_tiled_variant(1))
+    h.emu_set_async_mode(1 if mode == "lazy" else 0)
+    got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, 1)
+    check_s1_against_oracle(xq, xs, ws[0], ws[1], counts, cu, live, got)
