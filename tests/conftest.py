@@ -12,10 +12,19 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def emulating() -> bool:
+    """BGMOE_EMULATE=1 rehearses the GPU tests on the CPU emulator of tests/emu (no GPU visible, or not wanted): the
+    `dev` fixture is the CPU, the package's library handle is the emulation build, and the few torch.cuda calls
+    the tests and the host code make are stood in for.  A rehearsal of test and kernel logic, never a substitute
+    for the GPU run: speed, the hardware's rounding inside a matrix instruction and real memory ordering are not
+    what it shows."""
+    return os.environ.get("BGMOE_EMULATE", "0") == "1"
+
+
 def pytest_collection_modifyitems(config, items):
     """GPU tests are skipped (not failed) when no GPU is visible."""
     import torch
-    if torch.cuda.is_available():
+    if torch.cuda.is_available() or emulating():
         return
     skip = pytest.mark.skip(reason="no GPU visible")
     for item in items:
@@ -26,4 +35,12 @@ def pytest_collection_modifyitems(config, items):
 @pytest.fixture(scope="session")
 def dev():
     import torch
-    return torch.device("cuda:0")
+    return torch.device("cpu" if emulating() else "cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def _emulator_when_asked(request, monkeypatch):
+    if emulating() and "gpu" in request.keywords:
+        from tests import emu
+        emu.run_package_on_emulator(monkeypatch)
+    yield

@@ -43,3 +43,80 @@ def stats(h):
     out = (C.c_uint64 * 4)()
     h.emu_stats(out)
     return dict(zip(("launches", "blocks", "rendezvous", "async_loads"), [int(v) for v in out]))
+
+
+class _NoDeviceContext:
+    def __init__(self, *a, **k):
+        pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+class _NullStream:
+    cuda_stream = None
+
+    def __init__(self, *a, **k):
+        pass
+
+    def wait_event(self, ev):
+        pass
+
+    def wait_stream(self, st):
+        pass
+
+    def synchronize(self):
+        pass
+
+
+class _NullEvent:
+    def __init__(self, *a, **k):
+        pass
+
+    def record(self, stream=None):
+        pass
+
+    def synchronize(self):
+        pass
+
+    def wait(self, stream=None):
+        pass
+
+
+def run_package_on_emulator(monkeypatch):
+    """For a test: the package's host code (its ctypes layer classes) calls the emulation build instead of the GPU
+    library, with CPU tensors standing for device memory.  Patches, through pytest's monkeypatch, the library
+    handle, ``torch.cuda.current_stream`` / ``device`` / ``synchronize`` and the op wrappers' "is a CUDA tensor"
+    check; everything is undone when the test ends."""
+    import torch
+    from batchgen_amd import _lib
+    from batchgen_amd.kernels import _checks
+    h = load()
+    monkeypatch.setattr(_lib, "_lib", h)
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda *a, **k: _NullStream())
+    monkeypatch.setattr(torch.cuda, "device", _NoDeviceContext)
+    monkeypatch.setattr(torch.cuda, "synchronize", lambda *a, **k: None)
+    monkeypatch.setattr(torch.cuda, "Stream", _NullStream)
+    monkeypatch.setattr(torch.cuda, "Event", _NullEvent)
+    monkeypatch.setattr(torch.cuda, "stream", _NoDeviceContext)
+    # host code that asks a tensor whether it lives on the GPU (the emulated device memory is host memory)
+    monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
+
+    def tensor_only(t, name):
+        if not isinstance(t, torch.Tensor):
+            _checks.fail(f"{name} must be a tensor")
+    monkeypatch.setattr(_checks, "gpu", tensor_only)
+
+    from batchgen_amd.kernels import _workspace
+    pool = {}
+
+    def cpu_scratch(kind, device, need, floor=0):
+        buf = pool.get(kind)
+        if buf is None or buf.numel() < need:
+            buf = pool[kind] = torch.empty(max(int(need), int(floor)), dtype=torch.uint8)
+        return buf
+    monkeypatch.setattr(_workspace, "scratch", cpu_scratch)
+    return h

@@ -22,8 +22,17 @@ CLANG = "/opt/rocm/llvm/bin/clang++"
 
 # kernels that run under the emulator (their launch code and entry points included)
 SOURCES = ["gemm_fp8_skinny.hip", "gemm_fp8_tiled.hip", "gemm_fp8_tiled_k64.hip", "gemm_mxfp4_skinny.hip", "permute.hip",
-           "router_gemm.hip", "weight_repack.hip"]
+           "router_gemm.hip", "weight_repack.hip", "layer.hip", "act_quant.hip", "combine.hip", "router.hip",
+           "activation.hip", "norm_quant.hip", "gemm_fp8_dense.hip"]
 DYNAMIC_LDS = re.compile(r"extern\s+__shared__\s+(?:__align__\(\d+\)\s+)?(\w+)\s+(\w+)\[\];")
+# Lanes of a wave are not in lockstep under the emulator.  Where a kernel that a GPU has run passes data from lane to
+# lane through LDS with no rendezvous in between (on the GPU a wave's LDS accesses execute in order, and the source is
+# left as it is because an extra compiler barrier there changes the register allocation of a measured kernel), the
+# STAGED copy gets one: (file, text after which "emu::wave_sync();" is inserted).
+LOCKSTEP_POINTS = [
+    ("gemm_fp8_tiled.hip", "            *reinterpret_cast<uint2*>(patch + r16 * kEpiPitch + (16 * t + 4 * kq) * 2) = o;\n          }\n"),
+    ("gemm_fp8_tiled.hip", "              *reinterpret_cast<uint4*>(g.out + (row0 + tok0 + row) * g.n + col0 + (lane & 7) * 8) = v;\n          }\n"),
+]
 
 
 def _inputs():
@@ -53,6 +62,11 @@ def build(force: bool = False) -> str:
             continue
         text = open(os.path.join(CSRC, f)).read()
         text = DYNAMIC_LDS.sub(r"\1* const \2 = reinterpret_cast<\1*>(emu::dynamic_lds());", text)
+        for name, anchor in LOCKSTEP_POINTS:
+            if name == f:
+                if text.count(anchor) != 1:
+                    raise RuntimeError(f"{f}: the lockstep point {anchor!r} is not unique in the source any more")
+                text = text.replace(anchor, anchor + "          emu::wave_sync();\n")
         with open(os.path.join(stage, f.replace(".hip", ".cc")), "w") as out:
             out.write(text)
     shutil.copy(os.path.join(HERE, "bgmoe_async.h"), os.path.join(stage, "bgmoe_async.h"))

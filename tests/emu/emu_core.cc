@@ -42,7 +42,7 @@ emu_switch:
 namespace emu {
 namespace {
 
-enum Op { OP_NONE = 0, OP_SYNC, OP_SHFL, OP_BALLOT, OP_RFL, OP_RLANE, OP_MFMA16_F8, OP_MFMA32_F8, OP_MFMA16_BF16, OP_BARRIER };
+enum Op { OP_NONE = 0, OP_SYNC, OP_SHFL, OP_BALLOT, OP_RFL, OP_RLANE, OP_MFMA16_F8, OP_MFMA32_F8, OP_MFMA16_BF16, OP_DPP, OP_BARRIER };
 
 struct Pending { const uint8_t* src; uint8_t* dst; unsigned bytes; };
 
@@ -134,6 +134,26 @@ void perform(Fiber* wave, const std::vector<int>& who) {
     }
     case OP_RFL:
       for (int l : who) wave[l].out[0] = wave[who[0]].in[0];
+      break;
+    case OP_DPP:
+      // in: old, src, ctrl, row mask, bank mask, bound_ctrl.  A lane whose row (16 lanes) or bank (4 lanes) is masked
+      // out, or whose source lane does not exist or is not taking part, keeps `old` (0 with bound_ctrl).
+      for (int l : who) {
+        const int ctrl = (int)wave[l].in[2], rows = (int)wave[l].in[3], banks = (int)wave[l].in[4];
+        const int row = l >> 4, in_row = l & 15;
+        int src = -1;
+        if (ctrl < 0x100) src = (l & ~3) | ((ctrl >> (2 * (l & 3))) & 3);          // quad_perm
+        else if (ctrl == 0x140) src = (row << 4) | (15 - in_row);                    // row_mirror
+        else if (ctrl == 0x141) src = (row << 4) | (in_row & 8) | (7 - (in_row & 7));  // row_half_mirror
+        else if (ctrl == 0x142) src = row >= 1 ? ((row - 1) << 4) | 15 : -1;         // row_bcast15
+        else if (ctrl == 0x143) src = row >= 2 ? 31 : -1;                            // row_bcast31
+        else die("DPP control 0x%x is not emulated", ctrl);
+        bool present = false;
+        for (int m : who) present = present || m == src;
+        const bool enabled = ((rows >> row) & 1) && ((banks >> (in_row >> 2)) & 1);
+        if (enabled && present) wave[l].out[0] = wave[src].in[1];
+        else wave[l].out[0] = (enabled && wave[l].in[5]) ? 0u : wave[l].in[0];
+      }
       break;
     case OP_MFMA16_F8: {
       // A: lane l = row l % 16, K bytes 32 (l / 16) .. + 31; B likewise with its column; D[i][j]: lane j + 16 (i / 4),
@@ -371,6 +391,16 @@ __attribute__((noinline)) uint32_t readlane32(uint32_t v, int l) {
   g_cur->in[0] = v;
   g_cur->in[1] = (uint32_t)l;
   rendezvous(OP_RLANE, __builtin_return_address(0));
+  return g_cur->out[0];
+}
+__attribute__((noinline)) uint32_t update_dpp32(uint32_t old, uint32_t src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl) {
+  g_cur->in[0] = old;
+  g_cur->in[1] = src;
+  g_cur->in[2] = (uint32_t)ctrl;
+  g_cur->in[3] = (uint32_t)row_mask;
+  g_cur->in[4] = (uint32_t)bank_mask;
+  g_cur->in[5] = bound_ctrl;
+  rendezvous(OP_DPP, __builtin_return_address(0));
   return g_cur->out[0];
 }
 __attribute__((noinline)) uint64_t ballot(bool pred) {

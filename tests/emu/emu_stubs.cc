@@ -10,3 +10,17 @@ int bgmoe_internal_fp8_streamk(const bgmoe_fp8_act*, const bgmoe_fp8_weight*, co
                                void*, size_t, hipStream_t) {
   return BGMOE_ERR_WORKSPACE;
 }
+
+#include "bgmoe_common.h"
+
+int bgmoe_internal_init_fp8_streamk() { return BGMOE_OK; }
+
+extern "C" int bgmoe_version(void) { return 1; }
+extern "C" int bgmoe_init(void) {
+  int rc = bgmoe_internal_init_fp8_skinny();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_fp8_tiled();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_mxfp4();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_router_gemm();
+  if (rc == BGMOE_OK) rc = bgmoe_internal_init_permute();
+  return rc;
+}

@@ -64,6 +64,8 @@ uint32_t shfl32(uint32_t v, int src_lane);      // value of lane src_lane (mod 6
 uint64_t ballot(bool pred);
 uint32_t readfirstlane32(uint32_t v);
 uint32_t readlane32(uint32_t v, int lane);
+// v_mov_dpp: quad_perm (ctrl < 0x100), row_mirror 0x140, row_half_mirror 0x141, row_bcast15 0x142, row_bcast31 0x143
+uint32_t update_dpp32(uint32_t old, uint32_t src, int ctrl, int row_mask, int bank_mask, bool bound_ctrl);
 // matrix instructions: every lane passes its operand registers, gets its result registers
 void mfma_16x16x128_f8(const int32_t* a8, const int32_t* b8, const float* c4, float* d4);
 void mfma_32x32x64_f8(const int32_t* a8, const int32_t* b8, const float* c16, float* d16);
@@ -157,6 +159,8 @@ static inline T emu_from32(uint32_t u) { T t; static_assert(sizeof(T) == 4, "32-
 template <typename T>
 static inline uint32_t emu_to32(T t) { uint32_t u; static_assert(sizeof(T) == 4, "32-bit lane values only"); memcpy(&u, &t, 4); return u; }
 static inline unsigned long long __ballot(int pred) { return emu::ballot(pred != 0); }
+static inline int __any(int pred) { return emu::ballot(pred != 0) != 0; }
+static inline int __all(int pred) { return emu::ballot(pred == 0) == 0; }
 
 template <typename T>
 static inline T atomicAdd(T* p, T v) { const T old = *p; *p = old + v; return old; }
@@ -173,6 +177,8 @@ static inline T emu_readlane(T v, int l) { return emu_from32<T>(emu::readlane32(
 #define __builtin_amdgcn_readfirstlane(v) emu_readfirstlane(v)
 #define __builtin_amdgcn_readlane(v, l) emu_readlane((v), (l))
 #define __builtin_amdgcn_sched_barrier(x) ((void)0)
+#define __builtin_amdgcn_update_dpp(old, src, ctrl, rows, banks, bc) \
+  ((int)emu::update_dpp32((uint32_t)(old), (uint32_t)(src), (ctrl), (rows), (banks), (bc)))
 #define __builtin_amdgcn_fence(...) ((void)0)
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))

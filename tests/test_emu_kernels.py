@@ -240,3 +240,167 @@ def test_k64_split_tail_on_the_emulator(h, tiled_only, mode):
     h.emu_set_async_mode(1 if mode == "lazy" else 0)
     got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, 1)
     check_s1_against_oracle(xq, xs, ws[0], ws[1], counts, cu, live, got)
+
+
+# ---- MXFP4 (W4A16) kernels ------------------------------------------------------------------------------------------------
+def _mx_problem(seed, counts, n, k, align=16):
+    from oracle import mxfp4 as mx
+    counts, cu = _layout(counts, align)
+    m = max(int(cu[-1]), 1)
+    x = rand_bf16(torch.Generator().manual_seed(seed), m, k)
+    x16 = np.ascontiguousarray(x.view(torch.int16).numpy().view(np.uint16))
+    ws = []
+    for s in (seed + 1, seed + 2):
+        pk, sc = mx.quantize((0.02 * np.random.default_rng(s).standard_normal((len(counts), n, k))).astype(np.float32))
+        ws.append((np.ascontiguousarray(pk), np.ascontiguousarray(sc)))
+    live = np.zeros(m, dtype=bool)
+    for e, c in enumerate(counts):
+        live[cu[e]:cu[e] + c] = True
+    return counts, cu, m, x, x16, ws, live
+
+
+def _mx_weight(h, pk, sc, layout):
+    from batchgen_amd._lib import Mxfp4Weight
+    g, n, k2 = pk.shape
+    if layout == 1:
+        po, so = np.empty_like(pk), np.empty_like(sc)
+        ok(h, h.bgmoe_mxfp4_weight_repack(p(pk), p(sc), p(po), p(so), g, n, 2 * k2, None))
+        pk, sc = po, so
+    return (pk, sc), Mxfp4Weight(p(pk), n * k2, None, p(sc), n * sc.shape[2], None, layout, 0)
+
+
+def run_mx(h, counts, cu, m, x16, ws, n, k, layout, activation=0, row_pair=None, tokens=None, top_k=0):
+    keep, descs = [], []
+    for pk, sc in ws:
+        arrs, d = _mx_weight(h, pk, sc, layout)
+        keep.append(arrs)
+        descs.append(d)
+    out = np.full((m, n), 0x40E0, dtype=np.uint16)                        # bf16 7.0
+    ok(h, h.bgmoe_mxfp4_grouped_gemm(p(x16), C.byref(descs[0]), p(counts), p(cu), len(counts), m, n, k, p(out), None, 0, None))
+    hh = np.full((m, n), 0x40A0, dtype=np.uint16)                         # bf16 5.0
+    if row_pair is None:
+        ok(h, h.bgmoe_mxfp4_fused_s1(p(x16), C.byref(descs[0]), C.byref(descs[1]), p(counts), p(cu), len(counts), m, n, k,
+                                     p(hh), None, activation, 0, None))
+    else:
+        ok(h, h.bgmoe_mxfp4_fused_s1_gather(p(tokens), tokens.shape[0], p(row_pair), top_k, C.byref(descs[0]),
+                                            C.byref(descs[1]), p(counts), p(cu), len(counts), m, n, k, p(hh), None,
+                                            activation, 0, None))
+    return bf16_bits_to_f32(out), bf16_bits_to_f32(hh)
+
+
+MX_CASES = [((0, 1, 17, 33, 70), 256, 128), ((9, 40, 3), 128, 640), ((65, 2), 256, 896), ((20, 100), 384, 1664)]
+
+
+@pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
+@pytest.mark.parametrize("counts,n,k", MX_CASES, ids=[f"k{c[2]}" for c in MX_CASES])
+def test_mxfp4_kernel_and_its_second_shape_on_the_emulator(h, counts, n, k, layout):
+    """The proven shape (64-row items, three prefetch stages) against the oracle; then the second shape (32-row
+    items, six stages, a wait count that follows the depth; no GPU has run it): same bits, both activations --
+    1, 5, 7 and 13 K-blocks against the six stages."""
+    from oracle import situ as osi
+    counts, cu, m, x, x16, ws, live = _mx_problem(40 + n + k, counts, n, k)
+    want = run_mx(h, counts, cu, m, x16, ws, n, k, layout)
+    xf = oq.as_f32(x)
+    ref = og.grouped_gemm_mxfp4(xf, ws[0][0], ws[0][1], counts, cu, to_bf16=False)
+    np.testing.assert_allclose(want[0][live], ref[live], rtol=1e-2, atol=2e-3)
+    assert og.rel_frobenius(want[0][live], ref[live]) < 3e-3 and np.all(want[0][~live] == 7.0)
+    upv = og.grouped_gemm_mxfp4(xf, ws[1][0], ws[1][1], counts, cu, to_bf16=False)
+    assert og.rel_frobenius(want[1][live], (oq.silu_f32(ref) * upv)[live]) < 4e-3 and np.all(want[1][~live] == 5.0)
+    want_situ = run_mx(h, counts, cu, m, x16, ws, n, k, layout, activation=1)[1]
+    assert og.rel_frobenius(want_situ[live], osi.situ_fused(ref, upv)[live]) < 6e-3
+    try:
+        ok(h, h.bgmoe_set_mxfp4_variant(1))
+        got = run_mx(h, counts, cu, m, x16, ws, n, k, layout)
+        got_situ = run_mx(h, counts, cu, m, x16, ws, n, k, layout, activation=1)[1]
+    finally:
+        ok(h, h.bgmoe_set_mxfp4_variant(0))
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]) and np.array_equal(got_situ, want_situ)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("n_tok,top_k,e_total,start,el,mtp", [(96, 4, 24, 8, 6, 96), (200, 4, 8, 0, 6, 64), (1100, 8, 16, 4, 8, 700)])
+def test_index_only_dispatch_and_stage1_through_the_map_on_the_emulator(h, n_tok, top_k, e_total, start, el, mtp, variant):
+    """bgmoe_dispatch_index_3d against the oracle (counts, arrivals, positions, the inverse row -> pair map; the
+    third case takes the histogram / scan / rank launches), then the fused stage 1 reading its rows through the map
+    against the same kernel on the rows gathered by bgmoe_dispatch_scatter_3d: same bits.  No GPU has run either."""
+    from oracle import permute as op
+    rng = np.random.default_rng(n_tok)
+    ids = np.stack([rng.permutation(e_total)[:top_k] for _ in range(n_tok)]).astype(np.int32)
+    hdim, inter = 256, 128
+    nk = n_tok * top_k
+    ws_bytes = max(int(h.bgmoe_dispatch_workspace_bytes(nk, el)), 16)
+    wsp = np.zeros(ws_bytes, dtype=np.uint8)
+    counts = np.zeros(el, dtype=np.int32)
+    counters = np.zeros(el, dtype=np.int32)
+    pos = np.full(nk, -7, dtype=np.int32)
+    row_pair = np.full(el * mtp, 2 ** 30, dtype=np.int32)
+    ok(h, h.bgmoe_dispatch_index_3d(p(ids), n_tok, top_k, start, el, mtp, p(counts), p(counters), p(pos), p(row_pair), p(wsp),
+                                    ws_bytes, None))
+    want_counts, want_pos, arrivals = op.dispatch_masked_arrivals(ids, start, el, mtp)
+    want_pos = np.asarray(want_pos).reshape(-1)
+    assert np.array_equal(counts, want_counts) and np.array_equal(counters, arrivals) and np.array_equal(pos, want_pos)
+    want_rp = np.full(el * mtp, 2 ** 30, dtype=np.int32)
+    placed = np.nonzero(want_pos >= 0)[0]
+    want_rp[want_pos[placed]] = placed
+    assert np.array_equal(row_pair, want_rp)
+    if n_tok > 500:
+        return                                                  # the GEMM part at the two smaller sizes only
+    x = rand_bf16(torch.Generator().manual_seed(5), n_tok, hdim)
+    x16 = np.ascontiguousarray(x.view(torch.int16).numpy().view(np.uint16))
+    act = np.zeros((el * mtp, hdim), dtype=np.uint16)
+    counts2, counters2, pos2 = np.zeros_like(counts), np.zeros_like(counters), np.zeros_like(pos)
+    ok(h, h.bgmoe_dispatch_scatter_3d(p(x16), p(ids), n_tok, top_k, hdim, p(act), start, el, mtp, p(counts2), p(counters2),
+                                      p(pos2), p(wsp), ws_bytes, None))
+    assert np.array_equal(counts2, counts) and np.array_equal(pos2, pos)
+    from oracle import mxfp4 as mx
+    ws = []
+    for s in (1, 2):
+        pk, sc = mx.quantize((0.02 * np.random.default_rng(s).standard_normal((el, inter, hdim))).astype(np.float32))
+        ws.append((np.ascontiguousarray(pk), np.ascontiguousarray(sc)))
+    cu = (np.arange(el + 1) * mtp).astype(np.int32)
+    try:
+        ok(h, h.bgmoe_set_mxfp4_variant(variant))
+        want = run_mx(h, counts, cu, el * mtp, act, ws, inter, hdim, 1)[1]
+        got = run_mx(h, counts, cu, el * mtp, act, ws, inter, hdim, 1, row_pair=row_pair, tokens=x16, top_k=top_k)[1]
+    finally:
+        ok(h, h.bgmoe_set_mxfp4_variant(0))
+    assert np.array_equal(got, want)
+
+
+# ---- bf16 GEMM (router GEMM / linear layers) --------------------------------------------------------------------------------
+RG_PLANS = [(-1, -1), (-1, 0), (-1, 1), (-1, 2), (-1, 3), (-1, 4), (-1, 5)]      # chosen from the sizes; forced shapes; 5 = 128 x 64 tiles
+
+
+@pytest.mark.parametrize("mode", ["eager", "lazy"])
+@pytest.mark.parametrize("n,hd,e", [(129, 64, 64), (300, 1024, 100), (70, 512, 257), (256, 1536, 192)])
+def test_bf16_gemm_shapes_agree_bit_for_bit_on_the_emulator(h, n, hd, e, mode):
+    """Every launch shape of the bf16 GEMM computes the same chain per logit, so fp32 logits and bf16 outputs must be
+    the same bits whichever shape runs -- the proven ones among themselves (which is what says the emulator runs
+    this file correctly) and the 128-token x 64-output block tile that no GPU has run; and all of them the float64
+    product to 1e-5.  Shapes that a size does not admit fall back to the automatic choice inside the library."""
+    g = torch.Generator().manual_seed(n + hd + e)
+    x = rand_bf16(g, n, hd)
+    w = rand_bf16(g, e, hd, scale=0.05)
+    x16 = np.ascontiguousarray(x.view(torch.int16).numpy().view(np.uint16))
+    w16 = np.ascontiguousarray(w.view(torch.int16).numpy().view(np.uint16))
+    ws_bytes = max(int(h.bgmoe_router_gemm_workspace_bytes(n, hd, e)), 16)
+    ref = x.double().numpy() @ w.double().numpy().T
+    h.emu_set_async_mode(1 if mode == "lazy" else 0)
+    results = {}
+    try:
+        for plan in RG_PLANS:
+            ok(h, h.bgmoe_set_router_gemm_plan(*plan))
+            wsp = np.zeros(ws_bytes, dtype=np.uint8)
+            logits = np.full((n, e), 9.0, dtype=np.float32)
+            ok(h, h.bgmoe_router_gemm(p(x16), p(w16), n, hd, e, None, 0, 0, p(logits), p(wsp), ws_bytes, None))
+            out16 = np.zeros((n, e), dtype=np.uint16)
+            ok(h, h.bgmoe_bf16_linear(p(x16), p(w16), n, hd, e, p(out16), p(wsp), ws_bytes, None))
+            results[plan] = (logits, out16)
+    finally:
+        ok(h, h.bgmoe_set_router_gemm_plan(-1, -1))
+        h.emu_set_async_mode(0)
+    base = results[(-1, -1)]
+    assert np.linalg.norm(base[0] - ref) / np.linalg.norm(ref) < 1e-5
+    for plan, (lg, o16) in results.items():
+        assert np.array_equal(lg, base[0]), f"fp32 logits of plan {plan} differ"
+        assert np.array_equal(o16, base[1]), f"bf16 outputs of plan {plan} differ"

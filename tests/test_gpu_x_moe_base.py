@@ -9,6 +9,7 @@ import torch
 
 from oracle import gemm as og
 from oracle import layer as ol
+from oracle import quant as oq
 from tests.util import say
 
 pytestmark = pytest.mark.gpu
@@ -52,10 +53,20 @@ def test_template_layer_against_fused_layer_and_oracle(dev, n_group):
     fused = layer.forward_fused(xd).clone()
     assert torch.equal(layer._fused.topk_ids[:48], ids), "the fused call routes like gate()"
     a, b = out.float().cpu(), fused.float().cpu()
-    assert float((a - b).norm() / b.norm()) < 8e-3        # the shared expert's sums take another K order
-    ref = ol.moe_layer_fp8(x, None, None, None, wl.weights_to_numpy(w), 0, 16, layout="masked", max_tokens=64,
-                           shared=wl.weights_to_numpy(sh), routes=(ids.cpu().numpy(), wts.cpu().numpy()))
-    assert og.rel_frobenius(a.numpy(), ref["out"]) < 1e-2
+    # The template's shared expert is the reference's dense per-projection chain: gate and up leave their GEMM as
+    # bf16, SiLU and product are bf16 operations (the oracle's variant "iii"), and its sum with the routed part is
+    # rounded to bf16 twice.  The fused layer computes SwiGLU on the fp32 sums (variant "i") and adds everything in
+    # fp32.  A few percent of the intermediate's e4m3 bytes land on the neighbouring value between the two, so the
+    # two outputs differ by about one percent; each is held to the oracle of its own rounding.
+    assert float((a - b).norm() / b.norm()) < 3e-2
+    routes = (ids.cpu().numpy(), wts.cpu().numpy())
+    wn, sn = wl.weights_to_numpy(w), wl.weights_to_numpy(sh)
+    ref = ol.moe_layer_fp8(x, None, None, None, wn, 0, 16, layout="masked", max_tokens=64, shared=sn, routes=routes)
+    routed = ol.moe_layer_fp8(x, None, None, None, wn, 0, 16, layout="masked", max_tokens=64, shared=None, routes=routes)
+    dense = ol.moe_layer_fp8(x, None, None, None, wn, 0, 16, layout="masked", max_tokens=64, shared=sn, routes=routes,
+                             variant="iii")["y_shared"]
+    want_template = oq.bf16_round(oq.bf16_round(routed["out"]) + np.asarray(dense, dtype=np.float32)[:48])
+    assert og.rel_frobenius(a.numpy(), want_template) < 1e-2
     assert og.rel_frobenius(b.numpy(), ref["out"]) < 1e-2
     # the shared buffer manager changes nothing; 3-D input keeps its shape; too many tokens raise
     type(layer).init_buffer_manager(64, 1, 512, torch.device(dev))
