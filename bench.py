@@ -36,6 +36,7 @@ METRIC = "MoE layer TFLOP/s (FP8 prefill) & HBM GB/s (decode), % roofline, 1xMI3
 
 MIB = 1024 * 1024
 FLUSH_BYTES = 512 * MIB         # read between flushed replays: twice the 256 MiB last-level (Infinity) cache
+DEVICE = "cuda:0"               # the one GPU this benchmark runs on
 
 
 def traffic_record(key):
@@ -193,7 +194,7 @@ def bench_producer(a):
     import numpy as np
     import torch
     from batchgen_amd import _lib, workloads as wl
-    dev = torch.device("cuda:0")
+    dev = torch.device(DEVICE)
     torch.cuda.set_device(dev)
     if a.config is None:
         a.config = 1
@@ -415,7 +416,7 @@ def measure_layer(a, config, with_cpu):
     from batchgen_amd import _lib, workloads as wl
     from batchgen_amd.moe.fp8_layer import Fp8MoELayer
 
-    dev = torch.device("cuda:0")
+    dev = torch.device(DEVICE)
     torch.cuda.set_device(dev)
     cfg = wl.K3_LATENT if config == 5 else wl.CONFIGS[config]
     inp = wl.make_inputs(cfg, dev)

@@ -73,11 +73,17 @@ class _NullStream:
 
 
 class _NullEvent:
+    """torch.cuda.Event stand-in: the host's clock (the time the emulation took, of no meaning for the GPU)."""
+
     def __init__(self, *a, **k):
-        pass
+        self.t = 0.0
 
     def record(self, stream=None):
-        pass
+        import time
+        self.t = time.perf_counter()
+
+    def elapsed_time(self, other):
+        return max((other.t - self.t) * 1e3, 1e-6)
 
     def synchronize(self):
         pass
@@ -102,6 +108,8 @@ def run_package_on_emulator(monkeypatch):
     monkeypatch.setattr(torch.cuda, "Stream", _NullStream)
     monkeypatch.setattr(torch.cuda, "Event", _NullEvent)
     monkeypatch.setattr(torch.cuda, "stream", _NoDeviceContext)
+    monkeypatch.setattr(torch.cuda, "set_device", lambda *a, **k: None)
+    monkeypatch.setattr(torch.cuda, "empty_cache", lambda *a, **k: None)
     # host code that asks a tensor whether it lives on the GPU (the emulated device memory is host memory)
     monkeypatch.setattr(torch.Tensor, "is_cuda", property(lambda self: True))
 

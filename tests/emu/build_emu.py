@@ -23,7 +23,7 @@ CLANG = "/opt/rocm/llvm/bin/clang++"
 # kernels that run under the emulator (their launch code and entry points included)
 SOURCES = ["gemm_fp8_skinny.hip", "gemm_fp8_tiled.hip", "gemm_fp8_tiled_k64.hip", "gemm_mxfp4_skinny.hip", "permute.hip",
            "router_gemm.hip", "weight_repack.hip", "layer.hip", "act_quant.hip", "combine.hip", "router.hip",
-           "activation.hip", "norm_quant.hip", "gemm_fp8_dense.hip"]
+           "activation.hip", "norm_quant.hip", "gemm_fp8_dense.hip", "runtime.hip"]
 DYNAMIC_LDS = re.compile(r"extern\s+__shared__\s+(?:__align__\(\d+\)\s+)?(\w+)\s+(\w+)\[\];")
 # Lanes of a wave are not in lockstep under the emulator.  Where a kernel that a GPU has run passes data from lane to
 # lane through LDS with no rendezvous in between (on the GPU a wave's LDS accesses execute in order, and the source is

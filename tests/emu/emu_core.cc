@@ -491,20 +491,13 @@ uint8_t f32_to_e4m3(float f) {
 
 }  // namespace emu
 
-// ---- the pieces of the library's runtime that the staged kernel sources link against ---------------------------------
-static char g_error[512];
-void bgmoe_set_error(const char* fmt, ...) {
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(g_error, sizeof(g_error), fmt, ap);
-  va_end(ap);
+#include <chrono>
+double emu_now_ms() {
+  using clock = std::chrono::steady_clock;
+  return std::chrono::duration<double, std::milli>(clock::now().time_since_epoch()).count();
 }
-int bgmoe_check_launch(const char*) { return BGMOE_OK; }
-bool g_bgmoe_prof_on = false;
-void bgmoe_prof_mark(int, hipStream_t, bool) {}
 
 extern "C" {
-const char* bgmoe_last_error(void) { return g_error; }
 void emu_set_async_mode(int lazy) { emu::g_lazy = lazy != 0; }
 void emu_set_schedule(int mode) { emu::g_schedule = mode; }
 void emu_stats(uint64_t* out4) {

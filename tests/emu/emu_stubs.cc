@@ -1,5 +1,5 @@
-// TEST INFRASTRUCTURE: entry points of translation units that are not part of the emulation build, as far as the
-// staged sources refer to them.
+// TEST INFRASTRUCTURE: entry points of the one translation unit that is not part of the emulation build (the stream-K
+// form, whose prefetch ring is inline assembly), as far as the staged sources refer to them.
 #include <hip/hip_runtime.h>
 
 #include "../../include/bgmoe.h"
@@ -14,13 +14,3 @@ int bgmoe_internal_fp8_streamk(const bgmoe_fp8_act*, const bgmoe_fp8_weight*, co
 #include "bgmoe_common.h"
 
 int bgmoe_internal_init_fp8_streamk() { return BGMOE_OK; }
-
-extern "C" int bgmoe_version(void) { return 1; }
-extern "C" int bgmoe_init(void) {
-  int rc = bgmoe_internal_init_fp8_skinny();
-  if (rc == BGMOE_OK) rc = bgmoe_internal_init_fp8_tiled();
-  if (rc == BGMOE_OK) rc = bgmoe_internal_init_mxfp4();
-  if (rc == BGMOE_OK) rc = bgmoe_internal_init_router_gemm();
-  if (rc == BGMOE_OK) rc = bgmoe_internal_init_permute();
-  return rc;
-}

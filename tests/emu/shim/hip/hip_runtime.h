@@ -85,6 +85,15 @@ uint8_t f32_to_e4m3(float f);
 #define hipLaunchKernelGGL(kernel, grid, block, lds, stream, ...) \
   emu::launch((grid), (block), (size_t)(lds), [=]() { kernel(__VA_ARGS__); })
 
+// events carry the host's clock (what an emulated kernel takes on the CPU, of no meaning for the GPU)
+struct emu_event { double ms; };
+typedef emu_event* hipEvent_t;
+double emu_now_ms();
+static inline hipError_t hipEventCreate(hipEvent_t* e) { *e = new emu_event{0.0}; return hipSuccess; }
+static inline hipError_t hipEventRecord(hipEvent_t e, hipStream_t = nullptr) { e->ms = emu_now_ms(); return hipSuccess; }
+static inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
+static inline hipError_t hipEventElapsedTime(float* ms, hipEvent_t a, hipEvent_t b) { *ms = (float)(b->ms - a->ms); return hipSuccess; }
+static inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
 static inline hipError_t hipGetLastError() { return hipSuccess; }
 static inline const char* hipGetErrorString(hipError_t) { return "emulated"; }
 static inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }

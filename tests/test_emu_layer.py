@@ -61,3 +61,37 @@ def test_fp8_layer_on_the_emulator_matches_the_oracle(on_emulator, name):
     out = layer(inp["x"], inp["logits"]).clone()
     check_layer(layer, out, cfg, inp, w, sh)
     assert torch.equal(out, layer(inp["x"], inp["logits"]))            # reusable, deterministic
+
+
+def test_bench_measurement_code_on_the_emulator(on_emulator, monkeypatch):
+    """bench.py's measurement of both halves of the metric (timed passes, the cache-flushed decode passes, the
+    per-kernel timing pass, roofline and traffic objects, the JSON line) run through with configurations 1 and 2
+    scaled down and the emulator standing for the GPU: the times mean nothing, the code path and the accounting do."""
+    import json
+    from types import SimpleNamespace
+    import bench
+    small = {
+        1: wl.scaled(wl.CONFIGS[1], n_tokens=32, hidden=256, inter=128, shared_inter=128, max_tokens=32),
+        2: wl.scaled(wl.CONFIGS[2], n_tokens=300, hidden=256, inter=128, shared_inter=128),
+    }
+    monkeypatch.setattr(bench, "DEVICE", "cpu")
+    monkeypatch.setattr(bench, "FLUSH_BYTES", 1 << 20)
+    monkeypatch.setitem(wl.CONFIGS, 1, small[1])
+    monkeypatch.setitem(wl.CONFIGS, 2, small[2])
+    a = SimpleNamespace(steps=2, warmup=1, graph=False, copy_calibration=False, dense_backend=None, tiled_variant=0,
+                        tall_min_rows=0, mxfp4_variant=0, fold_gather=False, template=True, no_cpu_baseline=False)
+    for config in (1, 2):
+        out = bench.measure_layer(a, config, with_cpu=False)
+        line = json.loads(json.dumps(out))                       # everything in it serialises
+        decode = config == 1
+        assert line["unit"] == ("GB/s" if decode else "TFLOP/s") and line["value"] > 0 and line["ms_per_step"] > 0
+        assert line["config"]["workload"] == small[config].name and line["n_gpus"] == 1
+        roof = line["roofline"]
+        assert roof["bound"] == ("hbm" if decode else "mfma") and roof["achieved"] > 0 and 0 < roof["frac"]
+        assert ("cache_flushed" in line and "back_to_back" in line) == decode
+        if decode:
+            assert line["value"] == pytest.approx(line["cache_flushed"]["layer_hbm_GBps"])
+            assert line["timing"].startswith("median")
+        tl = line["template_layer"]                              # its own gate weights: other routes than the one-call layer's
+        assert tl["ms_per_step"] > 0 and 0 < tl["routed_rows"] <= small[config].n_tokens * small[config].top_k
+        assert sum(line["expert_counts"][:small[config].e_local]) == line["routed_rows"]
