@@ -3,6 +3,7 @@ package's ctypes signatures.  "Device memory" is host memory here: tests pass nu
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -22,6 +23,8 @@ def load():
         h.emu_set_async_mode.argtypes = [C.c_int]
         h.emu_set_schedule.argtypes = [C.c_int]
         h.emu_stats.argtypes = [C.c_void_p]
+        h.emu_guarded_alloc.restype, h.emu_guarded_alloc.argtypes = C.c_void_p, [C.c_size_t]
+        h.emu_guarded_free.argtypes = [C.c_void_p]
         h.emu_e4m3_to_f32.restype, h.emu_e4m3_to_f32.argtypes = C.c_float, [C.c_uint8]
         h.emu_f32_to_e4m3.restype, h.emu_f32_to_e4m3.argtypes = C.c_uint8, [C.c_float]
         _handle = h
@@ -128,3 +131,22 @@ def run_package_on_emulator(monkeypatch):
         return buf
     monkeypatch.setattr(_workspace, "scratch", cpu_scratch)
     return h
+
+
+def guarded(a: np.ndarray) -> np.ndarray:
+    """A copy of ``a`` in a buffer that ends at a page boundary with an inaccessible page behind it (and one in front):
+    a kernel that reads or writes past the end of the array faults at once, with a message that says by how much,
+    instead of quietly touching the neighbouring heap.  The size is rounded up to 16 bytes (slack at the front)."""
+    import weakref
+    h = load()
+    a = np.ascontiguousarray(a)
+    nbytes = max(a.nbytes, 16)
+    addr = h.emu_guarded_alloc(nbytes)
+    if not addr:
+        raise MemoryError("guarded allocation failed")
+    padded = (nbytes + 15) // 16 * 16
+    buf = (C.c_uint8 * a.nbytes).from_address(addr + padded - nbytes if a.nbytes else addr)
+    out = np.frombuffer(buf, dtype=a.dtype, count=a.size).reshape(a.shape)
+    out[...] = a
+    weakref.finalize(buf, h.emu_guarded_free, addr)
+    return out

@@ -497,7 +497,58 @@ double emu_now_ms() {
   return std::chrono::duration<double, std::milli>(clock::now().time_since_epoch()).count();
 }
 
+#include <signal.h>
+namespace {
+struct Guarded { uint8_t* base; size_t map_bytes; uint8_t* data; size_t bytes; };
+std::vector<Guarded> g_guarded;
+void on_segv(int, siginfo_t* info, void*) {
+  const uint8_t* a = static_cast<const uint8_t*>(info->si_addr);
+  for (const Guarded& g : g_guarded)
+    if (a >= g.base && a < g.base + g.map_bytes) {
+      fprintf(stderr, "emu: access %ld bytes %s a guarded buffer of %zu bytes\n",
+              a < g.data ? (long)(g.data - a) : (long)(a - (g.data + g.bytes)) + 1, a < g.data ? "in front of" : "past the end of",
+              g.bytes);
+      fflush(stderr);
+      abort();
+    }
+  fprintf(stderr, "emu: segmentation fault at %p (not next to a guarded buffer)\n", (const void*)a);
+  fflush(stderr);
+  abort();
+}
+}  // namespace
+
 extern "C" {
+// A buffer whose last byte is the last byte of a page, with an inaccessible page behind it and another in front of its
+// first page: an access past the end faults at once, and so does one more than a page's slack in front.  bytes is
+// rounded up to a multiple of 16 (the slack lies at the front).
+void* emu_guarded_alloc(size_t bytes) {
+  static bool handler = false;
+  if (!handler) {
+    struct sigaction sa;
+    memset(&sa, 0, sizeof(sa));
+    sa.sa_sigaction = on_segv;
+    sa.sa_flags = SA_SIGINFO;
+    sigaction(SIGSEGV, &sa, nullptr);
+    handler = true;
+  }
+  const size_t page = 4096, padded = (bytes + 15) & ~size_t(15);
+  const size_t body = (padded + page - 1) / page * page;
+  uint8_t* base = static_cast<uint8_t*>(mmap(nullptr, body + 2 * page, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0));
+  if (base == MAP_FAILED) return nullptr;
+  mprotect(base, page, PROT_NONE);
+  mprotect(base + page + body, page, PROT_NONE);
+  uint8_t* data = base + page + body - padded;
+  g_guarded.push_back(Guarded{base, body + 2 * page, data, padded});
+  return data;
+}
+void emu_guarded_free(void* data) {
+  for (size_t i = 0; i < g_guarded.size(); ++i)
+    if (g_guarded[i].data == data) {
+      munmap(g_guarded[i].base, g_guarded[i].map_bytes);
+      g_guarded.erase(g_guarded.begin() + (long)i);
+      return;
+    }
+}
 void emu_set_async_mode(int lazy) { emu::g_lazy = lazy != 0; }
 void emu_set_schedule(int mode) { emu::g_schedule = mode; }
 void emu_stats(uint64_t* out4) {

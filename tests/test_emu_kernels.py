@@ -2,7 +2,8 @@
 shuffles and barriers as rendezvous; asynchronous global -> LDS loads landing either at once or as late as the
 kernel's own waits allow).  Kernels a GPU has run are checked here against the oracle first -- that is what says the
 emulator executes this code correctly -- and the variants no GPU has run yet are then held to the same oracle and,
-where they promise it, to bit equality with the proven form."""
+where they promise it, to bit equality with the proven form.  Inputs and outputs live in guarded buffers (an
+inaccessible page right behind each array): a kernel that reads or writes past an array's end faults on the spot."""
 import ctypes as C
 
 import numpy as np
@@ -14,6 +15,7 @@ from oracle import fp8 as ofp8
 from oracle import gemm as og
 from oracle import quant as oq
 from tests import emu
+from tests.emu import guarded as G
 from tests.emu import ok, p
 from tests.util import rand_bf16
 
@@ -52,11 +54,12 @@ def _problem(seed, counts, n, k, nmat=1):
     live = np.zeros(m, dtype=bool)
     for e, c in enumerate(counts):
         live[cu[e]:cu[e] + c] = True
-    return counts, cu, m, np.ascontiguousarray(xq), np.ascontiguousarray(xs), ws, live
+    ws = [(G(wq), G(wsc.astype(np.float32))) for wq, wsc in ws]
+    return G(counts), G(cu), m, G(xq), G(xs), ws, live
 
 
 def _tile_major(h, wq):
-    out = np.empty_like(wq)
+    out = G(np.empty_like(wq))
     g, n, k = wq.shape
     ok(h, h.bgmoe_fp8_weight_repack(p(wq), p(out), g, n, k, None))
     return out
@@ -73,10 +76,10 @@ def _act(xq, xs):
 
 def run_gemm(h, counts, cu, m, xq, xs, w, n, k, layout=0, fill=7.0):
     wq, wsc = w
-    wq = np.ascontiguousarray(wq)
-    wsc = np.ascontiguousarray(wsc.astype(np.float32))
+    wq = G(wq)
+    wsc = G(wsc.astype(np.float32))
     out = np.full((m, n), np.float32(fill)).astype(np.float32)
-    out16 = (out.view(np.uint32) >> 16).astype(np.uint16)
+    out16 = G((out.view(np.uint32) >> 16).astype(np.uint16))
     a, b = _act(xq, xs), _weight(wq, wsc, layout)
     ok(h, h.bgmoe_fp8_grouped_gemm(C.byref(a), C.byref(b), p(counts), p(cu), len(counts), m, n, k, p(out16), None))
     return (out16.astype(np.uint32) << 16).view(np.float32)
@@ -102,18 +105,18 @@ def run_s1(h, counts, cu, m, xq, xs, wg, wu, n, k, layout=0):
     arrs = []
     descs = []
     for wq, wsc in (wg, wu):
-        wq = np.ascontiguousarray(wq)
+        wq = G(wq)
         if layout == 1:
             wq = _tile_major(h, wq)
-        wsc = np.ascontiguousarray(wsc.astype(np.float32))
+        wsc = G(wsc.astype(np.float32))
         arrs += [wq, wsc]
         descs.append(_weight(wq, wsc, layout))
     a = _act(xq, xs)
-    out16 = np.full((m, n), 0x40A0, dtype=np.uint16)                      # bf16 5.0
+    out16 = G(np.full((m, n), 0x40A0, dtype=np.uint16))                   # bf16 5.0
     ok(h, h.bgmoe_fp8_fused_s1(C.byref(a), C.byref(descs[0]), C.byref(descs[1]), p(counts), p(cu), len(counts), m, n, k,
                                p(out16), None, None, 0, 0, None))
-    hq = np.full((m, n), 0x55, dtype=np.uint8)
-    hs = np.full((n // 128, m), -3.0, dtype=np.float32)
+    hq = G(np.full((m, n), 0x55, dtype=np.uint8))
+    hs = G(np.full((n // 128, m), -3.0, dtype=np.float32))
     ok(h, h.bgmoe_fp8_fused_s1(C.byref(a), C.byref(descs[0]), C.byref(descs[1]), p(counts), p(cu), len(counts), m, n, k,
                                None, p(hq), p(hs), 1, m, None))
     return bf16_bits_to_f32(out16), hq, hs
@@ -248,22 +251,22 @@ def _mx_problem(seed, counts, n, k, align=16):
     counts, cu = _layout(counts, align)
     m = max(int(cu[-1]), 1)
     x = rand_bf16(torch.Generator().manual_seed(seed), m, k)
-    x16 = np.ascontiguousarray(x.view(torch.int16).numpy().view(np.uint16))
+    x16 = G(x.view(torch.int16).numpy().view(np.uint16))
     ws = []
     for s in (seed + 1, seed + 2):
         pk, sc = mx.quantize((0.02 * np.random.default_rng(s).standard_normal((len(counts), n, k))).astype(np.float32))
-        ws.append((np.ascontiguousarray(pk), np.ascontiguousarray(sc)))
+        ws.append((G(pk), G(sc)))
     live = np.zeros(m, dtype=bool)
     for e, c in enumerate(counts):
         live[cu[e]:cu[e] + c] = True
-    return counts, cu, m, x, x16, ws, live
+    return G(counts), G(cu), m, x, x16, ws, live
 
 
 def _mx_weight(h, pk, sc, layout):
     from batchgen_amd._lib import Mxfp4Weight
     g, n, k2 = pk.shape
     if layout == 1:
-        po, so = np.empty_like(pk), np.empty_like(sc)
+        po, so = G(np.empty_like(pk)), G(np.empty_like(sc))
         ok(h, h.bgmoe_mxfp4_weight_repack(p(pk), p(sc), p(po), p(so), g, n, 2 * k2, None))
         pk, sc = po, so
     return (pk, sc), Mxfp4Weight(p(pk), n * k2, None, p(sc), n * sc.shape[2], None, layout, 0)
@@ -275,9 +278,9 @@ def run_mx(h, counts, cu, m, x16, ws, n, k, layout, activation=0, row_pair=None,
         arrs, d = _mx_weight(h, pk, sc, layout)
         keep.append(arrs)
         descs.append(d)
-    out = np.full((m, n), 0x40E0, dtype=np.uint16)                        # bf16 7.0
+    out = G(np.full((m, n), 0x40E0, dtype=np.uint16))                     # bf16 7.0
     ok(h, h.bgmoe_mxfp4_grouped_gemm(p(x16), C.byref(descs[0]), p(counts), p(cu), len(counts), m, n, k, p(out), None, 0, None))
-    hh = np.full((m, n), 0x40A0, dtype=np.uint16)                         # bf16 5.0
+    hh = G(np.full((m, n), 0x40A0, dtype=np.uint16))                      # bf16 5.0
     if row_pair is None:
         ok(h, h.bgmoe_mxfp4_fused_s1(p(x16), C.byref(descs[0]), C.byref(descs[1]), p(counts), p(cu), len(counts), m, n, k,
                                      p(hh), None, activation, 0, None))
@@ -325,15 +328,15 @@ def test_index_only_dispatch_and_stage1_through_the_map_on_the_emulator(h, n_tok
     against the same kernel on the rows gathered by bgmoe_dispatch_scatter_3d: same bits.  No GPU has run either."""
     from oracle import permute as op
     rng = np.random.default_rng(n_tok)
-    ids = np.stack([rng.permutation(e_total)[:top_k] for _ in range(n_tok)]).astype(np.int32)
+    ids = G(np.stack([rng.permutation(e_total)[:top_k] for _ in range(n_tok)]).astype(np.int32))
     hdim, inter = 256, 128
     nk = n_tok * top_k
     ws_bytes = max(int(h.bgmoe_dispatch_workspace_bytes(nk, el)), 16)
-    wsp = np.zeros(ws_bytes, dtype=np.uint8)
-    counts = np.zeros(el, dtype=np.int32)
-    counters = np.zeros(el, dtype=np.int32)
-    pos = np.full(nk, -7, dtype=np.int32)
-    row_pair = np.full(el * mtp, 2 ** 30, dtype=np.int32)
+    wsp = G(np.zeros(ws_bytes, dtype=np.uint8))
+    counts = G(np.zeros(el, dtype=np.int32))
+    counters = G(np.zeros(el, dtype=np.int32))
+    pos = G(np.full(nk, -7, dtype=np.int32))
+    row_pair = G(np.full(el * mtp, 2 ** 30, dtype=np.int32))
     ok(h, h.bgmoe_dispatch_index_3d(p(ids), n_tok, top_k, start, el, mtp, p(counts), p(counters), p(pos), p(row_pair), p(wsp),
                                     ws_bytes, None))
     want_counts, want_pos, arrivals = op.dispatch_masked_arrivals(ids, start, el, mtp)
@@ -346,8 +349,8 @@ def test_index_only_dispatch_and_stage1_through_the_map_on_the_emulator(h, n_tok
     if n_tok > 500:
         return                                                  # the GEMM part at the two smaller sizes only
     x = rand_bf16(torch.Generator().manual_seed(5), n_tok, hdim)
-    x16 = np.ascontiguousarray(x.view(torch.int16).numpy().view(np.uint16))
-    act = np.zeros((el * mtp, hdim), dtype=np.uint16)
+    x16 = G(x.view(torch.int16).numpy().view(np.uint16))
+    act = G(np.zeros((el * mtp, hdim), dtype=np.uint16))
     counts2, counters2, pos2 = np.zeros_like(counts), np.zeros_like(counters), np.zeros_like(pos)
     ok(h, h.bgmoe_dispatch_scatter_3d(p(x16), p(ids), n_tok, top_k, hdim, p(act), start, el, mtp, p(counts2), p(counters2),
                                       p(pos2), p(wsp), ws_bytes, None))
@@ -356,8 +359,8 @@ def test_index_only_dispatch_and_stage1_through_the_map_on_the_emulator(h, n_tok
     ws = []
     for s in (1, 2):
         pk, sc = mx.quantize((0.02 * np.random.default_rng(s).standard_normal((el, inter, hdim))).astype(np.float32))
-        ws.append((np.ascontiguousarray(pk), np.ascontiguousarray(sc)))
-    cu = (np.arange(el + 1) * mtp).astype(np.int32)
+        ws.append((G(pk), G(sc)))
+    cu = G((np.arange(el + 1) * mtp).astype(np.int32))
     try:
         ok(h, h.bgmoe_set_mxfp4_variant(variant))
         want = run_mx(h, counts, cu, el * mtp, act, ws, inter, hdim, 1)[1]
@@ -381,8 +384,8 @@ def test_bf16_gemm_shapes_agree_bit_for_bit_on_the_emulator(h, n, hd, e, mode):
     g = torch.Generator().manual_seed(n + hd + e)
     x = rand_bf16(g, n, hd)
     w = rand_bf16(g, e, hd, scale=0.05)
-    x16 = np.ascontiguousarray(x.view(torch.int16).numpy().view(np.uint16))
-    w16 = np.ascontiguousarray(w.view(torch.int16).numpy().view(np.uint16))
+    x16 = G(x.view(torch.int16).numpy().view(np.uint16))
+    w16 = G(w.view(torch.int16).numpy().view(np.uint16))
     ws_bytes = max(int(h.bgmoe_router_gemm_workspace_bytes(n, hd, e)), 16)
     ref = x.double().numpy() @ w.double().numpy().T
     h.emu_set_async_mode(1 if mode == "lazy" else 0)
@@ -390,10 +393,10 @@ def test_bf16_gemm_shapes_agree_bit_for_bit_on_the_emulator(h, n, hd, e, mode):
     try:
         for plan in RG_PLANS:
             ok(h, h.bgmoe_set_router_gemm_plan(*plan))
-            wsp = np.zeros(ws_bytes, dtype=np.uint8)
-            logits = np.full((n, e), 9.0, dtype=np.float32)
+            wsp = G(np.zeros(ws_bytes, dtype=np.uint8))
+            logits = G(np.full((n, e), 9.0, dtype=np.float32))
             ok(h, h.bgmoe_router_gemm(p(x16), p(w16), n, hd, e, None, 0, 0, p(logits), p(wsp), ws_bytes, None))
-            out16 = np.zeros((n, e), dtype=np.uint16)
+            out16 = G(np.zeros((n, e), dtype=np.uint16))
             ok(h, h.bgmoe_bf16_linear(p(x16), p(w16), n, hd, e, p(out16), p(wsp), ws_bytes, None))
             results[plan] = (logits, out16)
     finally:
@@ -404,3 +407,22 @@ def test_bf16_gemm_shapes_agree_bit_for_bit_on_the_emulator(h, n, hd, e, mode):
     for plan, (lg, o16) in results.items():
         assert np.array_equal(lg, base[0]), f"fp32 logits of plan {plan} differ"
         assert np.array_equal(o16, base[1]), f"bf16 outputs of plan {plan} differ"
+
+
+def test_guarded_buffers_catch_an_overrun():
+    """The guard is real: a kernel given an output buffer one tile short dies on the spot with a message that names
+    the overrun (run in a child process: the emulator aborts)."""
+    import subprocess
+    import sys
+    code = (
+        "import numpy as np\n"
+        "from tests import emu\n"
+        "from tests.emu import guarded as G, p\n"
+        "h = emu.load()\n"
+        "src = G(np.zeros((1, 32, 128), dtype=np.uint8))\n"
+        "dst = G(np.zeros((1, 16, 128), dtype=np.uint8))\n"          # half of what the repack writes
+        "h.bgmoe_fp8_weight_repack(p(src), p(dst), 1, 32, 128, None)\n"
+        "print('not reached')\n")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=emu.os.path.dirname(emu.os.path.dirname(emu.os.path.dirname(emu.os.path.abspath(emu.__file__)))))
+    assert r.returncode != 0 and "not reached" not in r.stdout
+    assert "past the end of a guarded buffer" in r.stderr, r.stderr[-500:]
