@@ -1,0 +1,33 @@
+"""GPU test files that no GPU has executed yet, rehearsed on the CPU emulator (tests/emu) as part of the CPU suite:
+the same test functions, the package's own host code, CPU tensors standing for device memory (BGMOE_EMULATE=1, see
+tests/conftest.py).  What cannot be rehearsed is left out by name: tests of device-mismatch checks and of the compiled
+extension (they need real CUDA tensors), allocation counters of torch's CUDA allocator, graph capture, and the
+full-size shapes (too slow here).  A rehearsal shows that the test code and the kernels' logic hold together; the GPU
+run remains the parity test."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+REHEARSALS = [
+    ("tests/test_gpu_x_routes_and_argument_checks.py", "not reject_wrong_arguments"),
+    ("tests/test_gpu_x_moe_base.py", ""),
+    ("tests/test_gpu_x_dense_backend.py", "not full_size and not allocates_nothing and not 4096"),
+]
+
+
+@pytest.mark.parametrize("path,select", REHEARSALS, ids=[os.path.basename(p) for p, _ in REHEARSALS])
+def test_unrun_gpu_tests_pass_on_the_emulator(path, select):
+    from tests.emu.build_emu import build
+    build()                                                   # before the child, so that its time is the tests'
+    cmd = [sys.executable, "-m", "pytest", path, "-m", "gpu", "-q", "--tb=short", "-p", "no:cacheprovider"]
+    if select:
+        cmd += ["-k", select]
+    env = dict(os.environ, BGMOE_EMULATE="1")
+    r = subprocess.run(cmd, cwd=ROOT, env=env, capture_output=True, text=True, timeout=1500)
+    tail = (r.stdout + r.stderr)[-3000:]
+    assert r.returncode == 0, tail
+    assert " passed" in r.stdout and "failed" not in r.stdout.splitlines()[-1], tail
