@@ -435,13 +435,14 @@ __attribute__((noinline)) void mfma_16x16x32_bf16(const uint16_t* a8, const uint
   memcpy(d4, g_cur->out, 16);
 }
 
-void async_load(const void* base, uint32_t lane_off, uint32_t lds_base, unsigned bytes) {
+void async_load(const void* base, uint32_t lane_off, uint32_t lds_base, unsigned bytes, bool uniform_base) {
   Fiber* f = g_cur;
   ++g_stat_async;
   // base and LDS address are scalar operands of the instruction: every lane of the wave must pass the same
   UniformTag& tag = g_uniform[(size_t)f->lane.wave * kUniformSlots + f->async_seq % kUniformSlots];
-  if (!tag.used || tag.seq != f->async_seq) tag = UniformTag{f->async_seq, base, lds_base, true};
-  else if (tag.base != base || tag.lds != lds_base)
+  const void* tag_base = uniform_base ? base : nullptr;       // (a per-lane address form has no scalar base)
+  if (!tag.used || tag.seq != f->async_seq) tag = UniformTag{f->async_seq, tag_base, lds_base, true};
+  else if (tag.base != tag_base || tag.lds != lds_base)
     die("asynchronous load %u of wave %u: lane %u passes another base or LDS address than an earlier lane", f->async_seq,
         f->lane.wave, f->lane.lane);
   ++f->async_seq;

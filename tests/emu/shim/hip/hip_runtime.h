@@ -71,7 +71,7 @@ void mfma_16x16x128_f8(const int32_t* a8, const int32_t* b8, const float* c4, fl
 void mfma_32x32x64_f8(const int32_t* a8, const int32_t* b8, const float* c16, float* d16);
 void mfma_16x16x32_bf16(const uint16_t* a8, const uint16_t* b8, const float* c4, float* d4);
 // asynchronous global -> LDS loads (see bgmoe_async.h of this directory)
-void async_load(const void* base, uint32_t lane_off, uint32_t lds_base, unsigned bytes);
+void async_load(const void* base, uint32_t lane_off, uint32_t lds_base, unsigned bytes, bool uniform_base = true);
 void wait_vm(int n);
 float e4m3_to_f32(uint8_t b);
 uint8_t f32_to_e4m3(float f);
@@ -94,6 +94,8 @@ static inline hipError_t hipEventRecord(hipEvent_t e, hipStream_t = nullptr) { e
 static inline hipError_t hipEventSynchronize(hipEvent_t) { return hipSuccess; }
 static inline hipError_t hipEventElapsedTime(float* ms, hipEvent_t a, hipEvent_t b) { *ms = (float)(b->ms - a->ms); return hipSuccess; }
 static inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
+static inline hipError_t hipMemcpy(void* dst, const void* src, size_t n, int) { memcpy(dst, src, n); return hipSuccess; }
+static inline unsigned long long wall_clock64() { return (unsigned long long)(emu_now_ms() * 1e5); }
 static inline hipError_t hipGetLastError() { return hipSuccess; }
 static inline const char* hipGetErrorString(hipError_t) { return "emulated"; }
 static inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
@@ -173,6 +175,8 @@ static inline int __all(int pred) { return emu::ballot(pred == 0) == 0; }
 
 template <typename T>
 static inline T atomicAdd(T* p, T v) { const T old = *p; *p = old + v; return old; }
+template <typename T>
+static inline T atomicExch(T* p, T v) { const T old = *p; *p = v; return old; }
 template <typename T>
 static inline T atomicOr(T* p, T v) { const T old = *p; *p = old | v; return old; }
 template <typename T>
