@@ -138,5 +138,6 @@ def test_k64_variant_declines_short_k_and_bad_arguments(dev, k64):
     a = gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, cnt_d, cu_d, xs_t, ws_d, 16)
     assert lib().bgmoe_set_tiled_variant(0) == 0
     b = gm().fp8_blockwise_grouped_gemm(xq_d, wq_d, cnt_d, cu_d, xs_t, ws_d, 16)
-    assert torch.equal(a, b)
+    lv = torch.from_numpy(_live(counts, cu, m)).to(dev)          # (rows outside every group are never written)
+    assert torch.equal(a[lv], b[lv])
     assert lib().bgmoe_set_tiled_variant(3) != 0 and lib().bgmoe_set_tiled_variant(-1) != 0
