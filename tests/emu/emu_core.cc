@@ -39,6 +39,8 @@ emu_switch:
 .size emu_switch, .-emu_switch
 )");
 
+void emu_install_handlers();
+
 namespace emu {
 namespace {
 
@@ -366,6 +368,7 @@ Lane& lane() { return g_cur->lane; }
 uint8_t* dynamic_lds() { return g_dynamic_lds; }
 
 void launch(dim3 grid, dim3 block, size_t dynamic_lds_bytes, const std::function<void()>& body) {
+  emu_install_handlers();
   if (g_cur != nullptr) die("nested launch");
   if (dynamic_lds_bytes > sizeof(g_dynamic_lds)) die("%zu bytes of dynamic LDS", dynamic_lds_bytes);
   ++g_stat_launches;
@@ -498,8 +501,10 @@ double emu_now_ms() {
   return std::chrono::duration<double, std::milli>(clock::now().time_since_epoch()).count();
 }
 
+#include <execinfo.h>
 #include <signal.h>
 namespace {
+void install_segv_handler();
 struct Guarded { uint8_t* base; size_t map_bytes; uint8_t* data; size_t bytes; };
 std::vector<Guarded> g_guarded;
 void on_segv(int, siginfo_t* info, void*) {
@@ -512,26 +517,40 @@ void on_segv(int, siginfo_t* info, void*) {
       fflush(stderr);
       abort();
     }
-  fprintf(stderr, "emu: segmentation fault at %p (not next to a guarded buffer)\n", (const void*)a);
+  fprintf(stderr, "emu: segmentation fault at %p (not next to a guarded buffer%s)\n", (const void*)a,
+          a == nullptr ? "; address 0 is also what a 16-byte access to a pointer that is not 16-byte aligned reports on x86" : "");
+  if (emu::g_cur != nullptr)
+    fprintf(stderr, "emu: in launch %llu, block %u, thread %u\n", (unsigned long long)emu::g_stat_launches,
+            emu::g_cur->lane.bid.x, emu::g_cur->lane.tid.x);
+  void* frames[24];
+  const int n = backtrace(frames, 24);
+  backtrace_symbols_fd(frames, n, 2);
   fflush(stderr);
   abort();
 }
+void install_segv_handler() {
+  static bool handler = false;
+  if (handler) return;
+  static uint8_t alt[64 * 1024];
+  stack_t ss;
+  ss.ss_sp = alt; ss.ss_size = sizeof(alt); ss.ss_flags = 0;
+  sigaltstack(&ss, nullptr);                      // a fiber that overran its stack has none left for the handler
+  struct sigaction sa;
+  memset(&sa, 0, sizeof(sa));
+  sa.sa_sigaction = on_segv;
+  sa.sa_flags = SA_SIGINFO | SA_ONSTACK;
+  sigaction(SIGSEGV, &sa, nullptr);
+  handler = true;
+}
 }  // namespace
+void emu_install_handlers() { install_segv_handler(); }
 
 extern "C" {
 // A buffer whose last byte is the last byte of a page, with an inaccessible page behind it and another in front of its
 // first page: an access past the end faults at once, and so does one more than a page's slack in front.  bytes is
 // rounded up to a multiple of 16 (the slack lies at the front).
 void* emu_guarded_alloc(size_t bytes) {
-  static bool handler = false;
-  if (!handler) {
-    struct sigaction sa;
-    memset(&sa, 0, sizeof(sa));
-    sa.sa_sigaction = on_segv;
-    sa.sa_flags = SA_SIGINFO;
-    sigaction(SIGSEGV, &sa, nullptr);
-    handler = true;
-  }
+  install_segv_handler();
   const size_t page = 4096, padded = (bytes + 15) & ~size_t(15);
   const size_t body = (padded + page - 1) / page * page;
   uint8_t* base = static_cast<uint8_t*>(mmap(nullptr, body + 2 * page, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0));
