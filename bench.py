@@ -97,6 +97,9 @@ def parse():
     ap.add_argument("--mxfp4-variant", type=int, default=0, choices=[0, 1],
                     help="MXFP4 configurations: 0 = 64-row items with three prefetch stages (default), 1 = 32-row items "
                          "with six (bgmoe_set_mxfp4_variant)")
+    ap.add_argument("--bf16-gemm-plan", type=int, default=-1, choices=[-1, 0, 1, 2, 3, 4, 5],
+                    help="launch shape of the bf16 GEMM behind the router GEMM and the MXFP4 layers' linear layers "
+                         "(bgmoe_set_router_gemm_plan(-1, plan)): -1 = chosen from the sizes (default), 5 = 128 x 64 tiles")
     ap.add_argument("--fold-gather", action="store_true",
                     help="MXFP4 configurations: stage 1 reads its rows from the tokens through the dispatch's row -> pair "
                          "map instead of from a gathered copy (Mxfp4MoELayer(fold_gather=True))")
@@ -436,6 +439,7 @@ def measure_layer(a, config, with_cpu):
     _lib.check(_lib.lib().bgmoe_set_tiled_variant(int(getattr(a, "tiled_variant", 0))))
     _lib.check(_lib.lib().bgmoe_set_skinny_tall_min_rows(int(getattr(a, "tall_min_rows", 0))))
     _lib.check(_lib.lib().bgmoe_set_mxfp4_variant(int(getattr(a, "mxfp4_variant", 0))))
+    _lib.check(_lib.lib().bgmoe_set_router_gemm_plan(-1, int(getattr(a, "bf16_gemm_plan", -1))))
     x, logits = inp["x"], inp["logits"]
 
     for _ in range(a.warmup):
