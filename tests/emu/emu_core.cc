@@ -70,7 +70,10 @@ Fiber* g_cur = nullptr;
 void* g_sched_sp = nullptr;
 const std::function<void()>* g_body = nullptr;
 alignas(256) uint8_t g_dynamic_lds[160 * 1024];
+extern "C" uint8_t __start_emu_lds[], __stop_emu_lds[];     // the kernels' static __shared__ objects (linker symbols)
+__attribute__((section("emu_lds"), used)) uint8_t g_lds_section_anchor[16];   // the section exists whatever is staged
 bool g_lazy = false;
+size_t g_dynamic_bytes = 0;         // dynamic LDS the running launch asked for
 int g_schedule = 0;
 uint64_t g_stat_launches = 0, g_stat_blocks = 0, g_stat_rendezvous = 0, g_stat_async = 0;
 struct UniformTag { uint32_t seq; const void* base; uint32_t lds; bool used; };
@@ -358,7 +361,14 @@ uint8_t* lds_pointer(uint32_t lds32, unsigned bytes) {
   // kernels, g_dynamic_lds) lies in this shared object's data, whose upper address half g_dynamic_lds shares
   const uintptr_t hi = reinterpret_cast<uintptr_t>(g_dynamic_lds) & ~uintptr_t(0xffffffffu);
   uint8_t* p = reinterpret_cast<uint8_t*>(hi | lds32);
-  (void)bytes;
+  const bool in_static = p >= __start_emu_lds && p + 64u * bytes <= __stop_emu_lds;
+  const bool in_dynamic = p >= g_dynamic_lds && p < g_dynamic_lds + sizeof(g_dynamic_lds);
+  if (!in_static && !in_dynamic) die("asynchronous load to %p, which is no LDS address", (void*)p);
+  // a landing zone inside the dynamic LDS buffer must lie inside what the launch asked for
+  if (p >= g_dynamic_lds && p < g_dynamic_lds + sizeof(g_dynamic_lds) &&
+      (size_t)(p - g_dynamic_lds) + 64u * bytes > g_dynamic_bytes)
+    die("asynchronous load lands at dynamic LDS offset %zu + %u bytes, the launch asked for %zu bytes",
+        (size_t)(p - g_dynamic_lds), 64u * bytes, g_dynamic_bytes);
   return p;
 }
 
@@ -372,11 +382,16 @@ void launch(dim3 grid, dim3 block, size_t dynamic_lds_bytes, const std::function
   if (g_cur != nullptr) die("nested launch");
   if (dynamic_lds_bytes > sizeof(g_dynamic_lds)) die("%zu bytes of dynamic LDS", dynamic_lds_bytes);
   ++g_stat_launches;
+  g_dynamic_bytes = dynamic_lds_bytes;
   g_body = &body;
   for (unsigned z = 0; z < grid.z; ++z)
     for (unsigned y = 0; y < grid.y; ++y)
       for (unsigned x = 0; x < grid.x; ++x) {
         ++g_stat_blocks;
+        // a block finds no usable data in its LDS, dynamic or static: 0xFF bytes (NaN as e4m3, bf16 and fp32), so that a tile
+        // the block forgot to load cannot pass as the previous block's copy of it
+        memset(g_dynamic_lds, 0xFF, dynamic_lds_bytes);
+        memset(__start_emu_lds, 0xFF, (size_t)(__stop_emu_lds - __start_emu_lds));
         run_block(grid, block, dim3(x, y, z));
       }
   g_body = nullptr;

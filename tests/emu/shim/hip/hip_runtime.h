@@ -20,7 +20,9 @@
 #define __device__
 #define __host__
 #define __forceinline__ inline __attribute__((always_inline))
-#define __shared__ static
+// every __shared__ object lands in one ELF section, which the emulator poisons at the start of each block and uses
+// to tell LDS addresses from others
+#define __shared__ static __attribute__((section("emu_lds")))
 #define __launch_bounds__(...)
 #define __align__(n) __attribute__((aligned(n)))
 
