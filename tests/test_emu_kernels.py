@@ -426,3 +426,50 @@ def test_guarded_buffers_catch_an_overrun():
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, cwd=emu.os.path.dirname(emu.os.path.dirname(emu.os.path.dirname(emu.os.path.abspath(emu.__file__)))))
     assert r.returncode != 0 and "not reached" not in r.stdout
     assert "past the end of a guarded buffer" in r.stderr, r.stderr[-500:]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_through_the_new_variants(h, seed):
+    """Seeded random group sizes, widths, depths, layouts, load models and schedules through the three variants of the
+    FP8 / MXFP4 grouped kernels that no GPU has run (a longer private soak of the same generator found nothing)."""
+    rng = np.random.default_rng(4242 + seed)
+    kind = ("k64", "tall", "mx")[seed % 3]
+    try:
+        if kind == "k64":
+            counts = tuple(int(rng.choice([0, 1, 5, 127, 128, 129, 255, 256, 257, 300, 511, 513])) for _ in range(int(rng.integers(1, 5)))) + (3,)
+            n, k = int(rng.choice([128, 256, 384, 512])), int(rng.choice([256, 384, 512, 768]))
+            layout = int(rng.integers(0, 2))
+            counts, cu, m, xq, xs, ws, live = _problem(seed, counts, n, k, nmat=2)
+            ok(h, h.bgmoe_set_skinny_max_rows(0))
+            ok(h, h.bgmoe_set_tiled_variant(int(rng.choice([1, 2]))))
+            h.emu_set_async_mode(int(rng.integers(0, 2)))
+            h.emu_set_schedule(int(rng.integers(0, 3)))
+            got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+            check_s1_against_oracle(xq, xs, ws[0], ws[1], counts, cu, live, got)
+        elif kind == "tall":
+            counts = tuple(int(rng.choice([0, 1, 16, 31, 32, 33, 47, 64, 65, 96, 100, 128, 130, 200])) for _ in range(int(rng.integers(1, 7)))) + (40,)
+            n, k = int(rng.choice([128, 256, 384])), int(rng.choice([128, 256, 384, 640]))
+            layout = int(rng.integers(0, 2))
+            counts, cu, m, xq, xs, ws, live = _problem(seed, counts, n, k, nmat=2)
+            h.emu_set_schedule(int(rng.integers(0, 3)))
+            want = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+            ok(h, h.bgmoe_set_skinny_tall_min_rows(int(rng.choice([32, 40, 64, 100]))))
+            got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+            for a, b in zip(want, got):
+                assert np.array_equal(a, b)
+        else:
+            counts = tuple(int(rng.choice([0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 130])) for _ in range(int(rng.integers(1, 6)))) + (9,)
+            n, k = int(rng.choice([128, 256, 384])), int(rng.choice([128, 256, 640, 768, 896, 1152]))
+            layout = int(rng.integers(0, 2))
+            counts, cu, m, x, x16, ws, live = _mx_problem(seed, counts, n, k)
+            want = run_mx(h, counts, cu, m, x16, ws, n, k, layout)
+            ok(h, h.bgmoe_set_mxfp4_variant(1))
+            got = run_mx(h, counts, cu, m, x16, ws, n, k, layout)
+            assert np.array_equal(got[0], want[0]) and np.array_equal(got[1][live], want[1][live])
+    finally:
+        ok(h, h.bgmoe_set_mxfp4_variant(0))
+        ok(h, h.bgmoe_set_skinny_tall_min_rows(0))
+        ok(h, h.bgmoe_set_tiled_variant(0))
+        ok(h, h.bgmoe_set_skinny_max_rows(256))
+        h.emu_set_async_mode(0)
+        h.emu_set_schedule(0)
