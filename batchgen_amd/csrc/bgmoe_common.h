@@ -157,6 +157,9 @@ __device__ __forceinline__ intx4 gload_x4_stream(const void* p) {
 __device__ __forceinline__ float gload_f32(const float* p) {
   return *reinterpret_cast<const BGMOE_GLOBAL float*>((uintptr_t)p);
 }
+__device__ __forceinline__ uint32_t gload_u32(const void* p) {
+  return *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)p);
+}
 
 // ---- wave helpers ---------------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (BGMOE_WAVE - 1); }

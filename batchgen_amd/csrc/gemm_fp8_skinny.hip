@@ -222,6 +222,14 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
   // issue order: once at most the 8 weight loads of the youngest stage are outstanding, this wave's
   // tokens and weights of the stage about to be computed have landed; the barrier extends that to the
   // other waves' token loads and tells everybody that the slot refilled next is no longer being read.
+  // That count keeps at most two stages of weights in flight whatever NSTAGE is (one at the wait, the next
+  // issued behind it).  With more than three stages the wait is for the TOKENS of the stage about to be
+  // computed only: behind them in the queue are at least that stage's own 2*NT weight loads and those of
+  // the NSTAGE-2 younger stages (scale loads and the younger stages' token loads come on top, token loads
+  // of dead tiles are skipped: only weight loads are counted); the compiler's own counts hold the weights
+  // back until a stage's registers are read.
+  constexpr int kWaitLoads = NSTAGE <= 3 ? 2 * NT : 2 * NT * (NSTAGE - 1);
+  static_assert(kWaitLoads < 64, "the vector-memory counter has six bits");
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s) {
     issue_tokens(min(s, KB - 1), s);
@@ -231,7 +239,7 @@ __device__ __forceinline__ void fp8_skinny_item(const SkinnyArgs& g, const Bgmoe
   for (int kb0 = 0; kb0 < kb_main; kb0 += NSTAGE) {
 #pragma unroll
     for (int s = 0; s < NSTAGE; ++s) {
-      wait_vm<2 * NT>();
+      wait_vm<kWaitLoads>();
       block_barrier();
       issue_tokens(min(kb0 + s + NSTAGE - 1, KB - 1), (s + NSTAGE - 1) % NSTAGE);
       load_stage(st[(s + NSTAGE - 1) % NSTAGE], min(kb0 + s + NSTAGE - 1, KB - 1));
@@ -459,6 +467,17 @@ static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
   hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW, TALL>), grid, block, 0, st, g, vblocks);
 }
 
+// Prefetch depth of the plain GEMM's items (opt-in): 2 = one K-block ahead, as measured; 3 or 4 = two or three ahead
+// (the kernel has the registers: 17 per stage next to 32 accumulators), with the wait count that a deeper pipeline
+// needs (fp8_skinny_item).  Same chain per output element, so the same bits.
+static int g_skinny_gemm_stages = 2;
+
+extern "C" int bgmoe_set_skinny_gemm_stages(int stages) {
+  BGMOE_REQUIRE(stages >= 2 && stages <= 4, "set_skinny_gemm_stages: stages must be 2, 3 or 4");
+  g_skinny_gemm_stages = stages;
+  return BGMOE_OK;
+}
+
 // Stage 1 works on 32-row items (its epilogue keeps 16*TT x 8 fp32 results per lane alive next to the
 // prefetch stages); the plain GEMM on 64-row items, which halves the passes over the weights of groups
 // with more than 32 rows.
@@ -476,7 +495,14 @@ static void launch_variant(bool fused, int layout, int n, int groups, int64_t bo
     // 128-column items (two weight tiles per wave): twice as many, half as long as 256-column ones, which evens
     // out the last round of the persistent grid (measured: -5% to -10% on the down projection)
     const unsigned vb = bgmoe_item_grid((n + 127) / 128, groups, bound, hi, 64);
-    if (layout == BGMOE_W_TILE_MAJOR) launch_one<4, 2, false, BGMOE_W_TILE_MAJOR, 2>(vb, g, st);
+    const bool tile = layout == BGMOE_W_TILE_MAJOR;
+    if (g_skinny_gemm_stages == 4) {
+      if (tile) launch_one<4, 4, false, BGMOE_W_TILE_MAJOR, 2>(vb, g, st);
+      else launch_one<4, 4, false, BGMOE_W_ROW_MAJOR, 2>(vb, g, st);
+    } else if (g_skinny_gemm_stages == 3) {
+      if (tile) launch_one<4, 3, false, BGMOE_W_TILE_MAJOR, 2>(vb, g, st);
+      else launch_one<4, 3, false, BGMOE_W_ROW_MAJOR, 2>(vb, g, st);
+    } else if (tile) launch_one<4, 2, false, BGMOE_W_TILE_MAJOR, 2>(vb, g, st);
     else launch_one<4, 2, false, BGMOE_W_ROW_MAJOR, 2>(vb, g, st);
   }
 }
@@ -489,6 +515,10 @@ int bgmoe_internal_init_fp8_skinny() {
   skinny_resident<4, 2, false, BGMOE_W_ROW_MAJOR, 2>();
   skinny_resident<2, 3, true, BGMOE_W_TILE_MAJOR, 4, 4>();
   skinny_resident<2, 3, true, BGMOE_W_ROW_MAJOR, 4, 4>();
+  skinny_resident<4, 3, false, BGMOE_W_TILE_MAJOR, 2>();
+  skinny_resident<4, 3, false, BGMOE_W_ROW_MAJOR, 2>();
+  skinny_resident<4, 4, false, BGMOE_W_TILE_MAJOR, 2>();
+  skinny_resident<4, 4, false, BGMOE_W_ROW_MAJOR, 2>();
   return BGMOE_OK;
 }
 

@@ -148,10 +148,10 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
     for (int t = 0; t < NT; ++t) {
       if constexpr (LAYOUT == BGMOE_W_ROW_MAJOR) {
         s.A[t] = KEEP ? gload_x4(wp[t] + (kb << 6)) : gload_x4_stream(wp[t] + (kb << 6));
-        s.S[t] = *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)(sp[t] + (kb << 2)));
+        s.S[t] = gload_u32(sp[t] + (kb << 2));
       } else {
         s.A[t] = KEEP ? gload_x4(wp[t] + ((int64_t)kb << 10)) : gload_x4_stream(wp[t] + ((int64_t)kb << 10));
-        s.S[t] = *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)(sp[t] + (kb << 6)));
+        s.S[t] = gload_u32(sp[t] + (kb << 6));
       }
     }
   };

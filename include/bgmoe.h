@@ -517,6 +517,14 @@ int bgmoe_set_skinny_max_rows(int rows);
  * same bits.  Returns BGMOE_OK or BGMOE_ERR_ARG. */
 int bgmoe_set_skinny_tall_min_rows(int rows);
 
+/* Prefetch depth of the plain weight-streaming grouped GEMM, the down projection of a decode step (process-wide,
+ * opt-in; no counterpart in the reference).  stages = 2 (the default): an item loads one K-block ahead of the one it
+ * computes; 3 or 4: two or three ahead, i.e. two or three times the weight bytes in flight per block (the kernel keeps
+ * three blocks per CU with 3 stages, two with 4).  Every output element is computed by the same chain of operations
+ * whatever the depth: the results are the same bits.  Fused stage 1 is not affected (its three stages fill the
+ * register file).  Returns BGMOE_OK or BGMOE_ERR_ARG. */
+int bgmoe_set_skinny_gemm_stages(int stages);
+
 /* Fused stage 1: out = bf16( silu(X*Wg^T) * (X*Wu^T) ), fp32 gate and up.
  * Replaces `fp8_blockwise_fused_s1` / `_ptrs`
  * (grouped_fp8_blockwise_moe.py:423-560, fp8_blockwise_s1_kernel.cuh:425-607).

@@ -22,6 +22,7 @@ def load():
                 fn.restype, fn.argtypes = res, args
         h.emu_set_async_mode.argtypes = [C.c_int]
         h.emu_set_schedule.argtypes = [C.c_int]
+        h.emu_set_wait_slack.argtypes = [C.c_int]
         h.emu_stats.argtypes = [C.c_void_p]
         h.emu_guarded_alloc.restype, h.emu_guarded_alloc.argtypes = C.c_void_p, [C.c_size_t]
         h.emu_guarded_free.argtypes = [C.c_void_p]

@@ -44,6 +44,9 @@ STREAMK_ASM = [
      "emu::async_load(lane_ptr, 0, lds_base, 4, false);"),
     (re.compile(r'asm volatile\(""\s*:\s*"\+v"[^;]*;'), "(void)0;"),
 ]
+# The kernels' explicit global loads (bgmoe_common.h) report themselves to the emulator, which under its counted lazy
+# model gives them a place in the lane's queue of outstanding vector-memory operations.
+COUNTED_LOADS = re.compile(r"(__device__ __forceinline__ (?:intx4|float|uint32_t) gload_(?:x4|x4_stream|f32|u32)\([^)]*\) \{\n)")
 LOCKSTEP_POINTS = [
     ("gemm_fp8_tiled.hip", "            *reinterpret_cast<uint2*>(patch + r16 * kEpiPitch + (16 * t + 4 * kq) * 2) = o;\n          }\n"),
     ("gemm_fp8_tiled.hip", "              *reinterpret_cast<uint4*>(g.out + (row0 + tok0 + row) * g.n + col0 + (lane & 7) * 8) = v;\n          }\n"),
@@ -77,6 +80,10 @@ def build(force: bool = False) -> str:
             continue
         text = open(os.path.join(CSRC, f)).read()
         text = DYNAMIC_LDS.sub(r"\1* const \2 = reinterpret_cast<\1*>(emu::dynamic_lds());", text)
+        if f == "bgmoe_common.h":
+            text, hits = COUNTED_LOADS.subn(r"\1  emu::count_vm_load();\n", text)
+            if hits != 4:
+                raise RuntimeError(f"{f}: expected the four gload_* helpers, found {hits}")
         if f == "gemm_fp8_streamk.hip":
             for rx, body in STREAMK_ASM:
                 text, hits = rx.subn(body, text)

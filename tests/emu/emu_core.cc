@@ -73,6 +73,8 @@ alignas(256) uint8_t g_dynamic_lds[160 * 1024];
 extern "C" uint8_t __start_emu_lds[], __stop_emu_lds[];     // the kernels' static __shared__ objects (linker symbols)
 __attribute__((section("emu_lds"), used)) uint8_t g_lds_section_anchor[16];   // the section exists whatever is staged
 bool g_lazy = false;
+int g_wait_slack = 0;          // tests of the model itself: every wait_vm<N>(), N > 0, lets this many more loads stay out
+bool g_count_plain = false;     // lazy model: ordinary global loads take a place in the queue too
 size_t g_dynamic_bytes = 0;         // dynamic LDS the running launch asked for
 int g_schedule = 0;
 uint64_t g_stat_launches = 0, g_stat_blocks = 0, g_stat_rendezvous = 0, g_stat_async = 0;
@@ -94,7 +96,8 @@ constexpr int kUniformSlots = 64;
 void fiber_main() {
   (*g_body)();
   Fiber* f = g_cur;
-  for (const Pending& p : f->pending) memcpy(p.dst, p.src, p.bytes);   // whatever was still in flight lands
+  for (const Pending& p : f->pending)
+    if (p.bytes) memcpy(p.dst, p.src, p.bytes);                          // whatever was still in flight lands
   f->pending.clear();
   f->done = true;
   emu_switch(&f->sp, g_sched_sp);
@@ -470,13 +473,21 @@ void async_load(const void* base, uint32_t lane_off, uint32_t lds_base, unsigned
   else memcpy(dst, src, bytes);
 }
 
+// An ordinary global load issued through the kernels' gload_* helpers: its value is delivered at once (the compiler
+// places the wait for a register result itself), but under the counted lazy model it takes its place in the lane's
+// queue of outstanding vector-memory operations, so that a wait_vm<N>() counts what the hardware counts.
+void count_vm_load() {
+  if (g_lazy && g_count_plain) g_cur->pending.push_back(Pending{nullptr, nullptr, 0});
+}
+
 void wait_vm(int n) {
   Fiber* f = g_cur;
   if (!g_lazy) return;
-  const size_t keep = (size_t)(n < 0 ? 0 : n);
+  const size_t keep = (size_t)(n <= 0 ? 0 : n + g_wait_slack);
   if (f->pending.size() <= keep) return;
   const size_t land = f->pending.size() - keep;
-  for (size_t i = 0; i < land; ++i) memcpy(f->pending[i].dst, f->pending[i].src, f->pending[i].bytes);
+  for (size_t i = 0; i < land; ++i)
+    if (f->pending[i].bytes) memcpy(f->pending[i].dst, f->pending[i].src, f->pending[i].bytes);
   f->pending.erase(f->pending.begin(), f->pending.begin() + (long)land);
 }
 
@@ -584,7 +595,11 @@ void emu_guarded_free(void* data) {
       return;
     }
 }
-void emu_set_async_mode(int lazy) { emu::g_lazy = lazy != 0; }
+void emu_set_wait_slack(int loads) { emu::g_wait_slack = loads < 0 ? 0 : loads; }
+void emu_set_async_mode(int lazy) {                  // 0 eager, 1 lazy, 2 lazy with ordinary loads counted
+  emu::g_lazy = lazy != 0;
+  emu::g_count_plain = lazy == 2;
+}
 void emu_set_schedule(int mode) { emu::g_schedule = mode; }
 void emu_stats(uint64_t* out4) {
   out4[0] = emu::g_stat_launches; out4[1] = emu::g_stat_blocks; out4[2] = emu::g_stat_rendezvous; out4[3] = emu::g_stat_async;

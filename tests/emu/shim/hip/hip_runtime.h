@@ -75,6 +75,7 @@ void mfma_16x16x32_bf16(const uint16_t* a8, const uint16_t* b8, const float* c4,
 // asynchronous global -> LDS loads (see bgmoe_async.h of this directory)
 void async_load(const void* base, uint32_t lane_off, uint32_t lds_base, unsigned bytes, bool uniform_base = true);
 void wait_vm(int n);
+void count_vm_load();                           // an ordinary global load, for the counted lazy model
 float e4m3_to_f32(uint8_t b);
 uint8_t f32_to_e4m3(float f);
 }  // namespace emu

@@ -473,3 +473,100 @@ def test_random_shapes_through_the_new_variants(h, seed):
         ok(h, h.bgmoe_set_skinny_max_rows(256))
         h.emu_set_async_mode(0)
         h.emu_set_schedule(0)
+
+
+def run_plain_gemm(h, counts, cu, m, xq, xs, w, n, k, layout):
+    wq, wsc = w
+    if layout == 1:
+        wq = _tile_major(h, wq)
+    out16 = G(np.full((m, n), 0x40E0, dtype=np.uint16))                   # bf16 7.0
+    a, b = _act(xq, xs), _weight(wq, wsc, layout)
+    ok(h, h.bgmoe_fp8_grouped_gemm(C.byref(a), C.byref(b), p(counts), p(cu), len(counts), m, n, k, p(out16), None))
+    return np.array(out16)
+
+
+@pytest.fixture
+def streaming_knobs(h):
+    yield
+    ok(h, h.bgmoe_set_skinny_gemm_stages(2))
+    ok(h, h.bgmoe_set_mxfp4_variant(0))
+    ok(h, h.bgmoe_set_skinny_tall_min_rows(0))
+    h.emu_set_async_mode(0)
+    h.emu_set_schedule(0)
+    h.emu_set_wait_slack(0)
+
+
+@pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
+@pytest.mark.parametrize("k", [128, 256, 384, 640, 1152])
+def test_plain_streaming_gemm_at_every_prefetch_depth(h, streaming_knobs, k, layout):
+    """The down projection's kernel with two (a GPU has run it), three and four prefetch stages; 1 to 9 K-blocks, so
+    shorter than, equal to and longer than every ring.  Loads land at once, or as late as the kernel's hand-placed
+    waits allow with every global load of the item counted the way the hardware counts them (the deeper rings wait
+    for a different count than the proven one); three wave schedules.  One set of bits throughout."""
+    n = 256
+    counts, cu, m, xq, xs, ws, live = _problem(40 + k, (0, 1, 17, 40, 64, 70, 130), n, k)
+    want = run_plain_gemm(h, counts, cu, m, xq, xs, ws[0], n, k, layout)
+    ref = og.grouped_gemm_fp8(xq, xs, ws[0][0], ws[0][1], counts, cu, to_bf16=False)
+    got = bf16_bits_to_f32(want)
+    assert og.rel_frobenius(got[live], ref[live]) < 3e-3 and np.all(got[~live] == 7.0)
+    for stages in (2, 3, 4):
+        ok(h, h.bgmoe_set_skinny_gemm_stages(stages))
+        for mode, schedule in ((0, 1), (2, 0), (2, 2)):
+            h.emu_set_async_mode(mode)
+            h.emu_set_schedule(schedule)
+            out = run_plain_gemm(h, counts, cu, m, xq, xs, ws[0], n, k, layout)
+            assert np.array_equal(out, want), f"{stages} stages, load model {mode}, schedule {schedule}"
+
+
+@pytest.mark.parametrize("stages,slack", [(2, 16), (3, 16), (4, 16)])
+def test_counted_load_model_catches_a_wait_that_is_too_lenient(h, streaming_knobs, stages, slack):
+    """The negative control of the test above: the same kernels with every hand-placed wait loosened by `slack`
+    loads (in the emulator, not in the source) compute on token bytes that have not landed, and the result shows it."""
+    n, k = 128, 1152
+    counts, cu, m, xq, xs, ws, live = _problem(77, (64, 33), n, k)
+    want = run_plain_gemm(h, counts, cu, m, xq, xs, ws[0], n, k, 1)
+    ok(h, h.bgmoe_set_skinny_gemm_stages(stages))
+    h.emu_set_async_mode(2)
+    out = run_plain_gemm(h, counts, cu, m, xq, xs, ws[0], n, k, 1)
+    assert np.array_equal(out, want)
+    h.emu_set_wait_slack(slack)
+    out = run_plain_gemm(h, counts, cu, m, xq, xs, ws[0], n, k, 1)
+    assert not np.array_equal(out, want)
+
+
+@pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
+def test_streaming_kernels_with_loads_as_late_as_their_waits_allow(h, streaming_knobs, layout):
+    """Stage 1 (32-row and tall items) and the MXFP4 kernel (both shapes), whose hand-placed waits count their
+    ordinary weight loads as well: every global load of an item takes its place in the lane's queue, a token load
+    lands only when a wait leaves it no other choice.  Same bits as with loads that land at once."""
+    n, k = 256, 1152
+    counts, cu, m, xq, xs, ws, live = _problem(91, (1, 31, 33, 64, 100), n, k, nmat=2)
+    want = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+    mxc, mxcu, mxm, x, x16, mws, mlive = _mx_problem(92, (17, 33, 70), n, 1664)
+    mwant = run_mx(h, mxc, mxcu, mxm, x16, mws, n, 1664, layout)
+    for schedule in (0, 2):
+        h.emu_set_async_mode(2)
+        h.emu_set_schedule(schedule)
+        for tall_min in (0, 32):
+            ok(h, h.bgmoe_set_skinny_tall_min_rows(tall_min))
+            got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+            for a, b in zip(want, got):
+                assert np.array_equal(a, b), f"stage 1, tall_min {tall_min}, schedule {schedule}"
+        for variant in (0, 1):
+            ok(h, h.bgmoe_set_mxfp4_variant(variant))
+            got = run_mx(h, mxc, mxcu, mxm, x16, mws, n, 1664, layout)
+            assert np.array_equal(got[0], mwant[0]) and np.array_equal(got[1], mwant[1]), f"MXFP4 shape {variant}"
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_counted_load_model_catches_a_lenient_wait_in_the_mxfp4_kernel(h, streaming_knobs, variant):
+    n, k = 128, 1664
+    counts, cu, m, x, x16, ws, live = _mx_problem(93, (64, 20), n, k)
+    want = run_mx(h, counts, cu, m, x16, ws, n, k, 1)
+    ok(h, h.bgmoe_set_mxfp4_variant(variant))
+    h.emu_set_async_mode(2)
+    got = run_mx(h, counts, cu, m, x16, ws, n, k, 1)
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1])
+    h.emu_set_wait_slack(24)
+    got = run_mx(h, counts, cu, m, x16, ws, n, k, 1)
+    assert not (np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]))
