@@ -8,8 +8,9 @@
 //  * lazy: the copy happens only when a wait_vm<N>() of the issuing lane leaves it no other choice (all but the N
 //    youngest loads of that lane complete, in issue order) or when the lane ends -- the latest a load can land under
 //    the kernel's own waits, IF the kernel's wait counts count nothing but these loads.  A wait that is too lenient
-//    shows up as stale data.  Kernels whose wait counts also rely on ordinary loads in between (the weight-streaming
-//    kernels) are run eagerly only.
+//    shows up as stale data.  Kernels whose wait counts also count ordinary loads in between (the weight-streaming
+//    kernels) need the counted form of this model: the staged gload_* helpers report every ordinary global load, which
+//    then takes a place in the lane's queue although its value arrives at once.
 #pragma once
 #include "bgmoe_common.h"
 #include "bgmoe_hostdev.h"

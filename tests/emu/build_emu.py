@@ -1,9 +1,11 @@
 """TEST INFRASTRUCTURE: builds ``tests/emu/_build/libbgmoe_emu.so``, the library's kernel sources compiled as plain
 C++ for the host against the CPU emulator of this directory (``shim/hip/hip_runtime.h``, ``emu_core.cc``).
 
-The sources are staged unchanged except for two things the host compiler cannot take: ``bgmoe_async.h`` (gfx950
-inline assembly) is replaced by this directory's version with the same names, and a dynamic-LDS declaration
-(``extern __shared__ T name[];``) becomes a pointer to the emulator's LDS buffer.  Only tests load the result.
+The sources are staged unchanged except for what the host compiler cannot take -- ``bgmoe_async.h`` (gfx950 inline
+assembly) is replaced by this directory's version with the same names, a dynamic-LDS declaration
+(``extern __shared__ T name[];``) becomes a pointer to the emulator's LDS buffer, the stream-K form's assembly helpers
+get plain C++ bodies -- and for what the emulator has to be told: the explicit global loads of ``bgmoe_common.h``
+report themselves, and two lane-to-lane exchanges of a measured kernel get a rendezvous.  Only tests load the result.
 """
 from __future__ import annotations
 
