@@ -372,9 +372,8 @@ __global__ __launch_bounds__(256) void fp8_skinny_kernel(SkinnyArgs g, unsigned 
 // One weight matrix against m rows (host-known), K split over `ksplit` blocks per (n-tile, 64-row chunk): the
 // item function above on K-blocks [slice * per, ...), fp32 partial sums to g.part; splitk_reduce_kernel adds the
 // slices in ascending order.
-template <int LAYOUT, int TT>
+template <int LAYOUT, int TT, int NSTAGE = 2>
 __global__ __launch_bounds__(256) void fp8_dense_splitk_kernel(SkinnyArgs g, int m, int ksplit, int per) {
-  constexpr int NSTAGE = 2;
   __shared__ float s_amax[4][TT][16];
   __shared__ __align__(16) uint8_t s_ring[NSTAGE * TokSlot<TT>::kBytes];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
@@ -691,13 +690,24 @@ int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weig
   const int chunk_rows = m > 256 || (m > 128 && k >= 4096) ? 128 : 64;
   const unsigned blocks = (unsigned)(((n + 127) / 128) * ((m + chunk_rows - 1) / chunk_rows) * ksplit);
   const bool tile = w->layout == BGMOE_W_TILE_MAJOR;
+  // the prefetch depth follows bgmoe_set_skinny_gemm_stages for the 64-row chunks (the 128-row form has no registers
+  // for a third stage at two blocks per CU)
+#define BGMOE_SPLITK_LAUNCH(L_, TT_, NS_) \
+  hipLaunchKernelGGL((fp8_dense_splitk_kernel<L_, TT_, NS_>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per)
   if (chunk_rows == 128) {
-    if (tile) hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_TILE_MAJOR, 8>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
-    else hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_ROW_MAJOR, 8>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+    if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 8, 2);
+    else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 8, 2);
+  } else if (g_skinny_gemm_stages == 4) {
+    if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 4, 4);
+    else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 4, 4);
+  } else if (g_skinny_gemm_stages == 3) {
+    if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 4, 3);
+    else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 4, 3);
   } else {
-    if (tile) hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_TILE_MAJOR, 4>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
-    else hipLaunchKernelGGL((fp8_dense_splitk_kernel<BGMOE_W_ROW_MAJOR, 4>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per);
+    if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 4, 2);
+    else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 4, 2);
   }
+#undef BGMOE_SPLITK_LAUNCH
   int rc = bgmoe_check_launch("fp8_dense_gemm (split-K)");
   if (rc != BGMOE_OK || out == nullptr) return rc;         // out == nullptr: the caller consumes the partial sums
   const int64_t quads = m * n / 4;

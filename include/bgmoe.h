@@ -521,8 +521,9 @@ int bgmoe_set_skinny_tall_min_rows(int rows);
  * opt-in; no counterpart in the reference).  stages = 2 (the default): an item loads one K-block ahead of the one it
  * computes; 3 or 4: two or three ahead, i.e. two or three times the weight bytes in flight per block (the kernel keeps
  * three blocks per CU with 3 stages, two with 4).  Every output element is computed by the same chain of operations
- * whatever the depth: the results are the same bits.  Fused stage 1 is not affected (its three stages fill the
- * register file).  Returns BGMOE_OK or BGMOE_ERR_ARG. */
+ * whatever the depth: the results are the same bits.  The block-split form of bgmoe_fp8_dense_gemm follows the switch
+ * for its 64-row chunks.  Fused stage 1 is not affected (its three stages fill the register file).  Returns BGMOE_OK or
+ * BGMOE_ERR_ARG. */
 int bgmoe_set_skinny_gemm_stages(int stages);
 
 /* Fused stage 1: out = bf16( silu(X*Wg^T) * (X*Wu^T) ), fp32 gate and up.

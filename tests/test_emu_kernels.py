@@ -570,3 +570,36 @@ def test_counted_load_model_catches_a_lenient_wait_in_the_mxfp4_kernel(h, stream
     h.emu_set_wait_slack(24)
     got = run_mx(h, counts, cu, m, x16, ws, n, k, 1)
     assert not (np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]))
+
+
+@pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
+@pytest.mark.parametrize("m,n,k", [(70, 256, 1024), (100, 128, 2688), (40, 128, 4096)])
+def test_dense_split_k_gemm_at_every_prefetch_depth(h, streaming_knobs, m, n, k, layout):
+    """The one-weight GEMM's block-split form (K-slices of 8 blocks over blocks, fp32 partial sums, ordered sum): the
+    proven two-stage kernel against the oracle, then three and four stages under the counted late-load model -- slices
+    of 8, 5 and 8 K-blocks against rings of 2, 3 and 4."""
+    g = torch.Generator().manual_seed(300 + m + k)
+    xq, xs = oq.act_quant(rand_bf16(g, m, k))
+    wq, wsc = oq.weight_block_quant((0.02 * torch.randn(1, n, k, generator=g)).numpy())
+    xq, xs, wq, wsc = G(xq), G(xs), G(wq), G(wsc.astype(np.float32))
+    ref = og.grouped_gemm_fp8(xq, xs, wq, wsc, np.array([m], np.int32), np.array([0, m], np.int32), to_bf16=False)
+    wdev = _tile_major(h, wq) if layout == 1 else wq
+    need = int(h.bgmoe_fp8_dense_gemm_workspace(m, n, k, layout))
+    if need == 0:
+        pytest.skip("this shape is served by the wave-split kernel")
+    a = _act(xq, xs)
+
+    def run():
+        out = G(np.full((m, n), 0x40E0, dtype=np.uint16))
+        ws = G(np.full(need // 4, np.nan, dtype=np.float32))
+        ok(h, h.bgmoe_fp8_dense_gemm(C.byref(a), p(wdev), p(wsc), wsc.shape[2], layout, m, n, k, p(out), p(ws), need, None))
+        return np.array(out)
+
+    want = run()
+    assert og.rel_frobenius(bf16_bits_to_f32(want), ref) < 3e-3
+    for stages in (3, 4):
+        ok(h, h.bgmoe_set_skinny_gemm_stages(stages))
+        for mode, schedule in ((0, 1), (2, 0), (2, 2)):
+            h.emu_set_async_mode(mode)
+            h.emu_set_schedule(schedule)
+            assert np.array_equal(run(), want), f"{stages} stages, load model {mode}, schedule {schedule}"

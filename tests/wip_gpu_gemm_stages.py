@@ -72,3 +72,33 @@ def test_deeper_rings_in_the_layer(dev):
             assert torch.equal(layer(inp["x"], inp["logits"]), want)
     finally:
         check(lib().bgmoe_set_skinny_gemm_stages(2))
+
+
+@pytest.mark.parametrize("m,n,k", [(40, 512, 4224), (100, 1152, 1024), (128, 4096, 7168), (128, 7168, 2048)])
+def test_deeper_rings_in_the_dense_split_k_gemm(dev, m, n, k):
+    """The one-weight GEMM's block-split form with 64-row chunks follows the same switch."""
+    from batchgen_amd._lib import check, lib
+    from batchgen_amd.moe.shared_expert import fp8_gemm_nt
+    from oracle import quant as oq
+    from tests.util import rand_bf16
+    say("dense split-K prefetch depth", m, n, k)
+    g = torch.Generator().manual_seed(m + n + k)
+    xq, xs = oq.act_quant(rand_bf16(g, m, k).view(torch.int16).numpy().view(np.uint16), form="A")
+    wq, ws = oq.weight_block_quant((0.05 * torch.randn(1, n, k, generator=g)).numpy())
+    a = torch.from_numpy(xq).to(dev).view(torch.float8_e4m3fn)
+    b = torch.from_numpy(wq[0]).to(dev).view(torch.float8_e4m3fn)
+    sa, sb = torch.from_numpy(xs).to(dev), torch.from_numpy(ws[0]).to(dev)
+
+    def run():
+        d = torch.full((m, n), -7.0, dtype=torch.bfloat16, device=dev)
+        fp8_gemm_nt((a, sa), (b, sb), d)
+        torch.cuda.synchronize()
+        return d
+
+    want = run()
+    try:
+        for stages in (3, 4):
+            check(lib().bgmoe_set_skinny_gemm_stages(stages))
+            assert torch.equal(run(), want), f"output differs with {stages} prefetch stages"
+    finally:
+        check(lib().bgmoe_set_skinny_gemm_stages(2))
