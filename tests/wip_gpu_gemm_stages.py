@@ -83,7 +83,7 @@ def test_deeper_rings_in_the_dense_split_k_gemm(dev, m, n, k):
     from tests.util import rand_bf16
     say("dense split-K prefetch depth", m, n, k)
     g = torch.Generator().manual_seed(m + n + k)
-    xq, xs = oq.act_quant(rand_bf16(g, m, k).view(torch.int16).numpy().view(np.uint16), form="A")
+    xq, xs = oq.act_quant(rand_bf16(g, m, k).float().numpy(), form="A")
     wq, ws = oq.weight_block_quant((0.05 * torch.randn(1, n, k, generator=g)).numpy())
     a = torch.from_numpy(xq).to(dev).view(torch.float8_e4m3fn)
     b = torch.from_numpy(wq[0]).to(dev).view(torch.float8_e4m3fn)
