@@ -250,31 +250,60 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
 // Item width is chosen per launch on the device: with 4 weight tiles per wave (128 fused / 256 plain output
 // columns per item) when that already gives every resident block an item, else with 2 tiles per wave --
 // fp4 weight stages are small, so with few items twice as many narrower ones keep more loads in flight.
-template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool MAPPED = false>
+// TALL > 0 (mixed item heights): groups with more than 16 * TT rows are cut into items of 16 * TALL rows with
+// kMxTallStages prefetch stages, all others into items of 16 * TT rows with NSTAGE stages -- a small group gets the
+// deep pipeline, a larger one is still streamed once per 16 * TALL rows.  Every output element is computed by the
+// same chain of operations whatever the item height.
+constexpr int kMxTallStages = 3;
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool MAPPED, int NT, int TALL>
+__device__ __forceinline__ void mxfp4_run_item(const Mx4Args& g, const BgmoeItem& it, const uint8_t* ring, uint32_t ring_lds) {
+  if constexpr (TALL > 0) {
+    if (it.rows != 16 * TT) {               // wave-uniform: a tall group's item
+      if (it.cnt > 16 * TALL) mxfp4_item<TALL, kMxTallStages, FUSED, LAYOUT, true, NT, MAPPED>(g, it, ring, ring_lds);
+      else mxfp4_item<TALL, kMxTallStages, FUSED, LAYOUT, false, NT, MAPPED>(g, it, ring, ring_lds);
+      return;
+    }
+  }
+  if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, NT, MAPPED>(g, it, ring, ring_lds);
+  else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, NT, MAPPED>(g, it, ring, ring_lds);
+}
+
+template <int TT, int NSTAGE, bool FUSED, int LAYOUT, bool MAPPED = false, int TALL = 0>
 __global__ __launch_bounds__(256) void mxfp4_skinny_kernel(Mx4Args g, unsigned vblocks, unsigned slots) {
-  __shared__ __align__(16) uint8_t s_ring[NSTAGE * TT * 4096];
+  constexpr int kRingShort = NSTAGE * TT * 4096;
+  constexpr int kRingTall = TALL > 0 ? kMxTallStages * TALL * 4096 : 0;
+  __shared__ __align__(16) uint8_t s_ring[kRingShort > kRingTall ? kRingShort : kRingTall];
   const uint32_t ring_lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)s_ring);
   const int wide_cols = FUSED ? 128 : 256;
   const int ntiles_wide = (g.n + wide_cols - 1) / wide_cols;
-  const int chunks = bgmoe_total_chunks(g.seqlens, g.groups, g.lo, g.hi, 16 * TT);
+  const BgmoeTall tall{TALL > 0 ? 16 * TT : 0, 16 * TALL};      // tall above one short item's rows
+  const int chunks = bgmoe_total_chunks(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, tall);
   const bool narrow = (int64_t)chunks * ((ntiles_wide + 7) & ~7) < (int64_t)slots;   // slots: blocks resident at once
   if (narrow) {
     const int ntiles = (g.n + wide_cols / 2 - 1) / (wide_cols / 2);
     for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
-      const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, vb);
+      const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles, vb, tall);
       if (it.grp == BGMOE_ITEM_END) break;
       if (it.grp == BGMOE_ITEM_PAD) continue;
-      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 2, MAPPED>(g, it, s_ring, ring_lds);
-      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 2, MAPPED>(g, it, s_ring, ring_lds);
+      if constexpr (TALL > 0) {
+        mxfp4_run_item<TT, NSTAGE, FUSED, LAYOUT, MAPPED, 2, TALL>(g, it, s_ring, ring_lds);
+      } else {
+        if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 2, MAPPED>(g, it, s_ring, ring_lds);
+        else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 2, MAPPED>(g, it, s_ring, ring_lds);
+      }
       __syncthreads();                    // the token ring is reused by the next item
     }
   } else {
     for (unsigned vb = blockIdx.x; vb < vblocks; vb += gridDim.x) {
-      const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles_wide, vb);
+      const BgmoeItem it = bgmoe_decode_item(g.seqlens, g.groups, g.lo, g.hi, 16 * TT, ntiles_wide, vb, tall);
       if (it.grp == BGMOE_ITEM_END) break;
       if (it.grp == BGMOE_ITEM_PAD) continue;
-      if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 4, MAPPED>(g, it, s_ring, ring_lds);
-      else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 4, MAPPED>(g, it, s_ring, ring_lds);
+      if constexpr (TALL > 0) {
+        mxfp4_run_item<TT, NSTAGE, FUSED, LAYOUT, MAPPED, 4, TALL>(g, it, s_ring, ring_lds);
+      } else {
+        if (it.cnt > 16 * TT) mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, true, 4, MAPPED>(g, it, s_ring, ring_lds);
+        else mxfp4_item<TT, NSTAGE, FUSED, LAYOUT, false, 4, MAPPED>(g, it, s_ring, ring_lds);
+      }
       __syncthreads();
     }
   }
@@ -309,12 +338,12 @@ int check_w(const char* what, const bgmoe_mxfp4_weight* w) {
 }
 
 // blocks resident on the whole device at once, a multiple of 8 (queried once per kernel)
-template <int TT, int NS, bool FUSED, int LAYOUT, bool MAPPED = false>
+template <int TT, int NS, bool FUSED, int LAYOUT, bool MAPPED = false, int TALL = 0>
 unsigned mx_resident() {
   static unsigned resident = 0;
   if (resident == 0) {
     int per_cu = 0, dev = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT, MAPPED>, 256, 0) != hipSuccess || per_cu < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT, MAPPED, TALL>, 256, 0) != hipSuccess || per_cu < 1)
       per_cu = 1;
     if (hipGetDevice(&dev) != hipSuccess ||
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
@@ -325,15 +354,15 @@ unsigned mx_resident() {
   return resident;
 }
 
-template <int TT, int NS, bool FUSED, int LAYOUT, bool MAPPED = false>
+template <int TT, int NS, bool FUSED, int LAYOUT, bool MAPPED = false, int TALL = 0>
 void launch_one(unsigned vblocks, const Mx4Args& g, hipStream_t st) {
   // Twice as many blocks as fit at once: with up to two rounds of items every block has one item and the
   // hardware hands the second round out as blocks finish, which evens out items of unequal length (a 64-row
   // item takes 1.7x a 16-row one); beyond that the blocks stride.  Measured: skewed counts 14% faster,
   // uniform ones 3% slower (the late blocks' start-up).
-  const unsigned slots = mx_resident<TT, NS, FUSED, LAYOUT, MAPPED>();
+  const unsigned slots = mx_resident<TT, NS, FUSED, LAYOUT, MAPPED, TALL>();
   const dim3 grid(vblocks < 2 * slots ? vblocks : 2 * slots), block(256);
-  hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT, MAPPED>), grid, block, 0, st, g, vblocks,
+  hipLaunchKernelGGL((mxfp4_skinny_kernel<TT, NS, FUSED, LAYOUT, MAPPED, TALL>), grid, block, 0, st, g, vblocks,
                      vblocks < slots ? vblocks : slots);
 }
 
@@ -343,31 +372,35 @@ constexpr int kMxTT = 4;           // 64-row items: every group is streamed once
 // pay for three more stages (20 KB in flight per wave) at the same two blocks per CU and the same 48 KB token ring.
 // bf16 token rows weigh four times their weights, so a 32-row item is also the better-balanced unit.
 constexpr int kMxTT2 = 2, kMxNS2 = 6;
+// Mixed item heights (variant 2): the 64-row items' 64 accumulators and the 32-row items' prefetch stages share one
+// register budget, which leaves the 32-row items five stages at two blocks per CU.
+constexpr int kMxNSMixed = 5;
 int g_mx_variant = 0;
 
-template <int TT, int NS>
+template <int TT, int NS, int TALL = 0>
 void launch_shape(bool fused, bool tm, unsigned vblocks, const Mx4Args& g, hipStream_t st) {
   if (fused && g.row_pair != nullptr) {                  // stage 1 reading its rows through the row -> pair map
-    if (tm) launch_one<TT, NS, true, 1, true>(vblocks, g, st);
-    else launch_one<TT, NS, true, 0, true>(vblocks, g, st);
+    if (tm) launch_one<TT, NS, true, 1, true, TALL>(vblocks, g, st);
+    else launch_one<TT, NS, true, 0, true, TALL>(vblocks, g, st);
   } else if (fused) {
-    if (tm) launch_one<TT, NS, true, 1>(vblocks, g, st);
-    else launch_one<TT, NS, true, 0>(vblocks, g, st);
+    if (tm) launch_one<TT, NS, true, 1, false, TALL>(vblocks, g, st);
+    else launch_one<TT, NS, true, 0, false, TALL>(vblocks, g, st);
   } else {
-    if (tm) launch_one<TT, NS, false, 1>(vblocks, g, st);
-    else launch_one<TT, NS, false, 0>(vblocks, g, st);
+    if (tm) launch_one<TT, NS, false, 1, false, TALL>(vblocks, g, st);
+    else launch_one<TT, NS, false, 0, false, TALL>(vblocks, g, st);
   }
 }
 
 int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
-  const int tt = g_mx_variant == 1 ? kMxTT2 : kMxTT;
+  const int tt = g_mx_variant >= 1 ? kMxTT2 : kMxTT;      // (tall items only lower the item count: the same bound holds)
   const int ntile = fused ? 64 : 128;      // the narrow item width bounds the virtual block count of both widths
   const int64_t bound = g.row_bound > 0 && g.row_bound < m ? g.row_bound : m;
   const unsigned vblocks = bgmoe_item_grid((g.n + ntile - 1) / ntile, g.groups, bound, 0x7fffffff, 16 * tt);
   g.lo = 0; g.hi = 0x7fffffff;     // every group: more rows = more chunks (weights re-streamed)
   const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
   BgmoeProf prof(fused ? BGMOE_K_MXFP4_S1 : BGMOE_K_MXFP4_GEMM, st);
-  if (g_mx_variant == 1) launch_shape<kMxTT2, kMxNS2>(fused, tm, vblocks, g, st);
+  if (g_mx_variant == 2) launch_shape<kMxTT2, kMxNSMixed, kMxTT>(fused, tm, vblocks, g, st);
+  else if (g_mx_variant == 1) launch_shape<kMxTT2, kMxNS2>(fused, tm, vblocks, g, st);
   else launch_shape<kMxTT, 3>(fused, tm, vblocks, g, st);
   return bgmoe_check_launch("mxfp4 grouped gemm");
 }
@@ -399,12 +432,18 @@ int bgmoe_internal_init_mxfp4() {
   mx_resident<kMxTT2, kMxNS2, false, 0>();
   mx_resident<kMxTT2, kMxNS2, true, 1, true>();
   mx_resident<kMxTT2, kMxNS2, true, 0, true>();
+  mx_resident<kMxTT2, kMxNSMixed, true, 1, false, kMxTT>();
+  mx_resident<kMxTT2, kMxNSMixed, true, 0, false, kMxTT>();
+  mx_resident<kMxTT2, kMxNSMixed, false, 1, false, kMxTT>();
+  mx_resident<kMxTT2, kMxNSMixed, false, 0, false, kMxTT>();
+  mx_resident<kMxTT2, kMxNSMixed, true, 1, true, kMxTT>();
+  mx_resident<kMxTT2, kMxNSMixed, true, 0, true, kMxTT>();
   return BGMOE_OK;
 }
 
 extern "C" int bgmoe_set_mxfp4_variant(int variant) {
-  BGMOE_REQUIRE(variant == 0 || variant == 1, "set_mxfp4_variant: variant must be 0 (64-row items, three stages) or 1 "
-                                              "(32-row items, six stages), got %d", variant);
+  BGMOE_REQUIRE(variant >= 0 && variant <= 2, "set_mxfp4_variant: variant must be 0 (64-row items, three stages), 1 "
+                "(32-row items, six stages) or 2 (per group: 32-row items up to 32 rows, 64-row items above), got %d", variant);
   g_mx_variant = variant;
   return BGMOE_OK;
 }

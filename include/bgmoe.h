@@ -603,8 +603,10 @@ int bgmoe_mxfp4_fused_s1_gather(const uint16_t* x_tokens, int64_t n_tokens, cons
 /* Which shape of the MXFP4 weight-streaming kernel serves the calls above (process-wide, opt-in; no counterpart in
  * the reference): 0 = 64-row work items with a three-stage weight prefetch (the default), 1 = 32-row items with a
  * six-stage prefetch (2.5 times the weight bytes in flight per wave, groups above 32 rows pass over their weights
- * once per 32 rows).  Every output element is computed by the same chain of operations: same bits.
- * Returns BGMOE_OK or BGMOE_ERR_ARG. */
+ * once per 32 rows), 2 = the item height chosen per group on the device, in one launch: groups of at most 32 rows as
+ * 32-row items with a five-stage prefetch, larger groups as 64-row items with three stages (the 64-row items'
+ * accumulators and the 32-row items' stages share the register file, hence five).  Every output element is computed by
+ * the same chain of operations: same bits.  Returns BGMOE_OK or BGMOE_ERR_ARG. */
 int bgmoe_set_mxfp4_variant(int variant);
 
 /* DeepGEMM's contiguous m-grouped API describes the rows by a map `grouped_layout` [m] (row -> group, -1 on

@@ -55,14 +55,15 @@ def test_second_shape_gives_the_same_bits(dev, counts, n, k, layout):
     for e, c in enumerate(counts):
         live[cu[e]:cu[e] + c] = True
     lv = torch.from_numpy(live).to(dev)
-    try:
-        check(lib().bgmoe_set_mxfp4_variant(1))
-        got = run()
-    finally:
-        check(lib().bgmoe_set_mxfp4_variant(0))
-    assert torch.equal(got[0], want[0]), "plain GEMM (rows outside the groups included)"
-    for name, a, b in zip(("swiglu", "situ"), want[1:], got[1:]):
-        assert torch.equal(a[lv], b[lv]), f"fused stage 1 ({name})"
+    for variant in (1, 2):
+        try:
+            check(lib().bgmoe_set_mxfp4_variant(variant))
+            got = run()
+        finally:
+            check(lib().bgmoe_set_mxfp4_variant(0))
+        assert torch.equal(got[0], want[0]), f"shape {variant}: plain GEMM (rows outside the groups included)"
+        for name, a, b in zip(("swiglu", "situ"), want[1:], got[1:]):
+            assert torch.equal(a[lv], b[lv]), f"shape {variant}: fused stage 1 ({name})"
 
 
 @pytest.mark.parametrize("fold", [False, True], ids=["gathered", "folded_gather"])
@@ -75,10 +76,11 @@ def test_layer_on_the_second_shape(dev, fold):
     w, sh = wl.make_mxfp4_weights(cfg, dev)
     layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], fold_gather=fold)
     want = layer(inp["x"], inp["logits"]).clone()
-    try:
-        check(lib().bgmoe_set_mxfp4_variant(1))
-        got = layer(inp["x"], inp["logits"]).clone()
-    finally:
-        check(lib().bgmoe_set_mxfp4_variant(0))
-    assert torch.equal(got, want)
-    assert lib().bgmoe_set_mxfp4_variant(2) != 0 and lib().bgmoe_set_mxfp4_variant(-1) != 0
+    for variant in (1, 2):
+        try:
+            check(lib().bgmoe_set_mxfp4_variant(variant))
+            got = layer(inp["x"], inp["logits"]).clone()
+        finally:
+            check(lib().bgmoe_set_mxfp4_variant(0))
+        assert torch.equal(got, want), f"shape {variant}"
+    assert lib().bgmoe_set_mxfp4_variant(3) != 0 and lib().bgmoe_set_mxfp4_variant(-1) != 0
