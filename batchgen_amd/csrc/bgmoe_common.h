@@ -160,6 +160,13 @@ __device__ __forceinline__ float gload_f32(const float* p) {
 __device__ __forceinline__ uint32_t gload_u32(const void* p) {
   return *reinterpret_cast<const BGMOE_GLOBAL uint32_t*>((uintptr_t)p);
 }
+// The same for stores: a store through a generic pointer is a flat store, and while one is pending the compiler
+// turns every wait for a load into a full wait (flat operations may complete out of order), which drains a
+// software pipeline that runs into the next work item's loads.
+typedef unsigned int bgmoe_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void gstore_x2(void* p, uint2 v) {
+  *reinterpret_cast<BGMOE_GLOBAL bgmoe_u32x2*>((uintptr_t)p) = bgmoe_u32x2{v.x, v.y};
+}
 
 // ---- wave helpers ---------------------------------------------------------------
 __device__ __forceinline__ int lane_id() { return threadIdx.x & (BGMOE_WAVE - 1); }

@@ -231,7 +231,7 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
         uint2 o;
         o.x = pack2_bf16(h[0], h[1]);
         o.y = pack2_bf16(h[2], h[3]);
-        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * j + 4 * kq) = o;
+        gstore_x2(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * j + 4 * kq, o);
       }
     } else {
 #pragma unroll
@@ -240,7 +240,7 @@ __device__ __forceinline__ void mxfp4_item(const Mx4Args& g, const BgmoeItem& it
         uint2 o;
         o.x = pack2_bf16(acc[tt][t][0], acc[tt][t][1]);
         o.y = pack2_bf16(acc[tt][t][2], acc[tt][t][3]);
-        *reinterpret_cast<uint2*>(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * t + 4 * kq) = o;
+        gstore_x2(obase + (int64_t)tok * g.n + n0 + NW * wave + 16 * t + 4 * kq, o);
       }
     }
   }
