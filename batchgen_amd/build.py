@@ -64,11 +64,17 @@ def _compile(src: str, force: bool) -> str:
     cmd = [hipcc()] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
     if src in NO_SPILL:
         cmd.insert(-4, "-Rpass-analysis=kernel-resource-usage")
+    asm_job = _start_asm(src, obj) if src in NO_FLAT else None       # beside the compile, not after it
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
+        if asm_job:
+            asm_job.kill()
+            asm_job.communicate()
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
     if src in NO_SPILL:
         _check_no_spill(src, r.stderr, obj)
+    if asm_job:
+        _check_no_flat(src, obj, asm_job)
     return obj
 
 
@@ -78,6 +84,10 @@ def _compile(src: str, force: bool) -> str:
 # leave room for its 4 x 33 KB ring in the CU's 160 KB of LDS.  Checked on every build from the compiler's own
 # resource remarks; a kernel over budget fails the build.
 RESOURCE_GATES = {
+    # the weight-streaming kernels keep their prefetch stages in registers: two blocks per CU and no spills, whatever
+    # variant is added (a variant whose paths together need more than 256 registers drops to one block per CU)
+    "gemm_fp8_skinny.hip": dict(kernel="fp8_skinny_kernel", min_occupancy=2),
+    "gemm_mxfp4_skinny.hip": dict(kernel="mxfp4_skinny_kernel", min_occupancy=2),
     "gemm_fp8_streamk.hip": dict(kernel="fp8_streamk_kernel"),
     "gemm_fp8_tiled_k64.hip": dict(kernel="fp8_tiled_k64_kernel", max_vgprs=256, max_agprs=0,
                                    max_static_lds=163840 - 4 * (32768 + 1024), min_occupancy=2),
@@ -117,6 +127,32 @@ def _check_no_spill(src: str, remarks: str, obj: str) -> None:
     if bad or seen == 0:
         os.remove(obj)
         raise RuntimeError(f"{src}: kernel resource budget violated ({'; '.join(bad) or 'no resource remarks found'})")
+
+
+# The weight-streaming kernels run one work item into the next; a flat memory instruction (an access through a pointer
+# the compiler cannot place in the global address space) that is still pending makes the compiler wait for ALL loads at
+# the next use of a loaded register, which drains the next item's prefetch ring.  Their device assembly must hold none.
+NO_FLAT = ("gemm_fp8_skinny.hip", "gemm_mxfp4_skinny.hip")
+
+
+def _start_asm(src: str, obj: str):
+    cmd = [hipcc()] + FLAGS + ["--cuda-device-only", "-S", "-c", os.path.join(CSRC, src), "-o", obj[:-2] + ".s"]
+    return subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+
+
+def _check_no_flat(src: str, obj: str, job) -> None:
+    import re
+    asm = obj[:-2] + ".s"
+    _, err = job.communicate()
+    if job.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed for {src}:\n{err}")
+    with open(asm) as f:
+        found = sorted(set(re.findall(r"^\s*(flat_(?:load|store|atomic)\w*)", f.read(), re.M)))
+    os.remove(asm)
+    if found:
+        os.remove(obj)
+        raise RuntimeError(f"{src}: flat memory instructions in the device code ({', '.join(found)}): "
+                           "load and store through the gload_* / gstore_* helpers")
 
 
 # ---- PyTorch C++ extension modules (host code over the C ABI) --------------------------------------------------

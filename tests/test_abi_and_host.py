@@ -362,3 +362,28 @@ def test_moe_base_decode_template_on_a_toy_layer():
     cfg.phase = "prefill"
     with pytest.raises(NotImplementedError):
         layer(x)
+
+
+def test_build_gate_rejects_flat_memory_instructions(tmp_path):
+    """The streaming kernels' device assembly is scanned on every build: a flat load, store or atomic fails it (and
+    removes the object), directives and comments that merely contain the word do not."""
+    from batchgen_amd import build as b
+
+    class Done:
+        returncode = 0
+
+        def communicate(self):
+            return "", ""
+
+    def run(text):
+        obj = tmp_path / "k.o"
+        obj.write_bytes(b"x")
+        (tmp_path / "k.s").write_text(text)
+        b._check_no_flat("k.hip", str(obj), Done())
+        return obj
+
+    ok = run("\t.amdhsa_user_sgpr_flat_scratch_init 0\n\tglobal_store_dwordx2 v[0:1], v[2:3], off ; not flat_store\n")
+    assert ok.exists() and not (tmp_path / "k.s").exists()
+    with pytest.raises(RuntimeError, match="flat_store_dwordx2"):
+        run("\tglobal_load_dwordx4 v[0:3], v[4:5], off\n\tflat_store_dwordx2 v[0:1], v[2:3]\n")
+    assert not (tmp_path / "k.o").exists()
