@@ -91,6 +91,7 @@ _SIGS = {
     "bgmoe_set_skinny_max_rows": (i32, [i32]),
     "bgmoe_set_skinny_tall_min_rows": (i32, [i32]),
     "bgmoe_set_skinny_gemm_stages": (i32, [i32]),
+    "bgmoe_set_skinny_s1_stages": (i32, [i32]),
     "bgmoe_set_mxfp4_variant": (i32, [i32]),
     "bgmoe_set_tiled_variant": (i32, [i32]),
     "bgmoe_fp8_weight_repack": (i32, [vp, vp, i32, i32, i32, vp]),

@@ -477,6 +477,17 @@ extern "C" int bgmoe_set_skinny_gemm_stages(int stages) {
   return BGMOE_OK;
 }
 
+// Prefetch depth of fused stage 1 (opt-in): 3 = two K-blocks ahead, as measured; 4 = three ahead (220 VGPRs + 20
+// AGPRs, still two blocks per CU, no scratch), with the wait count a four-stage ring needs.  Same bits.  The tall-item
+// form keeps its own depths and takes precedence when both are switched on.
+static int g_skinny_s1_stages = 3;
+
+extern "C" int bgmoe_set_skinny_s1_stages(int stages) {
+  BGMOE_REQUIRE(stages == 3 || stages == 4, "set_skinny_s1_stages: stages must be 3 or 4");
+  g_skinny_s1_stages = stages;
+  return BGMOE_OK;
+}
+
 // Stage 1 works on 32-row items (its epilogue keeps 16*TT x 8 fp32 results per lane alive next to the
 // prefetch stages); the plain GEMM on 64-row items, which halves the passes over the weights of groups
 // with more than 32 rows.
@@ -488,6 +499,9 @@ static void launch_variant(bool fused, int layout, int n, int groups, int64_t bo
     if (g.tall_min > 0) {
       if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 3, true, BGMOE_W_TILE_MAJOR, 4, 4>(vb, g, st);
       else launch_one<2, 3, true, BGMOE_W_ROW_MAJOR, 4, 4>(vb, g, st);
+    } else if (g_skinny_s1_stages == 4) {
+      if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 4, true, BGMOE_W_TILE_MAJOR>(vb, g, st);
+      else launch_one<2, 4, true, BGMOE_W_ROW_MAJOR>(vb, g, st);
     } else if (layout == BGMOE_W_TILE_MAJOR) launch_one<2, 3, true, BGMOE_W_TILE_MAJOR>(vb, g, st);
     else launch_one<2, 3, true, BGMOE_W_ROW_MAJOR>(vb, g, st);
   } else {
@@ -514,6 +528,8 @@ int bgmoe_internal_init_fp8_skinny() {
   skinny_resident<4, 2, false, BGMOE_W_ROW_MAJOR, 2>();
   skinny_resident<2, 3, true, BGMOE_W_TILE_MAJOR, 4, 4>();
   skinny_resident<2, 3, true, BGMOE_W_ROW_MAJOR, 4, 4>();
+  skinny_resident<2, 4, true, BGMOE_W_TILE_MAJOR>();
+  skinny_resident<2, 4, true, BGMOE_W_ROW_MAJOR>();
   skinny_resident<4, 3, false, BGMOE_W_TILE_MAJOR, 2>();
   skinny_resident<4, 3, false, BGMOE_W_ROW_MAJOR, 2>();
   skinny_resident<4, 4, false, BGMOE_W_TILE_MAJOR, 2>();

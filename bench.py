@@ -110,6 +110,9 @@ def parse():
     ap.add_argument("--gemm-stages", type=int, default=2, choices=[2, 3, 4],
                     help="decode: prefetch depth of the weight-streaming down projection "
                          "(bgmoe_set_skinny_gemm_stages; 2 = the default)")
+    ap.add_argument("--s1-stages", type=int, default=3, choices=[3, 4],
+                    help="decode: prefetch depth of the weight-streaming fused stage 1 (bgmoe_set_skinny_s1_stages; "
+                         "3 = the default)")
     ap.add_argument("--template", action="store_true",
                     help="FP8 configurations: also time the layer as a model file runs it through the MoEBase template "
                          "(router GEMM + gate, routed experts behind the given routes, dense shared expert, add) and "
@@ -442,6 +445,7 @@ def measure_layer(a, config, with_cpu):
         layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
     _lib.check(_lib.lib().bgmoe_set_tiled_variant(int(getattr(a, "tiled_variant", 0))))
     _lib.check(_lib.lib().bgmoe_set_skinny_tall_min_rows(int(getattr(a, "tall_min_rows", 0))))
+    _lib.check(_lib.lib().bgmoe_set_skinny_s1_stages(int(getattr(a, "s1_stages", 3))))
     _lib.check(_lib.lib().bgmoe_set_skinny_gemm_stages(int(getattr(a, "gemm_stages", 2))))
     _lib.check(_lib.lib().bgmoe_set_mxfp4_variant(int(getattr(a, "mxfp4_variant", 0))))
     _lib.check(_lib.lib().bgmoe_set_router_gemm_plan(-1, int(getattr(a, "bf16_gemm_plan", -1))))

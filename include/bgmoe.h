@@ -526,6 +526,13 @@ int bgmoe_set_skinny_tall_min_rows(int rows);
  * BGMOE_ERR_ARG. */
 int bgmoe_set_skinny_gemm_stages(int stages);
 
+/* Prefetch depth of fused stage 1 of the weight-streaming kernel (process-wide, opt-in; no counterpart in the
+ * reference).  stages = 3 (the default): an item loads two K-blocks ahead of the one it computes; 4: three ahead (half
+ * again the weight bytes in flight per block, at the same two blocks per CU).  Same chain of operations per output
+ * element, same bits.  With tall items switched on (bgmoe_set_skinny_tall_min_rows) their form is used instead.
+ * Returns BGMOE_OK or BGMOE_ERR_ARG. */
+int bgmoe_set_skinny_s1_stages(int stages);
+
 /* Fused stage 1: out = bf16( silu(X*Wg^T) * (X*Wu^T) ), fp32 gate and up.
  * Replaces `fp8_blockwise_fused_s1` / `_ptrs`
  * (grouped_fp8_blockwise_moe.py:423-560, fp8_blockwise_s1_kernel.cuh:425-607).

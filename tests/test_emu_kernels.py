@@ -489,6 +489,7 @@ def run_plain_gemm(h, counts, cu, m, xq, xs, w, n, k, layout):
 @pytest.fixture
 def streaming_knobs(h):
     yield
+    ok(h, h.bgmoe_set_skinny_s1_stages(3))
     ok(h, h.bgmoe_set_skinny_gemm_stages(2))
     ok(h, h.bgmoe_set_mxfp4_variant(0))
     ok(h, h.bgmoe_set_skinny_tall_min_rows(0))
@@ -604,3 +605,27 @@ def test_dense_split_k_gemm_at_every_prefetch_depth(h, streaming_knobs, m, n, k,
             h.emu_set_async_mode(mode)
             h.emu_set_schedule(schedule)
             assert np.array_equal(run(), want), f"{stages} stages, load model {mode}, schedule {schedule}"
+
+
+@pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
+@pytest.mark.parametrize("k", [128, 384, 512, 640, 1152])
+def test_fused_stage1_with_four_prefetch_stages(h, streaming_knobs, k, layout):
+    """Fused stage 1 with a four-stage ring (no GPU has run it) against the proven three-stage form: bf16 output, e4m3
+    bytes and scales bit for bit; 1 to 9 K-blocks; loads at once and as late as the waits allow with every global load
+    counted; then the negative control -- the same run with every wait loosened by 24 loads must differ."""
+    n = 256
+    counts, cu, m, xq, xs, ws, live = _problem(500 + k, (0, 1, 31, 33, 64, 100), n, k, nmat=2)
+    want = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+    if k == 384:
+        check_s1_against_oracle(xq, xs, ws[0], ws[1], counts, cu, live, want)
+    ok(h, h.bgmoe_set_skinny_s1_stages(4))
+    for mode, schedule in ((0, 1), (2, 0), (2, 2)):
+        h.emu_set_async_mode(mode)
+        h.emu_set_schedule(schedule)
+        got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+        for name, a, b in zip(("bf16 output", "e4m3 bytes", "scales"), want, got):
+            assert np.array_equal(a, b), f"{name}: load model {mode}, schedule {schedule}"
+    if k >= 640:                             # long enough for the main loop of the four-stage ring
+        h.emu_set_wait_slack(24)
+        got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
+        assert not all(np.array_equal(a, b) for a, b in zip(want, got))

@@ -1,5 +1,6 @@
-"""The plain weight-streaming FP8 grouped GEMM (the down projection of a decode step) with a deeper prefetch ring
-(``bgmoe_set_skinny_gemm_stages``: 3 or 4 stages instead of 2, with the wait count a deeper ring needs).  Every output
+"""The weight-streaming FP8 kernels with deeper prefetch rings: the plain grouped GEMM (the down projection of a decode
+step; ``bgmoe_set_skinny_gemm_stages``: 3 or 4 stages instead of 2) and fused stage 1 (``bgmoe_set_skinny_s1_stages``:
+4 instead of 3), with the wait count a deeper ring needs.  Every output
 element is computed by the same chain of operations whatever the depth, so the output must equal the default
 kernel's bit for bit, rows outside every group untouched.  The rings' wait counts are exercised on the CPU emulator
 with every load landing as late as the waits allow (tests/test_emu_kernels.py).
@@ -101,4 +102,63 @@ def test_deeper_rings_in_the_dense_split_k_gemm(dev, m, n, k):
             check(lib().bgmoe_set_skinny_gemm_stages(stages))
             assert torch.equal(run(), want), f"output differs with {stages} prefetch stages"
     finally:
+        check(lib().bgmoe_set_skinny_gemm_stages(2))
+
+
+S1_CASES = [
+    ((0, 1, 31, 32, 33, 40, 64, 65, 100, 128, 129, 200, 256), 256, 512),
+    ((256, 14, 41, 65, 39, 35, 1), 2048, 7168),            # the benchmark layer's stage-1 shape, a folded shared expert
+    ((48,) * 9, 384, 128),                                 # one K-block
+    ((70, 3), 128, 384),                                   # three K-blocks: shorter than the four-stage ring
+    ((8,) * 32, 512, 1152),                                # nine K-blocks
+]
+
+
+@pytest.mark.parametrize("layout", ["row_major", "tile_major"])
+@pytest.mark.parametrize("counts,n,k", S1_CASES, ids=[f"case{i}" for i in range(len(S1_CASES))])
+def test_four_stage_fused_stage1_gives_the_same_bits(dev, counts, n, k, layout):
+    from batchgen_amd._lib import check, lib
+    say("fused stage 1, four prefetch stages", counts, n, k, layout)
+    counts, cu, m, xq, xs, ws = _make(6100 + n + k, counts, n, k, nmat=2)
+    (gq, gs), (uq, us) = ws
+    xq_d, xs_t, gq_d, gs_d = _dev(dev, xq, xs, gq, gs)
+    _, _, uq_d, us_d = _dev(dev, xq, xs, uq, us)
+    if layout == "tile_major":
+        gq_d, uq_d = gm().fp8_weight_repack(gq_d), gm().fp8_weight_repack(uq_d)
+    cnt_d, cu_d = torch.from_numpy(counts).to(dev), torch.from_numpy(cu).to(dev)
+
+    def run():
+        h = torch.full((m, n), 5.0, dtype=torch.bfloat16, device=dev)
+        gm().fp8_blockwise_fused_s1(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, 16, h, weight_layout=layout)
+        hq = torch.full((m, n), 0x55, dtype=torch.uint8, device=dev)
+        hs = torch.full((n // 128, m), -3.0, dtype=torch.float32, device=dev)
+        gm().fp8_blockwise_fused_s1_quant(xq_d, gq_d, uq_d, cnt_d, cu_d, xs_t, gs_d, us_d, hq, hs, weight_layout=layout)
+        torch.cuda.synchronize()
+        return h, hq, hs
+
+    want = run()
+    try:
+        check(lib().bgmoe_set_skinny_s1_stages(4))
+        got = run()
+    finally:
+        check(lib().bgmoe_set_skinny_s1_stages(3))
+    for name, a, b in zip(("bf16 output", "e4m3 bytes", "scales"), want, got):
+        assert torch.equal(a, b), f"{name} differ with four prefetch stages"
+
+
+def test_four_stage_stage1_in_the_layer(dev):
+    from batchgen_amd import workloads as wl
+    from batchgen_amd._lib import check, lib
+    from batchgen_amd.moe.fp8_layer import Fp8MoELayer
+    cfg = wl.scaled(wl.CONFIGS[1], hidden=1024, inter=512, shared_inter=512)
+    inp = wl.make_inputs(cfg, dev)
+    w, sh = wl.make_fp8_weights(cfg, dev)
+    layer = Fp8MoELayer(cfg, w, sh, inp["bias"])
+    want = layer(inp["x"], inp["logits"]).clone()
+    try:
+        check(lib().bgmoe_set_skinny_s1_stages(4))
+        check(lib().bgmoe_set_skinny_gemm_stages(3))
+        assert torch.equal(layer(inp["x"], inp["logits"]), want)
+    finally:
+        check(lib().bgmoe_set_skinny_s1_stages(3))
         check(lib().bgmoe_set_skinny_gemm_stages(2))
