@@ -375,6 +375,9 @@ constexpr int kMxTT2 = 2, kMxNS2 = 6;
 // Mixed item heights (variant 2): the 64-row items' 64 accumulators and the 32-row items' prefetch stages share one
 // register budget, which leaves the 32-row items five stages at two blocks per CU.
 constexpr int kMxNSMixed = 5;
+// The default item height with one more stage (variant 3): 64-row items keep every group of up to 64 rows a single pass
+// over its weights; the fourth stage costs 20 registers (171 + 64) and a 64 KB token ring, still two blocks per CU.
+constexpr int kMxNSDeep = 4;
 int g_mx_variant = 0;
 
 template <int TT, int NS, int TALL = 0>
@@ -399,7 +402,8 @@ int launch(bool fused, Mx4Args& g, int64_t m, hipStream_t st) {
   g.lo = 0; g.hi = 0x7fffffff;     // every group: more rows = more chunks (weights re-streamed)
   const bool tm = g.w0.layout == BGMOE_W_TILE_MAJOR;
   BgmoeProf prof(fused ? BGMOE_K_MXFP4_S1 : BGMOE_K_MXFP4_GEMM, st);
-  if (g_mx_variant == 2) launch_shape<kMxTT2, kMxNSMixed, kMxTT>(fused, tm, vblocks, g, st);
+  if (g_mx_variant == 3) launch_shape<kMxTT, kMxNSDeep>(fused, tm, vblocks, g, st);
+  else if (g_mx_variant == 2) launch_shape<kMxTT2, kMxNSMixed, kMxTT>(fused, tm, vblocks, g, st);
   else if (g_mx_variant == 1) launch_shape<kMxTT2, kMxNS2>(fused, tm, vblocks, g, st);
   else launch_shape<kMxTT, 3>(fused, tm, vblocks, g, st);
   return bgmoe_check_launch("mxfp4 grouped gemm");
@@ -432,6 +436,12 @@ int bgmoe_internal_init_mxfp4() {
   mx_resident<kMxTT2, kMxNS2, false, 0>();
   mx_resident<kMxTT2, kMxNS2, true, 1, true>();
   mx_resident<kMxTT2, kMxNS2, true, 0, true>();
+  mx_resident<kMxTT, kMxNSDeep, true, 1>();
+  mx_resident<kMxTT, kMxNSDeep, true, 0>();
+  mx_resident<kMxTT, kMxNSDeep, false, 1>();
+  mx_resident<kMxTT, kMxNSDeep, false, 0>();
+  mx_resident<kMxTT, kMxNSDeep, true, 1, true>();
+  mx_resident<kMxTT, kMxNSDeep, true, 0, true>();
   mx_resident<kMxTT2, kMxNSMixed, true, 1, false, kMxTT>();
   mx_resident<kMxTT2, kMxNSMixed, true, 0, false, kMxTT>();
   mx_resident<kMxTT2, kMxNSMixed, false, 1, false, kMxTT>();
@@ -442,8 +452,9 @@ int bgmoe_internal_init_mxfp4() {
 }
 
 extern "C" int bgmoe_set_mxfp4_variant(int variant) {
-  BGMOE_REQUIRE(variant >= 0 && variant <= 2, "set_mxfp4_variant: variant must be 0 (64-row items, three stages), 1 "
-                "(32-row items, six stages) or 2 (per group: 32-row items up to 32 rows, 64-row items above), got %d", variant);
+  BGMOE_REQUIRE(variant >= 0 && variant <= 3, "set_mxfp4_variant: variant must be 0 (64-row items, three stages), 1 "
+                "(32-row items, six stages), 2 (per group: 32-row items up to 32 rows, 64-row items above) or 3 (64-row "
+                "items, four stages), got %d", variant);
   g_mx_variant = variant;
   return BGMOE_OK;
 }

@@ -94,9 +94,9 @@ def parse():
     ap.add_argument("--tiled-variant", type=int, default=0, choices=[0, 1, 2],
                     help="which LDS-tiled kernel serves the prefill groups: 0 = K steps of 128 (default), 1 = K steps of "
                          "64 with in-place accumulation, 2 = the same with plain per-lane stores (bgmoe_set_tiled_variant)")
-    ap.add_argument("--mxfp4-variant", type=int, default=0, choices=[0, 1, 2],
+    ap.add_argument("--mxfp4-variant", type=int, default=0, choices=[0, 1, 2, 3],
                     help="MXFP4 configurations: 0 = 64-row items with three prefetch stages (default), 1 = 32-row items "
-                         "with six, 2 = per group: 32-row items (five stages) up to 32 rows, 64-row items above "
+                         "with six, 2 = per group: 32-row items (five stages) up to 32 rows, 64-row items above, 3 = 64-row items with four "
                          "(bgmoe_set_mxfp4_variant)")
     ap.add_argument("--bf16-gemm-plan", type=int, default=-1, choices=[-1, 0, 1, 2, 3, 4, 5],
                     help="launch shape of the bf16 GEMM behind the router GEMM and the MXFP4 layers' linear layers "

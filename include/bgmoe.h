@@ -612,7 +612,8 @@ int bgmoe_mxfp4_fused_s1_gather(const uint16_t* x_tokens, int64_t n_tokens, cons
  * six-stage prefetch (2.5 times the weight bytes in flight per wave, groups above 32 rows pass over their weights
  * once per 32 rows), 2 = the item height chosen per group on the device, in one launch: groups of at most 32 rows as
  * 32-row items with a five-stage prefetch, larger groups as 64-row items with three stages (the 64-row items'
- * accumulators and the 32-row items' stages share the register file, hence five).  Every output element is computed by
+ * accumulators and the 32-row items' stages share the register file, hence five), 3 = the default's 64-row items with a
+ * four-stage prefetch (a 64 KB token ring).  Every output element is computed by
  * the same chain of operations: same bits.  Returns BGMOE_OK or BGMOE_ERR_ARG. */
 int bgmoe_set_mxfp4_variant(int variant);
 

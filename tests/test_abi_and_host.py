@@ -111,9 +111,9 @@ def test_tuning_switches_check_their_arguments():
         assert h.bgmoe_set_skinny_s1_stages(bad) != 0 and b"3 or 4" in h.bgmoe_last_error()
     for good in (4, 3):
         assert h.bgmoe_set_skinny_s1_stages(good) == 0
-    for bad in (-1, 3):
+    for bad in (-1, 4):
         assert h.bgmoe_set_mxfp4_variant(bad) != 0 and b"variant" in h.bgmoe_last_error()
-    for good in (1, 2, 0):
+    for good in (1, 2, 3, 0):
         assert h.bgmoe_set_mxfp4_variant(good) == 0
 
 

@@ -311,7 +311,7 @@ def test_mxfp4_kernel_and_its_second_shape_on_the_emulator(h, counts, n, k, layo
     assert og.rel_frobenius(want[1][live], (oq.silu_f32(ref) * upv)[live]) < 4e-3 and np.all(want[1][~live] == 5.0)
     want_situ = run_mx(h, counts, cu, m, x16, ws, n, k, layout, activation=1)[1]
     assert og.rel_frobenius(want_situ[live], osi.situ_fused(ref, upv)[live]) < 6e-3
-    for variant in (1, 2):                  # 2: the item height per group (five stages up to 32 rows, 64-row items above)
+    for variant in (1, 2, 3):               # 2: the item height per group; 3: the default height with four stages
         try:
             ok(h, h.bgmoe_set_mxfp4_variant(variant))
             got = run_mx(h, counts, cu, m, x16, ws, n, k, layout)
@@ -321,7 +321,7 @@ def test_mxfp4_kernel_and_its_second_shape_on_the_emulator(h, counts, n, k, layo
         assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]) and np.array_equal(got_situ, want_situ), variant
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 @pytest.mark.parametrize("n_tok,top_k,e_total,start,el,mtp", [(96, 4, 24, 8, 6, 96), (200, 4, 8, 0, 6, 64), (1100, 8, 16, 4, 8, 700)])
 def test_index_only_dispatch_and_stage1_through_the_map_on_the_emulator(h, n_tok, top_k, e_total, start, el, mtp, variant):
     """bgmoe_dispatch_index_3d against the oracle (counts, arrivals, positions, the inverse row -> pair map; the
@@ -554,13 +554,13 @@ def test_streaming_kernels_with_loads_as_late_as_their_waits_allow(h, streaming_
             got = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
             for a, b in zip(want, got):
                 assert np.array_equal(a, b), f"stage 1, tall_min {tall_min}, schedule {schedule}"
-        for variant in (0, 1, 2):
+        for variant in (0, 1, 2, 3):
             ok(h, h.bgmoe_set_mxfp4_variant(variant))
             got = run_mx(h, mxc, mxcu, mxm, x16, mws, n, 1664, layout)
             assert np.array_equal(got[0], mwant[0]) and np.array_equal(got[1], mwant[1]), f"MXFP4 shape {variant}"
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
 def test_counted_load_model_catches_a_lenient_wait_in_the_mxfp4_kernel(h, streaming_knobs, variant):
     n, k = 128, 1664
     counts, cu, m, x, x16, ws, live = _mx_problem(93, (64, 20), n, k)

@@ -55,7 +55,7 @@ def test_second_shape_gives_the_same_bits(dev, counts, n, k, layout):
     for e, c in enumerate(counts):
         live[cu[e]:cu[e] + c] = True
     lv = torch.from_numpy(live).to(dev)
-    for variant in (1, 2):
+    for variant in (1, 2, 3):
         try:
             check(lib().bgmoe_set_mxfp4_variant(variant))
             got = run()
@@ -76,11 +76,11 @@ def test_layer_on_the_second_shape(dev, fold):
     w, sh = wl.make_mxfp4_weights(cfg, dev)
     layer = Mxfp4MoELayer(cfg, w, sh, inp["bias"], fold_gather=fold)
     want = layer(inp["x"], inp["logits"]).clone()
-    for variant in (1, 2):
+    for variant in (1, 2, 3):
         try:
             check(lib().bgmoe_set_mxfp4_variant(variant))
             got = layer(inp["x"], inp["logits"]).clone()
         finally:
             check(lib().bgmoe_set_mxfp4_variant(0))
         assert torch.equal(got, want), f"shape {variant}"
-    assert lib().bgmoe_set_mxfp4_variant(3) != 0 and lib().bgmoe_set_mxfp4_variant(-1) != 0
+    assert lib().bgmoe_set_mxfp4_variant(4) != 0 and lib().bgmoe_set_mxfp4_variant(-1) != 0
