@@ -706,11 +706,14 @@ int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weig
   const int chunk_rows = m > 256 || (m > 128 && k >= 4096) ? 128 : 64;
   const unsigned blocks = (unsigned)(((n + 127) / 128) * ((m + chunk_rows - 1) / chunk_rows) * ksplit);
   const bool tile = w->layout == BGMOE_W_TILE_MAJOR;
-  // the prefetch depth follows bgmoe_set_skinny_gemm_stages for the 64-row chunks (the 128-row form has no registers
-  // for a third stage at two blocks per CU)
+  // the prefetch depth follows bgmoe_set_skinny_gemm_stages (128-row chunks: three stages at most, a fourth 17 KB ring
+  // slot would pass the 64 KB of static LDS)
 #define BGMOE_SPLITK_LAUNCH(L_, TT_, NS_) \
   hipLaunchKernelGGL((fp8_dense_splitk_kernel<L_, TT_, NS_>), dim3(blocks), dim3(256), 0, st, g, (int)m, ksplit, per)
-  if (chunk_rows == 128) {
+  if (chunk_rows == 128 && g_skinny_gemm_stages >= 3) {
+    if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 8, 3);
+    else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 8, 3);
+  } else if (chunk_rows == 128) {
     if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 8, 2);
     else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 8, 2);
   } else if (g_skinny_gemm_stages == 4) {

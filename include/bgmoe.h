@@ -522,7 +522,7 @@ int bgmoe_set_skinny_tall_min_rows(int rows);
  * computes; 3 or 4: two or three ahead, i.e. two or three times the weight bytes in flight per block (the kernel keeps
  * three blocks per CU with 3 stages, two with 4).  Every output element is computed by the same chain of operations
  * whatever the depth: the results are the same bits.  The block-split form of bgmoe_fp8_dense_gemm follows the switch
- * for its 64-row chunks.  Fused stage 1 is not affected (its three stages fill the register file).  Returns BGMOE_OK or
+ * (its 128-row chunks take three stages at most).  Fused stage 1 is not affected (its three stages fill the register file).  Returns BGMOE_OK or
  * BGMOE_ERR_ARG. */
 int bgmoe_set_skinny_gemm_stages(int stages);
 

@@ -575,7 +575,7 @@ def test_counted_load_model_catches_a_lenient_wait_in_the_mxfp4_kernel(h, stream
 
 
 @pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
-@pytest.mark.parametrize("m,n,k", [(70, 256, 1024), (100, 128, 2688), (40, 128, 4096)])
+@pytest.mark.parametrize("m,n,k", [(70, 256, 1024), (100, 128, 2688), (40, 128, 4096), (150, 128, 4096), (300, 128, 1024)])
 def test_dense_split_k_gemm_at_every_prefetch_depth(h, streaming_knobs, m, n, k, layout):
     """The one-weight GEMM's block-split form (K-slices of 8 blocks over blocks, fp32 partial sums, ordered sum): the
     proven two-stage kernel against the oracle, then three and four stages under the counted late-load model -- slices

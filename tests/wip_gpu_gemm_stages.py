@@ -75,7 +75,8 @@ def test_deeper_rings_in_the_layer(dev):
         check(lib().bgmoe_set_skinny_gemm_stages(2))
 
 
-@pytest.mark.parametrize("m,n,k", [(40, 512, 4224), (100, 1152, 1024), (128, 4096, 7168), (128, 7168, 2048)])
+@pytest.mark.parametrize("m,n,k", [(40, 512, 4224), (100, 1152, 1024), (128, 4096, 7168), (128, 7168, 2048), (200, 512, 4224),
+                                    (300, 1152, 1024)])    # the last two: 128-row chunks
 def test_deeper_rings_in_the_dense_split_k_gemm(dev, m, n, k):
     """The one-weight GEMM's block-split form with 64-row chunks follows the same switch."""
     from batchgen_amd._lib import check, lib
