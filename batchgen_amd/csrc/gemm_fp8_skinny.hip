@@ -466,13 +466,13 @@ static void launch_one(unsigned vblocks, const SkinnyArgs& g, hipStream_t st) {
   hipLaunchKernelGGL((fp8_skinny_kernel<TT, NS, FUSED, LAYOUT, NTW, TALL>), grid, block, 0, st, g, vblocks);
 }
 
-// Prefetch depth of the plain GEMM's items (opt-in): 2 = one K-block ahead, as measured; 3 or 4 = two or three ahead
-// (the kernel has the registers: 17 per stage next to 32 accumulators), with the wait count that a deeper pipeline
-// needs (fp8_skinny_item).  Same chain per output element, so the same bits.
+// Prefetch depth of the plain GEMM's items (opt-in): 2 = one K-block ahead, as measured; 3, 4 or 6 = two, three or five
+// ahead (the kernel has the registers: 17 per stage next to 32 accumulators), with the wait count that a deeper
+// pipeline needs (fp8_skinny_item).  Same chain per output element, so the same bits.
 static int g_skinny_gemm_stages = 2;
 
 extern "C" int bgmoe_set_skinny_gemm_stages(int stages) {
-  BGMOE_REQUIRE(stages >= 2 && stages <= 4, "set_skinny_gemm_stages: stages must be 2, 3 or 4");
+  BGMOE_REQUIRE((stages >= 2 && stages <= 4) || stages == 6, "set_skinny_gemm_stages: stages must be 2, 3, 4 or 6");
   g_skinny_gemm_stages = stages;
   return BGMOE_OK;
 }
@@ -509,7 +509,10 @@ static void launch_variant(bool fused, int layout, int n, int groups, int64_t bo
     // out the last round of the persistent grid (measured: -5% to -10% on the down projection)
     const unsigned vb = bgmoe_item_grid((n + 127) / 128, groups, bound, hi, 64);
     const bool tile = layout == BGMOE_W_TILE_MAJOR;
-    if (g_skinny_gemm_stages == 4) {
+    if (g_skinny_gemm_stages == 6) {
+      if (tile) launch_one<4, 6, false, BGMOE_W_TILE_MAJOR, 2>(vb, g, st);
+      else launch_one<4, 6, false, BGMOE_W_ROW_MAJOR, 2>(vb, g, st);
+    } else if (g_skinny_gemm_stages == 4) {
       if (tile) launch_one<4, 4, false, BGMOE_W_TILE_MAJOR, 2>(vb, g, st);
       else launch_one<4, 4, false, BGMOE_W_ROW_MAJOR, 2>(vb, g, st);
     } else if (g_skinny_gemm_stages == 3) {
@@ -534,6 +537,8 @@ int bgmoe_internal_init_fp8_skinny() {
   skinny_resident<4, 3, false, BGMOE_W_ROW_MAJOR, 2>();
   skinny_resident<4, 4, false, BGMOE_W_TILE_MAJOR, 2>();
   skinny_resident<4, 4, false, BGMOE_W_ROW_MAJOR, 2>();
+  skinny_resident<4, 6, false, BGMOE_W_TILE_MAJOR, 2>();
+  skinny_resident<4, 6, false, BGMOE_W_ROW_MAJOR, 2>();
   return BGMOE_OK;
 }
 
@@ -716,7 +721,7 @@ int bgmoe_internal_fp8_dense_splitk(const bgmoe_fp8_act* a, const bgmoe_fp8_weig
   } else if (chunk_rows == 128) {
     if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 8, 2);
     else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 8, 2);
-  } else if (g_skinny_gemm_stages == 4) {
+  } else if (g_skinny_gemm_stages >= 4) {
     if (tile) BGMOE_SPLITK_LAUNCH(BGMOE_W_TILE_MAJOR, 4, 4);
     else BGMOE_SPLITK_LAUNCH(BGMOE_W_ROW_MAJOR, 4, 4);
   } else if (g_skinny_gemm_stages == 3) {

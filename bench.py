@@ -107,7 +107,7 @@ def parse():
     ap.add_argument("--tall-min-rows", type=int, default=0,
                     help="decode: groups with more rows than this run as 64-row stage-1 items of the weight-streaming "
                          "kernel (bgmoe_set_skinny_tall_min_rows; 0 = off, the default)")
-    ap.add_argument("--gemm-stages", type=int, default=2, choices=[2, 3, 4],
+    ap.add_argument("--gemm-stages", type=int, default=2, choices=[2, 3, 4, 6],
                     help="decode: prefetch depth of the weight-streaming down projection "
                          "(bgmoe_set_skinny_gemm_stages; 2 = the default)")
     ap.add_argument("--s1-stages", type=int, default=3, choices=[3, 4],

@@ -519,8 +519,8 @@ int bgmoe_set_skinny_tall_min_rows(int rows);
 
 /* Prefetch depth of the plain weight-streaming grouped GEMM, the down projection of a decode step (process-wide,
  * opt-in; no counterpart in the reference).  stages = 2 (the default): an item loads one K-block ahead of the one it
- * computes; 3 or 4: two or three ahead, i.e. two or three times the weight bytes in flight per block (the kernel keeps
- * three blocks per CU with 3 stages, two with 4).  Every output element is computed by the same chain of operations
+ * computes; 3, 4 or 6: two, three or five ahead, i.e. as many times the weight bytes in flight per block (the kernel
+ * keeps three blocks per CU with 3 stages, two with 4 or 6; bgmoe_fp8_dense_gemm takes 6 as 4).  Every output element is computed by the same chain of operations
  * whatever the depth: the results are the same bits.  The block-split form of bgmoe_fp8_dense_gemm follows the switch
  * (its 128-row chunks take three stages at most).  Fused stage 1 is not affected (its three stages fill the register file).  Returns BGMOE_OK or
  * BGMOE_ERR_ARG. */

@@ -103,9 +103,9 @@ def test_tuning_switches_check_their_arguments():
         assert h.bgmoe_set_skinny_tall_min_rows(bad) != 0 and b"at least 32" in h.bgmoe_last_error()
     for good in (32, 64, 200, 0):
         assert h.bgmoe_set_skinny_tall_min_rows(good) == 0
-    for bad in (-1, 0, 1, 5):
-        assert h.bgmoe_set_skinny_gemm_stages(bad) != 0 and b"2, 3 or 4" in h.bgmoe_last_error()
-    for good in (3, 4, 2):
+    for bad in (-1, 0, 1, 5, 7):
+        assert h.bgmoe_set_skinny_gemm_stages(bad) != 0 and b"2, 3, 4 or 6" in h.bgmoe_last_error()
+    for good in (3, 4, 6, 2):
         assert h.bgmoe_set_skinny_gemm_stages(good) == 0
     for bad in (0, 2, 5):
         assert h.bgmoe_set_skinny_s1_stages(bad) != 0 and b"3 or 4" in h.bgmoe_last_error()

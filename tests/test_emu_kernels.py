@@ -501,7 +501,7 @@ def streaming_knobs(h):
 @pytest.mark.parametrize("layout", [0, 1], ids=["row_major", "tile_major"])
 @pytest.mark.parametrize("k", [128, 256, 384, 640, 1152])
 def test_plain_streaming_gemm_at_every_prefetch_depth(h, streaming_knobs, k, layout):
-    """The down projection's kernel with two (a GPU has run it), three and four prefetch stages; 1 to 9 K-blocks, so
+    """The down projection's kernel with two (a GPU has run it), three, four and six prefetch stages; 1 to 9 K-blocks, so
     shorter than, equal to and longer than every ring.  Loads land at once, or as late as the kernel's hand-placed
     waits allow with every global load of the item counted the way the hardware counts them (the deeper rings wait
     for a different count than the proven one); three wave schedules.  One set of bits throughout."""
@@ -511,7 +511,7 @@ def test_plain_streaming_gemm_at_every_prefetch_depth(h, streaming_knobs, k, lay
     ref = og.grouped_gemm_fp8(xq, xs, ws[0][0], ws[0][1], counts, cu, to_bf16=False)
     got = bf16_bits_to_f32(want)
     assert og.rel_frobenius(got[live], ref[live]) < 3e-3 and np.all(got[~live] == 7.0)
-    for stages in (2, 3, 4):
+    for stages in (2, 3, 4, 6):
         ok(h, h.bgmoe_set_skinny_gemm_stages(stages))
         for mode, schedule in ((0, 1), (2, 0), (2, 2)):
             h.emu_set_async_mode(mode)
@@ -520,7 +520,7 @@ def test_plain_streaming_gemm_at_every_prefetch_depth(h, streaming_knobs, k, lay
             assert np.array_equal(out, want), f"{stages} stages, load model {mode}, schedule {schedule}"
 
 
-@pytest.mark.parametrize("stages,slack", [(2, 16), (3, 16), (4, 16)])
+@pytest.mark.parametrize("stages,slack", [(2, 16), (3, 16), (4, 16), (6, 24)])
 def test_counted_load_model_catches_a_wait_that_is_too_lenient(h, streaming_knobs, stages, slack):
     """The negative control of the test above: the same kernels with every hand-placed wait loosened by `slack`
     loads (in the emulator, not in the source) compute on token bytes that have not landed, and the result shows it."""

@@ -46,7 +46,7 @@ def test_deeper_rings_give_the_same_bits(dev, counts, n, k, layout):
 
     want = run()
     try:
-        for stages in (3, 4):
+        for stages in (3, 4, 6):
             check(lib().bgmoe_set_skinny_gemm_stages(stages))
             assert torch.equal(run(), want), f"output differs with {stages} prefetch stages"
     finally:
