@@ -541,11 +541,11 @@ def test_streaming_kernels_with_loads_as_late_as_their_waits_allow(h, streaming_
     """Stage 1 (32-row and tall items) and the MXFP4 kernel (both shapes), whose hand-placed waits count their
     ordinary weight loads as well: every global load of an item takes its place in the lane's queue, a token load
     lands only when a wait leaves it no other choice.  Same bits as with loads that land at once."""
-    n, k = 256, 1152
+    n, k = 256, 640
     counts, cu, m, xq, xs, ws, live = _problem(91, (1, 31, 33, 64, 100), n, k, nmat=2)
     want = run_s1(h, counts, cu, m, xq, xs, ws[0], ws[1], n, k, layout)
-    mxc, mxcu, mxm, x, x16, mws, mlive = _mx_problem(92, (17, 33, 70), n, 1664)
-    mwant = run_mx(h, mxc, mxcu, mxm, x16, mws, n, 1664, layout)
+    mxc, mxcu, mxm, x, x16, mws, mlive = _mx_problem(92, (17, 33, 70), n, 1152)
+    mwant = run_mx(h, mxc, mxcu, mxm, x16, mws, n, 1152, layout)
     for schedule in (0, 2):
         h.emu_set_async_mode(2)
         h.emu_set_schedule(schedule)
@@ -556,7 +556,7 @@ def test_streaming_kernels_with_loads_as_late_as_their_waits_allow(h, streaming_
                 assert np.array_equal(a, b), f"stage 1, tall_min {tall_min}, schedule {schedule}"
         for variant in (0, 1, 2, 3):
             ok(h, h.bgmoe_set_mxfp4_variant(variant))
-            got = run_mx(h, mxc, mxcu, mxm, x16, mws, n, 1664, layout)
+            got = run_mx(h, mxc, mxcu, mxm, x16, mws, n, 1152, layout)
             assert np.array_equal(got[0], mwant[0]) and np.array_equal(got[1], mwant[1]), f"MXFP4 shape {variant}"
 
 
