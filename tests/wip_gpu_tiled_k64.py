@@ -119,7 +119,8 @@ def test_k64_variant_against_the_k128_kernel_and_placement(dev):
     finally:
         check(lib().bgmoe_set_tiled_variant(0))
         check(lib().bgmoe_set_skinny_max_rows(256))
-    assert np.array_equal(outs[1], outs[2]), "the two epilogues of the K = 64 kernel store the same bits"
+    # (live rows only: the op allocates its output, rows outside every group hold whatever the allocation held)
+    assert np.array_equal(outs[1][live], outs[2][live]), "the two epilogues of the K = 64 kernel store the same bits"
     a, b = outs[0][live], outs[1][live]
     assert og.rel_frobenius(b, a) < 2e-3
     assert np.abs(a - b).max() <= 2.0 ** -6 * np.abs(a).max() + 1e-6
