@@ -391,3 +391,18 @@ def test_build_gate_rejects_flat_memory_instructions(tmp_path):
     with pytest.raises(RuntimeError, match="flat_store_dwordx2"):
         run("\tglobal_load_dwordx4 v[0:3], v[4:5], off\n\tflat_store_dwordx2 v[0:1], v[2:3]\n")
     assert not (tmp_path / "k.o").exists()
+
+
+def test_isa_audit_reads_rings_and_flat_instructions():
+    """The assembly reader behind `python -m batchgen_amd.isa_audit`: an innermost loop with barriers and matrix
+    instructions is a ring whose waits are listed in order; an enclosing loop is not reported again; flat memory
+    instructions are named."""
+    from batchgen_amd.isa_audit import audit
+    step = "\ts_waitcnt vmcnt(4)\n\ts_barrier\n\tglobal_load_dwordx4 v[0:3], v[4:5], off\n" + \
+           "\ts_waitcnt vmcnt(10)\n" + "\tv_mfma_f32_16x16x128_f8f6f4 a[0:3], v[0:7], v[8:15], a[0:3]\n" * 4
+    asm = ("_Z6kernelv: ; @_Z6kernelv\n.LBB0_1:\n\tflat_store_dwordx2 v[0:1], v[2:3]\n.LBB0_2:\n" + step * 2 +
+           "\ts_cbranch_scc1 .LBB0_2\n\ts_waitcnt vmcnt(0)\n\ts_cbranch_vccnz .LBB0_1\n\ts_endpgm\n")
+    (rec,) = audit(asm)
+    assert rec["kernel"] == "_Z6kernelv" and rec["flat"] == ["flat_store_dwordx2"]
+    (ring,) = rec["rings"]
+    assert ring["barriers"] == 2 and ring["mfma"] == 8 and ring["waits"] == [4, 10, 4, 10]
